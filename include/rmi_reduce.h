@@ -1,0 +1,234 @@
+/*
+ * rmi_reduce.h — C ABI of the MI355X (gfx950) dense-reduction library.
+ *
+ * Plain C: pointers, sizes and POD descriptors only.  Every entry point is
+ * stream-ordered, never synchronises the stream, never allocates device
+ * memory, never throws, and returns an rmi_status code.  Device pointers are
+ * ordinary HIP device addresses; `stream` is a hipStream_t passed as void*
+ * (NULL = the null stream).
+ *
+ * Each declaration names the interface of NVIDIA/raft (paths relative to
+ * cpp/include/raft) that it stands in for.  The reference has no FFI layer of
+ * its own for this path: its boundary is the header-template API, and the C++
+ * headers shipped beside this library keep those templates and lower them to
+ * the calls below.
+ */
+#ifndef RMI_REDUCE_H_
+#define RMI_REDUCE_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define RMI_ABI_VERSION 1
+
+#if defined(__GNUC__) || defined(__clang__)
+#define RMI_API __attribute__((visibility("default")))
+#else
+#define RMI_API
+#endif
+
+/* ---- status ----------------------------------------------------------- */
+typedef enum rmi_status {
+  RMI_OK                 = 0,
+  RMI_ERR_NULL           = 1, /* a required pointer is NULL                       */
+  RMI_ERR_BAD_ENUM       = 2, /* an enum field holds an unknown value             */
+  RMI_ERR_BAD_SHAPE      = 3, /* negative extent, or extent too large             */
+  RMI_ERR_UNSUPPORTED    = 4, /* dtype / functor combination has no kernel        */
+  RMI_ERR_WORKSPACE      = 5, /* workspace missing, too small or misaligned       */
+  RMI_ERR_ALIGNMENT      = 6, /* in/out pointer not aligned to its element size   */
+  RMI_ERR_LAUNCH         = 7, /* HIP reported an error at launch                  */
+  RMI_ERR_NO_DEVICE      = 8  /* no usable gfx950 device / code object            */
+} rmi_status;
+
+/* ---- element types ---------------------------------------------------- */
+/* KVP types are raft::KeyValuePair<Key,Value> (core/kvp.hpp:20-62): key
+ * first, then value, natural alignment: {i32,f32} = 8 B, {i32,f64} = 16 B
+ * (4 B padding after the key), {i64,f32} = 16 B (4 B tail padding),
+ * {i64,f64} = 16 B. */
+typedef enum rmi_dtype {
+  RMI_I8 = 0,
+  RMI_U8 = 1,
+  RMI_I32 = 2,
+  RMI_I64 = 3,
+  RMI_F16 = 4,
+  RMI_BF16 = 5,
+  RMI_F32 = 6,
+  RMI_F64 = 7,
+  RMI_KVP_I32_F32 = 8,
+  RMI_KVP_I32_F64 = 9,
+  RMI_KVP_I64_F32 = 10,
+  RMI_KVP_I64_F64 = 11,
+  RMI_DTYPE_COUNT_ = 12
+} rmi_dtype;
+
+/* ---- layout / axis ---------------------------------------------------- */
+/* raft::row_major / raft::col_major (core/mdspan_types.hpp:14-37) */
+typedef enum rmi_layout { RMI_ROW_MAJOR = 0, RMI_COL_MAJOR = 1 } rmi_layout;
+/* raft::Apply (linalg/linalg_types.hpp): ALONG_ROWS gives one output per row,
+ * ALONG_COLUMNS one output per column. */
+typedef enum rmi_apply { RMI_ALONG_ROWS = 0, RMI_ALONG_COLUMNS = 1 } rmi_apply;
+
+/* ---- functor vocabulary (core/operators.hpp:27-203,253-370) ------------ */
+/* main_op(value, index_along_reduced_axis) */
+typedef enum rmi_main_op {
+  RMI_MAIN_IDENTITY = 0, /* identity_op, cast_op<Out>                      */
+  RMI_MAIN_SQ       = 1, /* sq_op                                          */
+  RMI_MAIN_ABS      = 2, /* abs_op                                         */
+  RMI_MAIN_NZ       = 3, /* nz_op: x != 0 ? 1 : 0                          */
+  RMI_MAIN_KVP      = 4  /* (value, idx) -> KeyValuePair{idx, value}; the  */
+                         /* only main_op allowed with ARGMIN / ARGMAX      */
+} rmi_main_op;
+
+typedef enum rmi_reduce_op {
+  RMI_RED_ADD    = 0, /* add_op (compensated: linalg/reduce.cuh:25-27)     */
+  RMI_RED_MAX    = 1, /* max_op (NaN-ignoring, core/math.hpp:375-397)      */
+  RMI_RED_MIN    = 2, /* min_op                                            */
+  RMI_RED_ARGMAX = 3, /* argmax_op (core/operators.hpp:196-203)            */
+  RMI_RED_ARGMIN = 4  /* argmin_op (core/operators.hpp:187-194)            */
+} rmi_reduce_op;
+
+/* final_op(acc) applied once per output, in the output's arithmetic type
+ * (f32 for f16/bf16/f32 outputs, f64 for f64, i64 for integers). */
+typedef enum rmi_final_op {
+  RMI_FIN_IDENTITY  = 0,
+  RMI_FIN_SQRT      = 1, /* sqrt_op                                         */
+  RMI_FIN_ABS       = 2, /* abs_op                                          */
+  RMI_FIN_SQ        = 3, /* sq_op                                           */
+  RMI_FIN_MUL_CONST = 4, /* mul_const_op<Out>(final_scalar)                 */
+  RMI_FIN_DIV_CONST = 5, /* div_const_op<Out>(final_scalar)                 */
+  RMI_FIN_ADD_CONST = 6, /* add_const_op<Out>(final_scalar)                 */
+  RMI_FIN_SUB_CONST = 7, /* sub_const_op<Out>(final_scalar)                 */
+  /* acc, aux[k] -> |acc*final_scalar - aux[k]^2*final_scalar2|, and its
+   * square root: the epilogue of stats::vars / stats::stddev
+   * (stats/detail/stddev.cuh:46-59,91-101), fused into the reduction. */
+  RMI_FIN_VAR_FROM_SUMSQ    = 8,
+  RMI_FIN_STDDEV_FROM_SUMSQ = 9,
+  RMI_FIN_KEY = 10 /* key_op: KVP accumulator -> its key (integer output);
+                      matrix::argmax/argmin write the key only
+                      (matrix/detail/math.cuh:310)                         */
+} rmi_final_op;
+
+/* ---- scalar carrier for `init` ---------------------------------------- */
+typedef struct rmi_scalar {
+  double  f;   /* floating outputs: init value; KVP outputs: init.value      */
+  int64_t i;   /* integer outputs: init value;  KVP outputs: init.key        */
+} rmi_scalar;
+
+/* ---- the reduction descriptor ------------------------------------------
+ * Stands in for the template arguments and value arguments of
+ *   raft::linalg::reduce            (linalg/reduce.cuh:55-76,140-180)
+ *   raft::linalg::coalescedReduction (linalg/coalesced_reduction.cuh:55-70)
+ *   raft::linalg::stridedReduction   (linalg/strided_reduction.cuh:57-78)
+ * Semantics, for every output k and r running over the reduced axis:
+ *   acc_k   = reduce_op-fold over r of main_op(in[k,r], r)
+ *   acc_k   = reduce_op(init, acc_k)                  (init applied once)
+ *   if inplace: acc_k = reduce_op(out_old[k], acc_k)
+ *   out[k]  = final_op(acc_k)
+ */
+typedef struct rmi_reduce_desc {
+  int32_t in_dtype;    /* rmi_dtype of the matrix                             */
+  int32_t out_dtype;   /* rmi_dtype of the output vector                      */
+  int32_t layout;      /* rmi_layout                                          */
+  int32_t apply;       /* rmi_apply                                           */
+  int64_t n_rows;      /* data.extent(0)                                      */
+  int64_t n_cols;      /* data.extent(1)                                      */
+  int32_t main_op;     /* rmi_main_op                                         */
+  int32_t reduce_op;   /* rmi_reduce_op                                       */
+  int32_t final_op;    /* rmi_final_op                                        */
+  int32_t inplace;     /* 0 / 1                                               */
+  rmi_scalar init;     /* must be reduce_op's neutral element                 */
+  double final_scalar; /* constant of *_CONST; `ratio` of VAR/STDDEV          */
+  double final_scalar2;/* `ratio_mean` of VAR/STDDEV                          */
+  const void* final_aux; /* device vector (out_dtype, one per output) read by
+                            VAR/STDDEV (the mean); NULL otherwise            */
+  int32_t plan_hint;   /* rmi_plan_kind to force, or 0 = choose by shape      */
+  int32_t reserved;    /* must be 0                                           */
+} rmi_reduce_desc;
+
+/* ---- launch plans ------------------------------------------------------ */
+typedef enum rmi_plan_kind {
+  RMI_PLAN_AUTO       = 0,
+  RMI_PLAN_ROW_LANES  = 1, /* several whole rows per lane-load (rows <= 8 B..16 B)  */
+  RMI_PLAN_ROW_WAVE   = 2, /* 1..64 lanes of one wavefront per row                  */
+  RMI_PLAN_ROW_BLOCK  = 3, /* one 256-thread block per row, LDS tree                */
+  RMI_PLAN_ROW_SPLIT  = 4, /* several blocks per row + second pass over partials    */
+  RMI_PLAN_COL_TILE   = 5, /* column reduction: column-contiguous lanes, row ranges
+                              per block, LDS combine, second pass over partials    */
+  RMI_PLAN_EMPTY      = 6  /* nothing to read: outputs get final_op(init) only      */
+} rmi_plan_kind;
+
+typedef struct rmi_plan {
+  int32_t kind;            /* rmi_plan_kind actually chosen                   */
+  int32_t vec_bytes;       /* bytes per lane-load (16, or the element size)   */
+  int32_t lanes_per_row;   /* ROW_WAVE: lanes that share one row (1..64)      */
+  int32_t blocks_per_out;  /* ROW_SPLIT / COL_TILE: partials per output       */
+  int32_t block_threads;   /* threads per workgroup                           */
+  int32_t passes;          /* kernel launches (1 or 2)                        */
+  int64_t grid_blocks;     /* workgroups of the first launch                  */
+  int64_t n_outputs;       /* outputs produced                                */
+  int64_t reduce_len;      /* elements folded into each output                */
+  size_t  workspace_bytes; /* device workspace the plan needs (0 if none)     */
+} rmi_plan;
+
+/* ---- entry points ------------------------------------------------------ */
+
+/* ABI version of the loaded library (== RMI_ABI_VERSION it was built with). */
+RMI_API int rmi_abi_version(void);
+
+/* Human-readable text for a status code; never NULL. */
+RMI_API const char* rmi_status_string(int status);
+
+/* sizeof one element of an rmi_dtype, 0 for an unknown value. */
+RMI_API size_t rmi_dtype_size(int dtype);
+
+/* Plan chosen for `desc` on the current device (CU count is queried once and
+ * cached; with no device visible a 256-CU MI355X is assumed, so this call
+ * works on a host without a GPU).  Replaces the hard-coded Thin/Medium/Thick
+ * heuristics of linalg/detail/coalesced_reduction-inl.cuh:640-670 and the
+ * launch shapes of linalg/detail/strided_reduction.cuh:148-188. */
+RMI_API int rmi_plan_query(const rmi_reduce_desc* desc, rmi_plan* plan);
+
+/* Bytes of device workspace rmi_reduce needs for `desc` (0 for single-pass
+ * plans).  Replaces the internal rmm::device_uvector of
+ * linalg/detail/coalesced_reduction-inl.cuh:560. */
+RMI_API size_t rmi_reduce_workspace_bytes(const rmi_reduce_desc* desc);
+
+/* The reduction itself: replaces detail::reduce (linalg/detail/reduce.cuh:25-49),
+ * detail::coalescedReduction (linalg/detail/coalesced_reduction-inl.cuh:640-670)
+ * and detail::stridedReduction (linalg/detail/strided_reduction.cuh:129-196).
+ * `in`: n_rows*n_cols elements, contiguous in `layout`.  `out`: one element per
+ * output.  `workspace`: at least rmi_reduce_workspace_bytes(desc) bytes, 16-byte
+ * aligned, may be NULL when that is 0; its contents need no initialisation and
+ * are undefined afterwards.  Calls that share a workspace must be ordered on
+ * one stream. */
+RMI_API int rmi_reduce(const rmi_reduce_desc* desc,
+               const void* in,
+               void* out,
+               void* workspace,
+               size_t workspace_bytes,
+               void* stream);
+
+/* Whole-array map + reduce to one scalar: replaces detail::mapThenReduceImpl
+ * (linalg/detail/map_then_reduce.cuh:72-95) behind mapThenSumReduce /
+ * mapThenReduce / mapReduce / map_reduce (linalg/map_then_reduce.cuh:37-80,
+ * linalg/map_reduce.cuh:37-103).  *out = reduce_op(neutral, fold of
+ * main_op(in[i], i)), i < len.  Deterministic (no atomics).  Uses the
+ * descriptor fields in_dtype, out_dtype, main_op, reduce_op, final_op, init
+ * (= neutral), final_scalar; n_rows/n_cols/layout/apply are ignored. */
+RMI_API size_t rmi_map_reduce_workspace_bytes(const rmi_reduce_desc* desc, int64_t len);
+RMI_API int rmi_map_reduce(const rmi_reduce_desc* desc,
+                   int64_t len,
+                   const void* in,
+                   void* out,
+                   void* workspace,
+                   size_t workspace_bytes,
+                   void* stream);
+
+#ifdef __cplusplus
+} /* extern "C" */
+#endif
+#endif /* RMI_REDUCE_H_ */

@@ -1,0 +1,192 @@
+// C ABI of the reduction library (declared in include/rmi_reduce.h):
+// validation, plan selection, policy lookup, launch.
+#include <atomic>
+
+#include "rmi_launch.hpp"
+
+namespace rmi {
+namespace {
+
+// CU count of the current device, queried once per process.  Without a
+// visible device the MI355X figure is assumed so that planning works on a
+// build host.
+int cu_count()
+{
+  static std::atomic<int> cached{0};
+  int n = cached.load(std::memory_order_relaxed);
+  if (n > 0) return n;
+  int dev = 0;
+  hipDeviceProp_t prop;
+  if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess &&
+      prop.multiProcessorCount > 0) {
+    n = prop.multiProcessorCount;
+  } else {
+    (void)hipGetLastError();
+    n = 256;
+  }
+  cached.store(n, std::memory_order_relaxed);
+  return n;
+}
+
+run_fn lookup(const PolicyKey& k)
+{
+  switch (k.in_dtype) {
+    case RMI_I8: return lookup_i8(k);
+    case RMI_U8: return lookup_u8(k);
+    case RMI_I32: return lookup_i32(k);
+    case RMI_I64: return lookup_i64(k);
+    case RMI_F16: return lookup_f16(k);
+    case RMI_BF16: return lookup_bf16(k);
+    case RMI_F32: return lookup_f32(k);
+    case RMI_F64: return lookup_f64(k);
+    default: return nullptr;
+  }
+}
+
+bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
+
+int plan_for(const rmi_reduce_desc* desc, bool aligned16, PlanX& pl, PolicyKey& key)
+{
+  if (desc == nullptr) return RMI_ERR_NULL;
+  int acc_bytes = 8;
+  int rc        = classify(*desc, key, acc_bytes);
+  if (rc != RMI_OK) return rc;
+  if (lookup(key) == nullptr) return RMI_ERR_UNSUPPORTED;
+  return make_plan(*desc, key, acc_bytes, aligned16, cu_count(), pl);
+}
+
+int reduce_impl(const rmi_reduce_desc& d,
+                const void* in,
+                void* out,
+                void* ws,
+                size_t ws_bytes,
+                void* stream)
+{
+  PlanX pl;
+  PolicyKey key;
+  int rc = plan_for(&d, aligned(in, 16), pl, key);
+  if (rc != RMI_OK) return rc;
+  if (pl.n_out == 0) return RMI_OK;
+  if (out == nullptr) return RMI_ERR_NULL;
+  if (pl.len > 0 && in == nullptr) return RMI_ERR_NULL;
+  if (!aligned(in, dtype_size(d.in_dtype))) return RMI_ERR_ALIGNMENT;
+  const int out_es = dtype_size(d.out_dtype);
+  // a KVP with a 4-byte key and value is 4-byte aligned by the C rules
+  const size_t out_align = d.out_dtype == RMI_KVP_I32_F32 ? 4 : (out_es > 8 ? 8 : out_es);
+  if (!aligned(out, out_align)) return RMI_ERR_ALIGNMENT;
+  if (d.final_aux != nullptr && !aligned(d.final_aux, out_align)) return RMI_ERR_ALIGNMENT;
+  if (pl.ws_bytes > 0) {
+    if (ws == nullptr || ws_bytes < pl.ws_bytes) return RMI_ERR_WORKSPACE;
+    if (!aligned(ws, 16)) return RMI_ERR_WORKSPACE;
+  }
+
+  Problem pr{};
+  pr.in            = in;
+  pr.ws            = ws;
+  pr.epi.out       = out;
+  pr.epi.aux       = d.final_aux;
+  pr.epi.init_f    = d.init.f;
+  pr.epi.init_i    = d.init.i;
+  pr.epi.s1        = d.final_scalar;
+  pr.epi.s2        = d.final_scalar2;
+  pr.epi.out_dtype = d.out_dtype;
+  pr.epi.final_op  = d.final_op;
+  pr.epi.inplace   = d.inplace ? 1 : 0;
+  return lookup(key)(pl, pr, static_cast<hipStream_t>(stream));
+}
+
+// map_reduce is a one-row reduction over the contiguous dimension.
+rmi_reduce_desc as_single_row(const rmi_reduce_desc& d, int64_t len)
+{
+  rmi_reduce_desc r = d;
+  r.layout          = RMI_ROW_MAJOR;
+  r.apply           = RMI_ALONG_ROWS;
+  r.n_rows          = 1;
+  r.n_cols          = len;
+  r.inplace         = 0;
+  r.final_aux       = nullptr;
+  if (r.final_op == RMI_FIN_VAR_FROM_SUMSQ || r.final_op == RMI_FIN_STDDEV_FROM_SUMSQ)
+    r.final_op = -1;  // rejected by classify
+  return r;
+}
+
+}  // namespace
+}  // namespace rmi
+
+extern "C" {
+
+int rmi_abi_version(void) { return RMI_ABI_VERSION; }
+
+const char* rmi_status_string(int status)
+{
+  switch (status) {
+    case RMI_OK: return "ok";
+    case RMI_ERR_NULL: return "a required pointer is null";
+    case RMI_ERR_BAD_ENUM: return "descriptor holds an unknown enum value";
+    case RMI_ERR_BAD_SHAPE: return "extent is negative or too large";
+    case RMI_ERR_UNSUPPORTED: return "no kernel for this dtype / functor combination";
+    case RMI_ERR_WORKSPACE: return "workspace is missing, too small or misaligned";
+    case RMI_ERR_ALIGNMENT: return "pointer is not aligned to its element type";
+    case RMI_ERR_LAUNCH: return "HIP reported an error at kernel launch";
+    case RMI_ERR_NO_DEVICE: return "no usable gfx950 device";
+    default: return "unknown status";
+  }
+}
+
+size_t rmi_dtype_size(int dtype) { return (size_t)rmi::dtype_size(dtype); }
+
+int rmi_plan_query(const rmi_reduce_desc* desc, rmi_plan* plan)
+{
+  if (plan == nullptr) return RMI_ERR_NULL;
+  rmi::PlanX pl;
+  rmi::PolicyKey key;
+  const int rc = rmi::plan_for(desc, true, pl, key);
+  if (rc != RMI_OK) return rc;
+  rmi::export_plan(pl, *plan);
+  return RMI_OK;
+}
+
+size_t rmi_reduce_workspace_bytes(const rmi_reduce_desc* desc)
+{
+  // Whether the 16-byte-vector or the element-wise variant runs depends on the
+  // input pointer's alignment, known only at rmi_reduce time: size for both.
+  rmi::PlanX a, u;
+  rmi::PolicyKey key;
+  if (rmi::plan_for(desc, true, a, key) != RMI_OK) return 0;
+  if (rmi::plan_for(desc, false, u, key) != RMI_OK) return a.ws_bytes;
+  return a.ws_bytes > u.ws_bytes ? a.ws_bytes : u.ws_bytes;
+}
+
+int rmi_reduce(const rmi_reduce_desc* desc,
+               const void* in,
+               void* out,
+               void* workspace,
+               size_t workspace_bytes,
+               void* stream)
+{
+  if (desc == nullptr) return RMI_ERR_NULL;
+  return rmi::reduce_impl(*desc, in, out, workspace, workspace_bytes, stream);
+}
+
+size_t rmi_map_reduce_workspace_bytes(const rmi_reduce_desc* desc, int64_t len)
+{
+  if (desc == nullptr || len < 0) return 0;
+  const rmi_reduce_desc r = rmi::as_single_row(*desc, len);
+  return rmi_reduce_workspace_bytes(&r);
+}
+
+int rmi_map_reduce(const rmi_reduce_desc* desc,
+                   int64_t len,
+                   const void* in,
+                   void* out,
+                   void* workspace,
+                   size_t workspace_bytes,
+                   void* stream)
+{
+  if (desc == nullptr) return RMI_ERR_NULL;
+  if (len < 0) return RMI_ERR_BAD_SHAPE;
+  const rmi_reduce_desc r = rmi::as_single_row(*desc, len);
+  return rmi::reduce_impl(r, in, out, workspace, workspace_bytes, stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,414 @@
+// The gfx950 reduction kernels, templated on an accumulator policy
+// (rmi_device.hpp).  VEC16 = true: rows are read as 16-byte vectors
+// (global_load_dwordx4 per lane); false: one element per lane-load, used when
+// a row's byte length or the base pointer is not a multiple of 16.
+//
+//   row_lanes_kernel  K whole rows inside one 16-byte vector: no cross-lane step
+//   row_short_kernel  rows of at most G<=64 vectors: one vector per lane, G lanes
+//                     per row, 4 row-tiles in flight per wave
+//   row_wave_kernel   G<=64 lanes of one wave sweep a row, 4 loads in flight
+//   row_block_kernel  64*W threads per row chunk, B chunks per row; B == 1
+//                     writes outputs, B > 1 writes partials
+//   col_kernel        reduction along the strided dimension
+//   fold_kernel       second pass: partials[n_out][B] -> outputs
+#pragma once
+
+#include "rmi_device.hpp"
+
+namespace rmi {
+
+constexpr int kBlock = 256;  // threads per workgroup of every first-pass kernel
+constexpr int kUnroll = 4;   // independent 16-byte loads in flight per lane
+
+struct RowArgs {
+  const void* in;
+  void* partial;   // [n_out][B] accumulators, ROW_SPLIT only
+  i64 n_out;       // rows
+  i64 len;         // elements per row
+  i64 nvec;        // lane-loads per row: len/VEC (VEC16) or len (scalar)
+  i64 chunk;       // lane-loads per block chunk (row_block_kernel)
+  int G;           // lanes per row (row_short / row_wave)
+  int logG;
+  int B;           // chunks per row (row_block_kernel)
+  Epilogue epi;
+};
+
+struct ColArgs {
+  const void* in;
+  void* partial;      // [n_out][B] accumulators when B > 1
+  i64 n_out;          // D: length of the contiguous dimension
+  i64 len;            // N: number of strided rows folded
+  i64 nvec;           // lane-loads per row: D/VEC (VEC16) or D (scalar)
+  i64 rows_per_block; // rows owned by one blockIdx.y
+  int TX;             // lanes along the contiguous dimension (power of two <= 64)
+  int logTX;
+  int B;              // gridDim.y
+  Epilogue epi;
+};
+
+struct FoldArgs {
+  const void* partial;  // [n_out][B]
+  i64 n_out;
+  int B;
+  int LB;  // lanes per output (power of two <= 64)
+  int logLB;
+  Epilogue epi;
+};
+
+template <class P, bool VEC16>
+struct Loader {
+  using in_t                = typename P::in_t;
+  static constexpr int STEP = VEC16 ? P::VEC : 1;  // elements per lane-load
+};
+
+// A lane-load held in registers between issue and use.
+template <class P, bool VEC16>
+struct Held {
+  using in_t = typename P::in_t;
+  using type = std::conditional_t<VEC16, u32x4, typename In<in_t>::nat>;
+  static __device__ __forceinline__ type load(const void* in, i64 at)
+  {
+    if constexpr (VEC16) {
+      return load16(static_cast<const u32x4*>(in) + at);
+    } else {
+      return In<in_t>::ld(static_cast<const in_t*>(in) + at);
+    }
+  }
+  static __device__ __forceinline__ void push(typename P::acc_t& a, const type& x, i64 idx0)
+  {
+    if constexpr (VEC16) {
+      P::push_vec(a, x, idx0);
+    } else {
+      P::push(a, x, idx0);
+    }
+  }
+};
+
+// ---------------------------------------------------------------------------
+// K rows per 16-byte vector (row length VEC/K elements).  Lane-local.
+// ---------------------------------------------------------------------------
+template <class P, int K>
+__global__ __launch_bounds__(kBlock) void row_lanes_kernel(RowArgs a)
+{
+  using in_t      = typename P::in_t;
+  using acc_t     = typename P::acc_t;
+  constexpr int D = P::VEC / K;  // elements per row
+  const i64 nfull = a.n_out / K; // vectors made only of whole, in-range rows
+
+  u32x4 x[kUnroll];
+#pragma unroll
+  for (int u = 0; u < kUnroll; ++u) {
+    // consecutive lanes take consecutive vectors within each unroll slot
+    const i64 v = ((i64)blockIdx.x * kUnroll + u) * kBlock + threadIdx.x;
+    if (v < nfull) x[u] = load16(static_cast<const u32x4*>(a.in) + v);
+  }
+#pragma unroll
+  for (int u = 0; u < kUnroll; ++u) {
+    const i64 v = ((i64)blockIdx.x * kUnroll + u) * kBlock + threadIdx.x;
+    if (v < nfull) {
+      acc_t acc[K];
+      static_for<K>([&](auto r) {
+        acc[r] = P::neutral();
+        static_for<D>([&](auto j) {
+          P::push(acc[r], In<in_t>::template get<r * D + j>(x[u]), (i64)j);
+        });
+      });
+      static_for<K>([&](auto r) { finish<P>(a.epi, v * K + r, acc[r]); });
+    }
+  }
+  // Rows past the last whole vector (fewer than K of them): one lane each.
+  if (blockIdx.x == 0 && threadIdx.x < (unsigned)(a.n_out - nfull * K)) {
+    const i64 row = nfull * K + threadIdx.x;
+    acc_t acc     = P::neutral();
+    for (int j = 0; j < D; ++j)
+      P::push(acc, In<in_t>::ld(static_cast<const in_t*>(a.in) + row * D + j), (i64)j);
+    finish<P>(a.epi, row, acc);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Short rows: nvec <= G, one lane-load per lane per row, kUnroll tiles of
+// 64/G rows in flight per wave.
+// ---------------------------------------------------------------------------
+template <class P, bool VEC16>
+__global__ __launch_bounds__(kBlock) void row_short_kernel(RowArgs a)
+{
+  using acc_t     = typename P::acc_t;
+  using H         = Held<P, VEC16>;
+  constexpr int S = Loader<P, VEC16>::STEP;
+  const int lane  = threadIdx.x & (kWave - 1);
+  const i64 wid   = (i64)blockIdx.x * (kBlock / kWave) + (threadIdx.x >> 6);
+  const int G     = a.G;
+  const int R     = kWave >> a.logG;
+  const int c     = lane & (G - 1);
+  const int g     = lane >> a.logG;
+  const bool incol = c < a.nvec;
+
+  typename H::type x[kUnroll];
+  i64 row[kUnroll];
+#pragma unroll
+  for (int t = 0; t < kUnroll; ++t) {
+    row[t] = (wid * kUnroll + t) * R + g;
+    if (incol && row[t] < a.n_out) x[t] = H::load(a.in, row[t] * a.nvec + c);
+  }
+  acc_t acc[kUnroll];
+#pragma unroll
+  for (int t = 0; t < kUnroll; ++t) {
+    acc[t] = P::neutral();
+    if (incol && row[t] < a.n_out) H::push(acc[t], x[t], (i64)c * S);
+  }
+#pragma unroll
+  for (int t = 0; t < kUnroll; ++t)
+    group_allreduce<P>(acc[t], G);
+#pragma unroll
+  for (int t = 0; t < kUnroll; ++t) {
+    if (c == 0 && row[t] < a.n_out) finish<P>(a.epi, row[t], acc[t]);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// G lanes of one wave per row, looping over the row with kUnroll loads in
+// flight per lane.
+// ---------------------------------------------------------------------------
+template <class P, bool VEC16>
+__global__ __launch_bounds__(kBlock) void row_wave_kernel(RowArgs a)
+{
+  using acc_t     = typename P::acc_t;
+  using H         = Held<P, VEC16>;
+  constexpr int S = Loader<P, VEC16>::STEP;
+  const int lane  = threadIdx.x & (kWave - 1);
+  const i64 wid   = (i64)blockIdx.x * (kBlock / kWave) + (threadIdx.x >> 6);
+  const int G     = a.G;
+  const int R     = kWave >> a.logG;
+  const int c     = lane & (G - 1);
+  const i64 row   = wid * R + (lane >> a.logG);
+  const i64 nvec  = a.nvec;
+
+  acc_t acc = P::neutral();
+  if (row < a.n_out) {
+    const i64 base = row * nvec;
+    i64 v          = c;
+    for (; v + (kUnroll - 1) * G < nvec; v += kUnroll * G) {
+      typename H::type x[kUnroll];
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u)
+        x[u] = H::load(a.in, base + v + u * G);
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u)
+        H::push(acc, x[u], (v + u * G) * S);
+    }
+    if (v < nvec) {  // fewer than kUnroll lane-loads left for this lane
+      typename H::type x[kUnroll - 1];
+#pragma unroll
+      for (int u = 0; u < kUnroll - 1; ++u)
+        if (v + u * G < nvec) x[u] = H::load(a.in, base + v + u * G);
+#pragma unroll
+      for (int u = 0; u < kUnroll - 1; ++u)
+        if (v + u * G < nvec) H::push(acc, x[u], (v + u * G) * S);
+    }
+  }
+  group_allreduce<P>(acc, G);
+  if (c == 0 && row < a.n_out) finish<P>(a.epi, row, acc);
+}
+
+// ---------------------------------------------------------------------------
+// blockDim.x = 64*W threads per chunk of a row; B chunks per row.
+// ---------------------------------------------------------------------------
+template <class P, bool VEC16>
+__global__ __launch_bounds__(1024) void row_block_kernel(RowArgs a)
+{
+  using acc_t     = typename P::acc_t;
+  using H         = Held<P, VEC16>;
+  constexpr int S = Loader<P, VEC16>::STEP;
+  __shared__ acc_t sm[16];
+
+  const int T    = blockDim.x;
+  const int t    = threadIdx.x;
+  const u32 bid  = blockIdx.x;
+  const u32 urow = bid / (u32)a.B;
+  const int b    = (int)(bid - urow * (u32)a.B);
+  const i64 row  = urow;
+  const i64 v0   = (i64)b * a.chunk;
+  const i64 v1   = (v0 + a.chunk < a.nvec) ? (v0 + a.chunk) : a.nvec;
+  const i64 base = row * a.nvec;
+
+  acc_t acc = P::neutral();
+  i64 v     = v0 + t;
+  for (; v + (kUnroll - 1) * (i64)T < v1; v += (i64)kUnroll * T) {
+    typename H::type x[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u)
+      x[u] = H::load(a.in, base + v + (i64)u * T);
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u)
+      H::push(acc, x[u], (v + (i64)u * T) * S);
+  }
+  if (v < v1) {
+    typename H::type x[kUnroll - 1];
+#pragma unroll
+    for (int u = 0; u < kUnroll - 1; ++u)
+      if (v + (i64)u * T < v1) x[u] = H::load(a.in, base + v + (i64)u * T);
+#pragma unroll
+    for (int u = 0; u < kUnroll - 1; ++u)
+      if (v + (i64)u * T < v1) H::push(acc, x[u], (v + (i64)u * T) * S);
+  }
+
+  wave_allreduce<P>(acc);
+  const int W = T >> 6;
+  if (W > 1) {
+    if ((t & (kWave - 1)) == 0) sm[t >> 6] = acc;
+    __syncthreads();
+    if (t == 0) {
+      for (int w = 1; w < W; ++w)
+        P::merge(acc, sm[w]);
+    }
+  }
+  if (t == 0) {
+    if (a.B == 1) {
+      finish<P>(a.epi, row, acc);
+    } else {
+      static_cast<acc_t*>(a.partial)[row * a.B + b] = acc;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Reduction along the strided dimension of a [len][n_out] row-major array.
+// Thread (tx, ty): tx owns one lane-load wide group of adjacent columns for
+// the whole kernel, ty strides over the rows of this block's row range.
+// ---------------------------------------------------------------------------
+template <class P>
+__device__ __forceinline__ typename P::acc_t bperm_acc(const typename P::acc_t& a, int mask)
+{
+  using acc_t = typename P::acc_t;
+  static_assert(sizeof(acc_t) % 4 == 0, "accumulators are moved word by word");
+  constexpr int NW = sizeof(acc_t) / 4;
+  u32 w[NW];
+  __builtin_memcpy(w, &a, sizeof(acc_t));
+#pragma unroll
+  for (int i = 0; i < NW; ++i)
+    w[i] = (u32)__shfl_xor((int)w[i], mask, kWave);
+  acc_t r;
+  __builtin_memcpy(&r, w, sizeof(acc_t));
+  return r;
+}
+
+template <class P, bool VEC16>
+__global__ __launch_bounds__(kBlock) void col_kernel(ColArgs a)
+{
+  using acc_t     = typename P::acc_t;
+  using in_t      = typename P::in_t;
+  constexpr int S = VEC16 ? P::VEC : 1;
+  constexpr int W = kBlock / kWave;
+  __shared__ acc_t sm[W * kWave * S];
+
+  const int t    = threadIdx.x;
+  const int TX   = a.TX;
+  const int TY   = kBlock >> a.logTX;
+  const int tx   = t & (TX - 1);
+  const int ty   = t >> a.logTX;
+  const i64 cv   = (i64)blockIdx.x * TX + tx;
+  const i64 r0   = (i64)blockIdx.y * a.rows_per_block;
+  const i64 r1   = (r0 + a.rows_per_block < a.len) ? (r0 + a.rows_per_block) : a.len;
+  const bool live = cv < a.nvec;
+
+  acc_t acc[S];
+#pragma unroll
+  for (int j = 0; j < S; ++j)
+    acc[j] = P::neutral();
+
+  if (live) {
+    i64 r = r0 + ty;
+    if constexpr (VEC16) {
+      const u32x4* p = static_cast<const u32x4*>(a.in) + cv;
+      for (; r + (kUnroll - 1) * (i64)TY < r1; r += (i64)kUnroll * TY) {
+        u32x4 x[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u)
+          x[u] = load16(p + (r + (i64)u * TY) * a.nvec);
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u)
+          P::push_cols(acc, x[u], r + (i64)u * TY);
+      }
+      for (; r < r1; r += TY)
+        P::push_cols(acc, load16(p + r * a.nvec), r);
+    } else {
+      const in_t* p = static_cast<const in_t*>(a.in) + cv;
+      for (; r + (kUnroll - 1) * (i64)TY < r1; r += (i64)kUnroll * TY) {
+        typename In<in_t>::nat x[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u)
+          x[u] = In<in_t>::ld(p + (r + (i64)u * TY) * a.nvec);
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u)
+          P::push(acc[0], x[u], r + (i64)u * TY);
+      }
+      for (; r < r1; r += TY)
+        P::push(acc[0], In<in_t>::ld(p + r * a.nvec), r);
+    }
+  }
+
+  // lanes of one wave that share tx sit TX, 2*TX, ... apart
+  for (int m = TX; m < kWave; m <<= 1) {
+#pragma unroll
+    for (int j = 0; j < S; ++j)
+      P::merge(acc[j], bperm_acc<P>(acc[j], m));
+  }
+  // one value per (wave, tx, j) through LDS, folded by the block's first TX threads
+  const int lane = t & (kWave - 1);
+  const int wave = t >> 6;
+  constexpr int NW = W;  // every wave covers its own set of ty
+  if (lane < TX) {
+#pragma unroll
+    for (int j = 0; j < S; ++j)
+      sm[(wave * kWave + lane) * S + j] = acc[j];
+  }
+  __syncthreads();
+  if (t < TX && live) {
+#pragma unroll
+    for (int j = 0; j < S; ++j) {
+      acc_t r = sm[(0 * kWave + t) * S + j];
+      for (int w = 1; w < NW; ++w)
+        P::merge(r, sm[(w * kWave + t) * S + j]);
+      const i64 col = cv * S + j;
+      if (a.B == 1) {
+        finish<P>(a.epi, col, r);
+      } else {
+        static_cast<acc_t*>(a.partial)[col * a.B + blockIdx.y] = r;
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Second pass: LB lanes fold the B partials of one output in a fixed order,
+// then the epilogue.  B == 0 writes final_op(init) (empty reductions).
+// ---------------------------------------------------------------------------
+template <class P>
+__global__ __launch_bounds__(kBlock) void fold_kernel(FoldArgs a)
+{
+  using acc_t    = typename P::acc_t;
+  const i64 gtid = (i64)blockIdx.x * kBlock + threadIdx.x;
+  const i64 o    = gtid >> a.logLB;
+  const int lb   = (int)(gtid & (a.LB - 1));
+  acc_t acc      = P::neutral();
+  if (o < a.n_out) {
+    const acc_t* p = static_cast<const acc_t*>(a.partial) + o * a.B;
+    int b          = lb;
+    for (; b + (kUnroll - 1) * a.LB < a.B; b += kUnroll * a.LB) {
+      acc_t x[kUnroll];
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u)
+        x[u] = p[b + u * a.LB];
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u)
+        P::merge(acc, x[u]);
+    }
+    for (; b < a.B; b += a.LB)
+      P::merge(acc, p[b]);
+  }
+  group_allreduce<P>(acc, a.LB);
+  if (lb == 0 && o < a.n_out) finish<P>(a.epi, o, acc);
+}
+
+}  // namespace rmi

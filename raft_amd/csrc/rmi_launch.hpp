@@ -1,0 +1,224 @@
+// Host-side launch of one planned reduction for one accumulator policy.
+// Every policy instantiates run<P>; a per-input-type translation unit collects
+// them behind a lookup function so the policies compile in parallel.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include "rmi_kernels.hpp"
+#include "rmi_plan.hpp"
+
+namespace rmi {
+
+struct Problem {
+  const void* in;
+  void* ws;
+  Epilogue epi;
+};
+
+using run_fn = int (*)(const PlanX&, const Problem&, hipStream_t);
+
+template <class P>
+int launch_fold(const PlanX& pl, const Problem& pr, int B, hipStream_t st)
+{
+  FoldArgs f{};
+  f.partial = pr.ws;
+  f.n_out   = pl.n_out;
+  f.B       = B;
+  f.LB      = B >= 64 ? 64 : pow2ceil(B < 1 ? 1 : B);
+  f.logLB   = ilog2(f.LB);
+  f.epi     = pr.epi;
+  const int64_t threads = pl.n_out * f.LB;
+  const int64_t grid    = ceildiv(threads, kBlock);
+  if (grid > 0x7fffffffLL) return RMI_ERR_BAD_SHAPE;
+  hipLaunchKernelGGL((fold_kernel<P>), dim3((unsigned)grid), dim3(kBlock), 0, st, f);
+  return RMI_OK;
+}
+
+template <class P, int K>
+int launch_lanes(const PlanX& pl, const RowArgs& a, hipStream_t st)
+{
+  if constexpr (K <= P::VEC) {
+    hipLaunchKernelGGL(
+      (row_lanes_kernel<P, K>), dim3((unsigned)pl.grid_blocks), dim3(kBlock), 0, st, a);
+    return RMI_OK;
+  } else {
+    return RMI_ERR_UNSUPPORTED;
+  }
+}
+
+template <class P>
+int run(const PlanX& pl, const Problem& pr, hipStream_t st)
+{
+  static_assert(kBlock == kPlanBlock && kUnroll == kPlanUnroll,
+                "plan selector and kernels must agree on block size and unroll");
+  int rc = RMI_OK;
+  switch (pl.kind) {
+    case RMI_PLAN_EMPTY:
+      if (pl.n_out > 0) rc = launch_fold<P>(pl, pr, 0, st);
+      break;
+    case RMI_PLAN_ROW_LANES:
+    case RMI_PLAN_ROW_WAVE:
+    case RMI_PLAN_ROW_BLOCK:
+    case RMI_PLAN_ROW_SPLIT: {
+      RowArgs a{};
+      a.in      = pr.in;
+      a.partial = pr.ws;
+      a.n_out   = pl.n_out;
+      a.len     = pl.len;
+      a.nvec    = pl.nvec;
+      a.chunk   = pl.chunk;
+      a.G       = pl.G;
+      a.logG    = pl.logG;
+      a.B       = pl.B;
+      a.epi     = pr.epi;
+      const dim3 grid((unsigned)pl.grid_blocks);
+      if (pl.kind == RMI_PLAN_ROW_LANES) {
+        switch (pl.K) {
+          case 2: rc = launch_lanes<P, 2>(pl, a, st); break;
+          case 4: rc = launch_lanes<P, 4>(pl, a, st); break;
+          case 8: rc = launch_lanes<P, 8>(pl, a, st); break;
+          case 16: rc = launch_lanes<P, 16>(pl, a, st); break;
+          default: rc = RMI_ERR_UNSUPPORTED;
+        }
+      } else if (pl.kind == RMI_PLAN_ROW_WAVE) {
+        if (pl.short_rows) {
+          if (pl.vec16)
+            hipLaunchKernelGGL((row_short_kernel<P, true>), grid, dim3(kBlock), 0, st, a);
+          else
+            hipLaunchKernelGGL((row_short_kernel<P, false>), grid, dim3(kBlock), 0, st, a);
+        } else {
+          if (pl.vec16)
+            hipLaunchKernelGGL((row_wave_kernel<P, true>), grid, dim3(kBlock), 0, st, a);
+          else
+            hipLaunchKernelGGL((row_wave_kernel<P, false>), grid, dim3(kBlock), 0, st, a);
+        }
+      } else {
+        if (pl.vec16)
+          hipLaunchKernelGGL((row_block_kernel<P, true>), grid, dim3(pl.threads), 0, st, a);
+        else
+          hipLaunchKernelGGL((row_block_kernel<P, false>), grid, dim3(pl.threads), 0, st, a);
+        if (pl.kind == RMI_PLAN_ROW_SPLIT) rc = launch_fold<P>(pl, pr, pl.B, st);
+      }
+      break;
+    }
+    case RMI_PLAN_COL_TILE: {
+      ColArgs a{};
+      a.in             = pr.in;
+      a.partial        = pr.ws;
+      a.n_out          = pl.n_out;
+      a.len            = pl.len;
+      a.nvec           = pl.nvec;
+      a.rows_per_block = pl.rows_per_block;
+      a.TX             = pl.TX;
+      a.logTX          = pl.logTX;
+      a.B              = pl.B;
+      a.epi            = pr.epi;
+      const dim3 grid((unsigned)pl.gridx, (unsigned)pl.B);
+      if (pl.vec16)
+        hipLaunchKernelGGL((col_kernel<P, true>), grid, dim3(kBlock), 0, st, a);
+      else
+        hipLaunchKernelGGL((col_kernel<P, false>), grid, dim3(kBlock), 0, st, a);
+      if (pl.B > 1) rc = launch_fold<P>(pl, pr, pl.B, st);
+      break;
+    }
+    default: rc = RMI_ERR_BAD_ENUM;
+  }
+  if (rc != RMI_OK) return rc;
+  return hipGetLastError() == hipSuccess ? RMI_OK : RMI_ERR_LAUNCH;
+}
+
+// Policies offered for one input type, keyed by PolicyKey.
+template <class InT, bool IS_FLOAT_IN, bool IS_F64>
+run_fn lookup_for(const PolicyKey& k)
+{
+#define RMI_MAIN_CASES(MK)                           \
+  switch (k.main_op) {                               \
+    case RMI_MAIN_IDENTITY: MK(RMI_MAIN_IDENTITY);   \
+    case RMI_MAIN_SQ: MK(RMI_MAIN_SQ);               \
+    case RMI_MAIN_ABS: MK(RMI_MAIN_ABS);             \
+    case RMI_MAIN_NZ: MK(RMI_MAIN_NZ);               \
+    default: return nullptr;                         \
+  }
+#define RMI_MAIN3_CASES(MK)                          \
+  switch (k.main_op) {                               \
+    case RMI_MAIN_IDENTITY: MK(RMI_MAIN_IDENTITY);   \
+    case RMI_MAIN_SQ: MK(RMI_MAIN_SQ);               \
+    case RMI_MAIN_ABS: MK(RMI_MAIN_ABS);             \
+    default: return nullptr;                         \
+  }
+  switch (k.family) {
+    case kFamFloat:
+      if (k.red_op == RMI_RED_ADD) {
+        if constexpr (!IS_F64) {
+#define MK(M) return &run<PolF<InT, M, RMI_RED_ADD>>
+          RMI_MAIN_CASES(MK)
+#undef MK
+        }
+        return nullptr;
+      }
+      if constexpr (IS_FLOAT_IN) {
+        if (k.red_op == RMI_RED_MAX) {
+#define MK(M) return &run<PolF<InT, M, RMI_RED_MAX>>
+          RMI_MAIN3_CASES(MK)
+#undef MK
+        }
+        if (k.red_op == RMI_RED_MIN) {
+#define MK(M) return &run<PolF<InT, M, RMI_RED_MIN>>
+          RMI_MAIN3_CASES(MK)
+#undef MK
+        }
+      }
+      return nullptr;
+    case kFamKbn:
+      if constexpr (IS_F64) {
+#define MK(M) return &run<PolKbn<InT, M>>
+        RMI_MAIN_CASES(MK)
+#undef MK
+      }
+      return nullptr;
+    case kFamInt:
+      if constexpr (!IS_FLOAT_IN) {
+        if (k.red_op == RMI_RED_ADD) {
+#define MK(M) return &run<PolI<InT, M, RMI_RED_ADD>>
+          RMI_MAIN_CASES(MK)
+#undef MK
+        }
+        if (k.red_op == RMI_RED_MAX) {
+#define MK(M) return &run<PolI<InT, M, RMI_RED_MAX>>
+          RMI_MAIN3_CASES(MK)
+#undef MK
+        }
+        if (k.red_op == RMI_RED_MIN) {
+#define MK(M) return &run<PolI<InT, M, RMI_RED_MIN>>
+          RMI_MAIN3_CASES(MK)
+#undef MK
+        }
+      }
+      return nullptr;
+    case kFamKvp:
+      if constexpr (IS_FLOAT_IN) {
+        const bool is_max = k.red_op == RMI_RED_ARGMAX;
+        if (k.key64) {
+          return is_max ? &run<PolKvp<InT, int64_t, true>> : &run<PolKvp<InT, int64_t, false>>;
+        }
+        return is_max ? &run<PolKvp<InT, int32_t, true>> : &run<PolKvp<InT, int32_t, false>>;
+      }
+      return nullptr;
+    default: return nullptr;
+  }
+#undef RMI_MAIN_CASES
+#undef RMI_MAIN3_CASES
+}
+
+// one definition per input type, each in its own translation unit
+run_fn lookup_i8(const PolicyKey&);
+run_fn lookup_u8(const PolicyKey&);
+run_fn lookup_i32(const PolicyKey&);
+run_fn lookup_i64(const PolicyKey&);
+run_fn lookup_f16(const PolicyKey&);
+run_fn lookup_bf16(const PolicyKey&);
+run_fn lookup_f32(const PolicyKey&);
+run_fn lookup_f64(const PolicyKey&);
+
+}  // namespace rmi

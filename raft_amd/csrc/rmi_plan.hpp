@@ -1,0 +1,345 @@
+// Host-only: validation of a reduction descriptor and the choice of launch
+// plan by shape.  No HIP types here, so a plain g++ translation unit can use
+// and test it.
+//
+// The reference picks among Thin / Medium / Thick kernels with thresholds tied
+// to 32-lane warps and NVIDIA SM counts
+// (linalg/detail/coalesced_reduction-inl.cuh:302-326,640-670) and launches the
+// strided kernels with fixed block shapes
+// (linalg/detail/strided_reduction.cuh:148-188).  The selector below is
+// re-derived for 64-lane wavefronts, 16-byte lane loads and 256 CUs.
+#pragma once
+
+#include <stddef.h>
+#include <stdint.h>
+
+#include "rmi_reduce.h"
+
+namespace rmi {
+
+constexpr int kPlanBlock  = 256;
+constexpr int kPlanUnroll = 4;
+constexpr int kWavesPerCu = 32;  // 8 resident waves on each of the 4 SIMDs
+
+struct PlanX {
+  int kind        = RMI_PLAN_EMPTY;
+  bool strided    = false;  // reduce along the strided dimension
+  bool vec16      = false;  // 16-byte lane loads
+  bool short_rows = false;  // ROW_WAVE served by the one-load-per-lane kernel
+  int elem_bytes  = 0;
+  int step        = 1;  // elements per lane-load
+  int64_t n_out   = 0;
+  int64_t len     = 0;  // elements folded into one output
+  int64_t nvec    = 0;  // lane-loads along the contiguous dimension
+  int K           = 0;  // ROW_LANES: rows per 16-byte vector
+  int G           = 1;  // ROW_WAVE: lanes per row
+  int logG        = 0;
+  int threads     = kPlanBlock;  // ROW_BLOCK / ROW_SPLIT block size
+  int B           = 1;           // partials per output
+  int64_t chunk   = 0;           // ROW_SPLIT: lane-loads per block
+  int TX          = 1;           // COL_TILE
+  int logTX       = 0;
+  int64_t gridx   = 0;  // COL_TILE: blocks along the contiguous dimension
+  int64_t rows_per_block = 0;
+  int64_t grid_blocks    = 0;
+  int passes             = 1;
+  int acc_bytes          = 8;
+  size_t ws_bytes        = 0;
+};
+
+inline int dtype_size(int dt)
+{
+  switch (dt) {
+    case RMI_I8:
+    case RMI_U8: return 1;
+    case RMI_F16:
+    case RMI_BF16: return 2;
+    case RMI_I32:
+    case RMI_F32: return 4;
+    case RMI_I64:
+    case RMI_F64:
+    case RMI_KVP_I32_F32: return 8;
+    case RMI_KVP_I32_F64:
+    case RMI_KVP_I64_F32:
+    case RMI_KVP_I64_F64: return 16;
+    default: return 0;
+  }
+}
+
+inline bool is_float_dtype(int dt)
+{
+  return dt == RMI_F16 || dt == RMI_BF16 || dt == RMI_F32 || dt == RMI_F64;
+}
+inline bool is_int_dtype(int dt)
+{
+  return dt == RMI_I8 || dt == RMI_U8 || dt == RMI_I32 || dt == RMI_I64;
+}
+inline bool is_kvp_dtype(int dt) { return dt >= RMI_KVP_I32_F32 && dt <= RMI_KVP_I64_F64; }
+
+// Which accumulator family serves a descriptor.
+enum : int { kFamFloat = 0, kFamKbn = 1, kFamInt = 2, kFamKvp = 3 };
+
+struct PolicyKey {
+  int in_dtype = 0;
+  int family   = 0;
+  int main_op  = 0;
+  int red_op   = 0;
+  int key64    = 0;  // kFamKvp: 64-bit keys
+};
+
+inline int pow2ceil(int64_t x)
+{
+  int p = 1;
+  while (p < x)
+    p <<= 1;
+  return p;
+}
+inline int ilog2(int x)
+{
+  int l = 0;
+  while ((1 << l) < x)
+    ++l;
+  return l;
+}
+inline int64_t ceildiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// Validates enums, dtype/functor compatibility and shape; fills `key` and the
+// accumulator size.  Returns an rmi_status.
+inline int classify(const rmi_reduce_desc& d, PolicyKey& key, int& acc_bytes)
+{
+  if (d.in_dtype < 0 || d.in_dtype >= RMI_DTYPE_COUNT_ || d.out_dtype < 0 ||
+      d.out_dtype >= RMI_DTYPE_COUNT_)
+    return RMI_ERR_BAD_ENUM;
+  if (d.layout != RMI_ROW_MAJOR && d.layout != RMI_COL_MAJOR) return RMI_ERR_BAD_ENUM;
+  if (d.apply != RMI_ALONG_ROWS && d.apply != RMI_ALONG_COLUMNS) return RMI_ERR_BAD_ENUM;
+  if (d.main_op < RMI_MAIN_IDENTITY || d.main_op > RMI_MAIN_KVP) return RMI_ERR_BAD_ENUM;
+  if (d.reduce_op < RMI_RED_ADD || d.reduce_op > RMI_RED_ARGMIN) return RMI_ERR_BAD_ENUM;
+  if (d.final_op < RMI_FIN_IDENTITY || d.final_op > RMI_FIN_KEY) return RMI_ERR_BAD_ENUM;
+  if (d.plan_hint < RMI_PLAN_AUTO || d.plan_hint > RMI_PLAN_EMPTY) return RMI_ERR_BAD_ENUM;
+  if (d.reserved != 0) return RMI_ERR_BAD_ENUM;
+  if (d.n_rows < 0 || d.n_cols < 0) return RMI_ERR_BAD_SHAPE;
+  if (is_kvp_dtype(d.in_dtype)) return RMI_ERR_UNSUPPORTED;
+
+  const bool arg = d.reduce_op == RMI_RED_ARGMAX || d.reduce_op == RMI_RED_ARGMIN;
+  key.in_dtype   = d.in_dtype;
+  key.main_op    = d.main_op;
+  key.red_op     = d.reduce_op;
+  key.key64      = 0;
+  if (arg) {
+    // value -> {index, value}, arg-reduce, then either the pair or its key
+    if (d.main_op != RMI_MAIN_KVP) return RMI_ERR_UNSUPPORTED;
+    if (!is_float_dtype(d.in_dtype)) return RMI_ERR_UNSUPPORTED;
+    const bool val64 = d.in_dtype == RMI_F64;
+    if (d.final_op == RMI_FIN_KEY) {
+      if (d.out_dtype != RMI_I32 && d.out_dtype != RMI_I64) return RMI_ERR_UNSUPPORTED;
+      if (d.inplace) return RMI_ERR_UNSUPPORTED;
+      key.key64 = d.out_dtype == RMI_I64;
+    } else if (d.final_op == RMI_FIN_IDENTITY) {
+      if (!is_kvp_dtype(d.out_dtype)) return RMI_ERR_UNSUPPORTED;
+      const bool out_val64 = d.out_dtype == RMI_KVP_I32_F64 || d.out_dtype == RMI_KVP_I64_F64;
+      if (out_val64 != val64) return RMI_ERR_UNSUPPORTED;
+      key.key64 = d.out_dtype == RMI_KVP_I64_F32 || d.out_dtype == RMI_KVP_I64_F64;
+    } else {
+      return RMI_ERR_UNSUPPORTED;
+    }
+    key.family = kFamKvp;
+    acc_bytes  = (key.key64 || val64) ? 16 : 8;
+  } else {
+    if (d.main_op == RMI_MAIN_KVP || d.final_op == RMI_FIN_KEY) return RMI_ERR_UNSUPPORTED;
+    if (is_kvp_dtype(d.out_dtype)) return RMI_ERR_UNSUPPORTED;
+    if (is_float_dtype(d.out_dtype)) {
+      if (d.in_dtype == RMI_F64 && d.reduce_op == RMI_RED_ADD) {
+        key.family = kFamKbn;
+        acc_bytes  = 16;
+      } else {
+        // integers feeding a floating output are only summed (means, norms)
+        if (is_int_dtype(d.in_dtype) && d.reduce_op != RMI_RED_ADD) return RMI_ERR_UNSUPPORTED;
+        key.family = kFamFloat;
+        acc_bytes  = 8;
+      }
+      if ((d.final_op == RMI_FIN_VAR_FROM_SUMSQ || d.final_op == RMI_FIN_STDDEV_FROM_SUMSQ) &&
+          d.final_aux == nullptr)
+        return RMI_ERR_NULL;
+    } else {
+      // integer output: integer input, integer arithmetic end to end
+      if (!is_int_dtype(d.in_dtype)) return RMI_ERR_UNSUPPORTED;
+      if (d.out_dtype != RMI_I32 && d.out_dtype != RMI_I64) return RMI_ERR_UNSUPPORTED;
+      if (d.final_op == RMI_FIN_SQRT || d.final_op == RMI_FIN_VAR_FROM_SUMSQ ||
+          d.final_op == RMI_FIN_STDDEV_FROM_SUMSQ)
+        return RMI_ERR_UNSUPPORTED;
+      key.family = kFamInt;
+      acc_bytes  = 8;
+    }
+    if (d.main_op == RMI_MAIN_NZ && d.reduce_op != RMI_RED_ADD) return RMI_ERR_UNSUPPORTED;
+  }
+  return RMI_OK;
+}
+
+// Shape -> plan.  `aligned16`: the input base pointer is 16-byte aligned.
+// `hint`: an rmi_plan_kind to force where it is applicable to the shape.
+inline int make_plan(const rmi_reduce_desc& d,
+                     const PolicyKey& key,
+                     int acc_bytes,
+                     bool aligned16,
+                     int n_cu,
+                     PlanX& p)
+{
+  p            = PlanX{};
+  p.acc_bytes  = acc_bytes;
+  p.elem_bytes = dtype_size(d.in_dtype);
+  const int es = p.elem_bytes;
+  // (row-major, along rows) and (col-major, along columns) fold the contiguous
+  // dimension; the other two fold the strided one (linalg/detail/reduce.cuh:36-48).
+  const bool row_major = d.layout == RMI_ROW_MAJOR;
+  const bool along_rows = d.apply == RMI_ALONG_ROWS;
+  p.strided            = row_major != along_rows;
+  const int64_t contiguous = row_major ? d.n_cols : d.n_rows;
+  const int64_t other      = row_major ? d.n_rows : d.n_cols;
+  p.n_out = p.strided ? contiguous : other;
+  p.len   = p.strided ? other : contiguous;
+
+  if (key.family == kFamKvp && !key.key64 && p.len > (int64_t)INT32_MAX) return RMI_ERR_BAD_SHAPE;
+  if (p.n_out > ((int64_t)1 << 40) || p.len > ((int64_t)1 << 40)) return RMI_ERR_BAD_SHAPE;
+
+  const int64_t slots = (int64_t)n_cu * kWavesPerCu;
+  const int hint      = d.plan_hint;
+
+  if (p.n_out == 0) {
+    p.kind = RMI_PLAN_EMPTY;
+    p.passes = 0;
+    return RMI_OK;
+  }
+  if (p.len == 0) {
+    p.kind        = RMI_PLAN_EMPTY;
+    p.grid_blocks = ceildiv(p.n_out, kPlanBlock);
+    return RMI_OK;
+  }
+
+  const int64_t row_bytes = contiguous * es;
+  p.vec16                 = aligned16 && (row_bytes % 16 == 0);
+  p.step                  = p.vec16 ? 16 / es : 1;
+  p.nvec                  = contiguous / p.step;
+
+  if (p.strided) {
+    p.kind  = RMI_PLAN_COL_TILE;
+    p.TX    = (int)(p.nvec < 64 ? pow2ceil(p.nvec) : 64);
+    p.logTX = ilog2(p.TX);
+    const int TY = kPlanBlock / p.TX;
+    p.gridx      = ceildiv(p.nvec, p.TX);
+    // enough blocks to give every CU several, but at least two unrolled
+    // batches of rows per thread
+    int64_t B          = ceildiv((int64_t)n_cu * 8, p.gridx);
+    const int64_t maxB = ceildiv(p.len, (int64_t)TY * kPlanUnroll * 2);
+    if (B > maxB) B = maxB;
+    if (B < 1) B = 1;
+    if (B > 4096) B = 4096;
+    const int64_t quantum = (int64_t)TY * kPlanUnroll;
+    p.rows_per_block      = ceildiv(ceildiv(p.len, B), quantum) * quantum;
+    p.B                   = (int)ceildiv(p.len, p.rows_per_block);
+    p.grid_blocks         = p.gridx * p.B;
+    p.passes              = p.B > 1 ? 2 : 1;
+    p.ws_bytes            = p.B > 1 ? (size_t)p.n_out * p.B * acc_bytes : 0;
+    if (p.gridx > 0x7fffffffLL) return RMI_ERR_BAD_SHAPE;
+    return RMI_OK;
+  }
+
+  // ---- contiguous-dimension plans ----
+  // several whole rows per 16-byte vector
+  if (aligned16 && row_bytes < 16 && 16 % row_bytes == 0 &&
+      (hint == RMI_PLAN_AUTO || hint == RMI_PLAN_ROW_LANES)) {
+    p.kind        = RMI_PLAN_ROW_LANES;
+    p.vec16       = true;
+    p.step        = 16 / es;
+    p.K           = (int)(16 / row_bytes);
+    p.nvec        = 1;
+    p.grid_blocks = ceildiv(ceildiv(p.n_out, p.K), (int64_t)kPlanBlock * kPlanUnroll);
+    if (p.grid_blocks < 1) p.grid_blocks = 1;
+    return RMI_OK;
+  }
+
+  int kind = hint;
+  if (kind == RMI_PLAN_ROW_LANES || kind == RMI_PLAN_COL_TILE || kind == RMI_PLAN_EMPTY)
+    kind = RMI_PLAN_AUTO;
+  int threads = 64;
+  if (kind == RMI_PLAN_AUTO) {
+    if (p.nvec <= 4 * 64) {
+      kind = RMI_PLAN_ROW_WAVE;
+    } else {
+      // widen the team on a row until the machine's wave slots are filled,
+      // keeping at least kPlanUnroll lane-loads per thread
+      while (threads < 1024 && p.n_out * (threads / 64) < slots &&
+             p.nvec >= (int64_t)kPlanUnroll * threads * 4)
+        threads *= 4;
+      if (threads == 64) {
+        kind = RMI_PLAN_ROW_WAVE;
+      } else if (threads == 1024 && p.n_out * 16 < slots &&
+                 p.nvec >= (int64_t)2 * kPlanBlock * kPlanUnroll * 2) {
+        kind = RMI_PLAN_ROW_SPLIT;
+      } else {
+        kind = RMI_PLAN_ROW_BLOCK;
+      }
+    }
+  } else if (kind == RMI_PLAN_ROW_BLOCK) {
+    threads = kPlanBlock;
+  }
+
+  if (kind == RMI_PLAN_ROW_WAVE) {
+    p.kind = RMI_PLAN_ROW_WAVE;
+    if (p.nvec <= 8) {
+      p.short_rows = true;
+      p.G          = pow2ceil(p.nvec);
+    } else {
+      const int64_t g = ceildiv(p.nvec, kPlanUnroll);
+      p.G             = g >= 64 ? 64 : pow2ceil(g);
+      if (p.G < 8) p.G = 8;
+    }
+    p.logG               = ilog2(p.G);
+    const int64_t rows_w = (int64_t)(64 / p.G) * (p.short_rows ? kPlanUnroll : 1);
+    p.grid_blocks        = ceildiv(p.n_out, rows_w * (kPlanBlock / 64));
+  } else if (kind == RMI_PLAN_ROW_BLOCK) {
+    p.kind        = RMI_PLAN_ROW_BLOCK;
+    p.threads     = threads;
+    p.B           = 1;
+    p.chunk       = p.nvec;
+    p.grid_blocks = p.n_out;
+  } else {
+    p.kind    = RMI_PLAN_ROW_SPLIT;
+    p.threads = kPlanBlock;
+    const int64_t quantum = (int64_t)kPlanBlock * kPlanUnroll;
+    int64_t B             = ceildiv(slots, p.n_out * (kPlanBlock / 64));
+    const int64_t maxB    = p.nvec / (quantum * 2) > 1 ? p.nvec / (quantum * 2) : 1;
+    if (B > maxB) B = maxB;
+    if (B < 2) B = 2;
+    if (B > 4096) B = 4096;
+    p.chunk       = ceildiv(ceildiv(p.nvec, B), quantum) * quantum;
+    p.B           = (int)ceildiv(p.nvec, p.chunk);
+    p.grid_blocks = p.n_out * p.B;
+    if (p.B < 2) {  // the row is too short to split: one block per row
+      p.kind  = RMI_PLAN_ROW_BLOCK;
+      p.B     = 1;
+      p.chunk = p.nvec;
+    } else {
+      p.passes   = 2;
+      p.ws_bytes = (size_t)p.n_out * p.B * acc_bytes;
+    }
+  }
+  if (p.grid_blocks > 0x7fffffffLL) return RMI_ERR_BAD_SHAPE;
+  return RMI_OK;
+}
+
+inline void export_plan(const PlanX& p, rmi_plan& o)
+{
+  o.kind            = p.kind;
+  o.vec_bytes       = p.vec16 ? 16 : p.elem_bytes;
+  o.lanes_per_row   = p.kind == RMI_PLAN_ROW_WAVE ? p.G : 0;
+  o.blocks_per_out  = p.B;
+  o.block_threads   = (p.kind == RMI_PLAN_ROW_BLOCK || p.kind == RMI_PLAN_ROW_SPLIT) ? p.threads
+                                                                                      : kPlanBlock;
+  o.passes          = p.passes;
+  o.grid_blocks     = p.grid_blocks;
+  o.n_outputs       = p.n_out;
+  o.reduce_len      = p.len;
+  o.workspace_bytes = p.ws_bytes;
+}
+
+}  // namespace rmi

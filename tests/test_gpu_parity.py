@@ -1,0 +1,303 @@
+"""GPU results through the C ABI against the CPU oracle on the same seeded inputs:
+the shape grids of the reference's reduction tests, every launch plan, every dtype
+pairing, inplace, unaligned inputs and empty inputs."""
+import itertools
+
+import numpy as np
+import pytest
+
+from raft_amd import _capi as api
+from tests import _util as u
+
+pytestmark = pytest.mark.gpu
+
+LAYOUT_AXIS = list(itertools.product([api.ROW_MAJOR, api.COL_MAJOR],
+                                     [api.ALONG_ROWS, api.ALONG_COLUMNS]))
+
+
+def _rand(rng, dt, n, lo=-1.0, hi=1.0):
+    if dt == api.F32:
+        return rng.uniform(lo, hi, n).astype(np.float32)
+    if dt == api.F64:
+        return rng.uniform(lo, hi, n)
+    if dt == api.F16:
+        return rng.uniform(lo, hi, n).astype(np.float16)
+    if dt == api.BF16:
+        return u.to_bf16(rng.uniform(lo, hi, n).astype(np.float32))
+    if dt == api.I8:
+        return rng.integers(-128, 128, n, dtype=np.int8)
+    if dt == api.U8:
+        return rng.integers(0, 256, n, dtype=np.uint8)
+    if dt == api.I32:
+        return rng.integers(-100000, 100000, n, dtype=np.int32)
+    if dt == api.I64:
+        return rng.integers(-2**40, 2**40, n, dtype=np.int64)
+    raise ValueError(dt)
+
+
+# cpp/tests/linalg/reduce.cu:292-317: rows {11,1234} x cols {7,33,128,500}, 4 layout/axis
+# combinations, sq_op / add_op / sqrt_op, inplace=false then inplace=true on the same
+# output (:191-241).
+@pytest.mark.parametrize("in_dt,out_dt", [(api.F32, api.F32), (api.F64, api.F64),
+                                          (api.F32, api.F64)])
+@pytest.mark.parametrize("rows,cols", itertools.product([11, 1234], [7, 33, 128, 500]))
+def test_reduce_grid(gpu, in_dt, out_dt, rows, cols):
+    rng = np.random.default_rng(1234)
+    data = _rand(rng, in_dt, rows * cols)
+    for layout, apply in LAYOUT_AXIS:
+        d = api.make_desc(in_dt, out_dt, rows, cols, layout=layout, apply=apply,
+                          main_op=api.MAIN_SQ, final_op=api.FIN_SQRT)
+        first = u.check_against_oracle(d, data, label=f"{rows}x{cols} l{layout} a{apply}")
+        d.inplace = 1
+        u.check_against_oracle(d, data, old_raw=first,
+                               label=f"{rows}x{cols} l{layout} a{apply} inplace")
+
+
+# cpp/tests/linalg/reduce.cu:321-341 ("thick"): {3,9} x {17771,33333,100000}.
+@pytest.mark.parametrize("rows,cols", itertools.product([3, 9], [17771, 33333, 100000]))
+def test_reduce_thick(gpu, rows, cols):
+    rng = np.random.default_rng(1234)
+    data = _rand(rng, api.F32, rows * cols)
+    for layout, apply in LAYOUT_AXIS:
+        d = api.make_desc(api.F32, api.F32, rows, cols, layout=layout, apply=apply,
+                          main_op=api.MAIN_SQ, final_op=api.FIN_SQRT)
+        u.check_against_oracle(d, data, label=f"thick {rows}x{cols} l{layout} a{apply}")
+
+
+# cpp/tests/linalg/coalesced_reduction.cu:109-139: 10000 x {3..270}, 10 x 25000, ...
+@pytest.mark.parametrize("rows,cols", [(10000, c) for c in
+                                       (3, 5, 7, 9, 17, 31, 32, 33, 55, 63, 64, 65, 128, 270)]
+                         + [(10, 25000), (100, 4100), (1025, 2048), (5, 1 << 17)])
+@pytest.mark.parametrize("dt", [api.F32, api.F64])
+def test_coalesced_sweep(gpu, rows, cols, dt):
+    rng = np.random.default_rng(rows * 131 + cols)
+    data = _rand(rng, dt, rows * cols)
+    d = api.make_desc(dt, dt, rows, cols, main_op=api.MAIN_SQ)
+    first = u.check_against_oracle(d, data, label=f"coalesced {rows}x{cols}")
+    d.inplace = 1
+    u.check_against_oracle(d, data, old_raw=first, label=f"coalesced {rows}x{cols} inplace")
+
+
+# cpp/tests/linalg/strided_reduction.cu:94-102: 1024 x {32,64,128,256}; plus odd widths.
+@pytest.mark.parametrize("rows,cols", [(1024, c) for c in (32, 64, 128, 256)]
+                         + [(4097, 3), (100000, 2), (33333, 20), (777, 1000), (50, 20000)])
+@pytest.mark.parametrize("dt", [api.F32, api.F64])
+def test_strided_sweep(gpu, rows, cols, dt):
+    rng = np.random.default_rng(rows * 7 + cols)
+    data = _rand(rng, dt, rows * cols)
+    d = api.make_desc(dt, dt, rows, cols, apply=api.ALONG_COLUMNS, main_op=api.MAIN_SQ)
+    first = u.check_against_oracle(d, data, label=f"strided {rows}x{cols}")
+    d.inplace = 1
+    u.check_against_oracle(d, data, old_raw=first, label=f"strided {rows}x{cols} inplace")
+
+
+# Every row plan forced on a shape it applies to must agree with the oracle.
+@pytest.mark.parametrize("plan", [api.PLAN_ROW_WAVE, api.PLAN_ROW_BLOCK, api.PLAN_ROW_SPLIT])
+@pytest.mark.parametrize("rows,cols", [(37, 4096), (5, 70000), (300, 1000), (2, 262144 + 4)])
+@pytest.mark.parametrize("in_dt,out_dt,red", [(api.F32, api.F32, api.RED_ADD),
+                                              (api.F32, api.F32, api.RED_MAX),
+                                              (api.I8, api.I64, api.RED_ADD),
+                                              (api.F64, api.F64, api.RED_ADD)])
+def test_forced_row_plans(gpu, plan, rows, cols, in_dt, out_dt, red):
+    rng = np.random.default_rng(plan * 1000 + rows)
+    data = _rand(rng, in_dt, rows * cols)
+    init = {} if red == api.RED_ADD else dict(init_f=-np.inf)
+    d = api.make_desc(in_dt, out_dt, rows, cols, reduce_op=red, plan_hint=plan, **init)
+    u.check_against_oracle(d, data, label=f"plan {api.PLAN_NAME[plan]} {rows}x{cols}")
+
+
+# Input / output type pairings and functor triples.
+TYPE_CASES = [
+    (api.I8, api.I64), (api.I8, api.I32), (api.U8, api.I64), (api.I32, api.I64),
+    (api.I64, api.I64), (api.F16, api.F32), (api.F16, api.F16), (api.BF16, api.F32),
+    (api.BF16, api.BF16), (api.I8, api.F16), (api.I8, api.F32), (api.I32, api.F64),
+    (api.F32, api.F16), (api.F64, api.F32),
+]
+
+
+@pytest.mark.parametrize("in_dt,out_dt", TYPE_CASES)
+@pytest.mark.parametrize("main", [api.MAIN_IDENTITY, api.MAIN_SQ, api.MAIN_ABS, api.MAIN_NZ])
+def test_type_pairs_sum(gpu, in_dt, out_dt, main):
+    rng = np.random.default_rng(in_dt * 100 + out_dt * 10 + main)
+    for rows, cols, apply in [(257, 96, api.ALONG_ROWS), (64, 4096, api.ALONG_ROWS),
+                              (3000, 8, api.ALONG_ROWS), (2000, 48, api.ALONG_COLUMNS)]:
+        data = _rand(rng, in_dt, rows * cols)
+        if out_dt == api.F16 and in_dt in (api.I8, api.I32):
+            data = (data % 5).astype(data.dtype)  # keep sums inside f16's range
+        d = api.make_desc(in_dt, out_dt, rows, cols, apply=apply, main_op=main)
+        u.check_against_oracle(d, data, label=f"{api.DTYPE_NAME[in_dt]}->"
+                               f"{api.DTYPE_NAME[out_dt]} main{main} {rows}x{cols}")
+
+
+@pytest.mark.parametrize("in_dt,out_dt", [(api.F32, api.F32), (api.F64, api.F64),
+                                          (api.F16, api.F32), (api.BF16, api.F32),
+                                          (api.I8, api.I64), (api.I32, api.I32),
+                                          (api.I64, api.I64), (api.U8, api.I32)])
+@pytest.mark.parametrize("red", [api.RED_MAX, api.RED_MIN])
+@pytest.mark.parametrize("main", [api.MAIN_IDENTITY, api.MAIN_ABS, api.MAIN_SQ])
+def test_min_max(gpu, in_dt, out_dt, red, main):
+    rng = np.random.default_rng(in_dt + 17 * red + 5 * main)
+    big = 2**62
+    for rows, cols, apply in [(129, 200, api.ALONG_ROWS), (7, 9000, api.ALONG_ROWS),
+                              (5000, 4, api.ALONG_ROWS), (1500, 40, api.ALONG_COLUMNS)]:
+        data = _rand(rng, in_dt, rows * cols)
+        init = dict(init_f=-np.inf, init_i=-big) if red == api.RED_MAX else \
+            dict(init_f=np.inf, init_i=big)
+        d = api.make_desc(in_dt, out_dt, rows, cols, apply=apply, main_op=main, reduce_op=red,
+                          **init)
+        if out_dt == api.I32:
+            d.init.i = -2**31 if red == api.RED_MAX else 2**31 - 1
+        # identity / abs select one of the inputs: exact.  sq is squared in f64 and
+        # rounded once to the output type.
+        exact = out_dt in (api.F32, api.F64) and main != api.MAIN_SQ
+        u.check_against_oracle(d, data, tol=0.0 if exact else None,
+                               label=f"minmax {api.DTYPE_NAME[in_dt]} red{red} main{main}")
+
+
+# L1 / L2 / Linf norms (linalg/detail/norm.cuh:23-61), row and column, with and without sqrt;
+# cpp/tests/linalg/norm.cu:238-306 (incl. half -> float).
+@pytest.mark.parametrize("in_dt,out_dt", [(api.F32, api.F32), (api.F64, api.F64),
+                                          (api.F16, api.F32)])
+@pytest.mark.parametrize("norm", ["l1", "l2", "linf"])
+@pytest.mark.parametrize("fin", [api.FIN_IDENTITY, api.FIN_SQRT])
+def test_norms(gpu, in_dt, out_dt, norm, fin):
+    rng = np.random.default_rng(42)
+    main, red = {"l1": (api.MAIN_ABS, api.RED_ADD), "l2": (api.MAIN_SQ, api.RED_ADD),
+                 "linf": (api.MAIN_ABS, api.RED_MAX)}[norm]
+    for rows, cols in [(4, 8), (1024, 32), (1000, 100), (129, 1024), (37, 6000)]:
+        data = _rand(rng, in_dt, rows * cols, -10, 10)
+        for apply in (api.ALONG_ROWS, api.ALONG_COLUMNS):
+            d = api.make_desc(in_dt, out_dt, rows, cols, apply=apply, main_op=main,
+                              reduce_op=red, final_op=fin)
+            u.check_against_oracle(d, data, label=f"{norm} {rows}x{cols} a{apply}")
+
+
+# Key-value arg reductions: cpp/tests/linalg/reduce.cu:343-411 shapes, plus planted ties
+# (lowest index must win), NaN (never wins), all -inf rows and signed zeros.
+@pytest.mark.parametrize("in_dt,out_dt", [(api.F32, api.KVP_I32_F32), (api.F64, api.KVP_I32_F64),
+                                          (api.F32, api.KVP_I64_F32), (api.F64, api.KVP_I64_F64),
+                                          (api.F16, api.KVP_I32_F32), (api.BF16, api.KVP_I32_F32)])
+@pytest.mark.parametrize("red", [api.RED_ARGMAX, api.RED_ARGMIN])
+def test_kvp_arg_reduce(gpu, in_dt, out_dt, red):
+    rng = np.random.default_rng(1234 + red)
+    is_max = red == api.RED_ARGMAX
+    for rows, cols in itertools.product([11, 1234], [7, 33, 128, 500]):
+        data = _rand(rng, in_dt, rows * cols)
+        d = api.make_desc(in_dt, out_dt, rows, cols, main_op=api.MAIN_KVP, reduce_op=red,
+                          init_i=0, init_f=-np.inf if is_max else np.inf)
+        first = u.check_against_oracle(d, data, label=f"kvp {rows}x{cols}")
+        d.inplace = 1
+        u.check_against_oracle(d, data, old_raw=first, label=f"kvp {rows}x{cols} inplace")
+
+
+@pytest.mark.parametrize("plan", [api.PLAN_AUTO, api.PLAN_ROW_WAVE, api.PLAN_ROW_BLOCK,
+                                  api.PLAN_ROW_SPLIT])
+@pytest.mark.parametrize("cols", [64, 1000, 32000, 131072])
+def test_argmax_ties_and_specials(gpu, plan, cols):
+    rng = np.random.default_rng(cols)
+    rows = 48
+    m = rng.standard_normal((rows, cols)).astype(np.float32)
+    for r in range(rows):
+        kind = r % 6
+        if kind == 0:      # exact ties of the maximum at 2..4 positions
+            pos = rng.choice(cols, size=min(cols, 2 + r % 3), replace=False)
+            m[r, pos] = m[r].max() + 1.0
+        elif kind == 1:    # NaN scattered, never wins
+            m[r, rng.choice(cols, size=min(cols, 5), replace=False)] = np.nan
+        elif kind == 2:    # whole row -inf: init key wins
+            m[r, :] = -np.inf
+        elif kind == 3:    # signed zeros tie
+            m[r, :] = -1.0
+            pos = np.sort(rng.choice(cols, size=2, replace=False))
+            m[r, pos[0]] = -0.0
+            m[r, pos[1]] = 0.0
+        elif kind == 4:    # constant row: index 0
+            m[r, :] = 0.5
+        # kind 5: plain random
+    d = api.make_desc(api.F32, api.KVP_I32_F32, rows, cols, main_op=api.MAIN_KVP,
+                      reduce_op=api.RED_ARGMAX, init_i=0, init_f=-np.inf, plan_hint=plan)
+    raw = u.check_against_oracle(d, m.reshape(-1), label=f"ties cols={cols} plan={plan}")
+    # independent of the oracle: numpy's first-maximum rule on rows without NaN
+    for r in range(rows):
+        if r % 6 != 1:
+            assert int(raw["key"][r]) == int(np.argmax(m[r]))
+    dk = api.make_desc(api.F32, api.I32, rows, cols, main_op=api.MAIN_KVP,
+                       reduce_op=api.RED_ARGMAX, final_op=api.FIN_KEY, init_i=0,
+                       init_f=-np.inf, plan_hint=plan)
+    keys = u.gpu_reduce(dk, m.reshape(-1))
+    assert np.array_equal(keys, raw["key"])
+
+
+# Arg reduction along the strided dimension (the reference restricts KVP outputs to the
+# contiguous dimension, linalg/strided_reduction.cuh:70-77; here it is supported).
+def test_kvp_strided(gpu):
+    rng = np.random.default_rng(5)
+    rows, cols = 3000, 24
+    m = rng.standard_normal((rows, cols)).astype(np.float32)
+    m[17, 3] = m[2900, 3] = 9.0
+    d = api.make_desc(api.F32, api.KVP_I32_F32, rows, cols, apply=api.ALONG_COLUMNS,
+                      main_op=api.MAIN_KVP, reduce_op=api.RED_ARGMAX, init_i=0, init_f=-np.inf)
+    raw = u.check_against_oracle(d, m.reshape(-1), label="kvp strided")
+    assert int(raw["key"][3]) == 17
+
+
+# Inputs whose device address is not 16-byte aligned take the element-wise load path.
+@pytest.mark.parametrize("in_dt,out_dt", [(api.F32, api.F32), (api.I8, api.I64),
+                                          (api.BF16, api.F32), (api.F64, api.F64)])
+@pytest.mark.parametrize("rows,cols,apply", [(100, 256, api.ALONG_ROWS),
+                                             (9, 40000, api.ALONG_ROWS),
+                                             (2000, 8, api.ALONG_ROWS),
+                                             (4000, 64, api.ALONG_COLUMNS)])
+def test_unaligned_input(gpu, in_dt, out_dt, rows, cols, apply):
+    rng = np.random.default_rng(3)
+    data = _rand(rng, in_dt, rows * cols)
+    d = api.make_desc(in_dt, out_dt, rows, cols, apply=apply)
+    u.check_against_oracle(d, data, misalign_elems=1, label="unaligned")
+
+
+# Empty extents: no rows -> nothing written; no columns -> final_op(init) per output
+# (and red(old, init) when inplace).
+def test_empty_inputs(gpu):
+    data = np.zeros(0, dtype=np.float32)
+    d = api.make_desc(api.F32, api.F32, 0, 128)
+    assert u.gpu_reduce(d, data).size == 0
+    d = api.make_desc(api.F32, api.F32, 5, 0, init_f=2.0, final_op=api.FIN_SQ)
+    assert u.gpu_reduce(d, data).tolist() == [4.0] * 5
+    d = api.make_desc(api.F32, api.F32, 5, 0, init_f=0.0, inplace=True)
+    old = np.arange(5, dtype=np.float32)
+    assert u.gpu_reduce(d, data, old_raw=old).tolist() == old.tolist()
+    d = api.make_desc(api.F32, api.F32, 0, 7, apply=api.ALONG_COLUMNS, init_f=1.5)
+    assert u.gpu_reduce(d, data).tolist() == [1.5] * 7
+    di = api.make_desc(api.I8, api.I64, 3, 0, init_i=7)
+    assert u.gpu_reduce(di, np.zeros(0, dtype=np.int8)).tolist() == [7, 7, 7]
+
+
+# Mean with the reference's rounding of 1/N (stats/detail/mean.cuh:22,39), incl. the
+# int8 -> half case of cpp/tests/stats/mean.cu:177-185.
+@pytest.mark.parametrize("in_dt,out_dt", [(api.F32, api.F32), (api.F64, api.F64),
+                                          (api.F16, api.F32), (api.I8, api.F16)])
+@pytest.mark.parametrize("rows,cols", [(1024, 32), (1024, 64), (8000, 128), (20000, 2)])
+@pytest.mark.parametrize("row_major", [True, False])
+def test_mean(gpu, in_dt, out_dt, rows, cols, row_major):
+    rng = np.random.default_rng(rows + cols)
+    if in_dt == api.I8:
+        data = rng.integers(-20, 30, rows * cols, dtype=np.int8)
+    else:
+        data = _rand(rng, in_dt, rows * cols, -3, 5)
+    ratio = {api.F32: np.float32, api.F64: np.float64, api.F16: np.float16}[out_dt](1.0) / rows
+    d = api.make_desc(in_dt, out_dt, rows, cols, apply=api.ALONG_COLUMNS,
+                      layout=api.ROW_MAJOR if row_major else api.COL_MAJOR,
+                      final_op=api.FIN_MUL_CONST, final_scalar=float(ratio))
+    u.check_against_oracle(d, data, label="mean")
+
+
+# Results do not depend on run-to-run scheduling: no atomics anywhere.
+def test_bitwise_repeatable(gpu):
+    rng = np.random.default_rng(9)
+    for rows, cols, apply in [(4, 300000, api.ALONG_ROWS), (200000, 64, api.ALONG_COLUMNS),
+                              (50000, 128, api.ALONG_ROWS)]:
+        data = rng.standard_normal(rows * cols).astype(np.float32)
+        d = api.make_desc(api.F32, api.F32, rows, cols, apply=apply)
+        a = u.gpu_reduce(d, data)
+        for _ in range(3):
+            assert np.array_equal(a, u.gpu_reduce(d, data))

@@ -1,0 +1,275 @@
+"""Pins the CPU oracle (oracle/oracle.cpp): every known-answer fixture the reference's
+tests hold for the reduction path, plus closed forms and numpy routines on random
+inputs chosen so that a dropped term, a wrong stride or a swapped axis fails."""
+import itertools
+
+import numpy as np
+import pytest
+
+from raft_amd import _capi as api
+from tests import _util as u
+
+
+# cpp/tests/linalg/reduce.cu:108-177
+@pytest.mark.parametrize("layout,apply,expected", [
+    (api.ROW_MAJOR, api.ALONG_ROWS, [4, 8, 12]),
+    (api.ROW_MAJOR, api.ALONG_COLUMNS, [9, 10, 11, 12]),
+    (api.COL_MAJOR, api.ALONG_ROWS, [10, 11, 12]),
+    (api.COL_MAJOR, api.ALONG_COLUMNS, [3, 6, 9, 12]),
+])
+def test_simple_max_fixture(oracle, layout, apply, expected):
+    data = np.arange(1, 13, dtype=np.float32)
+    d = api.make_desc(api.F32, api.F32, 3, 4, layout=layout, apply=apply, reduce_op=api.RED_MAX)
+    assert u.oracle_reduce(d, data).tolist() == expected
+    out = np.zeros(len(expected), dtype=np.float32)
+    assert u.oracle_typed(d, data, out).tolist() == expected
+
+
+# cpp/tests/matrix/argmax.cu:71-75, argmin.cu:71-75
+def test_argmax_argmin_fixture(oracle):
+    data = np.array([0.1, 0.2, 0.3, 0.4, 0.4, 0.3, 0.2, 0.1, 0.2, 0.3, 0.5, 0.0], np.float32)
+    d = api.make_desc(api.F32, api.I32, 3, 4, main_op=api.MAIN_KVP, reduce_op=api.RED_ARGMAX,
+                      final_op=api.FIN_KEY, init_f=-np.inf)
+    assert u.oracle_reduce(d, data)[0].tolist() == [3, 0, 2]
+    out = np.zeros(3, dtype=np.int32)
+    assert u.oracle_typed(d, data, out).tolist() == [3, 0, 2]
+    d = api.make_desc(api.F32, api.I32, 3, 4, main_op=api.MAIN_KVP, reduce_op=api.RED_ARGMIN,
+                      final_op=api.FIN_KEY, init_f=np.inf)
+    assert u.oracle_reduce(d, data)[0].tolist() == [0, 3, 3]
+    assert u.oracle_typed(d, data, out).tolist() == [0, 3, 3]
+
+
+# cpp/tests/util/reduction.cu:167-171,179-181
+def test_vector64_fixture(oracle):
+    from tests.test_gpu_fixtures import VEC64
+    x = np.array(VEC64, dtype=np.int32)
+    for red, init, want in [(api.RED_MIN, 2**62, 0), (api.RED_MAX, -2**62, 5),
+                            (api.RED_ADD, 0, 158)]:
+        d = api.make_desc(api.I32, api.I64, 1, 64, reduce_op=red, init_i=init)
+        assert u.oracle_reduce(d, x).tolist() == [want]
+    xf = x.astype(np.float32)
+    d = api.make_desc(api.F32, api.KVP_I32_F32, 1, 64, main_op=api.MAIN_KVP,
+                      reduce_op=api.RED_ARGMAX, init_f=-np.inf)
+    k, v = u.oracle_reduce(d, xf)
+    assert (k[0], v[0]) == (15, 5.0)
+    d = api.make_desc(api.F32, api.KVP_I32_F32, 1, 64, main_op=api.MAIN_KVP,
+                      reduce_op=api.RED_ARGMIN, init_f=np.inf)
+    k, v = u.oracle_reduce(d, xf)
+    assert (k[0], v[0]) == (26, 0.0)
+
+
+# cpp/tests/core/operators_host.cpp:134-172: truth table of argmin_op / argmax_op on
+# a=(0,1.2) b=(0,3.4) c=(1,1.2), in both argument orders.  A two-element row plus
+# `init` plays the two operands.
+def _arg2(red, first, second):
+    """fold of [first, second] where each is (key, value): keys are forced through
+    init (key of `first`) and a one-element row whose index is the key of `second`."""
+    kf, vf = first
+    ks, vs = second
+    row = np.full(ks + 1, np.nan, dtype=np.float32)  # NaN never wins, pads the index
+    row[ks] = vs
+    d = api.make_desc(api.F32, api.KVP_I32_F32, 1, ks + 1, main_op=api.MAIN_KVP,
+                      reduce_op=red, init_i=kf, init_f=vf)
+    k, v = u.oracle_reduce(d, row)
+    return int(k[0]), float(np.float32(v[0]))
+
+
+def test_arg_op_truth_table(oracle):
+    a, b, c = (0, np.float32(1.2)), (0, np.float32(3.4)), (1, np.float32(1.2))
+    f = lambda kv: (kv[0], float(kv[1]))
+    for red, table in [
+        (api.RED_ARGMIN, [(a, b, a), (b, a, a), (a, c, a), (c, a, a), (b, c, c), (c, b, c)]),
+        (api.RED_ARGMAX, [(a, b, b), (b, a, b), (a, c, a), (c, a, a), (b, c, b), (c, b, b)]),
+    ]:
+        for x, y, want in table:
+            assert _arg2(red, x, y) == f(want), (red, x, y)
+
+
+# cpp/tests/stats/sum.cu:50-98: triples (3v, -vL, +vL) must still sum to rows*v.
+@pytest.mark.parametrize("npdt,dt,v,L", [(np.float32, api.F32, 1e-4, 1e7),
+                                         (np.float64, api.F64, 1e-6, 1e12)])
+def test_sum_compensation_fixture(oracle, npdt, dt, v, L):
+    rows, cols = 1024, 32
+    m = np.full((rows, cols), v, dtype=np.float64)
+    for r in range(2, rows, 3):
+        m[r], m[r - 1], m[r - 2] = v * L, -v * L, 3 * v
+    m = m.astype(npdt)
+    d = api.make_desc(dt, dt, rows, cols, apply=api.ALONG_COLUMNS)
+    # the typed implementation carries the reference's compensation term
+    out = np.zeros(cols, dtype=npdt)
+    u.oracle_typed(d, m.reshape(-1), out)
+    tol = 0.1 if npdt == np.float32 else 0.01
+    assert u.approx_ok(out, np.full(cols, rows * float(npdt(v))), tol).all()
+    # the fp64 oracle on fp32 data is exact to far below that
+    if npdt == np.float32:
+        seq = u.oracle_reduce(d, m.reshape(-1))
+        assert u.approx_ok(seq, np.full(cols, rows * float(np.float32(v))), 1e-6).all()
+
+
+# cpp/tests/stats/stddev.cu:139-150,187-190,198-202
+def test_stddev_fixtures(oracle):
+    rows, cols = 4096, 2
+    data = np.full(rows * cols, 1.25, dtype=np.float32)
+    mu = np.full(cols, 1.25)
+    for sample in (False, True):
+        r = 1.0 / (rows - 1 if sample else rows)
+        rm = r * rows if sample else 1.0
+        ds = api.make_desc(api.F32, api.F32, rows, cols, apply=api.ALONG_COLUMNS,
+                           main_op=api.MAIN_SQ, final_op=api.FIN_STDDEV_FROM_SUMSQ,
+                           final_scalar=r, final_scalar2=rm)
+        sd = u.oracle_reduce(ds, data, aux=mu)
+        assert np.all(np.abs(sd) < 1e-6)
+        ds.final_op = api.FIN_VAR_FROM_SUMSQ
+        var = u.oracle_reduce(ds, data, aux=mu)
+        assert np.allclose(np.sqrt(var), sd)
+
+
+# cpp/tests/linalg/map_then_reduce.cu:140-169
+def test_map_reduce_planted(oracle):
+    rng = np.random.default_rng(1234)
+    x = rng.uniform(2.0, 3.0, 1237).astype(np.float32)
+    x[42], x[337] = 1.0, 5.0
+    d = api.make_desc(api.F32, api.F32, 1, x.size, reduce_op=api.RED_MIN, init_f=np.inf)
+    assert u.oracle_reduce(d, x).tolist() == [1.0]
+    d = api.make_desc(api.F32, api.F32, 1, x.size, reduce_op=api.RED_MAX, init_f=-np.inf)
+    assert u.oracle_reduce(d, x).tolist() == [5.0]
+
+
+# What the mathematics fixes: numpy's own reductions on a non-square random matrix for
+# all four layout x axis combinations (a swapped stride or axis changes the answer).
+@pytest.mark.parametrize("layout,apply", itertools.product([api.ROW_MAJOR, api.COL_MAJOR],
+                                                           [api.ALONG_ROWS, api.ALONG_COLUMNS]))
+def test_against_numpy_closed_forms(oracle, layout, apply):
+    rng = np.random.default_rng(7)
+    rows, cols = 13, 29
+    m = rng.standard_normal((rows, cols))
+    flat = m.reshape(-1) if layout == api.ROW_MAJOR else m.T.reshape(-1)
+    flat = np.ascontiguousarray(flat)
+    ax = 1 if apply == api.ALONG_ROWS else 0
+    cases = [
+        (api.MAIN_IDENTITY, api.RED_ADD, api.FIN_IDENTITY, 0.0, m.sum(axis=ax)),
+        (api.MAIN_SQ, api.RED_ADD, api.FIN_SQRT, 0.0, np.linalg.norm(m, axis=ax)),
+        (api.MAIN_ABS, api.RED_ADD, api.FIN_IDENTITY, 0.0, np.abs(m).sum(axis=ax)),
+        (api.MAIN_ABS, api.RED_MAX, api.FIN_IDENTITY, 0.0, np.abs(m).max(axis=ax)),
+        (api.MAIN_IDENTITY, api.RED_MIN, api.FIN_IDENTITY, np.inf, m.min(axis=ax)),
+        (api.MAIN_NZ, api.RED_ADD, api.FIN_IDENTITY, 0.0, (m != 0).sum(axis=ax)),
+    ]
+    for main, red, fin, init, want in cases:
+        d = api.make_desc(api.F64, api.F64, rows, cols, layout=layout, apply=apply, main_op=main,
+                          reduce_op=red, final_op=fin, init_f=init)
+        got = u.oracle_reduce(d, flat)
+        assert np.allclose(got, want, rtol=1e-13, atol=0), (main, red)
+        out = np.zeros(len(want))
+        assert np.allclose(u.oracle_typed(d, flat, out), want, rtol=1e-13, atol=0)
+    # mean / population and sample stddev against numpy
+    n = m.shape[1 - ax] if False else (cols if ax == 1 else rows)
+    d = api.make_desc(api.F64, api.F64, rows, cols, layout=layout, apply=apply,
+                      final_op=api.FIN_MUL_CONST, final_scalar=1.0 / n)
+    mu = u.oracle_reduce(d, flat)
+    assert np.allclose(mu, m.mean(axis=ax), rtol=1e-13)
+    for sample in (False, True):
+        r = 1.0 / (n - 1 if sample else n)
+        rm = r * n if sample else 1.0
+        d = api.make_desc(api.F64, api.F64, rows, cols, layout=layout, apply=apply,
+                          main_op=api.MAIN_SQ, final_op=api.FIN_STDDEV_FROM_SUMSQ,
+                          final_scalar=r, final_scalar2=rm)
+        sd = u.oracle_reduce(d, flat, aux=mu)
+        assert np.allclose(sd, m.std(axis=ax, ddof=1 if sample else 0), rtol=1e-10)
+    # arg reductions against numpy's first-extremum rule, with planted ties
+    mt = m.copy()
+    mt[:, 5] = mt[:, 20] = 50.0
+    mt[3, :] = mt[9, :] = -50.0
+    flat_t = np.ascontiguousarray(mt.reshape(-1) if layout == api.ROW_MAJOR else mt.T.reshape(-1))
+    d = api.make_desc(api.F64, api.KVP_I64_F64, rows, cols, layout=layout, apply=apply,
+                      main_op=api.MAIN_KVP, reduce_op=api.RED_ARGMAX, init_f=-np.inf)
+    k, v = u.oracle_reduce(d, flat_t)
+    assert np.array_equal(k, np.argmax(mt, axis=ax)) and np.array_equal(v, mt.max(axis=ax))
+    d.reduce_op = api.RED_ARGMIN
+    d.init.f = np.inf
+    k, v = u.oracle_reduce(d, flat_t)
+    assert np.array_equal(k, np.argmin(mt, axis=ax)) and np.array_equal(v, mt.min(axis=ax))
+
+
+# inplace: dots = final(red(dots_old, acc)) -- tests/linalg/reduce.cuh:42-46
+def test_inplace_and_init(oracle):
+    x = np.arange(12, dtype=np.float64)
+    d = api.make_desc(api.F64, api.F64, 3, 4, main_op=api.MAIN_SQ, final_op=api.FIN_SQRT,
+                      inplace=True)
+    old = np.array([1.0, 2.0, 3.0])
+    want = np.sqrt(old + (x.reshape(3, 4) ** 2).sum(axis=1))
+    assert np.allclose(u.oracle_reduce(d, x, old=old), want, rtol=1e-15)
+    out = old.copy()
+    assert np.allclose(u.oracle_typed(d, x, out), want, rtol=1e-15)
+    di = api.make_desc(api.I32, api.I64, 3, 4, init_i=0, final_op=api.FIN_MUL_CONST,
+                       final_scalar=3)
+    xi = np.arange(12, dtype=np.int32)
+    assert u.oracle_reduce(di, xi).tolist() == (3 * xi.reshape(3, 4).sum(axis=1)).tolist()
+
+
+# integers: exact against numpy in int64, all integer input types
+@pytest.mark.parametrize("dt,npdt", [(api.I8, np.int8), (api.U8, np.uint8), (api.I32, np.int32),
+                                     (api.I64, np.int64)])
+def test_integer_sums_exact(oracle, dt, npdt):
+    rng = np.random.default_rng(11)
+    info = np.iinfo(npdt)
+    lo, hi = max(info.min, -2**40), min(info.max, 2**40)
+    m = rng.integers(lo, hi, (37, 1001), dtype=npdt)
+    for main, f in [(api.MAIN_IDENTITY, lambda a: a), (api.MAIN_ABS, np.abs)]:
+        d = api.make_desc(dt, api.I64, 37, 1001, main_op=main)
+        want = f(m.astype(np.int64)).sum(axis=1)
+        assert np.array_equal(u.oracle_reduce(d, m.reshape(-1)), want)
+        out = np.zeros(37, dtype=np.int64)
+        assert np.array_equal(u.oracle_typed(d, m.reshape(-1), out), want)
+
+
+# storage conversions against numpy's float16 and a bit-level bf16 rule
+def test_storage_conversions(oracle):
+    import ctypes as C
+    rng = np.random.default_rng(3)
+    x = np.concatenate([rng.standard_normal(4000).astype(np.float32) * 100,
+                        np.array([0.0, -0.0, 1e-8, -1e-8, 65504, 70000, 6e-8, np.inf, -np.inf],
+                                 dtype=np.float32)])
+    h = np.empty(x.size, dtype=np.uint16)
+    oracle.orc_f32_to_f16(x.ctypes.data, h.ctypes.data, x.size)
+    assert np.array_equal(h, x.astype(np.float16).view(np.uint16))
+    back = np.empty(x.size, dtype=np.float32)
+    oracle.orc_f16_to_f32(h.ctypes.data, back.ctypes.data, x.size)
+    assert np.array_equal(back, h.view(np.float16).astype(np.float32))
+    allh = np.arange(65536, dtype=np.uint16)
+    backall = np.empty(65536, dtype=np.float32)
+    oracle.orc_f16_to_f32(allh.ctypes.data, backall.ctypes.data, 65536)
+    ref = allh.view(np.float16).astype(np.float32)
+    assert np.array_equal(backall.view(np.uint32), ref.view(np.uint32))
+    b = u.to_bf16(x)
+    bits = x.view(np.uint32).astype(np.uint64)
+    want = ((bits + 0x7fff + ((bits >> 16) & 1)) >> 16).astype(np.uint16)
+    assert np.array_equal(b, want)
+    assert np.array_equal(u.from_bf16(b).view(np.uint32), b.astype(np.uint32) << 16)
+
+
+# the OpenMP implementation agrees with the sequential oracle on the benchmark's
+# kinds of input, to the build's floating tolerance / exactly for integers and keys
+def test_typed_matches_sequential(oracle):
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal(3000 * 128).astype(np.float32)
+    d = api.make_desc(api.F32, api.F32, 3000, 128, main_op=api.MAIN_SQ, final_op=api.FIN_SQRT)
+    out = np.zeros(3000, dtype=np.float32)
+    assert u.fp_close(u.oracle_typed(d, x, out), u.oracle_reduce(d, x)).all()
+    x = (3 + 2 * rng.standard_normal(40000 * 64)).astype(np.float32)
+    d = api.make_desc(api.F32, api.F32, 40000, 64, apply=api.ALONG_COLUMNS,
+                      final_op=api.FIN_MUL_CONST, final_scalar=1.0 / 40000)
+    out = np.zeros(64, dtype=np.float32)
+    assert u.fp_close(u.oracle_typed(d, x, out), u.oracle_reduce(d, x)).all()
+    m = rng.standard_normal((50, 32000)).astype(np.float32)
+    m[:, 100] = m[:, 31000] = 7.0
+    d = api.make_desc(api.F32, api.KVP_I32_F32, 50, 32000, main_op=api.MAIN_KVP,
+                      reduce_op=api.RED_ARGMAX, init_f=-np.inf)
+    out = np.zeros(50, dtype=u.KVP_NP[api.KVP_I32_F32])
+    u.oracle_typed(d, m.reshape(-1), out)
+    k, v = u.oracle_reduce(d, m.reshape(-1))
+    assert np.array_equal(out["key"], k) and (k == 100).all()
+    assert np.array_equal(out["value"].astype(np.float64), v)
+    xb = u.to_bf16(rng.uniform(-1, 1, 2 * 100000).astype(np.float32))
+    d = api.make_desc(api.BF16, api.F32, 2, 100000)
+    out = np.zeros(2, dtype=np.float32)
+    assert u.fp_close(u.oracle_typed(d, xb, out), u.oracle_reduce(d, xb)).all()
