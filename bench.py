@@ -1,0 +1,444 @@
+#!/usr/bin/env python3
+"""Benchmark of the dense-reduction path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--configs all|headline]
+
+A "step" is one reduction call (one pass of the hot path over one matrix).  The
+headline workload is the L2 row norm of a row-major fp32 1,000,000 x 128 matrix
+(N(0,1), sqrt fused); the other benchmark shapes are timed the same way and
+reported under "configs".  Inputs are generated on the device from fixed seeds and
+are resident in HBM before timing starts; consecutive steps read different
+buffers whose total size exceeds the 256 MB Infinity Cache, so every step streams
+from HBM.  Timing uses HIP events recorded on the stream the kernels run on.
+
+Prints one JSON line.  `roofline.achieved` = algorithmic bytes (input read once +
+output written once) / average launch duration.  `cpu_baseline` times the OpenMP
+host implementation of the same semantics (oracle/, kind "port") on this
+machine's cores.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+
+PEAK_HBM_GBPS = 8000.0  # MI355X published HBM3E bandwidth
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--configs", default="all",
+                    help="all | headline | comma list of cfg names (cfg1,cfg2,cfg3_mean,...)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-check", action="store_true", help="skip the correctness gate")
+    ap.add_argument("--only-kernel", default=None,
+                    help="run just this config's launches (for rocprofv3), no JSON extras")
+    return ap.parse_args()
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (the reduction path shards by rows "
+              "with no exchange; no multi-GPU figure is produced). Use --gpus 1.",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+
+    from raft_amd import _capi as api
+    from raft_amd import device as dev
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(3)
+    lib = api.load()
+    torch.cuda.set_device(0)
+    devc = torch.device("cuda:0")
+    stream = torch.cuda.current_stream()
+    sptr = stream.cuda_stream
+
+    def gen(seed):
+        g = torch.Generator(device=devc)
+        g.manual_seed(seed)
+        return g
+
+    # ------------------------------------------------------------------
+    # workloads
+    # ------------------------------------------------------------------
+    def mk_normal(rows, cols, seed, mean=0.0, std=1.0):
+        x = torch.randn(rows * cols, generator=gen(seed), device=devc, dtype=torch.float32)
+        if std != 1.0:
+            x.mul_(std)
+        if mean != 0.0:
+            x.add_(mean)
+        return x
+
+    def mk_uniform(rows, cols, seed):
+        x = torch.rand(rows * cols, generator=gen(seed), device=devc, dtype=torch.float32)
+        return x.mul_(2.0).sub_(1.0)
+
+    def mk_int8(rows, cols, seed):
+        return torch.randint(-128, 128, (rows * cols,), generator=gen(seed), device=devc,
+                             dtype=torch.int8)
+
+    def mk_bf16(rows, cols, seed):
+        return mk_uniform(rows, cols, seed).to(torch.bfloat16)
+
+    def mk_logits_with_ties(rows, cols, seed):
+        x = mk_normal(rows, cols, seed).view(rows, cols)
+        g = gen(seed + 1000)
+        n_tie = max(1, rows // 100)
+        tie_rows = torch.randperm(rows, generator=g, device=devc)[:n_tie]
+        mx = x[tie_rows].amax(dim=1)
+        for j in range(3):  # 1..3 further copies of the row maximum
+            pos = torch.randint(0, cols, (n_tie,), generator=g, device=devc)
+            keep = torch.rand(n_tie, generator=g, device=devc) < (1.0 if j == 0 else 0.5)
+            sel = tie_rows[keep]
+            x[sel, pos[keep]] = mx[keep]
+        return x.view(-1)
+
+    f32 = np.float32
+    WORK = {
+        # name: (description, maker, rows, cols, desc kwargs, out dtype bytes)
+        "cfg1": dict(desc="row sum fp32 10000x256 U[-1,1) seed 0", make=lambda s: mk_uniform(10000, 256, s),
+                     seed=0, rows=10000, cols=256, in_dt=api.F32, out_dt=api.F32, kw={}),
+        "cfg2": dict(desc="L2 row norm (sqrt) fp32 1000000x128 N(0,1)", make=lambda s: mk_normal(1000000, 128, s),
+                     seed=2, rows=1000000, cols=128, in_dt=api.F32, out_dt=api.F32,
+                     kw=dict(main_op=api.MAIN_SQ, final_op=api.FIN_SQRT)),
+        "cfg3_mean": dict(desc="column mean fp32 10000000x64 N(3,2)", make=lambda s: mk_normal(10000000, 64, s, 3.0, 2.0),
+                          seed=3, rows=10000000, cols=64, in_dt=api.F32, out_dt=api.F32,
+                          kw=dict(apply=api.ALONG_COLUMNS, final_op=api.FIN_MUL_CONST,
+                                  final_scalar=float(f32(1.0) / f32(10000000)))),
+        "cfg3_stddev": dict(desc="column stddev fp32 10000000x64 N(3,2)", make=lambda s: mk_normal(10000000, 64, s, 3.0, 2.0),
+                            seed=3, rows=10000000, cols=64, in_dt=api.F32, out_dt=api.F32,
+                            kw=dict(apply=api.ALONG_COLUMNS, main_op=api.MAIN_SQ,
+                                    final_op=api.FIN_STDDEV_FROM_SUMSQ,
+                                    final_scalar=float(f32(1.0) / f32(10000000)), final_scalar2=1.0),
+                            needs_mean=True),
+        "cfg4": dict(desc="row argmax (KVP int32,fp32) fp32 65536x32000 N(0,1), ties in 1% of rows",
+                     make=lambda s: mk_logits_with_ties(65536, 32000, s), seed=4, rows=65536, cols=32000,
+                     in_dt=api.F32, out_dt=api.KVP_I32_F32,
+                     kw=dict(main_op=api.MAIN_KVP, reduce_op=api.RED_ARGMAX, init_i=0,
+                             init_f=float("-inf"))),
+        "cfg5a": dict(desc="row sum int8->int64 4096x16384", make=lambda s: mk_int8(4096, 16384, s),
+                      seed=5, rows=4096, cols=16384, in_dt=api.I8, out_dt=api.I64, kw={}),
+        "cfg5b": dict(desc="row sum int8->int64 16777216x8", make=lambda s: mk_int8(16777216, 8, s),
+                      seed=6, rows=16777216, cols=8, in_dt=api.I8, out_dt=api.I64, kw={}),
+        "cfg5c": dict(desc="row sum bf16->fp32 8x4194304 (split rows, two passes)",
+                      make=lambda s: mk_bf16(8, 4194304, s), seed=7, rows=8, cols=4194304,
+                      in_dt=api.BF16, out_dt=api.F32, kw={}),
+    }
+    HEADLINE = "cfg2"
+
+    if args.configs == "all":
+        names = list(WORK)
+    elif args.configs == "headline":
+        names = [HEADLINE]
+    else:
+        names = [n for n in args.configs.split(",") if n]
+    if args.only_kernel:
+        names = [args.only_kernel]
+    if HEADLINE not in names and not args.only_kernel:
+        names.insert(0, HEADLINE)
+
+    def n_out(w):
+        return w["rows"] if w["kw"].get("apply", api.ALONG_ROWS) == api.ALONG_ROWS else w["cols"]
+
+    def alg_bytes(w):
+        return (w["rows"] * w["cols"] * api.DTYPE_SIZE[w["in_dt"]]
+                + n_out(w) * api.DTYPE_SIZE[w["out_dt"]])
+
+    TORCH_OUT = {api.F32: torch.float32, api.I64: torch.int64}
+
+    def run_config(name, steps, warmup, check=True):
+        w = WORK[name]
+        in_bytes = w["rows"] * w["cols"] * api.DTYPE_SIZE[w["in_dt"]]
+        # enough distinct inputs to defeat the 256 MB Infinity Cache, at most ~17 GB
+        nbuf = max(2, min(16, -(-(1 << 30) // in_bytes)))
+        bufs = [w["make"](w["seed"] + 7919 * i) for i in range(nbuf)]
+        no = n_out(w)
+        out_bytes = no * api.DTYPE_SIZE[w["out_dt"]]
+        outs = [torch.zeros(out_bytes, dtype=torch.uint8, device=devc) for _ in range(nbuf)]
+        kw = dict(w["kw"])
+        descs = []
+        aux = []
+        for i in range(nbuf):
+            d = api.make_desc(w["in_dt"], w["out_dt"], w["rows"], w["cols"], **kw)
+            if w.get("needs_mean"):
+                m = bufs[i].view(w["rows"], w["cols"]).mean(dim=0, dtype=torch.float64).to(torch.float32)
+                aux.append(m)
+                d.final_aux = m.data_ptr()
+            descs.append(d)
+        plan = api.plan_query(descs[0])
+        ws_bytes = lib.rmi_reduce_workspace_bytes(C.byref(descs[0]))
+        ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=devc)
+        wsp = ws.data_ptr()
+        in_ptrs = [b.data_ptr() for b in bufs]
+        out_ptrs = [o.data_ptr() for o in outs]
+        refs = [C.byref(d) for d in descs]
+        call = lib.rmi_reduce
+
+        def step(i):
+            j = i % nbuf
+            rc = call(refs[j], in_ptrs[j], out_ptrs[j], wsp, ws_bytes, sptr)
+            if rc != 0:
+                raise RuntimeError(f"{name}: rmi_reduce -> {api.status_string(rc)}")
+
+        for i in range(warmup):
+            step(i)
+        torch.cuda.synchronize()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        e0.record(stream)
+        for i in range(steps):
+            step(i)
+        e1.record(stream)
+        torch.cuda.synchronize()
+        wall_ms = (time.perf_counter() - t0) * 1e3
+        ev_ms = e0.elapsed_time(e1)
+        ms = ev_ms / steps
+        res = dict(workload=w["desc"], plan=api.PLAN_NAME[plan.kind], passes=plan.passes,
+                   grid_blocks=plan.grid_blocks, buffers=nbuf, ms_per_step=ms,
+                   wall_ms_per_step=wall_ms / steps,
+                   alg_bytes=alg_bytes(w), GBps=alg_bytes(w) / (ms * 1e-3) / 1e9,
+                   rows_per_s=w["rows"] / (ms * 1e-3))
+        res["pct_of_peak"] = 100.0 * res["GBps"] / PEAK_HBM_GBPS
+
+        # the same launches replayed from a HIP graph: removes host launch gaps, which
+        # dominate the shapes whose kernel is only a few microseconds long
+        try:
+            gsteps = max(nbuf, min(steps, 64))
+            side = torch.cuda.Stream()
+            side.wait_stream(stream)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.stream(side):
+                gptr = side.cuda_stream
+                with torch.cuda.graph(graph, stream=side):
+                    for i in range(gsteps):
+                        j = i % nbuf
+                        rc = call(refs[j], in_ptrs[j], out_ptrs[j], wsp, ws_bytes, gptr)
+                        assert rc == 0
+            stream.wait_stream(side)
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            reps = max(1, steps // gsteps)
+            e0.record(stream)
+            for _ in range(reps):
+                graph.replay()
+            e1.record(stream)
+            torch.cuda.synchronize()
+            gms = e0.elapsed_time(e1) / (reps * gsteps)
+            res["graph_ms_per_step"] = gms
+            res["graph_GBps"] = alg_bytes(w) / (gms * 1e-3) / 1e9
+            del graph
+        except Exception as ex:  # noqa: BLE001
+            res["graph_error"] = str(ex)[:200]
+
+        # same buffer every step (cache-resident when the input fits the Infinity Cache)
+        if in_bytes <= (256 << 20):
+            for i in range(5):
+                call(refs[0], in_ptrs[0], out_ptrs[0], wsp, ws_bytes, sptr)
+            torch.cuda.synchronize()
+            e0.record(stream)
+            for i in range(steps):
+                call(refs[0], in_ptrs[0], out_ptrs[0], wsp, ws_bytes, sptr)
+            e1.record(stream)
+            torch.cuda.synchronize()
+            cms = e0.elapsed_time(e1) / steps
+            res["same_buffer_ms_per_step"] = cms
+            res["same_buffer_GBps"] = alg_bytes(w) / (cms * 1e-3) / 1e9
+
+        if check:
+            res["check"] = check_config(name, w, bufs[0], outs[0], aux[0] if aux else None)
+        return res, bufs, outs
+
+    # ------------------------------------------------------------------
+    # correctness gate: oracle on a bounded sample + full-size properties
+    # ------------------------------------------------------------------
+    def check_config(name, w, buf, out_raw, aux):
+        from tests import _util as u
+        rows, cols = w["rows"], w["cols"]
+        info = {}
+        kw = dict(w["kw"])
+        if w["out_dt"] == api.KVP_I32_F32:
+            kv = out_raw.view(torch.int32).view(rows, 2)
+            keys = kv[:, 0].to(torch.int64)
+            vals = kv[:, 1].contiguous().view(torch.float32)
+            x = buf.view(rows, cols)
+            ok = True
+            for r0 in range(0, rows, 4096):
+                blk = x[r0:r0 + 4096]
+                mx = blk.amax(dim=1)
+                eq = blk == mx[:, None]
+                ar = torch.arange(cols, device=devc, dtype=torch.int64)
+                first = torch.where(eq, ar[None, :], torch.full((), cols, device=devc, dtype=torch.int64)).amin(dim=1)
+                ok &= bool(torch.equal(first, keys[r0:r0 + 4096]))
+                ok &= bool(torch.equal(mx, vals[r0:r0 + 4096]))
+            info["full_size_first_max_property"] = ok
+            ns = 256
+            sample = buf.view(rows, cols)[:ns].contiguous().cpu().numpy().reshape(-1)
+            d = api.make_desc(w["in_dt"], w["out_dt"], ns, cols, **kw)
+            ek, ev = u.oracle_reduce(d, sample)
+            gk = keys[:ns].cpu().numpy()
+            gv = vals[:ns].cpu().numpy().astype(np.float64)
+            info["oracle_sample_rows"] = ns
+            info["oracle_exact"] = bool(np.array_equal(gk, ek) and np.array_equal(gv, ev))
+            info["pass"] = ok and info["oracle_exact"]
+            return info
+        along_rows = kw.get("apply", api.ALONG_ROWS) == api.ALONG_ROWS
+        if along_rows:
+            ns = min(rows, max(1, (32 << 20) // (cols * api.DTYPE_SIZE[w["in_dt"]])))
+            tsample = buf.view(rows, cols)[:ns].contiguous()
+            sample = (tsample.view(torch.int16).cpu().numpy().view(np.uint16) if w["in_dt"] == api.BF16
+                      else tsample.cpu().numpy()).reshape(-1)
+            d = api.make_desc(w["in_dt"], w["out_dt"], ns, cols, **kw)
+            exp = u.oracle_reduce(d, sample)
+            got = out_raw.view(TORCH_OUT[w["out_dt"]])[:ns].cpu().numpy()
+            info["oracle_sample_rows"] = ns
+            if w["out_dt"] == api.I64:
+                info["oracle_exact"] = bool(np.array_equal(got, exp))
+                # full size: total of all row sums against an independent device reduction
+                tot = int(out_raw.view(torch.int64).sum().item())
+                ref = int(buf.view(-1).to(torch.int64).sum().item()) if buf.numel() <= (1 << 28) else \
+                    sum(int(c.to(torch.int64).sum().item()) for c in buf.view(-1).split(1 << 28))
+                info["full_size_checksum_equal"] = tot == ref
+                info["pass"] = info["oracle_exact"] and info["full_size_checksum_equal"]
+            else:
+                okv = u.fp_close(got, exp)
+                info["worst_rel_err_vs_fp64"] = u.worst_rel(got, exp)
+                info["pass"] = bool(okv.all())
+        else:
+            # strided: fp64 reference over the whole matrix on the device (independent
+            # implementation), plus the CPU oracle on the first 200k rows as its own problem
+            x = buf.view(rows, cols)
+            if name == "cfg3_mean":
+                ref = x.mean(dim=0, dtype=torch.float64).cpu().numpy()
+            else:
+                ref = x.to(torch.float64).std(dim=0, unbiased=False).cpu().numpy() \
+                    if rows * cols <= (1 << 28) else \
+                    torch.sqrt(torch.clamp((sum((c.to(torch.float64) ** 2).sum(dim=0) for c in x.split(1 << 21)) / rows)
+                               - x.mean(dim=0, dtype=torch.float64) ** 2, min=0)).cpu().numpy()
+            got = out_raw.view(torch.float32).cpu().numpy()
+            info["worst_rel_err_vs_fp64_full"] = u.worst_rel(got, ref)
+            ns = 200000
+            sub = x[:ns].contiguous()
+            d = api.make_desc(w["in_dt"], w["out_dt"], ns, cols, **{**kw, "final_scalar": 1.0 / ns})
+            d.final_scalar = float(np.float32(1.0) / np.float32(ns))
+            o = torch.zeros(cols, dtype=torch.float32, device=devc)
+            auxs = None
+            if w.get("needs_mean"):
+                auxs = sub.mean(dim=0, dtype=torch.float64).to(torch.float32)
+                d.final_aux = auxs.data_ptr()
+            dev.reduce(d, sub, o)
+            torch.cuda.synchronize()
+            exp = u.oracle_reduce(d, sub.cpu().numpy().reshape(-1),
+                                  aux=auxs.cpu().numpy().astype(np.float64) if auxs is not None else None)
+            info["oracle_sample_rows"] = ns
+            info["worst_rel_err_vs_fp64_sample"] = u.worst_rel(o.cpu().numpy(), exp)
+            info["pass"] = bool(u.fp_close(got, ref).all() and u.fp_close(o.cpu().numpy(), exp).all())
+        return info
+
+    # ------------------------------------------------------------------
+    # CPU baseline: the OpenMP host implementation on a bounded sample
+    # ------------------------------------------------------------------
+    def cpu_baseline(name, buf):
+        from tests import _util as u
+        w = WORK[name]
+        rows, cols = w["rows"], w["cols"]
+        es = api.DTYPE_SIZE[w["in_dt"]]
+        cap_bytes = 512 << 20
+        kw = dict(w["kw"])
+        ns = min(rows, max(1, cap_bytes // (cols * es)))
+        t = buf.view(rows, cols)[:ns].contiguous()
+        host = (t.view(torch.int16).cpu().numpy().view(np.uint16) if w["in_dt"] == api.BF16
+                else t.cpu().numpy()).reshape(-1)
+        if "final_scalar" in kw and name.startswith("cfg3"):
+            kw["final_scalar"] = float(np.float32(1.0) / np.float32(ns))
+        d = api.make_desc(w["in_dt"], w["out_dt"], ns, cols, **kw)
+        no = ns if kw.get("apply", api.ALONG_ROWS) == api.ALONG_ROWS else cols
+        out = np.zeros(no, dtype=u.out_numpy_dtype(w["out_dt"]))
+        auxh = np.full(no, 3.0, dtype=np.float32) if w.get("needs_mean") else None
+        threads = u.load_oracle().orc_max_threads()
+        try:
+            threads = min(threads, len(os.sched_getaffinity(0)))
+        except AttributeError:
+            pass
+        threads = max(1, threads)
+        u.oracle_typed(d, host, out, aux=auxh, threads=threads)  # warm-up, first touch
+        best = float("inf")
+        for _ in range(5):
+            t0 = time.perf_counter()
+            u.oracle_typed(d, host, out, aux=auxh, threads=threads)
+            best = min(best, time.perf_counter() - t0)
+        nbytes = ns * cols * es + no * api.DTYPE_SIZE[w["out_dt"]]
+        return dict(value=nbytes / best / 1e9, unit="GB/s", cores=threads, kind="port",
+                    sample=f"{ns} of {rows} rows x {cols} cols ({nbytes / 1e6:.0f} MB), "
+                           f"best of 5 after one warm-up, OpenMP schedule(static)",
+                    rows_per_s=ns / best, seconds=best)
+
+    # ------------------------------------------------------------------
+    if args.only_kernel:
+        run_config(args.only_kernel, args.steps, args.warmup, check=False)
+        return
+
+    results = {}
+    cpu = {}
+    for name in names:
+        steps = args.steps
+        res, bufs, outs = run_config(name, steps, args.warmup, check=not args.no_check)
+        results[name] = res
+        if not args.no_cpu:
+            cpu[name] = cpu_baseline(name, bufs[0])
+        del bufs, outs
+        torch.cuda.empty_cache()
+
+    head = results[HEADLINE]
+    line = {
+        "metric": "achieved HBM GB/s, L2 row norm fp32 1000000x128 (algorithmic bytes / kernel time)",
+        "value": head["GBps"],
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": head["ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": WORK[HEADLINE]["desc"], "plan": head["plan"],
+                   "buffers_rotated": head["buffers"], "timing": "hip events on the launch stream"},
+        "rows_per_s": head["rows_per_s"],
+        "pct_of_hbm_peak": head["pct_of_peak"],
+        "roofline": {"bound": "hbm", "achieved": head["GBps"], "peak": PEAK_HBM_GBPS,
+                     "unit": "GB/s", "frac": head["GBps"] / PEAK_HBM_GBPS,
+                     "traffic": MEASURED_TRAFFIC.get(HEADLINE)},
+        "cpu_baseline": cpu.get(HEADLINE),
+        "configs": results,
+        "cpu_baselines": cpu,
+        "device": torch.cuda.get_device_name(0),
+    }
+    print(json.dumps(line))
+
+
+# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs (see
+# profiles/), scaled by the same counters' reading for a copy kernel of known size.
+MEASURED_TRAFFIC: dict[str, float | None] = {}
+
+
+if __name__ == "__main__":
+    main()
