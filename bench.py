@@ -43,6 +43,9 @@ def parse_args():
     ap.add_argument("--no-check", action="store_true", help="skip the correctness gate")
     ap.add_argument("--only-kernel", default=None,
                     help="run just this config's launches (for rocprofv3), no JSON extras")
+    ap.add_argument("--calib-copy", action="store_true",
+                    help="with --only-kernel: also run 5 device copies of 512 MiB, the known-size "
+                         "kernel that rocprofv3 byte counters are scaled against")
     return ap.parse_args()
 
 
@@ -149,7 +152,7 @@ def main():
     else:
         names = [n for n in args.configs.split(",") if n]
     if args.only_kernel:
-        names = [args.only_kernel]
+        names = args.only_kernel.split(",")
     if HEADLINE not in names and not args.only_kernel:
         names.insert(0, HEADLINE)
 
@@ -392,7 +395,15 @@ def main():
 
     # ------------------------------------------------------------------
     if args.only_kernel:
-        run_config(args.only_kernel, args.steps, args.warmup, check=False)
+        for nm in args.only_kernel.split(","):
+            run_config(nm, args.steps, args.warmup, check=False)
+            torch.cuda.empty_cache()
+        if args.calib_copy:
+            a = torch.empty(512 << 20, dtype=torch.uint8, device=devc).random_(0, 255)
+            b = torch.empty_like(a)
+            for _ in range(5):
+                b.copy_(a)
+            torch.cuda.synchronize()
         return
 
     results = {}

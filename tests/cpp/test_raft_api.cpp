@@ -1,0 +1,611 @@
+// GPU tests of the C++ API layer: the reference's reduction-path tests restated
+// against the same names and signatures (raft::linalg::reduce, coalesced_reduction,
+// strided_reduction, norm, map_reduce, raft::stats::mean / stddev / vars / sum,
+// raft::matrix::argmax / argmin).  Expected values come from a sequential host
+// evaluation in double precision written here (the reference compares with naive
+// one-thread-per-output kernels, cpp/tests/linalg/reduce.cuh:27-178) and from the
+// reference's literal fixtures.
+#include <raft/core/device_mdarray.hpp>
+#include <raft/core/device_mdspan.hpp>
+#include <raft/core/device_resources.hpp>
+#include <raft/core/operators.hpp>
+#include <raft/linalg/coalesced_reduction.cuh>
+#include <raft/linalg/map_reduce.cuh>
+#include <raft/linalg/map_then_reduce.cuh>
+#include <raft/linalg/norm.cuh>
+#include <raft/linalg/reduce.cuh>
+#include <raft/linalg/strided_reduction.cuh>
+#include <raft/matrix/argmax.cuh>
+#include <raft/matrix/argmin.cuh>
+#include <raft/stats/mean.cuh>
+#include <raft/stats/stddev.cuh>
+#include <raft/stats/sum.cuh>
+#include <raft/util/cudart_utils.hpp>
+#include <raft/util/itertools.hpp>
+
+#include <cstdint>
+#include <random>
+
+#include "check.hpp"
+
+namespace {
+
+template <typename T>
+std::vector<T> to_host(const T* d, size_t n, hipStream_t s)
+{
+  std::vector<T> h(n);
+  raft::update_host(h.data(), d, n, s);
+  RAFT_HIP_TRY(hipStreamSynchronize(s));
+  return h;
+}
+
+template <typename T>
+std::vector<T> uniform(size_t n, double lo, double hi, unsigned long long seed)
+{
+  std::mt19937_64 g(seed);
+  std::uniform_real_distribution<double> d(lo, hi);
+  std::vector<T> v(n);
+  for (auto& x : v)
+    x = (T)d(g);
+  return v;
+}
+
+template <typename T>
+std::vector<T> normal(size_t n, double mu, double sigma, unsigned long long seed)
+{
+  std::mt19937_64 g(seed);
+  std::normal_distribution<double> d(mu, sigma);
+  std::vector<T> v(n);
+  for (auto& x : v)
+    x = (T)d(g);
+  return v;
+}
+
+// element (i, j) of an N x D matrix
+inline size_t at(bool row_major, size_t N, size_t D, size_t i, size_t j)
+{
+  return row_major ? i * D + j : i + j * N;
+}
+
+// dots = final(inplace ? red(old, fold) : fold), fold in double
+template <typename In, typename Main, typename Red, typename Fin>
+std::vector<double> host_reduce(const std::vector<In>& data, size_t N, size_t D, bool row_major,
+                                bool along_rows, double init, const std::vector<double>* old,
+                                Main main_op, Red red_op, Fin fin_op)
+{
+  const size_t n_out = along_rows ? N : D, len = along_rows ? D : N;
+  std::vector<double> out(n_out);
+  for (size_t k = 0; k < n_out; ++k) {
+    double acc = init;
+    for (size_t r = 0; r < len; ++r) {
+      const size_t idx = along_rows ? at(row_major, N, D, k, r) : at(row_major, N, D, r, k);
+      acc              = red_op(acc, main_op((double)data[idx], (int)r));
+    }
+    if (old) acc = red_op((*old)[k], acc);
+    out[k] = fin_op(acc);
+  }
+  return out;
+}
+
+template <typename T>
+bool all_close(const std::vector<T>& got, const std::vector<double>& want, double eps)
+{
+  if (got.size() != want.size()) return false;
+  t::CompareApprox<double> cmp(eps);
+  for (size_t i = 0; i < got.size(); ++i)
+    if (!cmp((double)got[i], want[i])) {
+      std::printf("  mismatch at %zu: got %.9g want %.9g\n", i, (double)got[i], want[i]);
+      return false;
+    }
+  return true;
+}
+
+// ---------------------------------------------------------------------------
+// cpp/tests/linalg/reduce.cu:106-178 simpleTest
+// ---------------------------------------------------------------------------
+template <typename T>
+void simple_max()
+{
+  raft::resources handle;
+  auto stream = raft::resource::get_cuda_stream(handle);
+  std::vector<T> data_h{1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12};
+  const std::uint32_t rows = 3, cols = 4;
+  for (int along_rows = 0; along_rows < 2; ++along_rows) {
+    auto output = raft::make_device_vector<T, std::uint32_t>(handle, along_rows ? rows : cols);
+    {
+      auto data = raft::make_device_matrix<T, std::uint32_t, raft::row_major>(handle, rows, cols);
+      raft::copy(data.data_handle(), data_h.data(), data.size(), stream);
+      std::vector<T> want;
+      if (along_rows) {
+        raft::linalg::reduce<raft::Apply::ALONG_ROWS>(handle, raft::make_const_mdspan(data.view()),
+                                                      output.view(), T(0), false,
+                                                      raft::identity_op(), raft::max_op(),
+                                                      raft::identity_op());
+        want = {4, 8, 12};
+      } else {
+        raft::linalg::reduce<raft::Apply::ALONG_COLUMNS>(
+          handle, raft::make_const_mdspan(data.view()), output.view(), T(0), false,
+          raft::identity_op(), raft::max_op(), raft::identity_op());
+        want = {9, 10, 11, 12};
+      }
+      CHECK(to_host(output.data_handle(), want.size(), stream) == want);
+    }
+    {
+      auto data = raft::make_device_matrix<T, std::uint32_t, raft::col_major>(handle, rows, cols);
+      raft::copy(data.data_handle(), data_h.data(), data.size(), stream);
+      std::vector<T> want;
+      if (along_rows) {
+        raft::linalg::reduce<raft::Apply::ALONG_ROWS>(handle, raft::make_const_mdspan(data.view()),
+                                                      output.view(), T(0), false,
+                                                      raft::identity_op(), raft::max_op(),
+                                                      raft::identity_op());
+        want = {10, 11, 12};
+      } else {
+        raft::linalg::reduce<raft::Apply::ALONG_COLUMNS>(
+          handle, raft::make_const_mdspan(data.view()), output.view(), T(0), false,
+          raft::identity_op(), raft::max_op(), raft::identity_op());
+        want = {3, 6, 9, 12};
+      }
+      CHECK(to_host(output.data_handle(), want.size(), stream) == want);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// cpp/tests/linalg/reduce.cu:180-341 fullTest: sq_op / add_op / sqrt_op, first
+// inplace=false then inplace=true on the same output.
+// ---------------------------------------------------------------------------
+template <typename In, typename Out, typename Idx>
+void reduce_full(double tol, std::vector<int> rows_list, std::vector<int> cols_list)
+{
+  raft::resources handle;
+  auto stream = raft::resource::get_cuda_stream(handle);
+  for (int rows : rows_list)
+    for (int cols : cols_list)
+      for (int rm = 0; rm < 2; ++rm)
+        for (int ar = 0; ar < 2; ++ar) {
+          const size_t len = (size_t)rows * cols;
+          auto data_h      = uniform<In>(len, -1.0, 1.0, 1234);
+          const Idx n_out  = ar ? rows : cols;
+          auto data_d      = raft::make_device_vector<In, Idx>(handle, (Idx)len);
+          auto dots        = raft::make_device_vector<Out, Idx>(handle, n_out);
+          raft::update_device(data_d.data_handle(), data_h.data(), len, stream);
+          auto sq   = [](double x, int) { return x * x; };
+          auto add  = [](double a, double b) { return a + b; };
+          auto sqr  = [](double x) { return std::sqrt(x); };
+          auto run  = [&](bool inplace) {
+            auto out_view = raft::make_device_vector_view<Out, Idx>(dots.data_handle(), n_out);
+            if (rm) {
+              auto v = raft::make_device_matrix_view<const In, Idx, raft::row_major>(
+                data_d.data_handle(), (Idx)rows, (Idx)cols);
+              if (ar) {
+                raft::linalg::reduce<raft::Apply::ALONG_ROWS>(handle, v, out_view, Out(0), inplace,
+                                                              raft::sq_op(), raft::add_op(),
+                                                              raft::sqrt_op());
+              } else {
+                raft::linalg::reduce<raft::Apply::ALONG_COLUMNS>(handle, v, out_view, Out(0),
+                                                                 inplace, raft::sq_op(),
+                                                                 raft::add_op(), raft::sqrt_op());
+              }
+            } else {
+              auto v = raft::make_device_matrix_view<const In, Idx, raft::col_major>(
+                data_d.data_handle(), (Idx)rows, (Idx)cols);
+              if (ar) {
+                raft::linalg::reduce<raft::Apply::ALONG_ROWS>(handle, v, out_view, Out(0), inplace,
+                                                              raft::sq_op(), raft::add_op(),
+                                                              raft::sqrt_op());
+              } else {
+                raft::linalg::reduce<raft::Apply::ALONG_COLUMNS>(handle, v, out_view, Out(0),
+                                                                 inplace, raft::sq_op(),
+                                                                 raft::add_op(), raft::sqrt_op());
+              }
+            }
+          };
+          run(false);
+          auto first = to_host(dots.data_handle(), (size_t)n_out, stream);
+          auto want  = host_reduce(data_h, rows, cols, rm, ar, 0.0, nullptr, sq, add, sqr);
+          CHECK(all_close(first, want, tol));
+          run(true);
+          std::vector<double> old(first.begin(), first.end());
+          auto want2 = host_reduce(data_h, rows, cols, rm, ar, 0.0, &old, sq, add, sqr);
+          CHECK(all_close(to_host(dots.data_handle(), (size_t)n_out, stream), want2, tol));
+        }
+}
+
+// ---------------------------------------------------------------------------
+// cpp/tests/linalg/reduce.cu:343-411: key-value arg-max through reduce().
+// ---------------------------------------------------------------------------
+template <typename T>
+void reduce_kvp()
+{
+  using KVP = raft::KeyValuePair<int, T>;
+  raft::resources handle;
+  auto stream = raft::resource::get_cuda_stream(handle);
+  for (int rows : {11, 1234})
+    for (int cols : {7, 33, 128, 500}) {
+      auto data_h = uniform<T>((size_t)rows * cols, -1.0, 1.0, 1234);
+      // exact ties: the lowest index must win
+      for (int r = 0; r < rows; r += 3) {
+        const int a = (r * 7) % cols, b = (r * 13 + 5) % cols;
+        data_h[(size_t)r * cols + a] = data_h[(size_t)r * cols + b] = T(2);
+      }
+      auto data = raft::make_device_matrix<T, int, raft::row_major>(handle, rows, cols);
+      auto dots = raft::make_device_vector<KVP, int>(handle, rows);
+      raft::update_device(data.data_handle(), data_h.data(), data_h.size(), stream);
+      raft::linalg::reduce<raft::Apply::ALONG_ROWS>(
+        handle, raft::make_const_mdspan(data.view()), dots.view(),
+        KVP(0, -std::numeric_limits<T>::infinity()), false, raft::value_to_kvp_op<int>(),
+        raft::argmax_op(), raft::identity_op());
+      auto got = to_host(dots.data_handle(), (size_t)rows, stream);
+      bool ok  = true;
+      for (int r = 0; r < rows; ++r) {
+        int best = 0;
+        for (int j = 1; j < cols; ++j)
+          if (data_h[(size_t)r * cols + j] > data_h[(size_t)r * cols + best]) best = j;
+        ok &= got[r].key == best && got[r].value == data_h[(size_t)r * cols + best];
+      }
+      CHECK(ok);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// cpp/tests/linalg/coalesced_reduction.cu, strided_reduction.cu
+// ---------------------------------------------------------------------------
+template <typename T>
+void coalesced_and_strided(double tol)
+{
+  raft::resources handle;
+  auto stream = raft::resource::get_cuda_stream(handle);
+  auto sq     = [](double x, int) { return x * x; };
+  auto add    = [](double a, double b) { return a + b; };
+  auto idf    = [](double x) { return x; };
+  const std::vector<std::pair<int, int>> shapes = {{10000, 3}, {10000, 17}, {10000, 32},
+                                                   {10000, 270}, {10, 25000}, {1024, 64},
+                                                   {1024, 256}, {9, 100000}};
+  for (auto [rows, cols] : shapes) {
+    auto data_h = uniform<T>((size_t)rows * cols, -1.0, 1.0, 1234);
+    auto data   = raft::make_device_matrix<T, int, raft::row_major>(handle, rows, cols);
+    raft::update_device(data.data_handle(), data_h.data(), data_h.size(), stream);
+    auto by_row = raft::make_device_vector<T, int>(handle, rows);
+    auto by_col = raft::make_device_vector<T, int>(handle, cols);
+    raft::linalg::coalesced_reduction(handle, raft::make_const_mdspan(data.view()), by_row.view(),
+                                      T(0), false, raft::sq_op());
+    CHECK(all_close(to_host(by_row.data_handle(), (size_t)rows, stream),
+                    host_reduce(data_h, rows, cols, true, true, 0.0, nullptr, sq, add, idf), tol));
+    raft::linalg::strided_reduction(handle, raft::make_const_mdspan(data.view()), by_col.view(),
+                                    T(0), false, raft::sq_op());
+    CHECK(all_close(to_host(by_col.data_handle(), (size_t)cols, stream),
+                    host_reduce(data_h, rows, cols, true, false, 0.0, nullptr, sq, add, idf), tol));
+    // pointer forms on a bare stream
+    raft::linalg::coalescedReduction(by_row.data_handle(), data.data_handle(), cols, rows, T(0),
+                                     stream, false, raft::abs_op());
+    auto absm = [](double x, int) { return std::fabs(x); };
+    CHECK(all_close(to_host(by_row.data_handle(), (size_t)rows, stream),
+                    host_reduce(data_h, rows, cols, true, true, 0.0, nullptr, absm, add, idf),
+                    tol));
+    raft::linalg::stridedReduction(by_col.data_handle(), data.data_handle(), cols, rows, T(0),
+                                   stream, false, raft::abs_op());
+    CHECK(all_close(to_host(by_col.data_handle(), (size_t)cols, stream),
+                    host_reduce(data_h, rows, cols, true, false, 0.0, nullptr, absm, add, idf),
+                    tol));
+  }
+}
+
+// ---------------------------------------------------------------------------
+// cpp/tests/linalg/norm.cu: L1 / L2 / Linf, rows and columns, with and without sqrt
+// ---------------------------------------------------------------------------
+template <typename T, typename OutT>
+void norms(double tol)
+{
+  using namespace raft::linalg;
+  raft::resources handle;
+  auto stream = raft::resource::get_cuda_stream(handle);
+  auto add    = [](double a, double b) { return a + b; };
+  auto mx     = [](double a, double b) { return std::max(a, b); };
+  auto idf    = [](double x) { return x; };
+  auto sqr    = [](double x) { return std::sqrt(x); };
+  auto sq     = [](double x, int) { return x * x; };
+  auto ab     = [](double x, int) { return std::fabs(x); };
+  for (auto [rows, cols] : std::vector<std::pair<int, int>>{{4, 8}, {1024, 32}, {1024, 64},
+                                                            {1000, 100}, {37, 1024}}) {
+    auto data_h = uniform<T>((size_t)rows * cols, -10.0, 10.0, 1234);
+    auto data   = raft::make_device_matrix<T, int, raft::row_major>(handle, rows, cols);
+    raft::update_device(data.data_handle(), data_h.data(), data_h.size(), stream);
+    auto in     = raft::make_const_mdspan(data.view());
+    auto by_row = raft::make_device_vector<OutT, int>(handle, rows);
+    auto by_col = raft::make_device_vector<OutT, int>(handle, cols);
+    auto rows_h = [&] { return to_host(by_row.data_handle(), (size_t)rows, stream); };
+    auto cols_h = [&] { return to_host(by_col.data_handle(), (size_t)cols, stream); };
+
+    norm<L1Norm, raft::Apply::ALONG_ROWS>(handle, in, by_row.view());
+    CHECK(all_close(rows_h(), host_reduce(data_h, rows, cols, true, true, 0, nullptr, ab, add, idf), tol));
+    norm<L2Norm, raft::Apply::ALONG_ROWS>(handle, in, by_row.view());
+    CHECK(all_close(rows_h(), host_reduce(data_h, rows, cols, true, true, 0, nullptr, sq, add, idf), tol));
+    norm<L2Norm, raft::Apply::ALONG_ROWS>(handle, in, by_row.view(), raft::sqrt_op());
+    CHECK(all_close(rows_h(), host_reduce(data_h, rows, cols, true, true, 0, nullptr, sq, add, sqr), tol));
+    norm<LinfNorm, raft::Apply::ALONG_ROWS>(handle, in, by_row.view());
+    CHECK(all_close(rows_h(), host_reduce(data_h, rows, cols, true, true, 0, nullptr, ab, mx, idf), tol));
+    norm<L1Norm, raft::Apply::ALONG_COLUMNS>(handle, in, by_col.view());
+    CHECK(all_close(cols_h(), host_reduce(data_h, rows, cols, true, false, 0, nullptr, ab, add, idf), tol));
+    norm<L2Norm, raft::Apply::ALONG_COLUMNS>(handle, in, by_col.view(), raft::sqrt_op());
+    CHECK(all_close(cols_h(), host_reduce(data_h, rows, cols, true, false, 0, nullptr, sq, add, sqr), tol));
+    norm<LinfNorm, raft::Apply::ALONG_COLUMNS>(handle, in, by_col.view());
+    CHECK(all_close(cols_h(), host_reduce(data_h, rows, cols, true, false, 0, nullptr, ab, mx, idf), tol));
+    // pointer forms
+    rowNorm<L2Norm, true>(by_row.data_handle(), data.data_handle(), cols, rows, stream,
+                          raft::sqrt_op());
+    CHECK(all_close(rows_h(), host_reduce(data_h, rows, cols, true, true, 0, nullptr, sq, add, sqr), tol));
+    colNorm<L1Norm, true>(by_col.data_handle(), data.data_handle(), cols, rows, stream);
+    CHECK(all_close(cols_h(), host_reduce(data_h, rows, cols, true, false, 0, nullptr, ab, add, idf), tol));
+  }
+}
+
+// ---------------------------------------------------------------------------
+// cpp/tests/stats/mean.cu, stddev.cu, sum.cu
+// ---------------------------------------------------------------------------
+template <typename T>
+void mean_stddev(double tol)
+{
+  raft::resources handle;
+  auto stream = raft::resource::get_cuda_stream(handle);
+  for (int rm = 0; rm < 2; ++rm)
+    for (auto [rows, cols] : std::vector<std::pair<int, int>>{{1024, 32}, {1024, 64}, {1024, 128},
+                                                              {1024, 256}, {100000, 2}, {31, 1},
+                                                              {1, 257}}) {
+      auto data_h = normal<T>((size_t)rows * cols, 1.0, 2.0, 1234);
+      auto data_d = raft::make_device_vector<T, int>(handle, rows * cols);
+      raft::update_device(data_d.data_handle(), data_h.data(), data_h.size(), stream);
+      auto mu  = raft::make_device_vector<T, int>(handle, cols);
+      auto sd  = raft::make_device_vector<T, int>(handle, cols);
+      auto var = raft::make_device_vector<T, int>(handle, cols);
+      auto sm  = raft::make_device_vector<T, int>(handle, cols);
+      auto mu_c = raft::make_device_vector_view<const T, int>(mu.data_handle(), cols);
+      std::vector<double> want_mu(cols, 0.0), want_sum(cols, 0.0);
+      for (int j = 0; j < cols; ++j) {
+        double s = 0;
+        for (int i = 0; i < rows; ++i)
+          s += (double)data_h[at(rm, rows, cols, i, j)];
+        want_sum[j] = s;
+        want_mu[j]  = s / rows;
+      }
+      for (int sample = 0; sample < 2; ++sample) {
+        if (sample && rows == 1) continue;
+        if (rm) {
+          auto v = raft::make_device_matrix_view<const T, int, raft::row_major>(
+            data_d.data_handle(), rows, cols);
+          raft::stats::mean(handle, v, mu.view());
+          raft::stats::stddev(handle, v, mu_c, sd.view(), (bool)sample);
+          raft::stats::vars(handle, v, mu_c, var.view(), (bool)sample);
+          raft::stats::sum(handle, v, sm.view());
+        } else {
+          auto v = raft::make_device_matrix_view<const T, int, raft::col_major>(
+            data_d.data_handle(), rows, cols);
+          raft::stats::mean(handle, v, mu.view());
+          raft::stats::stddev(handle, v, mu_c, sd.view(), (bool)sample);
+          raft::stats::vars(handle, v, mu_c, var.view(), (bool)sample);
+          raft::stats::sum(handle, v, sm.view());
+        }
+        auto mu_h = to_host(mu.data_handle(), (size_t)cols, stream);
+        CHECK(all_close(mu_h, want_mu, tol));
+        CHECK(all_close(to_host(sm.data_handle(), (size_t)cols, stream), want_sum, tol));
+        std::vector<double> want_sd(cols), want_var(cols);
+        for (int j = 0; j < cols; ++j) {
+          double ss = 0;
+          for (int i = 0; i < rows; ++i) {
+            const double x = (double)data_h[at(rm, rows, cols, i, j)];
+            ss += x * x;
+          }
+          const double r  = 1.0 / (sample ? rows - 1 : rows);
+          const double rmn = sample ? r * rows : 1.0;
+          want_var[j]     = std::fabs(ss * r - (double)mu_h[j] * (double)mu_h[j] * rmn);
+          want_sd[j]      = std::sqrt(want_var[j]);
+        }
+        // E[x^2] - mu^2 cancels: the reference checks stddev to 1e-1 of the generator's
+        // sigma (cpp/tests/stats/stddev.cu:120-182); here against the same formula in fp64
+        const double tol_sd = std::is_same_v<T, float> ? 2e-3 : 1e-7;
+        auto sd_h  = to_host(sd.data_handle(), (size_t)cols, stream);
+        auto var_h = to_host(var.data_handle(), (size_t)cols, stream);
+        CHECK(all_close(sd_h, want_sd, tol_sd));
+        CHECK(all_close(var_h, want_var, tol_sd));
+        // cpp/tests/stats/stddev.cu:198-202: sqrt(vars) == stddev
+        bool same = true;
+        for (int j = 0; j < cols; ++j)
+          same &= std::fabs(std::sqrt((double)var_h[j]) - (double)sd_h[j]) <= 1e-6 * (1 + sd_h[j]);
+        CHECK(same);
+      }
+    }
+}
+
+// cpp/tests/stats/mean.cu:177-185: int8 -> half
+void mean_int8_to_half()
+{
+  raft::resources handle;
+  auto stream    = raft::resource::get_cuda_stream(handle);
+  const int rows = 1024, cols = 64;
+  std::mt19937 g(1234);
+  std::uniform_int_distribution<int> d(-20, 30);
+  std::vector<std::int8_t> data_h((size_t)rows * cols);
+  for (auto& x : data_h)
+    x = (std::int8_t)d(g);
+  auto data = raft::make_device_matrix<std::int8_t, int, raft::row_major>(handle, rows, cols);
+  auto mu   = raft::make_device_vector<__half, int>(handle, cols);
+  raft::update_device(data.data_handle(), data_h.data(), data_h.size(), stream);
+  raft::stats::mean(handle, raft::make_const_mdspan(data.view()), mu.view());
+  auto mu_h = to_host(mu.data_handle(), (size_t)cols, stream);
+  bool ok   = true;
+  for (int j = 0; j < cols; ++j) {
+    double s = 0;
+    for (int i = 0; i < rows; ++i)
+      s += data_h[(size_t)i * cols + j];
+    ok &= std::fabs((double)__half2float(mu_h[j]) - s / rows) <= 0.02 + 2e-3 * std::fabs(s / rows);
+  }
+  CHECK(ok);
+}
+
+// cpp/tests/stats/sum.cu:50-98,139-140
+template <typename T>
+void sum_accuracy(T value, double large, double tol)
+{
+  raft::resources handle;
+  auto stream = raft::resource::get_cuda_stream(handle);
+  for (int rm = 0; rm < 2; ++rm)
+    for (auto [rows, cols] : std::vector<std::pair<int, int>>{{4, 5}, {1024, 32}, {1024, 256},
+                                                              {17, 5}, {7, 23}, {3, 97}, {1, 30}}) {
+      for (int compensate = 0; compensate < 2; ++compensate) {
+        const int len = rows * cols;
+        std::vector<T> data_h(len);
+        for (int i = 0; i < len; i++) {
+          data_h[i]     = T(double(value));
+          const int row = rm ? i / cols : i % rows;
+          if (compensate && row % 3 == 2) {
+            data_h[i]                      = T(double(value) * large);
+            data_h[rm ? (i - cols) : (i - 1)]     = T(-1 * double(value) * large);
+            data_h[rm ? (i - 2 * cols) : (i - 2)] = T(3.0 * double(value));
+          }
+        }
+        auto data_d = raft::make_device_vector<T, int>(handle, len);
+        auto out    = raft::make_device_vector<T, int>(handle, cols);
+        raft::update_device(data_d.data_handle(), data_h.data(), (size_t)len, stream);
+        if (rm) {
+          raft::stats::sum(handle,
+                           raft::make_device_matrix_view<const T, int, raft::row_major>(
+                             data_d.data_handle(), rows, cols),
+                           out.view());
+        } else {
+          raft::stats::sum(handle,
+                           raft::make_device_matrix_view<const T, int, raft::col_major>(
+                             data_d.data_handle(), rows, cols),
+                           out.view());
+        }
+        std::vector<double> want(cols, double(rows) * double(value));
+        CHECK(all_close(to_host(out.data_handle(), (size_t)cols, stream), want, tol));
+      }
+    }
+}
+
+// cpp/tests/matrix/argmax.cu:71-75, argmin.cu:71-75
+template <typename T>
+void arg_fixtures()
+{
+  raft::resources handle;
+  auto stream = raft::resource::get_cuda_stream(handle);
+  std::vector<T> h{T(0.1), T(0.2), T(0.3), T(0.4), T(0.4), T(0.3),
+                   T(0.2), T(0.1), T(0.2), T(0.3), T(0.5), T(0.0)};
+  auto in  = raft::make_device_matrix<T, std::uint32_t, raft::row_major>(handle, 3, 4);
+  auto out = raft::make_device_vector<int, std::uint32_t>(handle, 3);
+  raft::update_device(in.data_handle(), h.data(), h.size(), stream);
+  auto in_c = raft::make_device_matrix_view<const T, std::uint32_t, raft::row_major>(
+    in.data_handle(), 3, 4);
+  raft::matrix::argmax(handle, in_c, out.view());
+  CHECK((to_host(out.data_handle(), 3, stream) == std::vector<int>{3, 0, 2}));
+  raft::matrix::argmin(handle, in_c, out.view());
+  CHECK((to_host(out.data_handle(), 3, stream) == std::vector<int>{0, 3, 3}));
+  auto out64 = raft::make_device_vector<std::int64_t, std::uint32_t>(handle, 3);
+  raft::matrix::argmax(handle, in_c, out64.view());
+  CHECK((to_host(out64.data_handle(), 3, stream) == std::vector<std::int64_t>{3, 0, 2}));
+}
+
+// cpp/tests/linalg/map_then_reduce.cu:101-169
+void map_reduce_cases()
+{
+  raft::resources handle;
+  auto stream = raft::resource::get_cuda_stream(handle);
+  {
+    const int len = 1 << 20;
+    auto h        = uniform<float>(len, -1.0, 1.0, 1234);
+    auto in       = raft::make_device_vector<float, int>(handle, len);
+    auto out      = raft::make_device_scalar<float>(handle);
+    raft::update_device(in.data_handle(), h.data(), h.size(), stream);
+    raft::linalg::mapThenSumReduce(out.data_handle(), (size_t)len, raft::identity_op(), stream,
+                                   in.data_handle());
+    double want = 0;
+    for (float x : h)
+      want += x;
+    CHECK(std::fabs((double)to_host(out.data_handle(), 1, stream)[0] - want) <= 1e-3);
+    raft::linalg::mapThenSumReduce(out.data_handle(), (size_t)len, raft::sq_op(), stream,
+                                   in.data_handle());
+    want = 0;
+    for (float x : h)
+      want += (double)x * x;
+    CHECK(std::fabs((double)to_host(out.data_handle(), 1, stream)[0] - want) <= 1e-3 * want);
+  }
+  {
+    const int len = 1237;
+    auto h        = uniform<float>(len, 2.0, 3.0, 1234);
+    h[42]         = 1.0f;
+    h[337]        = 5.0f;
+    auto in       = raft::make_device_vector<float, int>(handle, len);
+    auto out      = raft::make_device_scalar<float>(handle);
+    raft::update_device(in.data_handle(), h.data(), h.size(), stream);
+    auto in_c = raft::make_device_vector_view<const float, int>(in.data_handle(), len);
+    raft::linalg::map_reduce(handle, in_c, out.view(), std::numeric_limits<float>::max(),
+                             raft::identity_op(), raft::min_op());
+    CHECK(to_host(out.data_handle(), 1, stream)[0] == 1.0f);
+    raft::linalg::map_reduce(handle, in_c, out.view(), std::numeric_limits<float>::lowest(),
+                             raft::identity_op(), raft::max_op());
+    CHECK(to_host(out.data_handle(), 1, stream)[0] == 5.0f);
+  }
+}
+
+// a second handle on a stream of its own, reused across many calls that need the
+// handle-owned workspace (split rows, column partials)
+void handle_workspace_reuse()
+{
+  hipStream_t s;
+  RAFT_HIP_TRY(hipStreamCreate(&s));
+  {
+    raft::device_resources handle(s);
+    const int rows = 4, cols = 1 << 20;
+    auto h    = uniform<float>((size_t)rows * cols, -1.0, 1.0, 99);
+    auto data = raft::make_device_matrix<float, int, raft::row_major>(handle, rows, cols);
+    auto out  = raft::make_device_vector<float, int>(handle, rows);
+    raft::update_device(data.data_handle(), h.data(), h.size(), s);
+    auto add = [](double a, double b) { return a + b; };
+    auto idm = [](double x, int) { return x; };
+    auto idf = [](double x) { return x; };
+    auto want = host_reduce(h, rows, cols, true, true, 0.0, nullptr, idm, add, idf);
+    for (int rep = 0; rep < 5; ++rep) {
+      raft::linalg::reduce<raft::Apply::ALONG_ROWS>(handle, raft::make_const_mdspan(data.view()),
+                                                    out.view(), 0.0f);
+      CHECK(all_close(to_host(out.data_handle(), (size_t)rows, s), want, 1e-5));
+    }
+  }
+  RAFT_HIP_TRY(hipStreamDestroy(s));
+}
+
+}  // namespace
+
+TEST_CASE(ReduceSimpleF) { simple_max<float>(); }
+TEST_CASE(ReduceSimpleD) { simple_max<double>(); }
+TEST_CASE(ReduceTestFFI32) { reduce_full<float, float, int>(2e-6, {11, 1234}, {7, 33, 128, 500}); }
+TEST_CASE(ReduceTestFFU32) { reduce_full<float, float, std::uint32_t>(2e-6, {11, 1234}, {7, 33, 128, 500}); }
+TEST_CASE(ReduceTestFFI64) { reduce_full<float, float, std::int64_t>(2e-6, {11, 1234}, {7, 33, 128, 500}); }
+TEST_CASE(ReduceTestFFU64) { reduce_full<float, float, std::uint64_t>(2e-6, {11, 1234}, {7, 33, 128, 500}); }
+TEST_CASE(ReduceTestDDI32) { reduce_full<double, double, int>(1e-9, {11, 1234}, {7, 33, 128, 500}); }
+TEST_CASE(ReduceTestFDI32) { reduce_full<float, double, int>(1e-9, {11, 1234}, {7, 33, 128, 500}); }
+TEST_CASE(ReduceTestFFThick) { reduce_full<float, float, int>(1e-4, {3, 9}, {17771, 33333, 100000}); }
+TEST_CASE(ReduceTestKVPIF) { reduce_kvp<float>(); }
+TEST_CASE(ReduceTestKVPID) { reduce_kvp<double>(); }
+TEST_CASE(CoalescedStridedF) { coalesced_and_strided<float>(2e-6); }
+TEST_CASE(CoalescedStridedD) { coalesced_and_strided<double>(1e-9); }
+TEST_CASE(NormF) { norms<float, float>(1e-5); }
+TEST_CASE(NormD) { norms<double, double>(1e-9); }
+TEST_CASE(MeanStddevF) { mean_stddev<float>(1e-5); }
+TEST_CASE(MeanStddevD) { mean_stddev<double>(1e-9); }
+TEST_CASE(MeanInt8ToHalf) { mean_int8_to_half(); }
+TEST_CASE(SumAccuracyF) { sum_accuracy<float>(0.0001f, 1e7, 0.001); }
+TEST_CASE(SumAccuracyD) { sum_accuracy<double>(0.000001, 1e12, 0.0001); }
+TEST_CASE(ArgFixturesF) { arg_fixtures<float>(); }
+TEST_CASE(ArgFixturesD) { arg_fixtures<double>(); }
+TEST_CASE(MapReduce) { map_reduce_cases(); }
+TEST_CASE(HandleWorkspaceReuse) { handle_workspace_reuse(); }
+
+int main()
+{
+  int n = 0;
+  if (hipGetDeviceCount(&n) != hipSuccess || n == 0) {
+    std::printf("no GPU visible\n");
+    return 2;
+  }
+  return t::run_all();
+}

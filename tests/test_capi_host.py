@@ -1,0 +1,150 @@
+"""CPU-side checks of the C ABI: the library loads, exports every symbol that
+include/rmi_reduce.h declares, validates descriptors and plans the benchmark shapes
+as designed.  No kernel is launched here."""
+import ctypes as C
+import re
+from pathlib import Path
+
+import pytest
+
+from raft_amd import _capi as api
+
+ROOT = Path(__file__).resolve().parent.parent
+
+
+def test_library_exports_every_declared_symbol():
+    header = (ROOT / "include" / "rmi_reduce.h").read_text()
+    declared = set(re.findall(r"RMI_API\s+[\w\s\*]+?\b(rmi_\w+)\s*\(", header))
+    assert declared, "no RMI_API declarations found"
+    assert declared == set(api.SYMBOLS), (declared ^ set(api.SYMBOLS))
+    lib = api.load()
+    for name in declared:
+        assert getattr(lib, name) is not None
+    assert lib.rmi_abi_version() == 1
+
+
+def test_struct_layouts_match_the_header(tmp_path):
+    # the header must compile as plain C, and the ctypes mirrors must have the sizes and
+    # field offsets the C compiler gives the two PODs
+    import subprocess
+    fields_d = [n for n, _ in api.ReduceDesc._fields_]
+    fields_p = [n for n, _ in api.Plan._fields_]
+    src = tmp_path / "layout.c"
+    lines = ['#include <stdio.h>', '#include <stddef.h>', '#include "rmi_reduce.h"', 'int main(void){',
+             'printf("%zu %zu\\n", sizeof(rmi_reduce_desc), sizeof(rmi_plan));']
+    lines += [f'printf("%zu\\n", offsetof(rmi_reduce_desc, {f}));' for f in fields_d]
+    lines += [f'printf("%zu\\n", offsetof(rmi_plan, {f}));' for f in fields_p]
+    lines += ['return 0;}']
+    src.write_text("\n".join(lines))
+    exe = tmp_path / "layout"
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", f"-I{ROOT / 'include'}", str(src),
+                    "-o", str(exe)], check=True)
+    out = subprocess.run([str(exe)], capture_output=True, text=True, check=True).stdout.split()
+    assert [int(out[0]), int(out[1])] == [C.sizeof(api.ReduceDesc), C.sizeof(api.Plan)]
+    offs = [int(x) for x in out[2:]]
+    want = [getattr(api.ReduceDesc, f).offset for f in fields_d] + \
+           [getattr(api.Plan, f).offset for f in fields_p]
+    assert offs == want
+    lib = api.load()
+    for dt, size in api.DTYPE_SIZE.items():
+        assert lib.rmi_dtype_size(dt) == size
+    assert lib.rmi_dtype_size(99) == 0
+
+
+def test_status_strings():
+    lib = api.load()
+    seen = {lib.rmi_status_string(i).decode() for i in range(9)}
+    assert len(seen) == 9 and "ok" in seen
+    assert lib.rmi_status_string(1234).decode() == "unknown status"
+
+
+BENCH_SHAPES = [
+    # in, out, rows, cols, kwargs, expected plan, expected passes
+    (api.F32, api.F32, 10000, 256, {}, api.PLAN_ROW_WAVE, 1),
+    (api.F32, api.F32, 1000000, 128, dict(main_op=api.MAIN_SQ, final_op=api.FIN_SQRT),
+     api.PLAN_ROW_WAVE, 1),
+    (api.F32, api.F32, 10000000, 64, dict(apply=api.ALONG_COLUMNS), api.PLAN_COL_TILE, 2),
+    (api.F32, api.KVP_I32_F32, 65536, 32000,
+     dict(main_op=api.MAIN_KVP, reduce_op=api.RED_ARGMAX), api.PLAN_ROW_WAVE, 1),
+    (api.I8, api.I64, 4096, 16384, {}, api.PLAN_ROW_BLOCK, 1),
+    (api.I8, api.I64, 16777216, 8, {}, api.PLAN_ROW_LANES, 1),
+    (api.BF16, api.F32, 8, 4194304, {}, api.PLAN_ROW_SPLIT, 2),
+]
+
+
+@pytest.mark.parametrize("in_dt,out_dt,rows,cols,kw,plan,passes", BENCH_SHAPES)
+def test_plans_of_benchmark_shapes(in_dt, out_dt, rows, cols, kw, plan, passes):
+    d = api.make_desc(in_dt, out_dt, rows, cols, **kw)
+    p = api.plan_query(d)
+    assert p.kind == plan and p.passes == passes
+    assert p.vec_bytes == 16
+    n_out = cols if kw.get("apply") == api.ALONG_COLUMNS else rows
+    assert p.n_outputs == n_out and p.reduce_len == rows * cols // n_out
+    ws = api.load().rmi_reduce_workspace_bytes(C.byref(d))
+    assert (ws > 0) == (passes == 2)
+    assert ws >= p.workspace_bytes
+    assert p.grid_blocks >= 1
+
+
+def test_plan_hints_and_fallbacks():
+    # a forced split on a short row degrades to one block per row
+    d = api.make_desc(api.F32, api.F32, 10, 512, plan_hint=api.PLAN_ROW_SPLIT)
+    p = api.plan_query(d)
+    assert p.kind == api.PLAN_ROW_BLOCK and p.passes == 1 and p.workspace_bytes == 0
+    d = api.make_desc(api.F32, api.F32, 4, 1 << 20, plan_hint=api.PLAN_ROW_SPLIT)
+    p = api.plan_query(d)
+    assert p.kind == api.PLAN_ROW_SPLIT and p.blocks_per_out >= 2
+    assert p.workspace_bytes == 4 * p.blocks_per_out * 8
+    # rows of 7 floats (28 B) cannot be read as 16-byte vectors
+    p = api.plan_query(api.make_desc(api.F32, api.F32, 1000, 7))
+    assert p.vec_bytes == 4 and p.kind == api.PLAN_ROW_WAVE
+    # f64 sums carry a 16-byte (sum, compensation) accumulator through the partials
+    d = api.make_desc(api.F64, api.F64, 4, 1 << 20, plan_hint=api.PLAN_ROW_SPLIT)
+    p = api.plan_query(d)
+    assert p.workspace_bytes == 4 * p.blocks_per_out * 16
+    # column-major along rows is a strided fold
+    p = api.plan_query(api.make_desc(api.F32, api.F32, 64, 100000, layout=api.COL_MAJOR))
+    assert p.kind == api.PLAN_COL_TILE and p.n_outputs == 64
+
+
+@pytest.mark.parametrize("kw,status", [
+    (dict(in_dtype=77), api.ERR_BAD_ENUM),
+    (dict(layout=5), api.ERR_BAD_ENUM),
+    (dict(reduce_op=9), api.ERR_BAD_ENUM),
+    (dict(n_rows=-3), api.ERR_BAD_SHAPE),
+    (dict(out_dtype=api.I64), api.ERR_UNSUPPORTED),             # float in, int out
+    (dict(out_dtype=api.KVP_I32_F32), api.ERR_UNSUPPORTED),     # KVP out needs an arg-reduce
+    (dict(reduce_op=api.RED_ARGMAX), api.ERR_UNSUPPORTED),      # arg-reduce needs MAIN_KVP
+    (dict(reduce_op=api.RED_ARGMAX, main_op=api.MAIN_KVP, out_dtype=api.KVP_I32_F64),
+     api.ERR_UNSUPPORTED),                                      # value type mismatch
+    (dict(final_op=api.FIN_STDDEV_FROM_SUMSQ), api.ERR_NULL),   # needs final_aux
+    (dict(in_dtype=api.KVP_I32_F32), api.ERR_UNSUPPORTED),
+    (dict(reserved=1), api.ERR_BAD_ENUM),
+])
+def test_descriptor_validation(kw, status):
+    d = api.make_desc(api.F32, api.F32, 100, 100)
+    for k, v in kw.items():
+        setattr(d, k, v)
+    p = api.Plan()
+    assert api.load().rmi_plan_query(C.byref(d), C.byref(p)) == status
+
+
+def test_null_and_workspace_errors_without_a_launch():
+    lib = api.load()
+    p = api.Plan()
+    assert lib.rmi_plan_query(None, C.byref(p)) == api.ERR_NULL
+    d = api.make_desc(api.F32, api.F32, 100, 100)
+    assert lib.rmi_plan_query(C.byref(d), None) == api.ERR_NULL
+    assert lib.rmi_reduce(None, None, None, None, 0, None) == api.ERR_NULL
+    # the checks below return before anything is launched
+    assert lib.rmi_reduce(C.byref(d), 0x1000, None, None, 0, None) == api.ERR_NULL
+    assert lib.rmi_reduce(C.byref(d), None, 0x1000, None, 0, None) == api.ERR_NULL
+    assert lib.rmi_reduce(C.byref(d), 0x1002, 0x1000, None, 0, None) == api.ERR_ALIGNMENT
+    assert lib.rmi_reduce(C.byref(d), 0x1000, 0x1002, None, 0, None) == api.ERR_ALIGNMENT
+    d = api.make_desc(api.BF16, api.F32, 8, 4194304)
+    assert lib.rmi_reduce(C.byref(d), 0x1000, 0x2000, None, 0, None) == api.ERR_WORKSPACE
+    assert lib.rmi_reduce(C.byref(d), 0x1000, 0x2000, 0x3000, 16, None) == api.ERR_WORKSPACE
+    assert lib.rmi_map_reduce(C.byref(d), -1, None, None, None, 0, None) == api.ERR_BAD_SHAPE
+    # zero outputs: success, nothing to do
+    d = api.make_desc(api.F32, api.F32, 0, 100)
+    assert lib.rmi_reduce(C.byref(d), None, None, None, 0, None) == api.OK

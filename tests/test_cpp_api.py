@@ -1,0 +1,33 @@
+"""Runs the C++ API test programs (tests/cpp/*.cpp, built by raft_amd.build).
+
+test_raft_host needs no GPU: functor vocabulary, views, precondition errors, plan
+selector.  test_raft_api restates the reference's reduction-path tests against the
+kept raft:: names and runs on the GPU."""
+import subprocess
+from pathlib import Path
+
+import pytest
+
+BIN = Path(__file__).resolve().parent / "cpp" / "bin"
+
+
+def _run(name, timeout):
+    exe = BIN / name
+    if not exe.exists():
+        from raft_amd import build
+        build.build_cpp_tests()
+    proc = subprocess.run([str(exe)], capture_output=True, text=True, timeout=timeout)
+    tail = "\n".join(proc.stdout.splitlines()[-40:])
+    assert proc.returncode == 0, f"{name} failed (rc={proc.returncode}):\n{tail}\n{proc.stderr[-2000:]}"
+    return proc.stdout
+
+
+def test_cpp_host_layer():
+    out = _run("test_raft_host", 60)
+    assert "0 failed" in out
+
+
+@pytest.mark.gpu
+def test_cpp_api_on_gpu(gpu):
+    out = _run("test_raft_api", 600)
+    assert "0 failed" in out
