@@ -92,6 +92,12 @@ int reduce_impl(const rmi_reduce_desc& d,
   pr.epi.out_dtype = d.out_dtype;
   pr.epi.final_op  = d.final_op;
   pr.epi.inplace   = d.inplace ? 1 : 0;
+  const bool natural_out =
+    key.family == kFamKvp
+      ? false
+      : (key.family == kFamInt ? true : (d.out_dtype == RMI_F32 || d.out_dtype == RMI_F64));
+  pr.epi.plain         = (!d.inplace && d.final_op == RMI_FIN_IDENTITY && natural_out) ? 1 : 0;
+  pr.epi.out_aligned16 = aligned(out, 16) ? 1 : 0;
   return lookup(key)(pl, pr, static_cast<hipStream_t>(stream));
 }
 

@@ -551,6 +551,11 @@ struct Epilogue {
   int out_dtype;
   int final_op;
   int inplace;
+  // Set by the host when final_op is the identity, inplace is off and the output
+  // is stored in the accumulator's own family (f32 / f64, i32 / i64, key-value
+  // pair): the common case, kept free of the general epilogue's branches.
+  int plain;
+  int out_aligned16;  // the output pointer is 16-byte aligned
 };
 
 __device__ __forceinline__ float bf16_to_f32(uint16_t b) { return as_f32((u32)b << 16); }
@@ -644,6 +649,14 @@ struct out_kvp {
   V value;
 };
 
+// Outputs use ordinary stores: small or strided non-temporal stores bypass the
+// L2's write combining and measured slower on every shape.
+template <class T>
+__device__ __forceinline__ void store_stream(T* p, T v)
+{
+  *p = v;
+}
+
 template <class P>
 __device__ __forceinline__ void finish(const Epilogue& e, i64 k, typename P::acc_t acc)
 {
@@ -651,6 +664,14 @@ __device__ __forceinline__ void finish(const Epilogue& e, i64 k, typename P::acc
   if constexpr (P::CLS == kClsFloat) {
     acc_t a = P::from_f64(e.init_f);
     P::merge(a, acc);
+    if (e.plain) {
+      if (e.out_dtype == RMI_F32) {
+        store_stream(static_cast<float*>(e.out) + k, (float)P::to_f64(a));
+      } else {
+        store_stream(static_cast<double*>(e.out) + k, P::to_f64(a));
+      }
+      return;
+    }
     if (e.inplace) {
       acc_t o = P::from_f64(load_out_f64(e.out, e.out_dtype, k));
       P::merge(o, a);
@@ -660,6 +681,14 @@ __device__ __forceinline__ void finish(const Epilogue& e, i64 k, typename P::acc
   } else if constexpr (P::CLS == kClsInt) {
     acc_t a = e.init_i;
     P::merge(a, acc);
+    if (e.plain) {
+      if (e.out_dtype == RMI_I64) {
+        store_stream(static_cast<i64*>(e.out) + k, (i64)a);
+      } else {
+        store_stream(static_cast<int32_t*>(e.out) + k, (int32_t)a);
+      }
+      return;
+    }
     if (e.inplace) {
       acc_t o = e.out_dtype == RMI_I64 ? static_cast<const i64*>(e.out)[k]
                                        : (i64) static_cast<const int32_t*>(e.out)[k];
@@ -690,6 +719,33 @@ __device__ __forceinline__ void finish(const Epilogue& e, i64 k, typename P::acc
     o[k].key   = a.key;
     o[k].value = a.value;
   }
+}
+
+// K results for the consecutive outputs k0 .. k0+K-1 held by one lane.  Pairs of
+// int64 results leave as one 16-byte store when the epilogue is plain.
+template <class P, int K>
+__device__ __forceinline__ void finish_run(const Epilogue& e, i64 k0, typename P::acc_t (&acc)[K])
+{
+  if constexpr (P::CLS == kClsInt && (K % 2 == 0)) {
+    if (e.plain && e.out_dtype == RMI_I64 && e.out_aligned16) {
+#pragma unroll
+      for (int r = 0; r < K; r += 2) {
+        i64 a = e.init_i, b = e.init_i;
+        P::merge(a, acc[r]);
+        P::merge(b, acc[r + 1]);
+        u32x4 v;
+        v[0] = (u32)(u64)a;
+        v[1] = (u32)((u64)a >> 32);
+        v[2] = (u32)(u64)b;
+        v[3] = (u32)((u64)b >> 32);
+        *reinterpret_cast<u32x4*>(static_cast<i64*>(e.out) + k0 + r) = v;
+      }
+      return;
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < K; ++r)
+    finish<P>(e, k0 + r, acc[r]);
 }
 
 }  // namespace rmi

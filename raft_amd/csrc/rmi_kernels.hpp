@@ -39,7 +39,6 @@ struct ColArgs {
   i64 n_out;          // D: length of the contiguous dimension
   i64 len;            // N: number of strided rows folded
   i64 nvec;           // lane-loads per row: D/VEC (VEC16) or D (scalar)
-  i64 rows_per_block; // rows owned by one blockIdx.y
   int TX;             // lanes along the contiguous dimension (power of two <= 64)
   int logTX;
   int B;              // gridDim.y
@@ -84,6 +83,23 @@ struct Held {
   }
 };
 
+// Accumulator held by lane `src` of the wave (ds_bpermute, word by word).
+template <class P>
+__device__ __forceinline__ typename P::acc_t shfl_acc(const typename P::acc_t& a, int src)
+{
+  using acc_t = typename P::acc_t;
+  static_assert(sizeof(acc_t) % 4 == 0, "accumulators are moved word by word");
+  constexpr int NW = sizeof(acc_t) / 4;
+  u32 w[NW];
+  __builtin_memcpy(w, &a, sizeof(acc_t));
+#pragma unroll
+  for (int i = 0; i < NW; ++i)
+    w[i] = (u32)__shfl((int)w[i], src, kWave);
+  acc_t r;
+  __builtin_memcpy(&r, w, sizeof(acc_t));
+  return r;
+}
+
 // ---------------------------------------------------------------------------
 // K rows per 16-byte vector (row length VEC/K elements).  Lane-local.
 // ---------------------------------------------------------------------------
@@ -113,7 +129,7 @@ __global__ __launch_bounds__(kBlock) void row_lanes_kernel(RowArgs a)
           P::push(acc[r], In<in_t>::template get<r * D + j>(x[u]), (i64)j);
         });
       });
-      static_for<K>([&](auto r) { finish<P>(a.epi, v * K + r, acc[r]); });
+      finish_run<P, K>(a.epi, v * K, acc);
     }
   }
   // Rows past the last whole vector (fewer than K of them): one lane each.
@@ -160,9 +176,36 @@ __global__ __launch_bounds__(kBlock) void row_short_kernel(RowArgs a)
 #pragma unroll
   for (int t = 0; t < kUnroll; ++t)
     group_allreduce<P>(acc[t], G);
+
+  // Every lane of a group now holds its row's result.  Hand the results to lanes
+  // so that consecutive lanes own consecutive rows: the wave's kUnroll*R outputs
+  // then leave as one contiguous run per store instead of R-element pieces.
+  const i64 wave_row0 = wid * kUnroll * R;
+  if (G == 1) {
+#pragma unroll
+    for (int t = 0; t < kUnroll; ++t)
+      if (row[t] < a.n_out) finish<P>(a.epi, row[t], acc[t]);
+    return;
+  }
+  const int logR   = 6 - a.logG;
+  const int src    = (lane & (R - 1)) << a.logG;  // first lane of group (lane % R)
+  const int my_sub = lane >> logR;                // which R-run of a 64-row span this lane serves
+  acc_t mine[kUnroll];
 #pragma unroll
   for (int t = 0; t < kUnroll; ++t) {
-    if (c == 0 && row[t] < a.n_out) finish<P>(a.epi, row[t], acc[t]);
+    const acc_t v = shfl_acc<P>(acc[t], src);
+    const int s   = (t << logR) >> 6;                   // 64-row span that tile t falls in
+    const int sub = t - ((s << 6) >> logR);             // position of tile t inside that span
+#pragma unroll
+    for (int sc = 0; sc < kUnroll; ++sc)
+      if (s == sc && my_sub == sub) mine[sc] = v;
+  }
+  const int spans = (kUnroll * R + kWave - 1) >> 6;
+#pragma unroll
+  for (int sc = 0; sc < kUnroll; ++sc) {
+    const int q = lane + (sc << 6);
+    if (sc < spans && q < kUnroll * R && wave_row0 + q < a.n_out)
+      finish<P>(a.epi, wave_row0 + q, mine[sc]);
   }
 }
 
@@ -275,7 +318,7 @@ __global__ __launch_bounds__(1024) void row_block_kernel(RowArgs a)
 // ---------------------------------------------------------------------------
 // Reduction along the strided dimension of a [len][n_out] row-major array.
 // Thread (tx, ty): tx owns one lane-load wide group of adjacent columns for
-// the whole kernel, ty strides over the rows of this block's row range.
+// the whole kernel, ty strides over the rows of the tiles dealt to this block.
 // ---------------------------------------------------------------------------
 template <class P>
 __device__ __forceinline__ typename P::acc_t bperm_acc(const typename P::acc_t& a, int mask)
@@ -308,9 +351,11 @@ __global__ __launch_bounds__(kBlock) void col_kernel(ColArgs a)
   const int tx   = t & (TX - 1);
   const int ty   = t >> a.logTX;
   const i64 cv   = (i64)blockIdx.x * TX + tx;
-  const i64 r0   = (i64)blockIdx.y * a.rows_per_block;
-  const i64 r1   = (r0 + a.rows_per_block < a.len) ? (r0 + a.rows_per_block) : a.len;
   const bool live = cv < a.nvec;
+  // Row tiles of TY*kUnroll rows are dealt round-robin over blockIdx.y, so at any
+  // moment the blocks of the grid read one compact, advancing window of the matrix.
+  const i64 RT     = (i64)TY * kUnroll;
+  const i64 n_full = a.len / RT;
 
   acc_t acc[S];
 #pragma unroll
@@ -318,10 +363,10 @@ __global__ __launch_bounds__(kBlock) void col_kernel(ColArgs a)
     acc[j] = P::neutral();
 
   if (live) {
-    i64 r = r0 + ty;
     if constexpr (VEC16) {
       const u32x4* p = static_cast<const u32x4*>(a.in) + cv;
-      for (; r + (kUnroll - 1) * (i64)TY < r1; r += (i64)kUnroll * TY) {
+      for (i64 tile = blockIdx.y; tile < n_full; tile += a.B) {
+        const i64 r = tile * RT + ty;
         u32x4 x[kUnroll];
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u)
@@ -330,11 +375,14 @@ __global__ __launch_bounds__(kBlock) void col_kernel(ColArgs a)
         for (int u = 0; u < kUnroll; ++u)
           P::push_cols(acc, x[u], r + (i64)u * TY);
       }
-      for (; r < r1; r += TY)
-        P::push_cols(acc, load16(p + r * a.nvec), r);
+      if ((i64)blockIdx.y == n_full % a.B) {  // the rows past the last whole tile
+        for (i64 r = n_full * RT + ty; r < a.len; r += TY)
+          P::push_cols(acc, load16(p + r * a.nvec), r);
+      }
     } else {
       const in_t* p = static_cast<const in_t*>(a.in) + cv;
-      for (; r + (kUnroll - 1) * (i64)TY < r1; r += (i64)kUnroll * TY) {
+      for (i64 tile = blockIdx.y; tile < n_full; tile += a.B) {
+        const i64 r = tile * RT + ty;
         typename In<in_t>::nat x[kUnroll];
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u)
@@ -343,8 +391,10 @@ __global__ __launch_bounds__(kBlock) void col_kernel(ColArgs a)
         for (int u = 0; u < kUnroll; ++u)
           P::push(acc[0], x[u], r + (i64)u * TY);
       }
-      for (; r < r1; r += TY)
-        P::push(acc[0], In<in_t>::ld(p + r * a.nvec), r);
+      if ((i64)blockIdx.y == n_full % a.B) {
+        for (i64 r = n_full * RT + ty; r < a.len; r += TY)
+          P::push(acc[0], In<in_t>::ld(p + r * a.nvec), r);
+      }
     }
   }
 

@@ -109,7 +109,6 @@ int run(const PlanX& pl, const Problem& pr, hipStream_t st)
       a.n_out          = pl.n_out;
       a.len            = pl.len;
       a.nvec           = pl.nvec;
-      a.rows_per_block = pl.rows_per_block;
       a.TX             = pl.TX;
       a.logTX          = pl.logTX;
       a.B              = pl.B;

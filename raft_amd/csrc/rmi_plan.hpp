@@ -40,7 +40,6 @@ struct PlanX {
   int TX          = 1;           // COL_TILE
   int logTX       = 0;
   int64_t gridx   = 0;  // COL_TILE: blocks along the contiguous dimension
-  int64_t rows_per_block = 0;
   int64_t grid_blocks    = 0;
   int passes             = 1;
   int acc_bytes          = 8;
@@ -226,16 +225,15 @@ inline int make_plan(const rmi_reduce_desc& d,
     p.logTX = ilog2(p.TX);
     const int TY = kPlanBlock / p.TX;
     p.gridx      = ceildiv(p.nvec, p.TX);
-    // enough blocks to give every CU several, but at least two unrolled
-    // batches of rows per thread
-    int64_t B          = ceildiv((int64_t)n_cu * 8, p.gridx);
-    const int64_t maxB = ceildiv(p.len, (int64_t)TY * kPlanUnroll * 2);
+    // row tiles of TY*unroll rows are dealt round-robin to B blocks: enough blocks
+    // to give every CU several, but at least two tiles per block
+    const int64_t tile_rows = (int64_t)TY * kPlanUnroll;
+    int64_t B               = ceildiv((int64_t)n_cu * 8, p.gridx);
+    const int64_t maxB      = ceildiv(p.len, tile_rows * 2);
     if (B > maxB) B = maxB;
     if (B < 1) B = 1;
     if (B > 4096) B = 4096;
-    const int64_t quantum = (int64_t)TY * kPlanUnroll;
-    p.rows_per_block      = ceildiv(ceildiv(p.len, B), quantum) * quantum;
-    p.B                   = (int)ceildiv(p.len, p.rows_per_block);
+    p.B = (int)B;
     p.grid_blocks         = p.gridx * p.B;
     p.passes              = p.B > 1 ? 2 : 1;
     p.ws_bytes            = p.B > 1 ? (size_t)p.n_out * p.B * acc_bytes : 0;
