@@ -665,6 +665,9 @@ __device__ __forceinline__ void finish(const Epilogue& e, i64 k, typename P::acc
     acc_t a = P::from_f64(e.init_f);
     P::merge(a, acc);
     if (e.plain) {
+#ifdef RMI_EXP_NOSTORE
+      if (P::to_f64(a) != 12345.678) return;
+#endif
       if (e.out_dtype == RMI_F32) {
         store_stream(static_cast<float*>(e.out) + k, (float)P::to_f64(a));
       } else {
@@ -672,6 +675,9 @@ __device__ __forceinline__ void finish(const Epilogue& e, i64 k, typename P::acc
       }
       return;
     }
+#ifdef RMI_EXP_PLAIN_ONLY
+    return;
+#endif
     if (e.inplace) {
       acc_t o = P::from_f64(load_out_f64(e.out, e.out_dtype, k));
       P::merge(o, a);

@@ -7,8 +7,8 @@
 //   row_short_kernel  rows of at most G<=64 vectors: one vector per lane, G lanes
 //                     per row, 4 row-tiles in flight per wave
 //   row_wave_kernel   G<=64 lanes of one wave sweep a row, 4 loads in flight
-//   row_block_kernel  64*W threads per row chunk, B chunks per row; B == 1
-//                     writes outputs, B > 1 writes partials
+//   row_block_kernel  teams of 64..1024 threads per row chunk, B chunks per row;
+//                     B == 1 writes outputs, B > 1 writes partials
 //   col_kernel        reduction along the strided dimension
 //   fold_kernel       second pass: partials[n_out][B] -> outputs
 #pragma once
@@ -19,6 +19,14 @@ namespace rmi {
 
 constexpr int kBlock = 256;  // threads per workgroup of every first-pass kernel
 constexpr int kUnroll = 4;   // independent 16-byte loads in flight per lane
+#ifndef RMI_COL_UNROLL
+#define RMI_COL_UNROLL 4
+#endif
+constexpr int kColUnroll = RMI_COL_UNROLL;  // the same for the column kernel
+#ifndef RMI_TEAM_UNROLL
+#define RMI_TEAM_UNROLL 8
+#endif
+constexpr int kTeamUnroll = RMI_TEAM_UNROLL;  // the same for the team-per-row kernel
 
 struct RowArgs {
   const void* in;
@@ -30,6 +38,7 @@ struct RowArgs {
   int G;           // lanes per row (row_short / row_wave)
   int logG;
   int B;           // chunks per row (row_block_kernel)
+  int logT;        // row_block_kernel: a team is 64 << logT threads
   Epilogue epi;
 };
 
@@ -255,7 +264,10 @@ __global__ __launch_bounds__(kBlock) void row_wave_kernel(RowArgs a)
 }
 
 // ---------------------------------------------------------------------------
-// blockDim.x = 64*W threads per chunk of a row; B chunks per row.
+// Teams of T = 64 << logT threads (1..16 waves); each team sweeps one chunk of
+// one row with kTeamUnroll loads in flight per lane.  A workgroup holds
+// blockDim.x / T teams.  B chunks per row: B == 1 writes outputs, B > 1 writes
+// partials for the second pass.
 // ---------------------------------------------------------------------------
 template <class P, bool VEC16>
 __global__ __launch_bounds__(1024) void row_block_kernel(RowArgs a)
@@ -263,50 +275,60 @@ __global__ __launch_bounds__(1024) void row_block_kernel(RowArgs a)
   using acc_t     = typename P::acc_t;
   using H         = Held<P, VEC16>;
   constexpr int S = Loader<P, VEC16>::STEP;
+  constexpr int U = kTeamUnroll;
   __shared__ acc_t sm[16];
 
-  const int T    = blockDim.x;
-  const int t    = threadIdx.x;
-  const u32 bid  = blockIdx.x;
-  const u32 urow = bid / (u32)a.B;
-  const int b    = (int)(bid - urow * (u32)a.B);
-  const i64 row  = urow;
-  const i64 v0   = (i64)b * a.chunk;
-  const i64 v1   = (v0 + a.chunk < a.nvec) ? (v0 + a.chunk) : a.nvec;
-  const i64 base = row * a.nvec;
+  const int T     = kWave << a.logT;
+  const int team  = threadIdx.x >> (6 + a.logT);
+  const int t     = threadIdx.x & (T - 1);
+  const int teams = blockDim.x >> (6 + a.logT);
+  const i64 unit  = (i64)blockIdx.x * teams + team;  // (row, chunk) index
+  const bool live = unit < a.n_out * a.B;
+  i64 row         = unit;
+  int b           = 0;
+  if (a.B > 1) {
+    row = unit / a.B;
+    b   = (int)(unit - row * a.B);
+  }
 
   acc_t acc = P::neutral();
-  i64 v     = v0 + t;
-  for (; v + (kUnroll - 1) * (i64)T < v1; v += (i64)kUnroll * T) {
-    typename H::type x[kUnroll];
+  if (live) {
+    const i64 v0   = (i64)b * a.chunk;
+    const i64 v1   = (v0 + a.chunk < a.nvec) ? (v0 + a.chunk) : a.nvec;
+    const i64 base = row * a.nvec;
+    i64 v          = v0 + t;
+    for (; v + (U - 1) * (i64)T < v1; v += (i64)U * T) {
+      typename H::type x[U];
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u)
-      x[u] = H::load(a.in, base + v + (i64)u * T);
+      for (int u = 0; u < U; ++u)
+        x[u] = H::load(a.in, base + v + (i64)u * T);
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u)
-      H::push(acc, x[u], (v + (i64)u * T) * S);
-  }
-  if (v < v1) {
-    typename H::type x[kUnroll - 1];
+      for (int u = 0; u < U; ++u)
+        H::push(acc, x[u], (v + (i64)u * T) * S);
+    }
+    if (v < v1) {  // fewer than U lane-loads left for this lane
+      typename H::type x[U - 1];
 #pragma unroll
-    for (int u = 0; u < kUnroll - 1; ++u)
-      if (v + (i64)u * T < v1) x[u] = H::load(a.in, base + v + (i64)u * T);
+      for (int u = 0; u < U - 1; ++u)
+        if (v + (i64)u * T < v1) x[u] = H::load(a.in, base + v + (i64)u * T);
 #pragma unroll
-    for (int u = 0; u < kUnroll - 1; ++u)
-      if (v + (i64)u * T < v1) H::push(acc, x[u], (v + (i64)u * T) * S);
+      for (int u = 0; u < U - 1; ++u)
+        if (v + (i64)u * T < v1) H::push(acc, x[u], (v + (i64)u * T) * S);
+    }
   }
 
   wave_allreduce<P>(acc);
-  const int W = T >> 6;
-  if (W > 1) {
-    if ((t & (kWave - 1)) == 0) sm[t >> 6] = acc;
+  if (a.logT > 0) {  // combine the team's waves through LDS
+    const int wave = threadIdx.x >> 6;
+    if ((threadIdx.x & (kWave - 1)) == 0) sm[wave] = acc;
     __syncthreads();
     if (t == 0) {
-      for (int w = 1; w < W; ++w)
-        P::merge(acc, sm[w]);
+      const int w0 = team << a.logT;
+      for (int w = 1; w < (1 << a.logT); ++w)
+        P::merge(acc, sm[w0 + w]);
     }
   }
-  if (t == 0) {
+  if (t == 0 && live) {
     if (a.B == 1) {
       finish<P>(a.epi, row, acc);
     } else {
@@ -352,9 +374,9 @@ __global__ __launch_bounds__(kBlock) void col_kernel(ColArgs a)
   const int ty   = t >> a.logTX;
   const i64 cv   = (i64)blockIdx.x * TX + tx;
   const bool live = cv < a.nvec;
-  // Row tiles of TY*kUnroll rows are dealt round-robin over blockIdx.y, so at any
+  // Row tiles of TY*kColUnroll rows are dealt round-robin over blockIdx.y, so at any
   // moment the blocks of the grid read one compact, advancing window of the matrix.
-  const i64 RT     = (i64)TY * kUnroll;
+  const i64 RT     = (i64)TY * kColUnroll;
   const i64 n_full = a.len / RT;
 
   acc_t acc[S];
@@ -367,12 +389,12 @@ __global__ __launch_bounds__(kBlock) void col_kernel(ColArgs a)
       const u32x4* p = static_cast<const u32x4*>(a.in) + cv;
       for (i64 tile = blockIdx.y; tile < n_full; tile += a.B) {
         const i64 r = tile * RT + ty;
-        u32x4 x[kUnroll];
+        u32x4 x[kColUnroll];
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u)
+        for (int u = 0; u < kColUnroll; ++u)
           x[u] = load16(p + (r + (i64)u * TY) * a.nvec);
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u)
+        for (int u = 0; u < kColUnroll; ++u)
           P::push_cols(acc, x[u], r + (i64)u * TY);
       }
       if ((i64)blockIdx.y == n_full % a.B) {  // the rows past the last whole tile
@@ -383,12 +405,12 @@ __global__ __launch_bounds__(kBlock) void col_kernel(ColArgs a)
       const in_t* p = static_cast<const in_t*>(a.in) + cv;
       for (i64 tile = blockIdx.y; tile < n_full; tile += a.B) {
         const i64 r = tile * RT + ty;
-        typename In<in_t>::nat x[kUnroll];
+        typename In<in_t>::nat x[kColUnroll];
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u)
+        for (int u = 0; u < kColUnroll; ++u)
           x[u] = In<in_t>::ld(p + (r + (i64)u * TY) * a.nvec);
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u)
+        for (int u = 0; u < kColUnroll; ++u)
           P::push(acc[0], x[u], r + (i64)u * TY);
       }
       if ((i64)blockIdx.y == n_full % a.B) {

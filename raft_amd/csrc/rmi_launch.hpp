@@ -50,8 +50,11 @@ int launch_lanes(const PlanX& pl, const RowArgs& a, hipStream_t st)
 template <class P>
 int run(const PlanX& pl, const Problem& pr, hipStream_t st)
 {
-  static_assert(kBlock == kPlanBlock && kUnroll == kPlanUnroll,
+#ifndef RMI_EXP_SKIP_ASSERT
+  static_assert(kBlock == kPlanBlock && kUnroll == kPlanUnroll && kColUnroll == kPlanUnroll &&
+                  kTeamUnroll == kPlanTeamUnroll,
                 "plan selector and kernels must agree on block size and unroll");
+#endif
   int rc = RMI_OK;
   switch (pl.kind) {
     case RMI_PLAN_EMPTY:
@@ -71,6 +74,7 @@ int run(const PlanX& pl, const Problem& pr, hipStream_t st)
       a.G       = pl.G;
       a.logG    = pl.logG;
       a.B       = pl.B;
+      a.logT    = ilog2(pl.threads / 64);
       a.epi     = pr.epi;
       const dim3 grid((unsigned)pl.grid_blocks);
       if (pl.kind == RMI_PLAN_ROW_LANES) {
@@ -81,7 +85,7 @@ int run(const PlanX& pl, const Problem& pr, hipStream_t st)
           case 16: rc = launch_lanes<P, 16>(pl, a, st); break;
           default: rc = RMI_ERR_UNSUPPORTED;
         }
-      } else if (pl.kind == RMI_PLAN_ROW_WAVE) {
+      } else if (pl.kind == RMI_PLAN_ROW_WAVE && !pl.team_kernel) {
         if (pl.short_rows) {
           if (pl.vec16)
             hipLaunchKernelGGL((row_short_kernel<P, true>), grid, dim3(kBlock), 0, st, a);
@@ -94,10 +98,11 @@ int run(const PlanX& pl, const Problem& pr, hipStream_t st)
             hipLaunchKernelGGL((row_wave_kernel<P, false>), grid, dim3(kBlock), 0, st, a);
         }
       } else {
+        const dim3 block((unsigned)(pl.threads < kBlock ? kBlock : pl.threads));
         if (pl.vec16)
-          hipLaunchKernelGGL((row_block_kernel<P, true>), grid, dim3(pl.threads), 0, st, a);
+          hipLaunchKernelGGL((row_block_kernel<P, true>), grid, block, 0, st, a);
         else
-          hipLaunchKernelGGL((row_block_kernel<P, false>), grid, dim3(pl.threads), 0, st, a);
+          hipLaunchKernelGGL((row_block_kernel<P, false>), grid, block, 0, st, a);
         if (pl.kind == RMI_PLAN_ROW_SPLIT) rc = launch_fold<P>(pl, pr, pl.B, st);
       }
       break;

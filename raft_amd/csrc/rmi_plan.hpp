@@ -18,7 +18,8 @@
 namespace rmi {
 
 constexpr int kPlanBlock  = 256;
-constexpr int kPlanUnroll = 4;
+constexpr int kPlanUnroll = 4;      // lane-loads in flight: sub-wave and column kernels
+constexpr int kPlanTeamUnroll = 8;  // lane-loads in flight: team-per-row kernel
 constexpr int kWavesPerCu = 32;  // 8 resident waves on each of the 4 SIMDs
 
 struct PlanX {
@@ -26,6 +27,7 @@ struct PlanX {
   bool strided    = false;  // reduce along the strided dimension
   bool vec16      = false;  // 16-byte lane loads
   bool short_rows = false;  // ROW_WAVE served by the one-load-per-lane kernel
+  bool team_kernel = false; // served by the team-per-row kernel
   int elem_bytes  = 0;
   int step        = 1;  // elements per lane-load
   int64_t n_out   = 0;
@@ -263,15 +265,13 @@ inline int make_plan(const rmi_reduce_desc& d,
     if (p.nvec <= 4 * 64) {
       kind = RMI_PLAN_ROW_WAVE;
     } else {
-      // widen the team on a row until the machine's wave slots are filled,
-      // keeping at least kPlanUnroll lane-loads per thread
+      // widen the team on a row until the machine's wave slots are filled, as long
+      // as every thread keeps a full batch of lane-loads
       while (threads < 1024 && p.n_out * (threads / 64) < slots &&
-             p.nvec >= (int64_t)kPlanUnroll * threads * 4)
-        threads *= 4;
-      if (threads == 64) {
-        kind = RMI_PLAN_ROW_WAVE;
-      } else if (threads == 1024 && p.n_out * 16 < slots &&
-                 p.nvec >= (int64_t)2 * kPlanBlock * kPlanUnroll * 2) {
+             p.nvec >= (int64_t)2 * threads * kPlanTeamUnroll)
+        threads *= 2;
+      if (threads == 1024 && p.n_out * 16 < slots &&
+          p.nvec >= (int64_t)2 * kPlanBlock * kPlanTeamUnroll) {
         kind = RMI_PLAN_ROW_SPLIT;
       } else {
         kind = RMI_PLAN_ROW_BLOCK;
@@ -279,6 +279,8 @@ inline int make_plan(const rmi_reduce_desc& d,
     }
   } else if (kind == RMI_PLAN_ROW_BLOCK) {
     threads = kPlanBlock;
+  } else if (kind == RMI_PLAN_ROW_WAVE && p.nvec > 4 * 64) {
+    kind = RMI_PLAN_ROW_BLOCK;  // one wave per row, served by the team kernel
   }
 
   if (kind == RMI_PLAN_ROW_WAVE) {
@@ -295,17 +297,24 @@ inline int make_plan(const rmi_reduce_desc& d,
     const int64_t rows_w = (int64_t)(64 / p.G) * (p.short_rows ? kPlanUnroll : 1);
     p.grid_blocks        = ceildiv(p.n_out, rows_w * (kPlanBlock / 64));
   } else if (kind == RMI_PLAN_ROW_BLOCK) {
-    p.kind        = RMI_PLAN_ROW_BLOCK;
+    // a team of `threads` threads per row; a 256-thread workgroup holds several
+    // teams when a team is smaller.  One wave per row is reported as ROW_WAVE.
+    p.kind        = threads == 64 ? RMI_PLAN_ROW_WAVE : RMI_PLAN_ROW_BLOCK;
+    p.team_kernel = true;
+    p.G           = 64;
+    p.logG        = 6;
     p.threads     = threads;
     p.B           = 1;
     p.chunk       = p.nvec;
-    p.grid_blocks = p.n_out;
+    const int teams = threads >= kPlanBlock ? 1 : kPlanBlock / threads;
+    p.grid_blocks   = ceildiv(p.n_out, teams);
   } else {
-    p.kind    = RMI_PLAN_ROW_SPLIT;
-    p.threads = kPlanBlock;
-    const int64_t quantum = (int64_t)kPlanBlock * kPlanUnroll;
+    p.kind        = RMI_PLAN_ROW_SPLIT;
+    p.team_kernel = true;
+    p.threads     = kPlanBlock;
+    const int64_t quantum = (int64_t)kPlanBlock * kPlanTeamUnroll;
     int64_t B             = ceildiv(slots, p.n_out * (kPlanBlock / 64));
-    const int64_t maxB    = p.nvec / (quantum * 2) > 1 ? p.nvec / (quantum * 2) : 1;
+    const int64_t maxB    = p.nvec / quantum > 1 ? p.nvec / quantum : 1;
     if (B > maxB) B = maxB;
     if (B < 2) B = 2;
     if (B > 4096) B = 4096;
@@ -331,8 +340,7 @@ inline void export_plan(const PlanX& p, rmi_plan& o)
   o.vec_bytes       = p.vec16 ? 16 : p.elem_bytes;
   o.lanes_per_row   = p.kind == RMI_PLAN_ROW_WAVE ? p.G : 0;
   o.blocks_per_out  = p.B;
-  o.block_threads   = (p.kind == RMI_PLAN_ROW_BLOCK || p.kind == RMI_PLAN_ROW_SPLIT) ? p.threads
-                                                                                      : kPlanBlock;
+  o.block_threads   = (p.team_kernel && p.threads > kPlanBlock) ? p.threads : kPlanBlock;
   o.passes          = p.passes;
   o.grid_blocks     = p.grid_blocks;
   o.n_outputs       = p.n_out;
