@@ -96,7 +96,10 @@ int reduce_impl(const rmi_reduce_desc& d,
     key.family == kFamKvp
       ? false
       : (key.family == kFamInt ? true : (d.out_dtype == RMI_F32 || d.out_dtype == RMI_F64));
-  pr.epi.plain         = (!d.inplace && d.final_op == RMI_FIN_IDENTITY && natural_out) ? 1 : 0;
+  const bool simple_final =
+    d.final_op == RMI_FIN_IDENTITY ||
+    (key.family != kFamInt && (d.final_op == RMI_FIN_SQRT || d.final_op == RMI_FIN_MUL_CONST));
+  pr.epi.plain         = (!d.inplace && simple_final && natural_out) ? 1 : 0;
   pr.epi.out_aligned16 = aligned(out, 16) ? 1 : 0;
   return lookup(key)(pl, pr, static_cast<hipStream_t>(stream));
 }

@@ -551,9 +551,10 @@ struct Epilogue {
   int out_dtype;
   int final_op;
   int inplace;
-  // Set by the host when final_op is the identity, inplace is off and the output
-  // is stored in the accumulator's own family (f32 / f64, i32 / i64, key-value
-  // pair): the common case, kept free of the general epilogue's branches.
+  // Set by the host when inplace is off, the output is stored in the accumulator's
+  // own family (f32 / f64, i32 / i64) and final_op is the identity (floating
+  // outputs: also sqrt or a multiplication by a constant): the common cases, kept
+  // free of the general epilogue's branches.
   int plain;
   int out_aligned16;  // the output pointer is 16-byte aligned
 };
@@ -665,19 +666,21 @@ __device__ __forceinline__ void finish(const Epilogue& e, i64 k, typename P::acc
     acc_t a = P::from_f64(e.init_f);
     P::merge(a, acc);
     if (e.plain) {
-#ifdef RMI_EXP_NOSTORE
-      if (P::to_f64(a) != 12345.678) return;
-#endif
+      // identity, sqrt or a multiplication by a constant, stored as f32 or f64:
+      // the epilogues of sums, L2 norms and means
       if (e.out_dtype == RMI_F32) {
-        store_stream(static_cast<float*>(e.out) + k, (float)P::to_f64(a));
+        float y = (float)P::to_f64(a);
+        if (e.final_op == RMI_FIN_SQRT) y = sqrt(y);
+        if (e.final_op == RMI_FIN_MUL_CONST) y = y * (float)e.s1;
+        store_stream(static_cast<float*>(e.out) + k, y);
       } else {
-        store_stream(static_cast<double*>(e.out) + k, P::to_f64(a));
+        double y = P::to_f64(a);
+        if (e.final_op == RMI_FIN_SQRT) y = sqrt(y);
+        if (e.final_op == RMI_FIN_MUL_CONST) y = y * e.s1;
+        store_stream(static_cast<double*>(e.out) + k, y);
       }
       return;
     }
-#ifdef RMI_EXP_PLAIN_ONLY
-    return;
-#endif
     if (e.inplace) {
       acc_t o = P::from_f64(load_out_f64(e.out, e.out_dtype, k));
       P::merge(o, a);

@@ -4,7 +4,7 @@
 // a row's byte length or the base pointer is not a multiple of 16.
 //
 //   row_lanes_kernel  K whole rows inside one 16-byte vector: no cross-lane step
-//   row_short_kernel  rows of at most G<=64 vectors: one vector per lane, G lanes
+//   row_short_kernel  rows of at most G<=8 vectors: one vector per lane, G lanes
 //                     per row, 4 row-tiles in flight per wave
 //   row_wave_kernel   G<=64 lanes of one wave sweep a row, 4 loads in flight
 //   row_block_kernel  teams of 64..1024 threads per row chunk, B chunks per row;
@@ -387,15 +387,30 @@ __global__ __launch_bounds__(kBlock) void col_kernel(ColArgs a)
   if (live) {
     if constexpr (VEC16) {
       const u32x4* p = static_cast<const u32x4*>(a.in) + cv;
-      for (i64 tile = blockIdx.y; tile < n_full; tile += a.B) {
-        const i64 r = tile * RT + ty;
-        u32x4 x[kColUnroll];
+      // two tiles in flight: the loads of the next tile are issued before the
+      // current one is accumulated
+      i64 tile = blockIdx.y;
+      u32x4 x[kColUnroll];
+      if (tile < n_full) {
 #pragma unroll
         for (int u = 0; u < kColUnroll; ++u)
-          x[u] = load16(p + (r + (i64)u * TY) * a.nvec);
+          x[u] = load16(p + (tile * RT + ty + (i64)u * TY) * a.nvec);
+      }
+      while (tile < n_full) {
+        const i64 next = tile + a.B;
+        u32x4 y[kColUnroll];
+        if (next < n_full) {
+#pragma unroll
+          for (int u = 0; u < kColUnroll; ++u)
+            y[u] = load16(p + (next * RT + ty + (i64)u * TY) * a.nvec);
+        }
 #pragma unroll
         for (int u = 0; u < kColUnroll; ++u)
-          P::push_cols(acc, x[u], r + (i64)u * TY);
+          P::push_cols(acc, x[u], tile * RT + ty + (i64)u * TY);
+#pragma unroll
+        for (int u = 0; u < kColUnroll; ++u)
+          x[u] = y[u];
+        tile = next;
       }
       if ((i64)blockIdx.y == n_full % a.B) {  // the rows past the last whole tile
         for (i64 r = n_full * RT + ty; r < a.len; r += TY)

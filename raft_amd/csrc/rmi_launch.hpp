@@ -77,6 +77,7 @@ int run(const PlanX& pl, const Problem& pr, hipStream_t st)
       a.logT    = ilog2(pl.threads / 64);
       a.epi     = pr.epi;
       const dim3 grid((unsigned)pl.grid_blocks);
+      const unsigned lds = (unsigned)pl.lds_reserve;
       if (pl.kind == RMI_PLAN_ROW_LANES) {
         switch (pl.K) {
           case 2: rc = launch_lanes<P, 2>(pl, a, st); break;
@@ -93,7 +94,7 @@ int run(const PlanX& pl, const Problem& pr, hipStream_t st)
             hipLaunchKernelGGL((row_short_kernel<P, false>), grid, dim3(kBlock), 0, st, a);
         } else {
           if (pl.vec16)
-            hipLaunchKernelGGL((row_wave_kernel<P, true>), grid, dim3(kBlock), 0, st, a);
+            hipLaunchKernelGGL((row_wave_kernel<P, true>), grid, dim3(kBlock), lds, st, a);
           else
             hipLaunchKernelGGL((row_wave_kernel<P, false>), grid, dim3(kBlock), 0, st, a);
         }

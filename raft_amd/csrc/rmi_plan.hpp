@@ -21,6 +21,11 @@ constexpr int kPlanBlock  = 256;
 constexpr int kPlanUnroll = 4;      // lane-loads in flight: sub-wave and column kernels
 constexpr int kPlanTeamUnroll = 8;  // lane-loads in flight: team-per-row kernel
 constexpr int kWavesPerCu = 32;  // 8 resident waves on each of the 4 SIMDs
+// Workgroups per CU of the persistent column kernel.  Measured on MI355X: with two
+// tiles in flight per workgroup, 2 per CU (8 waves) sustains ~7.1 TB/s; 4 and 8 per CU
+// lose 2 and 8 points to queueing in the memory system.
+constexpr int kColBlocksPerCu = 2;
+constexpr int kLdsPerCu       = 160 * 1024;  // LDS bytes of one gfx950 CU
 
 struct PlanX {
   int kind        = RMI_PLAN_EMPTY;
@@ -44,6 +49,7 @@ struct PlanX {
   int64_t gridx   = 0;  // COL_TILE: blocks along the contiguous dimension
   int64_t grid_blocks    = 0;
   int passes             = 1;
+  int lds_reserve        = 0;  // dynamic LDS bytes reserved only to cap occupancy
   int acc_bytes          = 8;
   size_t ws_bytes        = 0;
 };
@@ -227,10 +233,10 @@ inline int make_plan(const rmi_reduce_desc& d,
     p.logTX = ilog2(p.TX);
     const int TY = kPlanBlock / p.TX;
     p.gridx      = ceildiv(p.nvec, p.TX);
-    // row tiles of TY*unroll rows are dealt round-robin to B blocks: enough blocks
-    // to give every CU several, but at least two tiles per block
+    // row tiles of TY*unroll rows are dealt round-robin to B blocks: kColBlocksPerCu
+    // blocks per CU, but at least two tiles per block
     const int64_t tile_rows = (int64_t)TY * kPlanUnroll;
-    int64_t B               = ceildiv((int64_t)n_cu * 8, p.gridx);
+    int64_t B               = ceildiv((int64_t)n_cu * kColBlocksPerCu, p.gridx);
     const int64_t maxB      = ceildiv(p.len, tile_rows * 2);
     if (B > maxB) B = maxB;
     if (B < 1) B = 1;
@@ -296,6 +302,15 @@ inline int make_plan(const rmi_reduce_desc& d,
     p.logG               = ilog2(p.G);
     const int64_t rows_w = (int64_t)(64 / p.G) * (p.short_rows ? kPlanUnroll : 1);
     p.grid_blocks        = ceildiv(p.n_out, rows_w * (kPlanBlock / 64));
+    if (!p.short_rows && p.vec16) {
+      // Bytes in flight per CU are what the memory system is sensitive to: about
+      // 80 KB (5 workgroups of 256 lanes x 4 loads x 16 B) sustains the most; the
+      // default 8 resident workgroups lose 3-4 points to queueing.  A dynamic LDS
+      // reservation the kernel never touches caps the resident workgroups.
+      const int64_t loads_per_lane = ceildiv(p.nvec, p.G);
+      if (loads_per_lane >= 4) p.lds_reserve = kLdsPerCu / 5 - 768;
+      else if (loads_per_lane == 3) p.lds_reserve = kLdsPerCu / 6 - 768;
+    }
   } else if (kind == RMI_PLAN_ROW_BLOCK) {
     // a team of `threads` threads per row; a 256-thread workgroup holds several
     // teams when a team is smaller.  One wave per row is reported as ROW_WAVE.
