@@ -219,6 +219,7 @@ def main():
                    alg_bytes=alg_bytes(w), GBps=alg_bytes(w) / (ms * 1e-3) / 1e9,
                    rows_per_s=w["rows"] / (ms * 1e-3))
         res["pct_of_peak"] = 100.0 * res["GBps"] / PEAK_HBM_GBPS
+        res["hbm_traffic_bytes_rocprof"] = MEASURED_TRAFFIC.get(name)
 
         # the same launches replayed from a HIP graph: removes host launch gaps, which
         # dominate the shapes whose kernel is only a few microseconds long
@@ -406,6 +407,24 @@ def main():
             torch.cuda.synchronize()
         return
 
+    def launch_floor_us():
+        # the fixed cost of one launch: a reduction whose data is a few KB, same call path
+        x = torch.zeros(64 * 64, dtype=torch.float32, device=devc)
+        o = torch.zeros(64, dtype=torch.float32, device=devc)
+        d = api.make_desc(api.F32, api.F32, 64, 64)
+        ref = C.byref(d)
+        for _ in range(20):
+            lib.rmi_reduce(ref, x.data_ptr(), o.data_ptr(), None, 0, sptr)
+        torch.cuda.synchronize()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for _ in range(200):
+            lib.rmi_reduce(ref, x.data_ptr(), o.data_ptr(), None, 0, sptr)
+        e1.record(stream)
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / 200 * 1e3
+
     results = {}
     cpu = {}
     for name in names:
@@ -439,6 +458,7 @@ def main():
                      "unit": "GB/s", "frac": head["GBps"] / PEAK_HBM_GBPS,
                      "traffic": MEASURED_TRAFFIC.get(HEADLINE)},
         "cpu_baseline": cpu.get(HEADLINE),
+        "launch_floor_us": launch_floor_us(),
         "configs": results,
         "cpu_baselines": cpu,
         "device": torch.cuda.get_device_name(0),
@@ -448,7 +468,10 @@ def main():
 
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs (see
 # profiles/), scaled by the same counters' reading for a copy kernel of known size.
-MEASURED_TRAFFIC: dict[str, float | None] = {}
+MEASURED_TRAFFIC: dict[str, float | None] = {
+    "cfg1": 10.33e6, "cfg2": 516.04e6, "cfg3_mean": 2561.36e6, "cfg3_stddev": 2561.37e6,
+    "cfg4": 8388.84e6, "cfg5a": 67.26e6, "cfg5b": 268.57e6, "cfg5c": 67.30e6,
+}
 
 
 if __name__ == "__main__":

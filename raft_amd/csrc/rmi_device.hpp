@@ -650,8 +650,8 @@ struct out_kvp {
   V value;
 };
 
-// Outputs use ordinary stores: small or strided non-temporal stores bypass the
-// L2's write combining and measured slower on every shape.
+// Single outputs use ordinary stores: small or strided non-temporal stores bypass
+// the L2's write combining and measured slower on every shape.
 template <class T>
 __device__ __forceinline__ void store_stream(T* p, T v)
 {
@@ -747,7 +747,8 @@ __device__ __forceinline__ void finish_run(const Epilogue& e, i64 k0, typename P
         v[1] = (u32)((u64)a >> 32);
         v[2] = (u32)(u64)b;
         v[3] = (u32)((u64)b >> 32);
-        *reinterpret_cast<u32x4*>(static_cast<i64*>(e.out) + k0 + r) = v;
+        // whole 16-byte lane stores, contiguous across the wave: streamed past the caches
+        __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(static_cast<i64*>(e.out) + k0 + r));
       }
       return;
     }

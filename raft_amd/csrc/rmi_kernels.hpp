@@ -19,14 +19,8 @@ namespace rmi {
 
 constexpr int kBlock = 256;  // threads per workgroup of every first-pass kernel
 constexpr int kUnroll = 4;   // independent 16-byte loads in flight per lane
-#ifndef RMI_COL_UNROLL
-#define RMI_COL_UNROLL 4
-#endif
-constexpr int kColUnroll = RMI_COL_UNROLL;  // the same for the column kernel
-#ifndef RMI_TEAM_UNROLL
-#define RMI_TEAM_UNROLL 8
-#endif
-constexpr int kTeamUnroll = RMI_TEAM_UNROLL;  // the same for the team-per-row kernel
+constexpr int kColUnroll  = 4;  // rows per lane and tile in the column kernel
+constexpr int kTeamUnroll = 8;  // loads in flight per lane in the team-per-row kernel
 
 struct RowArgs {
   const void* in;

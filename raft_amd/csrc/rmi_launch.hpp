@@ -50,11 +50,9 @@ int launch_lanes(const PlanX& pl, const RowArgs& a, hipStream_t st)
 template <class P>
 int run(const PlanX& pl, const Problem& pr, hipStream_t st)
 {
-#ifndef RMI_EXP_SKIP_ASSERT
   static_assert(kBlock == kPlanBlock && kUnroll == kPlanUnroll && kColUnroll == kPlanUnroll &&
                   kTeamUnroll == kPlanTeamUnroll,
                 "plan selector and kernels must agree on block size and unroll");
-#endif
   int rc = RMI_OK;
   switch (pl.kind) {
     case RMI_PLAN_EMPTY:
