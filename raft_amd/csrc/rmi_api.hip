@@ -45,14 +45,14 @@ run_fn lookup(const PolicyKey& k)
 
 bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 
-int plan_for(const rmi_reduce_desc* desc, bool aligned16, PlanX& pl, PolicyKey& key)
+int plan_for(const rmi_reduce_desc* desc, PlanX& pl, PolicyKey& key)
 {
   if (desc == nullptr) return RMI_ERR_NULL;
   int acc_bytes = 8;
   int rc        = classify(*desc, key, acc_bytes);
   if (rc != RMI_OK) return rc;
   if (lookup(key) == nullptr) return RMI_ERR_UNSUPPORTED;
-  return make_plan(*desc, key, acc_bytes, aligned16, cu_count(), pl);
+  return make_plan(*desc, key, acc_bytes, cu_count(), pl);
 }
 
 int reduce_impl(const rmi_reduce_desc& d,
@@ -64,7 +64,7 @@ int reduce_impl(const rmi_reduce_desc& d,
 {
   PlanX pl;
   PolicyKey key;
-  int rc = plan_for(&d, aligned(in, 16), pl, key);
+  int rc = plan_for(&d, pl, key);
   if (rc != RMI_OK) return rc;
   if (pl.n_out == 0) return RMI_OK;
   if (out == nullptr) return RMI_ERR_NULL;
@@ -149,7 +149,7 @@ int rmi_plan_query(const rmi_reduce_desc* desc, rmi_plan* plan)
   if (plan == nullptr) return RMI_ERR_NULL;
   rmi::PlanX pl;
   rmi::PolicyKey key;
-  const int rc = rmi::plan_for(desc, true, pl, key);
+  const int rc = rmi::plan_for(desc, pl, key);
   if (rc != RMI_OK) return rc;
   rmi::export_plan(pl, *plan);
   return RMI_OK;
@@ -157,13 +157,10 @@ int rmi_plan_query(const rmi_reduce_desc* desc, rmi_plan* plan)
 
 size_t rmi_reduce_workspace_bytes(const rmi_reduce_desc* desc)
 {
-  // Whether the 16-byte-vector or the element-wise variant runs depends on the
-  // input pointer's alignment, known only at rmi_reduce time: size for both.
-  rmi::PlanX a, u;
+  rmi::PlanX pl;
   rmi::PolicyKey key;
-  if (rmi::plan_for(desc, true, a, key) != RMI_OK) return 0;
-  if (rmi::plan_for(desc, false, u, key) != RMI_OK) return a.ws_bytes;
-  return a.ws_bytes > u.ws_bytes ? a.ws_bytes : u.ws_bytes;
+  if (rmi::plan_for(desc, pl, key) != RMI_OK) return 0;
+  return pl.ws_bytes;
 }
 
 int rmi_reduce(const rmi_reduce_desc* desc,

@@ -31,10 +31,14 @@ using f16_t = _Float16;
 // ---------------------------------------------------------------------------
 // Loads
 // ---------------------------------------------------------------------------
+// 16 bytes at any byte address: gfx950 runs global memory in unaligned access
+// mode, so one global_load_dwordx4 serves aligned and unaligned addresses alike.
+typedef u32x4 u32x4_unaligned __attribute__((aligned(1)));
+
 __device__ __forceinline__ u32x4 load16(const void* p)
 {
   // One global_load_dwordx4 per lane; streamed once, so mark it non-temporal.
-  return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+  return __builtin_nontemporal_load(reinterpret_cast<const u32x4_unaligned*>(p));
 }
 
 __device__ __forceinline__ float as_f32(u32 w) { return __uint_as_float(w); }
@@ -511,6 +515,35 @@ struct PolKvp {
     return acc_t{xchg<SEL>(a.key), xchg<SEL>(a.value)};
   }
 };
+
+// ---------------------------------------------------------------------------
+// The last, overlapping vector of a row whose length is not a multiple of VEC:
+// it ends exactly at the row's end, so its first `skip` elements were already
+// folded by the previous whole vector and only elements j >= skip count.
+// ---------------------------------------------------------------------------
+template <class P>
+__device__ __forceinline__ void push_vec_from(typename P::acc_t& a,
+                                              const u32x4& v,
+                                              i64 idx0,
+                                              int skip)
+{
+  using in_t = typename P::in_t;
+  static_for<P::VEC>([&](auto j) {
+    if (j >= skip) P::push(a, In<in_t>::template get<j>(v), idx0 + j);
+  });
+}
+
+template <class P>
+__device__ __forceinline__ void push_cols_from(typename P::acc_t (&a)[P::VEC],
+                                               const u32x4& v,
+                                               i64 idx,
+                                               int skip)
+{
+  using in_t = typename P::in_t;
+  static_for<P::VEC>([&](auto j) {
+    if (j >= skip) P::push(a[j], In<in_t>::template get<j>(v), idx);
+  });
+}
 
 // ---------------------------------------------------------------------------
 // Wave-level all-reduce over groups of G lanes (G a power of two, 1..64).

@@ -1,12 +1,14 @@
 // The gfx950 reduction kernels, templated on an accumulator policy
-// (rmi_device.hpp).  VEC16 = true: rows are read as 16-byte vectors
-// (global_load_dwordx4 per lane); false: one element per lane-load, used when
-// a row's byte length or the base pointer is not a multiple of 16.
+// (rmi_device.hpp).  VEC16 = true: a row is read as 16-byte vectors
+// (global_load_dwordx4 per lane, at any byte alignment); a row length that is not
+// a multiple of the vector width ends with one more vector that overlaps the
+// previous one and counts only its new elements.  false: one element per
+// lane-load, used for rows shorter than 16 bytes.
 //
 //   row_lanes_kernel  K whole rows inside one 16-byte vector: no cross-lane step
 //   row_short_kernel  rows of at most G<=8 vectors: one vector per lane, G lanes
 //                     per row, 4 row-tiles in flight per wave
-//   row_wave_kernel   G<=64 lanes of one wave sweep a row, 4 loads in flight
+//   row_wave_kernel   G<=64 lanes of one wave per row, at most 4 loads per lane
 //   row_block_kernel  teams of 64..1024 threads per row chunk, B chunks per row;
 //                     B == 1 writes outputs, B > 1 writes partials
 //   col_kernel        reduction along the strided dimension
@@ -17,18 +19,20 @@
 
 namespace rmi {
 
-constexpr int kBlock = 256;  // threads per workgroup of every first-pass kernel
-constexpr int kUnroll = 4;   // independent 16-byte loads in flight per lane
-constexpr int kColUnroll  = 4;  // rows per lane and tile in the column kernel
-constexpr int kTeamUnroll = 8;  // loads in flight per lane in the team-per-row kernel
+constexpr int kBlock      = 256;  // threads per workgroup (the team kernel may use up to 1024)
+constexpr int kUnroll     = 4;    // independent 16-byte loads in flight per lane
+constexpr int kColUnroll  = 4;    // rows per lane and tile in the column kernel
+constexpr int kTeamUnroll = 8;    // loads in flight per lane in the team-per-row kernel
 
 struct RowArgs {
   const void* in;
   void* partial;   // [n_out][B] accumulators, ROW_SPLIT only
   i64 n_out;       // rows
   i64 len;         // elements per row
-  i64 nvec;        // lane-loads per row: len/VEC (VEC16) or len (scalar)
-  i64 chunk;       // lane-loads per block chunk (row_block_kernel)
+  i64 row_bytes;   // len * sizeof(element)
+  i64 nvec;        // whole lane-loads per row: len / VEC (VEC16) or len (element-wise)
+  i64 chunk;       // lane-loads per team chunk (row_block_kernel)
+  int tail;        // VEC16: elements after the last whole vector (len % VEC)
   int G;           // lanes per row (row_short / row_wave)
   int logG;
   int B;           // chunks per row (row_block_kernel)
@@ -38,13 +42,15 @@ struct RowArgs {
 
 struct ColArgs {
   const void* in;
-  void* partial;      // [n_out][B] accumulators when B > 1
-  i64 n_out;          // D: length of the contiguous dimension
-  i64 len;            // N: number of strided rows folded
-  i64 nvec;           // lane-loads per row: D/VEC (VEC16) or D (scalar)
-  int TX;             // lanes along the contiguous dimension (power of two <= 64)
+  void* partial;   // [n_out][B] accumulators when B > 1
+  i64 n_out;       // D: length of the contiguous dimension
+  i64 len;         // N: number of strided rows folded
+  i64 row_bytes;   // D * sizeof(element)
+  i64 nvec;        // whole lane-loads per row: D / VEC (VEC16) or D (element-wise)
+  int tail;        // VEC16: columns after the last whole vector (D % VEC)
+  int TX;          // lanes along the contiguous dimension (power of two <= 64)
   int logTX;
-  int B;              // gridDim.y
+  int B;           // gridDim.y
   Epilogue epi;
 };
 
@@ -57,23 +63,19 @@ struct FoldArgs {
   Epilogue epi;
 };
 
-template <class P, bool VEC16>
-struct Loader {
-  using in_t                = typename P::in_t;
-  static constexpr int STEP = VEC16 ? P::VEC : 1;  // elements per lane-load
-};
-
-// A lane-load held in registers between issue and use.
+// A lane-load held in registers between issue and use.  `row` points at the first
+// byte of a row, `v` counts lane-loads from there.
 template <class P, bool VEC16>
 struct Held {
-  using in_t = typename P::in_t;
-  using type = std::conditional_t<VEC16, u32x4, typename In<in_t>::nat>;
-  static __device__ __forceinline__ type load(const void* in, i64 at)
+  using in_t                = typename P::in_t;
+  using type                = std::conditional_t<VEC16, u32x4, typename In<in_t>::nat>;
+  static constexpr int STEP = VEC16 ? P::VEC : 1;  // elements per lane-load
+  static __device__ __forceinline__ type load(const char* row, i64 v)
   {
     if constexpr (VEC16) {
-      return load16(static_cast<const u32x4*>(in) + at);
+      return load16(row + v * 16);
     } else {
-      return In<in_t>::ld(static_cast<const in_t*>(in) + at);
+      return In<in_t>::ld(reinterpret_cast<const in_t*>(row) + v);
     }
   }
   static __device__ __forceinline__ void push(typename P::acc_t& a, const type& x, i64 idx0)
@@ -82,6 +84,34 @@ struct Held {
       P::push_vec(a, x, idx0);
     } else {
       P::push(a, x, idx0);
+    }
+  }
+  // Lane-load `v` of a row of `nvec` whole vectors and `tail` further elements:
+  // v < nvec is whole vector v; v == nvec is the overlapping last vector that ends
+  // at the row's end (VEC16 rows hold at least one whole vector).
+  static __device__ __forceinline__ type load_any(const char* row, i64 v, i64 nvec, i64 len)
+  {
+    if constexpr (VEC16) {
+      return load16(v < nvec ? row + v * 16 : row + (len - P::VEC) * (i64)sizeof(in_t));
+    } else {
+      return In<in_t>::ld(reinterpret_cast<const in_t*>(row) + v);
+    }
+  }
+  static __device__ __forceinline__ void push_any(typename P::acc_t& a,
+                                                  const type& x,
+                                                  i64 v,
+                                                  i64 nvec,
+                                                  i64 len,
+                                                  int tail)
+  {
+    if constexpr (VEC16) {
+      if (v < nvec) {
+        P::push_vec(a, x, v * P::VEC);
+      } else {
+        push_vec_from<P>(a, x, len - P::VEC, P::VEC - tail);
+      }
+    } else {
+      P::push(a, x, v);
     }
   }
 };
@@ -103,6 +133,23 @@ __device__ __forceinline__ typename P::acc_t shfl_acc(const typename P::acc_t& a
   return r;
 }
 
+// Accumulator of lane (lane ^ mask).
+template <class P>
+__device__ __forceinline__ typename P::acc_t bperm_acc(const typename P::acc_t& a, int mask)
+{
+  using acc_t = typename P::acc_t;
+  static_assert(sizeof(acc_t) % 4 == 0, "accumulators are moved word by word");
+  constexpr int NW = sizeof(acc_t) / 4;
+  u32 w[NW];
+  __builtin_memcpy(w, &a, sizeof(acc_t));
+#pragma unroll
+  for (int i = 0; i < NW; ++i)
+    w[i] = (u32)__shfl_xor((int)w[i], mask, kWave);
+  acc_t r;
+  __builtin_memcpy(&r, w, sizeof(acc_t));
+  return r;
+}
+
 // ---------------------------------------------------------------------------
 // K rows per 16-byte vector (row length VEC/K elements).  Lane-local.
 // ---------------------------------------------------------------------------
@@ -113,13 +160,14 @@ __global__ __launch_bounds__(kBlock) void row_lanes_kernel(RowArgs a)
   using acc_t     = typename P::acc_t;
   constexpr int D = P::VEC / K;  // elements per row
   const i64 nfull = a.n_out / K; // vectors made only of whole, in-range rows
+  const char* inb = static_cast<const char*>(a.in);
 
   u32x4 x[kUnroll];
 #pragma unroll
   for (int u = 0; u < kUnroll; ++u) {
     // consecutive lanes take consecutive vectors within each unroll slot
     const i64 v = ((i64)blockIdx.x * kUnroll + u) * kBlock + threadIdx.x;
-    if (v < nfull) x[u] = load16(static_cast<const u32x4*>(a.in) + v);
+    if (v < nfull) x[u] = load16(inb + v * 16);
   }
 #pragma unroll
   for (int u = 0; u < kUnroll; ++u) {
@@ -154,27 +202,29 @@ __global__ __launch_bounds__(kBlock) void row_short_kernel(RowArgs a)
 {
   using acc_t     = typename P::acc_t;
   using H         = Held<P, VEC16>;
-  constexpr int S = Loader<P, VEC16>::STEP;
+  const char* inb = static_cast<const char*>(a.in);
   const int lane  = threadIdx.x & (kWave - 1);
   const i64 wid   = (i64)blockIdx.x * (kBlock / kWave) + (threadIdx.x >> 6);
   const int G     = a.G;
   const int R     = kWave >> a.logG;
   const int c     = lane & (G - 1);
   const int g     = lane >> a.logG;
-  const bool incol = c < a.nvec;
+  const i64 nload  = a.nvec + (a.tail > 0 ? 1 : 0);  // the tail is one more lane-load
+  const bool incol = c < nload;
 
   typename H::type x[kUnroll];
   i64 row[kUnroll];
 #pragma unroll
   for (int t = 0; t < kUnroll; ++t) {
     row[t] = (wid * kUnroll + t) * R + g;
-    if (incol && row[t] < a.n_out) x[t] = H::load(a.in, row[t] * a.nvec + c);
+    if (incol && row[t] < a.n_out)
+      x[t] = H::load_any(inb + row[t] * a.row_bytes, c, a.nvec, a.len);
   }
   acc_t acc[kUnroll];
 #pragma unroll
   for (int t = 0; t < kUnroll; ++t) {
     acc[t] = P::neutral();
-    if (incol && row[t] < a.n_out) H::push(acc[t], x[t], (i64)c * S);
+    if (incol && row[t] < a.n_out) H::push_any(acc[t], x[t], c, a.nvec, a.len, a.tail);
   }
 #pragma unroll
   for (int t = 0; t < kUnroll; ++t)
@@ -213,15 +263,16 @@ __global__ __launch_bounds__(kBlock) void row_short_kernel(RowArgs a)
 }
 
 // ---------------------------------------------------------------------------
-// G lanes of one wave per row, looping over the row with kUnroll loads in
-// flight per lane.
+// G lanes of one wave per row, kUnroll loads in flight per lane.  The plan
+// gives every lane at most kUnroll lane-loads per row (nvec <= kUnroll*G); the
+// loop is there for forced plans.
 // ---------------------------------------------------------------------------
 template <class P, bool VEC16>
 __global__ __launch_bounds__(kBlock) void row_wave_kernel(RowArgs a)
 {
   using acc_t     = typename P::acc_t;
   using H         = Held<P, VEC16>;
-  constexpr int S = Loader<P, VEC16>::STEP;
+  constexpr int S = H::STEP;
   const int lane  = threadIdx.x & (kWave - 1);
   const i64 wid   = (i64)blockIdx.x * (kBlock / kWave) + (threadIdx.x >> 6);
   const int G     = a.G;
@@ -232,25 +283,26 @@ __global__ __launch_bounds__(kBlock) void row_wave_kernel(RowArgs a)
 
   acc_t acc = P::neutral();
   if (row < a.n_out) {
-    const i64 base = row * nvec;
+    const char* rp = static_cast<const char*>(a.in) + row * a.row_bytes;
     i64 v          = c;
     for (; v + (kUnroll - 1) * G < nvec; v += kUnroll * G) {
       typename H::type x[kUnroll];
 #pragma unroll
       for (int u = 0; u < kUnroll; ++u)
-        x[u] = H::load(a.in, base + v + u * G);
+        x[u] = H::load(rp, v + u * G);
 #pragma unroll
       for (int u = 0; u < kUnroll; ++u)
         H::push(acc, x[u], (v + u * G) * S);
     }
-    if (v < nvec) {  // fewer than kUnroll lane-loads left for this lane
-      typename H::type x[kUnroll - 1];
+    const i64 nload = nvec + (a.tail > 0 ? 1 : 0);  // the tail is one more lane-load
+    if (v < nload) {  // fewer than kUnroll lane-loads left for this lane
+      typename H::type x[kUnroll];
 #pragma unroll
-      for (int u = 0; u < kUnroll - 1; ++u)
-        if (v + u * G < nvec) x[u] = H::load(a.in, base + v + u * G);
+      for (int u = 0; u < kUnroll; ++u)
+        if (v + u * G < nload) x[u] = H::load_any(rp, v + u * G, nvec, a.len);
 #pragma unroll
-      for (int u = 0; u < kUnroll - 1; ++u)
-        if (v + u * G < nvec) H::push(acc, x[u], (v + u * G) * S);
+      for (int u = 0; u < kUnroll; ++u)
+        if (v + u * G < nload) H::push_any(acc, x[u], v + u * G, nvec, a.len, a.tail);
     }
   }
   group_allreduce<P>(acc, G);
@@ -268,7 +320,7 @@ __global__ __launch_bounds__(1024) void row_block_kernel(RowArgs a)
 {
   using acc_t     = typename P::acc_t;
   using H         = Held<P, VEC16>;
-  constexpr int S = Loader<P, VEC16>::STEP;
+  constexpr int S = H::STEP;
   constexpr int U = kTeamUnroll;
   __shared__ acc_t sm[16];
 
@@ -289,13 +341,13 @@ __global__ __launch_bounds__(1024) void row_block_kernel(RowArgs a)
   if (live) {
     const i64 v0   = (i64)b * a.chunk;
     const i64 v1   = (v0 + a.chunk < a.nvec) ? (v0 + a.chunk) : a.nvec;
-    const i64 base = row * a.nvec;
+    const char* rp = static_cast<const char*>(a.in) + row * a.row_bytes;
     i64 v          = v0 + t;
     for (; v + (U - 1) * (i64)T < v1; v += (i64)U * T) {
       typename H::type x[U];
 #pragma unroll
       for (int u = 0; u < U; ++u)
-        x[u] = H::load(a.in, base + v + (i64)u * T);
+        x[u] = H::load(rp, v + (i64)u * T);
 #pragma unroll
       for (int u = 0; u < U; ++u)
         H::push(acc, x[u], (v + (i64)u * T) * S);
@@ -304,11 +356,14 @@ __global__ __launch_bounds__(1024) void row_block_kernel(RowArgs a)
       typename H::type x[U - 1];
 #pragma unroll
       for (int u = 0; u < U - 1; ++u)
-        if (v + (i64)u * T < v1) x[u] = H::load(a.in, base + v + (i64)u * T);
+        if (v + (i64)u * T < v1) x[u] = H::load(rp, v + (i64)u * T);
 #pragma unroll
       for (int u = 0; u < U - 1; ++u)
         if (v + (i64)u * T < v1) H::push(acc, x[u], (v + (i64)u * T) * S);
     }
+    // the overlapping last vector of the row goes to the team that owns the last chunk
+    if (a.tail > 0 && b == a.B - 1 && t == 0)
+      H::push_any(acc, H::load_any(rp, a.nvec, a.nvec, a.len), a.nvec, a.nvec, a.len, a.tail);
   }
 
   wave_allreduce<P>(acc);
@@ -335,23 +390,13 @@ __global__ __launch_bounds__(1024) void row_block_kernel(RowArgs a)
 // Reduction along the strided dimension of a [len][n_out] row-major array.
 // Thread (tx, ty): tx owns one lane-load wide group of adjacent columns for
 // the whole kernel, ty strides over the rows of the tiles dealt to this block.
+// Persistent: kColBlocksPerCu workgroups per CU; row tiles of TY*kColUnroll rows
+// are dealt round-robin over blockIdx.y, so at any moment the grid reads one
+// compact, advancing window of the matrix, and a workgroup's next tile is in
+// flight while it accumulates the current one.  (The loop holds no stores, which
+// is what lets loads stay in flight across iterations: gfx9 counts loads and
+// stores in one in-order counter.)
 // ---------------------------------------------------------------------------
-template <class P>
-__device__ __forceinline__ typename P::acc_t bperm_acc(const typename P::acc_t& a, int mask)
-{
-  using acc_t = typename P::acc_t;
-  static_assert(sizeof(acc_t) % 4 == 0, "accumulators are moved word by word");
-  constexpr int NW = sizeof(acc_t) / 4;
-  u32 w[NW];
-  __builtin_memcpy(w, &a, sizeof(acc_t));
-#pragma unroll
-  for (int i = 0; i < NW; ++i)
-    w[i] = (u32)__shfl_xor((int)w[i], mask, kWave);
-  acc_t r;
-  __builtin_memcpy(&r, w, sizeof(acc_t));
-  return r;
-}
-
 template <class P, bool VEC16>
 __global__ __launch_bounds__(kBlock) void col_kernel(ColArgs a)
 {
@@ -361,34 +406,40 @@ __global__ __launch_bounds__(kBlock) void col_kernel(ColArgs a)
   constexpr int W = kBlock / kWave;
   __shared__ acc_t sm[W * kWave * S];
 
-  const int t    = threadIdx.x;
-  const int TX   = a.TX;
-  const int TY   = kBlock >> a.logTX;
-  const int tx   = t & (TX - 1);
-  const int ty   = t >> a.logTX;
-  const i64 cv   = (i64)blockIdx.x * TX + tx;
-  const bool live = cv < a.nvec;
-  // Row tiles of TY*kColUnroll rows are dealt round-robin over blockIdx.y, so at any
-  // moment the blocks of the grid read one compact, advancing window of the matrix.
+  const int t      = threadIdx.x;
+  const int TX     = a.TX;
+  const int TY     = kBlock >> a.logTX;
+  const int tx     = t & (TX - 1);
+  const int ty     = t >> a.logTX;
+  const i64 cv     = (i64)blockIdx.x * TX + tx;
+  const bool whole = cv < a.nvec;                          // a full lane-load of columns
+  const bool part  = VEC16 && cv == a.nvec && a.tail > 0;  // the last, partial group
   const i64 RT     = (i64)TY * kColUnroll;
   const i64 n_full = a.len / RT;
+  const char* inb  = static_cast<const char*>(a.in);
 
   acc_t acc[S];
 #pragma unroll
   for (int j = 0; j < S; ++j)
     acc[j] = P::neutral();
 
-  if (live) {
-    if constexpr (VEC16) {
-      const u32x4* p = static_cast<const u32x4*>(a.in) + cv;
-      // two tiles in flight: the loads of the next tile are issued before the
-      // current one is accumulated
+  if constexpr (VEC16) {
+    // `skip` > 0 marks the partial group: its vector ends at the row's end and its
+    // first `skip` columns belong to the previous group.
+    auto sweep = [&](const char* p, int skip) {
+      auto take = [&](const u32x4& v, i64 r) {
+        if (skip == 0) {
+          P::push_cols(acc, v, r);
+        } else {
+          push_cols_from<P>(acc, v, r, skip);
+        }
+      };
       i64 tile = blockIdx.y;
       u32x4 x[kColUnroll];
       if (tile < n_full) {
 #pragma unroll
         for (int u = 0; u < kColUnroll; ++u)
-          x[u] = load16(p + (tile * RT + ty + (i64)u * TY) * a.nvec);
+          x[u] = load16(p + (tile * RT + ty + (i64)u * TY) * a.row_bytes);
       }
       while (tile < n_full) {
         const i64 next = tile + a.B;
@@ -396,11 +447,11 @@ __global__ __launch_bounds__(kBlock) void col_kernel(ColArgs a)
         if (next < n_full) {
 #pragma unroll
           for (int u = 0; u < kColUnroll; ++u)
-            y[u] = load16(p + (next * RT + ty + (i64)u * TY) * a.nvec);
+            y[u] = load16(p + (next * RT + ty + (i64)u * TY) * a.row_bytes);
         }
 #pragma unroll
         for (int u = 0; u < kColUnroll; ++u)
-          P::push_cols(acc, x[u], tile * RT + ty + (i64)u * TY);
+          take(x[u], tile * RT + ty + (i64)u * TY);
 #pragma unroll
         for (int u = 0; u < kColUnroll; ++u)
           x[u] = y[u];
@@ -408,24 +459,29 @@ __global__ __launch_bounds__(kBlock) void col_kernel(ColArgs a)
       }
       if ((i64)blockIdx.y == n_full % a.B) {  // the rows past the last whole tile
         for (i64 r = n_full * RT + ty; r < a.len; r += TY)
-          P::push_cols(acc, load16(p + r * a.nvec), r);
+          take(load16(p + r * a.row_bytes), r);
       }
-    } else {
-      const in_t* p = static_cast<const in_t*>(a.in) + cv;
-      for (i64 tile = blockIdx.y; tile < n_full; tile += a.B) {
-        const i64 r = tile * RT + ty;
-        typename In<in_t>::nat x[kColUnroll];
+    };
+    if (whole) {
+      sweep(inb + cv * 16, 0);
+    } else if (part) {
+      sweep(inb + (a.n_out - S) * (i64)sizeof(in_t), S - a.tail);
+    }
+  } else if (whole) {
+    const in_t* p = reinterpret_cast<const in_t*>(inb) + cv;
+    for (i64 tile = blockIdx.y; tile < n_full; tile += a.B) {
+      const i64 r = tile * RT + ty;
+      typename In<in_t>::nat x[kColUnroll];
 #pragma unroll
-        for (int u = 0; u < kColUnroll; ++u)
-          x[u] = In<in_t>::ld(p + (r + (i64)u * TY) * a.nvec);
+      for (int u = 0; u < kColUnroll; ++u)
+        x[u] = In<in_t>::ld(p + (r + (i64)u * TY) * a.n_out);
 #pragma unroll
-        for (int u = 0; u < kColUnroll; ++u)
-          P::push(acc[0], x[u], r + (i64)u * TY);
-      }
-      if ((i64)blockIdx.y == n_full % a.B) {
-        for (i64 r = n_full * RT + ty; r < a.len; r += TY)
-          P::push(acc[0], In<in_t>::ld(p + r * a.nvec), r);
-      }
+      for (int u = 0; u < kColUnroll; ++u)
+        P::push(acc[0], x[u], r + (i64)u * TY);
+    }
+    if ((i64)blockIdx.y == n_full % a.B) {
+      for (i64 r = n_full * RT + ty; r < a.len; r += TY)
+        P::push(acc[0], In<in_t>::ld(p + r * a.n_out), r);
     }
   }
 
@@ -438,24 +494,29 @@ __global__ __launch_bounds__(kBlock) void col_kernel(ColArgs a)
   // one value per (wave, tx, j) through LDS, folded by the block's first TX threads
   const int lane = t & (kWave - 1);
   const int wave = t >> 6;
-  constexpr int NW = W;  // every wave covers its own set of ty
   if (lane < TX) {
 #pragma unroll
     for (int j = 0; j < S; ++j)
       sm[(wave * kWave + lane) * S + j] = acc[j];
   }
   __syncthreads();
-  if (t < TX && live) {
+  if (t < TX && (whole || part)) {
+    // the partial group holds the row's last S columns; its first S - tail are
+    // already covered by the group before it
+    const int first = whole ? 0 : S - a.tail;
+    const i64 col0  = whole ? cv * S : a.n_out - S;
 #pragma unroll
     for (int j = 0; j < S; ++j) {
-      acc_t r = sm[(0 * kWave + t) * S + j];
-      for (int w = 1; w < NW; ++w)
-        P::merge(r, sm[(w * kWave + t) * S + j]);
-      const i64 col = cv * S + j;
-      if (a.B == 1) {
-        finish<P>(a.epi, col, r);
-      } else {
-        static_cast<acc_t*>(a.partial)[col * a.B + blockIdx.y] = r;
+      if (j >= first) {
+        acc_t r = sm[(0 * kWave + t) * S + j];
+        for (int w = 1; w < W; ++w)
+          P::merge(r, sm[(w * kWave + t) * S + j]);
+        const i64 col = col0 + j;
+        if (a.B == 1) {
+          finish<P>(a.epi, col, r);
+        } else {
+          static_cast<acc_t*>(a.partial)[col * a.B + blockIdx.y] = r;
+        }
       }
     }
   }

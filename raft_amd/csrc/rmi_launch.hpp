@@ -67,7 +67,9 @@ int run(const PlanX& pl, const Problem& pr, hipStream_t st)
       a.partial = pr.ws;
       a.n_out   = pl.n_out;
       a.len     = pl.len;
+      a.row_bytes = pl.row_bytes;
       a.nvec    = pl.nvec;
+      a.tail    = pl.tail;
       a.chunk   = pl.chunk;
       a.G       = pl.G;
       a.logG    = pl.logG;
@@ -112,7 +114,9 @@ int run(const PlanX& pl, const Problem& pr, hipStream_t st)
       a.partial        = pr.ws;
       a.n_out          = pl.n_out;
       a.len            = pl.len;
+      a.row_bytes      = pl.row_bytes;
       a.nvec           = pl.nvec;
+      a.tail           = pl.tail;
       a.TX             = pl.TX;
       a.logTX          = pl.logTX;
       a.B              = pl.B;

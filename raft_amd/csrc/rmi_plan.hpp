@@ -37,7 +37,9 @@ struct PlanX {
   int step        = 1;  // elements per lane-load
   int64_t n_out   = 0;
   int64_t len     = 0;  // elements folded into one output
-  int64_t nvec    = 0;  // lane-loads along the contiguous dimension
+  int64_t nvec    = 0;  // whole lane-loads along the contiguous dimension
+  int tail        = 0;  // vec16: elements after the last whole vector
+  int64_t row_bytes = 0; // bytes of one row of the contiguous dimension
   int K           = 0;  // ROW_LANES: rows per 16-byte vector
   int G           = 1;  // ROW_WAVE: lanes per row
   int logG        = 0;
@@ -182,12 +184,10 @@ inline int classify(const rmi_reduce_desc& d, PolicyKey& key, int& acc_bytes)
   return RMI_OK;
 }
 
-// Shape -> plan.  `aligned16`: the input base pointer is 16-byte aligned.
-// `hint`: an rmi_plan_kind to force where it is applicable to the shape.
+// Shape -> plan.  desc.plan_hint forces a plan kind where it applies to the shape.
 inline int make_plan(const rmi_reduce_desc& d,
                      const PolicyKey& key,
                      int acc_bytes,
-                     bool aligned16,
                      int n_cu,
                      PlanX& p)
 {
@@ -222,17 +222,23 @@ inline int make_plan(const rmi_reduce_desc& d,
     return RMI_OK;
   }
 
+  // Rows of at least 16 bytes are read as 16-byte vectors (at any alignment)
+  // plus up to VEC-1 tail elements; shorter rows element by element.
   const int64_t row_bytes = contiguous * es;
-  p.vec16                 = aligned16 && (row_bytes % 16 == 0);
+  p.row_bytes             = row_bytes;
+  p.vec16                 = row_bytes >= 16;
   p.step                  = p.vec16 ? 16 / es : 1;
   p.nvec                  = contiguous / p.step;
+  p.tail                  = (int)(contiguous % p.step);
+  // lane-loads a row needs, counting the tail elements as one more
+  const int64_t nload = p.nvec + (p.tail > 0 ? 1 : 0);
 
   if (p.strided) {
     p.kind  = RMI_PLAN_COL_TILE;
-    p.TX    = (int)(p.nvec < 64 ? pow2ceil(p.nvec) : 64);
+    p.TX    = (int)(nload < 64 ? pow2ceil(nload) : 64);
     p.logTX = ilog2(p.TX);
     const int TY = kPlanBlock / p.TX;
-    p.gridx      = ceildiv(p.nvec, p.TX);
+    p.gridx      = ceildiv(nload, p.TX);
     // row tiles of TY*unroll rows are dealt round-robin to B blocks: kColBlocksPerCu
     // blocks per CU, but at least two tiles per block
     const int64_t tile_rows = (int64_t)TY * kPlanUnroll;
@@ -251,13 +257,14 @@ inline int make_plan(const rmi_reduce_desc& d,
 
   // ---- contiguous-dimension plans ----
   // several whole rows per 16-byte vector
-  if (aligned16 && row_bytes < 16 && 16 % row_bytes == 0 &&
+  if (row_bytes < 16 && 16 % row_bytes == 0 &&
       (hint == RMI_PLAN_AUTO || hint == RMI_PLAN_ROW_LANES)) {
     p.kind        = RMI_PLAN_ROW_LANES;
     p.vec16       = true;
     p.step        = 16 / es;
     p.K           = (int)(16 / row_bytes);
     p.nvec        = 1;
+    p.tail        = 0;
     p.grid_blocks = ceildiv(ceildiv(p.n_out, p.K), (int64_t)kPlanBlock * kPlanUnroll);
     if (p.grid_blocks < 1) p.grid_blocks = 1;
     return RMI_OK;
@@ -268,7 +275,7 @@ inline int make_plan(const rmi_reduce_desc& d,
     kind = RMI_PLAN_AUTO;
   int threads = 64;
   if (kind == RMI_PLAN_AUTO) {
-    if (p.nvec <= 4 * 64) {
+    if (nload <= 4 * 64) {
       kind = RMI_PLAN_ROW_WAVE;
     } else {
       // widen the team on a row until the machine's wave slots are filled, as long
@@ -285,17 +292,17 @@ inline int make_plan(const rmi_reduce_desc& d,
     }
   } else if (kind == RMI_PLAN_ROW_BLOCK) {
     threads = kPlanBlock;
-  } else if (kind == RMI_PLAN_ROW_WAVE && p.nvec > 4 * 64) {
+  } else if (kind == RMI_PLAN_ROW_WAVE && nload > 4 * 64) {
     kind = RMI_PLAN_ROW_BLOCK;  // one wave per row, served by the team kernel
   }
 
   if (kind == RMI_PLAN_ROW_WAVE) {
     p.kind = RMI_PLAN_ROW_WAVE;
-    if (p.nvec <= 8) {
+    if (nload <= 8) {
       p.short_rows = true;
-      p.G          = pow2ceil(p.nvec);
+      p.G          = pow2ceil(nload);  // lane c == nvec loads the overlapping last vector
     } else {
-      const int64_t g = ceildiv(p.nvec, kPlanUnroll);
+      const int64_t g = ceildiv(nload, kPlanUnroll);
       p.G             = g >= 64 ? 64 : pow2ceil(g);
       if (p.G < 8) p.G = 8;
     }
@@ -307,7 +314,7 @@ inline int make_plan(const rmi_reduce_desc& d,
       // 80 KB (5 workgroups of 256 lanes x 4 loads x 16 B) sustains the most; the
       // default 8 resident workgroups lose 3-4 points to queueing.  A dynamic LDS
       // reservation the kernel never touches caps the resident workgroups.
-      const int64_t loads_per_lane = ceildiv(p.nvec, p.G);
+      const int64_t loads_per_lane = ceildiv(nload, p.G);
       if (loads_per_lane >= 4) p.lds_reserve = kLdsPerCu / 5 - 768;
       else if (loads_per_lane == 3) p.lds_reserve = kLdsPerCu / 6 - 768;
     }

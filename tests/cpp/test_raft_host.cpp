@@ -154,7 +154,9 @@ TEST_CASE(plan_selector)
   p = plan(RMI_F32, RMI_KVP_I32_F32, 65536, 32000, RMI_ALONG_ROWS, RMI_RED_ARGMAX, RMI_MAIN_KVP);
   CHECK(p.kind == RMI_PLAN_ROW_WAVE && p.lanes_per_row == 64);
   p = plan(RMI_F32, RMI_F32, 100, 7);
-  CHECK(p.vec_bytes == 4);  // rows of 28 bytes cannot use 16-byte lane loads
+  CHECK(p.vec_bytes == 16);  // 28-byte rows: one 16-byte lane load and three tail elements
+  p = plan(RMI_F32, RMI_F32, 100, 3);
+  CHECK(p.vec_bytes == 4);  // 12-byte rows are read element by element
   p = plan(RMI_F32, RMI_F32, 5, 0);
   CHECK(p.kind == RMI_PLAN_EMPTY);
   rmi_reduce_desc bad{};

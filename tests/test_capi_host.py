@@ -95,8 +95,11 @@ def test_plan_hints_and_fallbacks():
     p = api.plan_query(d)
     assert p.kind == api.PLAN_ROW_SPLIT and p.blocks_per_out >= 2
     assert p.workspace_bytes == 4 * p.blocks_per_out * 8
-    # rows of 7 floats (28 B) cannot be read as 16-byte vectors
+    # rows of 7 floats (28 B) are one 16-byte vector plus three tail elements;
+    # rows of 3 floats (12 B) are read element by element
     p = api.plan_query(api.make_desc(api.F32, api.F32, 1000, 7))
+    assert p.vec_bytes == 16 and p.kind == api.PLAN_ROW_WAVE
+    p = api.plan_query(api.make_desc(api.F32, api.F32, 1000, 3))
     assert p.vec_bytes == 4 and p.kind == api.PLAN_ROW_WAVE
     # f64 sums carry a 16-byte (sum, compensation) accumulator through the partials
     d = api.make_desc(api.F64, api.F64, 4, 1 << 20, plan_hint=api.PLAN_ROW_SPLIT)
