@@ -424,14 +424,16 @@ __global__ __launch_bounds__(kBlock) void col_kernel(ColArgs a)
     acc[j] = P::neutral();
 
   if constexpr (VEC16) {
-    // `skip` > 0 marks the partial group: its vector ends at the row's end and its
-    // first `skip` columns belong to the previous group.
-    auto sweep = [&](const char* p, int skip) {
+    // MASKED: the row length is not a multiple of the vector width.  The partial
+    // group's vector ends at the row's end and its first `skip` columns belong to the
+    // group before it; all lanes then run the masked accumulate (skip == 0 for whole
+    // groups) so that a wave stays on one instruction stream.
+    auto sweep = [&](const char* p, int skip, auto masked) {
       auto take = [&](const u32x4& v, i64 r) {
-        if (skip == 0) {
-          P::push_cols(acc, v, r);
-        } else {
+        if constexpr (decltype(masked)::value) {
           push_cols_from<P>(acc, v, r, skip);
+        } else {
+          P::push_cols(acc, v, r);
         }
       };
       i64 tile = blockIdx.y;
@@ -462,10 +464,11 @@ __global__ __launch_bounds__(kBlock) void col_kernel(ColArgs a)
           take(load16(p + r * a.row_bytes), r);
       }
     };
-    if (whole) {
-      sweep(inb + cv * 16, 0);
-    } else if (part) {
-      sweep(inb + (a.n_out - S) * (i64)sizeof(in_t), S - a.tail);
+    if (a.tail == 0) {
+      if (whole) sweep(inb + cv * 16, 0, std::false_type{});
+    } else if (whole || part) {
+      const char* p = whole ? inb + cv * 16 : inb + (a.n_out - S) * (i64)sizeof(in_t);
+      sweep(p, whole ? 0 : S - a.tail, std::true_type{});
     }
   } else if (whole) {
     const in_t* p = reinterpret_cast<const in_t*>(inb) + cv;
