@@ -332,10 +332,20 @@ struct kbn_t {
   double c;
 };
 
+// One compensated step.  The reference picks between (s - t) + x and (x - t) + s by
+// comparing magnitudes; both are the exact rounding error of s + x.  Knuth's
+// branch-free two-sum yields the same exact error with two more additions and no
+// compare / select, which is cheaper on the f64 pipe.
+__device__ __forceinline__ double two_sum_err(double s, double x, double t)
+{
+  const double bp = t - s;
+  return (s - (t - bp)) + (x - bp);
+}
+
 __device__ __forceinline__ void kbn_add(kbn_t& a, double x)
 {
   const double t = a.s + x;
-  a.c += (fabs(a.s) >= fabs(x)) ? ((a.s - t) + x) : ((x - t) + a.s);
+  a.c += two_sum_err(a.s, x, t);
   a.s = t;
 }
 
@@ -363,7 +373,7 @@ struct PolKbn {
   static __device__ __forceinline__ void merge(acc_t& a, const acc_t& b)
   {
     const double t = a.s + b.s;
-    const double e = (fabs(a.s) >= fabs(b.s)) ? ((a.s - t) + b.s) : ((b.s - t) + a.s);
+    const double e = two_sum_err(a.s, b.s, t);
     a.c            = (a.c + b.c) + e;
     a.s            = t;
   }
