@@ -17,6 +17,10 @@
 
 #include "rmi_reduce.h"
 
+#if defined(__HIPCC__)
+#include <raft/linalg/detail/rmi_generic.hpp>
+#endif
+
 namespace raft {
 
 // bfloat16 storage (1 sign, 8 exponent, 7 mantissa bits) for inputs and outputs
@@ -271,8 +275,8 @@ void reduce(const resources* res,
             bool along_rows,
             OutType init,
             bool inplace,
-            const MainLambda&,
-            const ReduceLambda&,
+            const MainLambda& main_op,
+            const ReduceLambda& reduce_op,
             const FinalLambda& final_op,
             int final_override         = -1,
             double scalar1             = 0.0,
@@ -280,18 +284,41 @@ void reduce(const resources* res,
             const void* final_aux      = nullptr,
             int out_dtype_override     = -1)
 {
-  static_assert(main_tag<MainLambda>::value >= 0,
-                "main_op is not one of the functors the reduction library implements "
-                "(identity_op, cast_op, sq_op, abs_op, nz_op, value_to_kvp_op); arbitrary "
-                "device lambdas cannot cross the C ABI");
-  static_assert(reduce_tag<ReduceLambda>::value >= 0,
-                "reduce_op is not one of add_op, max_op, min_op, argmax_op, argmin_op");
-  static_assert(final_tag<FinalLambda>::value >= 0,
-                "final_op is not one of identity_op, sqrt_op, abs_op, sq_op, key_op, "
-                "mul/div/add/sub_const_op");
+  // Functor and element types the library implements go through the C ABI; anything
+  // else is instantiated in this translation unit when it is compiled by hipcc.
+  constexpr bool lowered = main_tag<MainLambda>::value >= 0 &&
+                           reduce_tag<ReduceLambda>::value >= 0 &&
+                           final_tag<FinalLambda>::value >= 0 &&
+                           dtype_of<std::remove_cv_t<InType>>::value >= 0 &&
+                           dtype_of<std::remove_cv_t<OutType>>::value >= 0;
+  if constexpr (!lowered) {
+#if defined(__HIPCC__)
+    (void)res;
+    generic::reduce(stream, dots, data, n_rows, n_cols, row_major, along_rows, init, inplace,
+                    main_op, reduce_op, final_op);
+    return;
+#else
+    static_assert(main_tag<MainLambda>::value >= 0,
+                  "main_op is not one of the functors the reduction library implements "
+                  "(identity_op, cast_op, sq_op, abs_op, nz_op, value_to_kvp_op); compile this "
+                  "translation unit with hipcc to use arbitrary device functors");
+    static_assert(reduce_tag<ReduceLambda>::value >= 0,
+                  "reduce_op is not one of add_op, max_op, min_op, argmax_op, argmin_op; compile "
+                  "this translation unit with hipcc to use arbitrary device functors");
+    static_assert(final_tag<FinalLambda>::value >= 0,
+                  "final_op is not one of identity_op, sqrt_op, abs_op, sq_op, key_op, "
+                  "mul/div/add/sub_const_op; compile this translation unit with hipcc to use "
+                  "arbitrary device functors");
+    static_assert(dtype_of<std::remove_cv_t<InType>>::value >= 0 &&
+                    dtype_of<std::remove_cv_t<OutType>>::value >= 0,
+                  "element type not supported by the reduction library; compile this translation "
+                  "unit with hipcc to reduce arbitrary trivially copyable types");
+#endif
+  } else {
   rmi_reduce_desc d{};
-  d.in_dtype      = dtype<InType>();
-  d.out_dtype     = out_dtype_override >= 0 ? out_dtype_override : dtype<OutType>();
+  d.in_dtype      = dtype_of<std::remove_cv_t<InType>>::value;
+  d.out_dtype     = out_dtype_override >= 0 ? out_dtype_override
+                                            : dtype_of<std::remove_cv_t<OutType>>::value;
   d.layout        = row_major ? RMI_ROW_MAJOR : RMI_COL_MAJOR;
   d.apply         = along_rows ? RMI_ALONG_ROWS : RMI_ALONG_COLUMNS;
   d.n_rows        = n_rows;
@@ -309,6 +336,9 @@ void reduce(const resources* res,
   const size_t ws_bytes = rmi_reduce_workspace_bytes(&d);
   workspace_lease ws(res, stream, ws_bytes);
   check(rmi_reduce(&d, data, dots, ws.data(), ws.size(), stream), "rmi_reduce");
+  (void)main_op;
+  (void)reduce_op;
+  }
 }
 
 }  // namespace detail::rmi

@@ -1,0 +1,308 @@
+// Reductions with ARBITRARY device functors, for translation units compiled by
+// hipcc.  The closed functor vocabulary goes through the C ABI of the reduction
+// library; anything else (device lambdas, caller-defined functor structs, output
+// types the library does not know) cannot cross a C ABI and is instantiated here,
+// in the caller's translation unit, the way the reference instantiates all of its
+// kernels (linalg/detail/coalesced_reduction-inl.cuh, detail/strided_reduction.cuh).
+//
+// Semantics are the reference's: every participating lane starts from `init`
+// (which therefore has to be reduce_op's neutral element), main_op receives the
+// index along the reduced axis, and
+//   dots[k] = final_op(inplace ? reduce_op(dots[k], acc) : acc).
+// Unlike the reference there are no atomics: partial results of the strided and
+// split plans are folded in a fixed order, so results are repeatable.
+//
+// The kernels are wave64 / gfx950 code: 16-byte lane loads for arithmetic element
+// types, ds_bpermute butterflies on 32-bit words for accumulators of any trivially
+// copyable type, LDS across waves.  They are simpler than the library's tuned
+// kernels (no compensated sums: accumulation happens in OutType with the caller's
+// reduce_op, exactly as written).
+#pragma once
+
+#if !defined(__HIPCC__)
+#error "rmi_generic.hpp holds device code: include it only from hipcc translation units"
+#endif
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <type_traits>
+
+#include <raft/core/error.hpp>
+
+namespace raft::detail::rmi::generic {
+
+constexpr int kWave  = 64;
+constexpr int kBlock = 256;
+
+template <typename T>
+__device__ __forceinline__ T shfl_xor_any(const T& v, int mask)
+{
+  static_assert(std::is_trivially_copyable_v<T>, "accumulators must be trivially copyable");
+  constexpr int NW = (sizeof(T) + 3) / 4;
+  std::uint32_t w[NW] = {};
+  __builtin_memcpy(w, &v, sizeof(T));
+#pragma unroll
+  for (int i = 0; i < NW; ++i)
+    w[i] = (std::uint32_t)__shfl_xor((int)w[i], mask, kWave);
+  T r;
+  __builtin_memcpy(&r, w, sizeof(T));
+  return r;
+}
+
+// all-reduce over groups of G lanes (G a power of two <= 64); reduce_op must be
+// commutative for every lane to end with the same value, which the callers below
+// do not rely on: only lane 0 of a group uses the result.
+template <typename T, typename Red>
+__device__ __forceinline__ T group_reduce(T acc, int G, Red& red)
+{
+  for (int m = G >> 1; m >= 1; m >>= 1)
+    acc = red(acc, shfl_xor_any(acc, m));
+  return acc;
+}
+
+// elements per 16-byte lane load, or 1 when the element type is not a power-of-two
+// sized arithmetic type
+template <typename In>
+constexpr int vec_width()
+{
+  if constexpr (std::is_arithmetic_v<In> && (sizeof(In) == 1 || sizeof(In) == 2 ||
+                                             sizeof(In) == 4 || sizeof(In) == 8)) {
+    return 16 / (int)sizeof(In);
+  } else {
+    return 1;
+  }
+}
+
+// acc = fold of main_op(row[j], j) for j = first, first + stride, ... over whole
+// 16-byte vectors, then the tail elements
+template <typename In, typename Out, typename Idx, typename Main, typename Red>
+__device__ __forceinline__ Out sweep_row(const In* row, Idx D, int first, int stride, Out acc,
+                                         Main& main_op, Red& red)
+{
+  constexpr int V = vec_width<In>();
+  if constexpr (V > 1) {
+    const Idx nvec = D / V;
+    for (Idx v = first; v < nvec; v += stride) {
+      In x[V];  // one 16-byte lane load at any element-aligned address
+      __builtin_memcpy(x, reinterpret_cast<const char*>(row) + (std::size_t)v * 16, 16);
+#pragma unroll
+      for (int j = 0; j < V; ++j)
+        acc = red(acc, static_cast<Out>(main_op(x[j], static_cast<Idx>(v * V + j))));
+    }
+    for (Idx j = nvec * V + first; j < D; j += stride)
+      acc = red(acc, static_cast<Out>(main_op(row[j], j)));
+  } else {
+    for (Idx j = first; j < D; j += stride)
+      acc = red(acc, static_cast<Out>(main_op(row[j], j)));
+  }
+  return acc;
+}
+
+// G lanes of a wave per row (rows are contiguous, D elements each)
+template <typename In, typename Out, typename Idx, typename Main, typename Red, typename Fin>
+__global__ __launch_bounds__(kBlock) void rows_group_kernel(Out* dots, const In* data, Idx D,
+                                                            Idx N, Out init, bool inplace,
+                                                            Main main_op, Red red, Fin fin,
+                                                            int G, int logG)
+{
+  const int lane         = threadIdx.x & (kWave - 1);
+  const std::int64_t wid = (std::int64_t)blockIdx.x * (kBlock / kWave) + (threadIdx.x >> 6);
+  const int c            = lane & (G - 1);
+  const std::int64_t row = wid * (kWave >> logG) + (lane >> logG);
+  Out acc                = init;
+  if (row < (std::int64_t)N) acc = sweep_row<In, Out, Idx>(data + row * D, D, c, G, acc, main_op, red);
+  acc = group_reduce(acc, G, red);
+  if (c == 0 && row < (std::int64_t)N) dots[row] = fin(inplace ? red(dots[row], acc) : acc);
+}
+
+// one 256-thread workgroup per chunk of a row; B chunks per row.  B == 1 writes the
+// outputs, B > 1 writes partials[row * B + b].
+template <typename In, typename Out, typename Idx, typename Main, typename Red, typename Fin>
+__global__ __launch_bounds__(kBlock) void rows_block_kernel(Out* dots, Out* partial,
+                                                            const In* data, Idx D, Idx N, Out init,
+                                                            bool inplace, Main main_op, Red red,
+                                                            Fin fin, int B, std::int64_t chunk)
+{
+  __shared__ Out sm[kBlock / kWave];
+  const std::int64_t row = blockIdx.x / B;
+  const int b            = blockIdx.x % B;
+  const std::int64_t j0  = (std::int64_t)b * chunk;
+  const std::int64_t j1  = j0 + chunk < (std::int64_t)D ? j0 + chunk : (std::int64_t)D;
+  Out acc                = init;
+  for (std::int64_t j = j0 + threadIdx.x; j < j1; j += kBlock)
+    acc = red(acc, static_cast<Out>(main_op(data[row * D + j], static_cast<Idx>(j))));
+  acc = group_reduce(acc, kWave, red);
+  if ((threadIdx.x & (kWave - 1)) == 0) sm[threadIdx.x >> 6] = acc;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < kBlock / kWave; ++w)
+      acc = red(acc, sm[w]);
+    if (B == 1) {
+      dots[row] = fin(inplace ? red(dots[row], acc) : acc);
+    } else {
+      partial[row * B + b] = acc;
+    }
+  }
+}
+
+// strided: data is N rows of D contiguous elements, one output per column.
+// blockDim = (TX, 256/TX); blockIdx.y owns row tiles dealt round-robin.
+template <typename In, typename Out, typename Idx, typename Main, typename Red, typename Fin>
+__global__ __launch_bounds__(kBlock) void cols_kernel(Out* dots, Out* partial, const In* data,
+                                                      Idx D, Idx N, Out init, bool inplace,
+                                                      Main main_op, Red red, Fin fin, int TX,
+                                                      int logTX, int B)
+{
+  __shared__ Out sm[kBlock];
+  const int tx           = threadIdx.x & (TX - 1);
+  const int ty           = threadIdx.x >> logTX;
+  const int TY           = kBlock >> logTX;
+  const std::int64_t col = (std::int64_t)blockIdx.x * TX + tx;
+  Out acc                = init;
+  if (col < (std::int64_t)D) {
+    for (std::int64_t r = (std::int64_t)blockIdx.y * TY + ty; r < (std::int64_t)N;
+         r += (std::int64_t)B * TY)
+      acc = red(acc, static_cast<Out>(main_op(data[r * D + col], static_cast<Idx>(r))));
+  }
+  sm[threadIdx.x] = acc;
+  __syncthreads();
+  for (int s = TY >> 1; s >= 1; s >>= 1) {
+    if (ty < s) sm[threadIdx.x] = red(sm[threadIdx.x], sm[threadIdx.x + (s << logTX)]);
+    __syncthreads();
+  }
+  if (ty == 0 && col < (std::int64_t)D) {
+    if (B == 1) {
+      dots[col] = fin(inplace ? red(dots[col], sm[tx]) : sm[tx]);
+    } else {
+      partial[col * B + blockIdx.y] = sm[tx];
+    }
+  }
+}
+
+// second pass over partials[n_out][B], one thread per output, fixed order
+template <typename Out, typename Red, typename Fin>
+__global__ __launch_bounds__(kBlock) void fold_kernel(Out* dots, const Out* partial,
+                                                      std::int64_t n_out, int B, Out init,
+                                                      bool inplace, Red red, Fin fin)
+{
+  const std::int64_t o = (std::int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (o >= n_out) return;
+  Out acc = init;
+  for (int b = 0; b < B; ++b)
+    acc = red(acc, partial[o * B + b]);
+  dots[o] = fin(inplace ? red(dots[o], acc) : acc);
+}
+
+inline int pow2ceil(std::int64_t x)
+{
+  int p = 1;
+  while (p < x)
+    p <<= 1;
+  return p;
+}
+inline int ilog2(int x)
+{
+  int l = 0;
+  while ((1 << l) < x)
+    ++l;
+  return l;
+}
+
+inline void check_launch(const char* what)
+{
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess)
+    throw raft::hip_error(std::string("HIP error encountered at: ") + what + ": " +
+                          hipGetErrorString(e));
+}
+
+// dots[N] from N contiguous rows of D elements
+template <typename In, typename Out, typename Idx, typename Main, typename Red, typename Fin>
+void coalesced(Out* dots, const In* data, Idx D, Idx N, Out init, hipStream_t stream, bool inplace,
+               Main main_op, Red red, Fin fin)
+{
+  if (N <= 0) return;
+  constexpr int V           = vec_width<In>();
+  const std::int64_t nloads = ((std::int64_t)D + V - 1) / V;
+  if (nloads <= 256 || (std::int64_t)N >= 8192) {
+    // lanes per row: about four loads per lane
+    std::int64_t g = (nloads + 3) / 4;
+    const int G    = g >= 64 ? 64 : pow2ceil(g < 1 ? 1 : g);
+    const int rows_per_block = (kWave / G) * (kBlock / kWave);
+    const std::int64_t grid  = ((std::int64_t)N + rows_per_block - 1) / rows_per_block;
+    hipLaunchKernelGGL((rows_group_kernel<In, Out, Idx, Main, Red, Fin>), dim3((unsigned)grid),
+                       dim3(kBlock), 0, stream, dots, data, D, N, init, inplace, main_op, red, fin,
+                       G, ilog2(G));
+    check_launch("rows_group_kernel");
+    return;
+  }
+  // few long rows: split each into B chunks so that the grid fills the device
+  std::int64_t B = (2048 + (std::int64_t)N - 1) / (std::int64_t)N;
+  const std::int64_t max_b = ((std::int64_t)D + 4 * kBlock - 1) / (4 * kBlock);
+  if (B > max_b) B = max_b;
+  if (B < 1) B = 1;
+  const std::int64_t chunk = ((std::int64_t)D + B - 1) / B;
+  B                        = ((std::int64_t)D + chunk - 1) / chunk;
+  Out* partial             = nullptr;
+  if (B > 1) RAFT_HIP_TRY(hipMallocAsync((void**)&partial, sizeof(Out) * (std::size_t)N * B, stream));
+  hipLaunchKernelGGL((rows_block_kernel<In, Out, Idx, Main, Red, Fin>),
+                     dim3((unsigned)((std::int64_t)N * B)), dim3(kBlock), 0, stream, dots, partial,
+                     data, D, N, init, inplace, main_op, red, fin, (int)B, chunk);
+  check_launch("rows_block_kernel");
+  if (B > 1) {
+    hipLaunchKernelGGL((fold_kernel<Out, Red, Fin>),
+                       dim3((unsigned)(((std::int64_t)N + kBlock - 1) / kBlock)), dim3(kBlock), 0,
+                       stream, dots, partial, (std::int64_t)N, (int)B, init, inplace, red, fin);
+    check_launch("fold_kernel");
+    RAFT_HIP_TRY(hipFreeAsync(partial, stream));
+  }
+}
+
+// dots[D] from N rows of D contiguous elements (one output per column)
+template <typename In, typename Out, typename Idx, typename Main, typename Red, typename Fin>
+void strided(Out* dots, const In* data, Idx D, Idx N, Out init, hipStream_t stream, bool inplace,
+             Main main_op, Red red, Fin fin)
+{
+  if (D <= 0) return;
+  const int TX             = D >= 64 ? 64 : pow2ceil(D);
+  const int TY             = kBlock / TX;
+  const std::int64_t gridx = ((std::int64_t)D + TX - 1) / TX;
+  std::int64_t B           = (1024 + gridx - 1) / gridx;
+  const std::int64_t max_b = ((std::int64_t)N + 4 * TY - 1) / (4 * TY);
+  if (B > max_b) B = max_b;
+  if (B < 1) B = 1;
+  if (B > 4096) B = 4096;
+  Out* partial = nullptr;
+  if (B > 1) RAFT_HIP_TRY(hipMallocAsync((void**)&partial, sizeof(Out) * (std::size_t)D * B, stream));
+  hipLaunchKernelGGL((cols_kernel<In, Out, Idx, Main, Red, Fin>),
+                     dim3((unsigned)gridx, (unsigned)B), dim3(kBlock), 0, stream, dots, partial,
+                     data, D, N, init, inplace, main_op, red, fin, TX, ilog2(TX), (int)B);
+  check_launch("cols_kernel");
+  if (B > 1) {
+    hipLaunchKernelGGL((fold_kernel<Out, Red, Fin>),
+                       dim3((unsigned)(((std::int64_t)D + kBlock - 1) / kBlock)), dim3(kBlock), 0,
+                       stream, dots, partial, (std::int64_t)D, (int)B, init, inplace, red, fin);
+    check_launch("fold_kernel");
+    RAFT_HIP_TRY(hipFreeAsync(partial, stream));
+  }
+}
+
+// layout x axis dispatch of linalg/detail/reduce.cuh:36-48
+template <typename In, typename Out, typename Main, typename Red, typename Fin>
+void reduce(hipStream_t stream, Out* dots, const In* data, std::int64_t n_rows,
+            std::int64_t n_cols, bool row_major, bool along_rows, Out init, bool inplace,
+            Main main_op, Red red, Fin fin)
+{
+  using Idx = std::int64_t;
+  if (row_major == along_rows) {
+    // fold the contiguous dimension
+    const Idx D = row_major ? n_cols : n_rows, N = row_major ? n_rows : n_cols;
+    coalesced<In, Out, Idx>(dots, data, D, N, init, stream, inplace, main_op, red, fin);
+  } else {
+    const Idx D = row_major ? n_cols : n_rows, N = row_major ? n_rows : n_cols;
+    strided<In, Out, Idx>(dots, data, D, N, init, stream, inplace, main_op, red, fin);
+  }
+}
+
+}  // namespace raft::detail::rmi::generic

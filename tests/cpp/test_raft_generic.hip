@@ -1,0 +1,285 @@
+// GPU tests of the header-template fallback: reductions whose functors or element
+// types are outside the library's vocabulary (device lambdas, caller-defined functor
+// structs, KeyValuePair<int, short>) are instantiated in this translation unit by
+// hipcc.  Cases follow the reference's callers of that kind: the test-local ValueToKVP
+// / ArgMaxOp of cpp/tests/linalg/reduce.cu:346-411 and the capturing lambda of
+// stats/detail/stddev.cuh:46-47.
+#include <raft/core/device_mdarray.hpp>
+#include <raft/core/device_mdspan.hpp>
+#include <raft/core/operators.hpp>
+#include <raft/linalg/coalesced_reduction.cuh>
+#include <raft/linalg/map_reduce.cuh>
+#include <raft/linalg/reduce.cuh>
+#include <raft/linalg/strided_reduction.cuh>
+#include <raft/util/cudart_utils.hpp>
+
+#include <cstdint>
+#include <random>
+
+#include "check.hpp"
+
+namespace {
+
+template <typename T>
+std::vector<T> to_host(const T* d, size_t n, hipStream_t s)
+{
+  std::vector<T> h(n);
+  raft::update_host(h.data(), d, n, s);
+  RAFT_HIP_TRY(hipStreamSynchronize(s));
+  return h;
+}
+
+template <typename T>
+std::vector<T> uniform(size_t n, double lo, double hi, unsigned long long seed)
+{
+  std::mt19937_64 g(seed);
+  std::uniform_real_distribution<double> d(lo, hi);
+  std::vector<T> v(n);
+  for (auto& x : v)
+    x = (T)d(g);
+  return v;
+}
+
+inline size_t at(bool row_major, size_t N, size_t D, size_t i, size_t j)
+{
+  return row_major ? i * D + j : i + j * N;
+}
+
+// the test-local functors of cpp/tests/linalg/reduce.cu:346-358
+template <typename T, typename IdxT = int>
+struct ValueToKVP {
+  HDI raft::KeyValuePair<IdxT, T> operator()(T value, IdxT idx) const { return {idx, value}; }
+};
+template <typename T1, typename T2>
+struct ArgMaxOp {
+  HDI raft::KeyValuePair<T1, T2> operator()(raft::KeyValuePair<T1, T2> a,
+                                            raft::KeyValuePair<T1, T2> b) const
+  {
+    return (a.value > b.value || (a.value == b.value && a.key <= b.key)) ? a : b;
+  }
+};
+
+bool close(double a, double b, double eps)
+{
+  const double d = std::fabs(a - b), m = std::max(std::fabs(a), std::fabs(b));
+  return d <= eps || d / m <= eps;
+}
+
+}  // namespace
+
+// device lambdas as main_op and final_op, all four layout x axis combinations
+TEST_CASE(LambdaMainAndFinal)
+{
+  raft::resources handle;
+  auto stream = raft::resource::get_cuda_stream(handle);
+  for (auto [rows, cols] : std::vector<std::pair<int, int>>{{11, 7}, {1234, 33}, {1234, 128},
+                                                            {37, 500}, {5, 70001}, {20011, 24}}) {
+    auto h = uniform<float>((size_t)rows * cols, -1.0, 1.0, 1234);
+    auto d = raft::make_device_vector<float, int>(handle, rows * cols);
+    raft::update_device(d.data_handle(), h.data(), h.size(), stream);
+    for (int rm = 0; rm < 2; ++rm)
+      for (int ar = 0; ar < 2; ++ar) {
+        const int n_out = ar ? rows : cols, len = ar ? cols : rows;
+        auto out = raft::make_device_vector<float, int>(handle, n_out);
+        auto main_op = [] __device__(float a, int i) { return a * a + 0.001f * (float)(i % 7); };
+        auto fin_op  = [] __device__(float x) { return 0.5f * x + 1.0f; };
+        auto ov      = out.view();
+        if (rm) {
+          auto v = raft::make_device_matrix_view<const float, int, raft::row_major>(
+            d.data_handle(), rows, cols);
+          if (ar)
+            raft::linalg::reduce<raft::Apply::ALONG_ROWS>(handle, v, ov, 0.0f, false, main_op,
+                                                          raft::add_op(), fin_op);
+          else
+            raft::linalg::reduce<raft::Apply::ALONG_COLUMNS>(handle, v, ov, 0.0f, false, main_op,
+                                                             raft::add_op(), fin_op);
+        } else {
+          auto v = raft::make_device_matrix_view<const float, int, raft::col_major>(
+            d.data_handle(), rows, cols);
+          if (ar)
+            raft::linalg::reduce<raft::Apply::ALONG_ROWS>(handle, v, ov, 0.0f, false, main_op,
+                                                          raft::add_op(), fin_op);
+          else
+            raft::linalg::reduce<raft::Apply::ALONG_COLUMNS>(handle, v, ov, 0.0f, false, main_op,
+                                                             raft::add_op(), fin_op);
+        }
+        auto got = to_host(out.data_handle(), (size_t)n_out, stream);
+        bool ok  = true;
+        for (int k = 0; k < n_out; ++k) {
+          double acc = 0;
+          for (int r = 0; r < len; ++r) {
+            const double x = h[ar ? at(rm, rows, cols, k, r) : at(rm, rows, cols, r, k)];
+            acc += x * x + 0.001 * (r % 7);
+          }
+          ok &= close(got[k], 0.5 * acc + 1.0, 2e-4);
+        }
+        CHECK(ok);
+      }
+  }
+}
+
+// cpp/tests/linalg/reduce.cu:360-400: KeyValuePair<int, short> / <int, float> / <int, double>
+// arg-max with the test's own functors, inplace = false then true
+template <typename T>
+void kvp_custom()
+{
+  using KVP = raft::KeyValuePair<int, T>;
+  raft::resources handle;
+  auto stream = raft::resource::get_cuda_stream(handle);
+  for (int rows : {11, 1234})
+    for (int cols : {7, 33, 128, 500}) {
+      std::mt19937 g(1234);
+      std::uniform_int_distribution<int> di(-3000, 3000);
+      std::vector<T> h((size_t)rows * cols);
+      for (auto& x : h)
+        x = (T)di(g);
+      auto d    = raft::make_device_matrix<T, int, raft::row_major>(handle, rows, cols);
+      auto dots = raft::make_device_vector<KVP, int>(handle, rows);
+      raft::update_device(d.data_handle(), h.data(), h.size(), stream);
+      for (int inplace = 0; inplace < 2; ++inplace) {
+        raft::linalg::reduce<raft::Apply::ALONG_ROWS>(
+          handle, raft::make_const_mdspan(d.view()), dots.view(), KVP(0, std::numeric_limits<T>::lowest()),
+          (bool)inplace, ValueToKVP<T, int>(), ArgMaxOp<int, T>(), raft::identity_op());
+        auto got = to_host(dots.data_handle(), (size_t)rows, stream);
+        bool ok  = true;
+        for (int r = 0; r < rows; ++r) {
+          int best = 0;
+          for (int j = 1; j < cols; ++j)
+            if (h[(size_t)r * cols + j] > h[(size_t)r * cols + best]) best = j;
+          ok &= got[r].key == best && got[r].value == h[(size_t)r * cols + best];
+        }
+        CHECK(ok);
+      }
+    }
+}
+TEST_CASE(KvpShortCustomFunctors) { kvp_custom<short>(); }
+TEST_CASE(KvpFloatCustomFunctors) { kvp_custom<float>(); }
+TEST_CASE(KvpDoubleCustomFunctors) { kvp_custom<double>(); }
+
+// stats/detail/stddev.cuh:46-47: a capturing lambda as main_op of a column reduction
+TEST_CASE(CapturingLambdaColumns)
+{
+  raft::resources handle;
+  auto stream    = raft::resource::get_cuda_stream(handle);
+  const int rows = 50000, cols = 48;
+  auto h         = uniform<float>((size_t)rows * cols, -2.0, 3.0, 7);
+  auto d         = raft::make_device_matrix<float, int, raft::row_major>(handle, rows, cols);
+  auto out       = raft::make_device_vector<float, int>(handle, cols);
+  raft::update_device(d.data_handle(), h.data(), h.size(), stream);
+  const float shift = 0.25f;
+  raft::linalg::strided_reduction(
+    handle, raft::make_const_mdspan(d.view()), out.view(), 0.0f, false,
+    [shift] __device__(float a, int) { return (a - shift) * (a - shift); });
+  auto got = to_host(out.data_handle(), (size_t)cols, stream);
+  bool ok  = true;
+  for (int j = 0; j < cols; ++j) {
+    double acc = 0;
+    for (int i = 0; i < rows; ++i) {
+      const double x = (double)h[(size_t)i * cols + j] - shift;
+      acc += x * x;
+    }
+    ok &= close(got[j], acc, 5e-4);
+  }
+  CHECK(ok);
+}
+
+// an element type the library has no kernel for (int16) with library functors, and a
+// custom reduce_op (product) over doubles: long rows (split) and many short rows
+TEST_CASE(UnknownTypesAndReduceOps)
+{
+  raft::resources handle;
+  auto stream = raft::resource::get_cuda_stream(handle);
+  {
+    const int rows = 3, cols = 300000;
+    std::mt19937 g(5);
+    std::uniform_int_distribution<int> di(-100, 100);
+    std::vector<std::int16_t> h((size_t)rows * cols);
+    for (auto& x : h)
+      x = (std::int16_t)di(g);
+    auto d   = raft::make_device_matrix<std::int16_t, int, raft::row_major>(handle, rows, cols);
+    auto out = raft::make_device_vector<long long, int>(handle, rows);
+    raft::update_device(d.data_handle(), h.data(), h.size(), stream);
+    raft::linalg::coalesced_reduction(handle, raft::make_const_mdspan(d.view()), out.view(), 0LL,
+                                      false, raft::cast_op<long long>(), raft::add_op());
+    auto got = to_host(out.data_handle(), (size_t)rows, stream);
+    for (int r = 0; r < rows; ++r) {
+      long long s = 0;
+      for (int j = 0; j < cols; ++j)
+        s += h[(size_t)r * cols + j];
+      CHECK(got[r] == s);
+    }
+  }
+  {
+    const int rows = 4000, cols = 9;
+    auto h   = uniform<double>((size_t)rows * cols, 0.9, 1.1, 11);
+    auto d   = raft::make_device_matrix<double, int, raft::row_major>(handle, rows, cols);
+    auto out = raft::make_device_vector<double, int>(handle, rows);
+    raft::update_device(d.data_handle(), h.data(), h.size(), stream);
+    raft::linalg::reduce<raft::Apply::ALONG_ROWS>(handle, raft::make_const_mdspan(d.view()),
+                                                  out.view(), 1.0, false, raft::identity_op(),
+                                                  raft::mul_op());
+    auto got = to_host(out.data_handle(), (size_t)rows, stream);
+    bool ok  = true;
+    for (int r = 0; r < rows; ++r) {
+      double p = 1;
+      for (int j = 0; j < cols; ++j)
+        p *= h[(size_t)r * cols + j];
+      ok &= close(got[r], p, 1e-12);
+    }
+    CHECK(ok);
+  }
+}
+
+// library functors still take the C ABI path from a hipcc translation unit
+TEST_CASE(VocabularyStillLowered)
+{
+  raft::resources handle;
+  auto stream    = raft::resource::get_cuda_stream(handle);
+  const int rows = 1000, cols = 128;
+  auto h         = uniform<float>((size_t)rows * cols, -1.0, 1.0, 3);
+  auto d         = raft::make_device_matrix<float, int, raft::row_major>(handle, rows, cols);
+  auto out       = raft::make_device_vector<float, int>(handle, rows);
+  raft::update_device(d.data_handle(), h.data(), h.size(), stream);
+  raft::linalg::reduce<raft::Apply::ALONG_ROWS>(handle, raft::make_const_mdspan(d.view()),
+                                                out.view(), 0.0f, false, raft::sq_op(),
+                                                raft::add_op(), raft::sqrt_op());
+  auto got = to_host(out.data_handle(), (size_t)rows, stream);
+  bool ok  = true;
+  for (int r = 0; r < rows; ++r) {
+    double s = 0;
+    for (int j = 0; j < cols; ++j)
+      s += (double)h[(size_t)r * cols + j] * h[(size_t)r * cols + j];
+    ok &= close(got[r], std::sqrt(s), 1e-6);
+  }
+  CHECK(ok);
+}
+
+// map_reduce with a device lambda
+TEST_CASE(MapReduceLambda)
+{
+  raft::resources handle;
+  auto stream   = raft::resource::get_cuda_stream(handle);
+  const int len = 1 << 20;
+  auto h        = uniform<float>(len, -1.0, 1.0, 9);
+  auto in       = raft::make_device_vector<float, int>(handle, len);
+  auto out      = raft::make_device_scalar<float>(handle);
+  raft::update_device(in.data_handle(), h.data(), h.size(), stream);
+  auto in_c = raft::make_device_vector_view<const float, int>(in.data_handle(), len);
+  raft::linalg::map_reduce(handle, in_c, out.view(), 0.0f,
+                           [] __device__(float x, int) { return x > 0.0f ? x : 0.0f; },
+                           raft::add_op());
+  double want = 0;
+  for (float x : h)
+    want += x > 0 ? x : 0;
+  CHECK(close(to_host(out.data_handle(), 1, stream)[0], want, 1e-4));
+}
+
+int main()
+{
+  int n = 0;
+  if (hipGetDeviceCount(&n) != hipSuccess || n == 0) {
+    std::printf("no GPU visible\n");
+    return 2;
+  }
+  return t::run_all();
+}

@@ -2,7 +2,8 @@
 
 test_raft_host needs no GPU: functor vocabulary, views, precondition errors, plan
 selector.  test_raft_api restates the reference's reduction-path tests against the
-kept raft:: names and runs on the GPU."""
+kept raft:: names and runs on the GPU.  test_raft_generic is compiled by hipcc and
+covers functors outside the library's vocabulary."""
 import subprocess
 from pathlib import Path
 
@@ -30,4 +31,12 @@ def test_cpp_host_layer():
 @pytest.mark.gpu
 def test_cpp_api_on_gpu(gpu):
     out = _run("test_raft_api", 600)
+    assert "0 failed" in out
+
+
+@pytest.mark.gpu
+def test_cpp_generic_functors_on_gpu(gpu):
+    """Device lambdas, caller-defined functors and KeyValuePair<int, short>, instantiated in
+    a hipcc translation unit by the header fallback (tests/cpp/test_raft_generic.hip)."""
+    out = _run("test_raft_generic", 600)
     assert "0 failed" in out
