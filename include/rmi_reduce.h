@@ -228,6 +228,21 @@ RMI_API int rmi_map_reduce(const rmi_reduce_desc* desc,
                    size_t workspace_bytes,
                    void* stream);
 
+/* Row normalisation fused with its norm: out[i, :] = in[i, :] / norm_i with
+ * norm_i = final_op(reduce_op(init, fold over j of main_op(in[i, j]))); rows whose
+ * norm is <= eps (or NaN) are left untouched.  Replaces detail::coalesced_normalize
+ * (linalg/detail/normalize.cuh:36-197) behind raft::linalg::row_normalize
+ * (linalg/normalize.cuh:48-110).  Uses the descriptor fields in_dtype (also the
+ * output's type: F16, BF16, F32 or F64), n_rows, n_cols, main_op (IDENTITY, SQ, ABS),
+ * reduce_op (ADD, MAX, MIN), final_op (IDENTITY or SQRT) and init.f; the matrix is
+ * row-major.  The division happens in the element's arithmetic (f32 for f16 / bf16).
+ * `out` may be `in`.  Needs no workspace. */
+RMI_API int rmi_row_normalize(const rmi_reduce_desc* desc,
+                              const void* in,
+                              void* out,
+                              double eps,
+                              void* stream);
+
 #ifdef __cplusplus
 } /* extern "C" */
 #endif

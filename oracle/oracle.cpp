@@ -32,6 +32,8 @@
 //   map-then-reduce: include/raft/linalg/detail/map_then_reduce.cuh:47-95
 //   arg-reduce, key-only output, init (0, -/+inf):
 //       include/raft/matrix/detail/math.cuh:292-352
+//   row normalisation: include/raft/linalg/detail/normalize.cuh:36-57,
+//       include/raft/linalg/normalize.cuh:91-107
 //
 // Pinned by (tests/test_oracle.py): the closed-form fixtures of
 // tests/linalg/reduce.cu:108-177, tests/matrix/argmax.cu:71-75,
@@ -697,6 +699,36 @@ ORC_API int orc_reduce_typed(const rmi_reduce_desc* d,
     case RMI_BF16: return typed_in(*d, (const bf16*)in, out, aux, threads);
     case RMI_F32: return typed_in(*d, (const float*)in, out, aux, threads);
     case RMI_F64: return typed_in(*d, (const double*)in, out, aux, threads);
+    default: return RMI_ERR_UNSUPPORTED;
+  }
+}
+
+// Row normalisation in fp64: out[i, :] = in[i, :] / norm_i, rows with norm_i <= eps
+// untouched (cpp/include/raft/linalg/detail/normalize.cuh:36-57).  `out` holds the
+// previous contents on entry, as doubles.
+template <class T>
+static int normalize_seq(const rmi_reduce_desc& d, const T* in, double* out, double eps)
+{
+  for (int64_t i = 0; i < d.n_rows; ++i) {
+    double acc = d.init.f;
+    for (int64_t j = 0; j < d.n_cols; ++j)
+      acc = red_f(d.reduce_op, acc, main_f(d.main_op, Elem<T>::f64(in[i * d.n_cols + j])));
+    const double norm = d.final_op == RMI_FIN_SQRT ? sqrt(acc) : acc;
+    if (!(norm > eps)) continue;
+    for (int64_t j = 0; j < d.n_cols; ++j)
+      out[i * d.n_cols + j] = Elem<T>::f64(in[i * d.n_cols + j]) / norm;
+  }
+  return RMI_OK;
+}
+
+ORC_API int orc_row_normalize(const rmi_reduce_desc* d, const void* in, double* out, double eps)
+{
+  if (!d) return RMI_ERR_NULL;
+  switch (d->in_dtype) {
+    case RMI_F16: return normalize_seq(*d, (const f16*)in, out, eps);
+    case RMI_BF16: return normalize_seq(*d, (const bf16*)in, out, eps);
+    case RMI_F32: return normalize_seq(*d, (const float*)in, out, eps);
+    case RMI_F64: return normalize_seq(*d, (const double*)in, out, eps);
     default: return RMI_ERR_UNSUPPORTED;
   }
 }

@@ -195,4 +195,42 @@ int rmi_map_reduce(const rmi_reduce_desc* desc,
   return rmi::reduce_impl(r, in, out, workspace, workspace_bytes, stream);
 }
 
+int rmi_row_normalize(const rmi_reduce_desc* desc,
+                      const void* in,
+                      void* out,
+                      double eps,
+                      void* stream)
+{
+  using namespace rmi;
+  if (desc == nullptr) return RMI_ERR_NULL;
+  const rmi_reduce_desc& d = *desc;
+  if (d.n_rows < 0 || d.n_cols < 0) return RMI_ERR_BAD_SHAPE;
+  if (d.final_op != RMI_FIN_IDENTITY && d.final_op != RMI_FIN_SQRT) return RMI_ERR_UNSUPPORTED;
+  norm_fn fn = nullptr;
+  switch (d.in_dtype) {
+    case RMI_F16: fn = lookup_norm_f16(d.main_op, d.reduce_op); break;
+    case RMI_BF16: fn = lookup_norm_bf16(d.main_op, d.reduce_op); break;
+    case RMI_F32: fn = lookup_norm_f32(d.main_op, d.reduce_op); break;
+    case RMI_F64: fn = lookup_norm_f64(d.main_op, d.reduce_op); break;
+    default: return d.in_dtype >= 0 && d.in_dtype < RMI_DTYPE_COUNT_ ? RMI_ERR_UNSUPPORTED
+                                                                     : RMI_ERR_BAD_ENUM;
+  }
+  if (fn == nullptr) return RMI_ERR_UNSUPPORTED;
+  if (d.n_rows == 0 || d.n_cols == 0) return RMI_OK;
+  if (in == nullptr || out == nullptr) return RMI_ERR_NULL;
+  const int es = dtype_size(d.in_dtype);
+  if (!aligned(in, es) || !aligned(out, es)) return RMI_ERR_ALIGNMENT;
+  const NormPlan pl = make_norm_plan(d.n_rows, d.n_cols, es);
+  NormArgs a{};
+  a.in        = in;
+  a.out       = out;
+  a.n_rows    = d.n_rows;
+  a.len       = d.n_cols;
+  a.row_bytes = d.n_cols * es;
+  a.final_op  = d.final_op;
+  a.init      = d.init.f;
+  a.eps       = eps;
+  return fn(pl, a, static_cast<hipStream_t>(stream));
+}
+
 }  // extern "C"

@@ -6,6 +6,7 @@
 #include <hip/hip_runtime.h>
 
 #include "rmi_kernels.hpp"
+#include "rmi_normalize.hpp"
 #include "rmi_plan.hpp"
 
 namespace rmi {
@@ -135,6 +136,101 @@ int run(const PlanX& pl, const Problem& pr, hipStream_t st)
   return hipGetLastError() == hipSuccess ? RMI_OK : RMI_ERR_LAUNCH;
 }
 
+// ---- row normalisation -----------------------------------------------------------
+struct NormPlan {
+  bool vec16   = false;
+  bool team    = false;
+  int G        = 1;
+  int logG     = 0;
+  int threads  = kBlock;
+  int64_t grid = 0;
+  int64_t nvec = 0;
+  int tail     = 0;
+};
+
+inline NormPlan make_norm_plan(int64_t n_rows, int64_t len, int elem_bytes)
+{
+  NormPlan p;
+  const int64_t row_bytes = len * elem_bytes;
+  p.vec16                 = row_bytes >= 16;
+  const int step          = p.vec16 ? 16 / elem_bytes : 1;
+  p.nvec                  = len / step;
+  p.tail                  = (int)(len % step);
+  const int64_t nload     = p.nvec + (p.tail > 0 ? 1 : 0);
+  if (nload <= (int64_t)kUnroll * kWave) {
+    const int64_t g = ceildiv(nload, kUnroll);
+    p.G             = g >= 64 ? 64 : pow2ceil(g < 1 ? 1 : g);
+    p.logG          = ilog2(p.G);
+    p.grid          = ceildiv(n_rows, (int64_t)(kWave / p.G) * (kBlock / kWave));
+  } else {
+    p.team    = true;
+    p.threads = nload >= (int64_t)4 * 1024 * kUnroll ? 1024 : kBlock;
+    p.grid    = n_rows;
+  }
+  return p;
+}
+
+using norm_fn = int (*)(const NormPlan&, const NormArgs&, hipStream_t);
+
+template <class P>
+int run_normalize(const NormPlan& pl, const NormArgs& args, hipStream_t st)
+{
+  NormArgs a = args;
+  a.nvec     = pl.nvec;
+  a.tail     = pl.tail;
+  a.G        = pl.G;
+  a.logG     = pl.logG;
+  if (pl.grid > 0x7fffffffLL) return RMI_ERR_BAD_SHAPE;
+  const dim3 grid((unsigned)pl.grid);
+  if (!pl.team) {
+    if (pl.vec16)
+      hipLaunchKernelGGL((normalize_wave_kernel<P, true>), grid, dim3(kBlock), 0, st, a);
+    else
+      hipLaunchKernelGGL((normalize_wave_kernel<P, false>), grid, dim3(kBlock), 0, st, a);
+  } else {
+    // rows of 4 KB and more always hold whole vectors
+    hipLaunchKernelGGL((normalize_team_kernel<P, true>), grid, dim3(pl.threads), 0, st, a);
+  }
+  return hipGetLastError() == hipSuccess ? RMI_OK : RMI_ERR_LAUNCH;
+}
+
+// Norm functor pairs offered for one floating input type: (identity | sq | abs) with
+// (add | max | min).
+template <class InT, bool IS_F64>
+norm_fn lookup_norm_for(int main_op, int red_op)
+{
+#define RMI_NORM_MAIN(RED_POLICY)                                   \
+  switch (main_op) {                                                \
+    case RMI_MAIN_IDENTITY: return &run_normalize<RED_POLICY(RMI_MAIN_IDENTITY)>; \
+    case RMI_MAIN_SQ: return &run_normalize<RED_POLICY(RMI_MAIN_SQ)>;             \
+    case RMI_MAIN_ABS: return &run_normalize<RED_POLICY(RMI_MAIN_ABS)>;           \
+    default: return nullptr;                                        \
+  }
+  if (red_op == RMI_RED_ADD) {
+    if constexpr (IS_F64) {
+#define POL(M) PolKbn<InT, M>
+      RMI_NORM_MAIN(POL)
+#undef POL
+    } else {
+#define POL(M) PolF<InT, M, RMI_RED_ADD>
+      RMI_NORM_MAIN(POL)
+#undef POL
+    }
+  }
+  if (red_op == RMI_RED_MAX) {
+#define POL(M) PolF<InT, M, RMI_RED_MAX>
+    RMI_NORM_MAIN(POL)
+#undef POL
+  }
+  if (red_op == RMI_RED_MIN) {
+#define POL(M) PolF<InT, M, RMI_RED_MIN>
+    RMI_NORM_MAIN(POL)
+#undef POL
+  }
+#undef RMI_NORM_MAIN
+  return nullptr;
+}
+
 // Policies offered for one input type, keyed by PolicyKey.
 template <class InT, bool IS_FLOAT_IN, bool IS_F64>
 run_fn lookup_for(const PolicyKey& k)
@@ -227,5 +323,9 @@ run_fn lookup_f16(const PolicyKey&);
 run_fn lookup_bf16(const PolicyKey&);
 run_fn lookup_f32(const PolicyKey&);
 run_fn lookup_f64(const PolicyKey&);
+norm_fn lookup_norm_f16(int main_op, int red_op);
+norm_fn lookup_norm_bf16(int main_op, int red_op);
+norm_fn lookup_norm_f32(int main_op, int red_op);
+norm_fn lookup_norm_f64(int main_op, int red_op);
 
 }  // namespace rmi

@@ -1,0 +1,217 @@
+// Row normalisation fused with its norm: out[i, :] = in[i, :] / norm_i, where
+// norm_i = final_op(reduce_op-fold of main_op(in[i, j])) and rows whose norm is
+// <= eps are left untouched (linalg/detail/normalize.cuh:36-57,112-134 of the
+// reference).  Rows of up to 256 lane-loads stay in registers between the reduction
+// and the scaling, so the matrix is read once and written once; longer rows are
+// swept twice by one team (the second sweep finds the row in the caches).
+#pragma once
+
+#include "rmi_kernels.hpp"
+
+namespace rmi {
+
+struct NormArgs {
+  const void* in;
+  void* out;
+  i64 n_rows;
+  i64 len;
+  i64 row_bytes;
+  i64 nvec;    // whole lane-loads per row
+  int tail;    // elements after the last whole vector
+  int G;       // lanes per row (wave kernel)
+  int logG;
+  int logT;    // team kernel: 64 << logT threads per row
+  int final_op;
+  double init;
+  double eps;
+};
+
+// Element stores, the inverse of In<T>::get.
+template <class T>
+struct Put;
+template <>
+struct Put<float> {
+  template <int J>
+  static __device__ __forceinline__ void at(u32x4& v, float x)
+  {
+    v[J] = as_u32(x);
+  }
+  static __device__ __forceinline__ void st(float* p, float x) { *p = x; }
+};
+template <>
+struct Put<double> {
+  template <int J>
+  static __device__ __forceinline__ void at(u32x4& v, double x)
+  {
+    v[2 * J]     = (u32)__double2loint(x);
+    v[2 * J + 1] = (u32)__double2hiint(x);
+  }
+  static __device__ __forceinline__ void st(double* p, double x) { *p = x; }
+};
+template <>
+struct Put<f16_t> {
+  static __device__ __forceinline__ u32 bits(float x)
+  {
+    const f16_t h = (f16_t)x;
+    uint16_t b;
+    __builtin_memcpy(&b, &h, 2);
+    return b;
+  }
+  template <int J>
+  static __device__ __forceinline__ void at(u32x4& v, float x)
+  {
+    if constexpr (J & 1) {
+      v[J / 2] = (v[J / 2] & 0xffffu) | (bits(x) << 16);
+    } else {
+      v[J / 2] = (v[J / 2] & 0xffff0000u) | bits(x);
+    }
+  }
+  static __device__ __forceinline__ void st(f16_t* p, float x) { *p = (f16_t)x; }
+};
+template <>
+struct Put<bf16_t> {
+  template <int J>
+  static __device__ __forceinline__ void at(u32x4& v, float x)
+  {
+    const u32 b = f32_to_bf16(x);
+    if constexpr (J & 1) {
+      v[J / 2] = (v[J / 2] & 0xffffu) | (b << 16);
+    } else {
+      v[J / 2] = (v[J / 2] & 0xffff0000u) | b;
+    }
+  }
+  static __device__ __forceinline__ void st(bf16_t* p, float x) { p->bits = f32_to_bf16(x); }
+};
+
+__device__ __forceinline__ void store16(void* p, const u32x4& v)
+{
+  *reinterpret_cast<u32x4_unaligned*>(p) = v;
+}
+
+// norm of a row from its folded accumulator, in the element's own arithmetic
+template <class P>
+__device__ __forceinline__ typename P::nat row_norm(const NormArgs& a, typename P::acc_t acc)
+{
+  using nat               = typename P::nat;
+  typename P::acc_t total = P::from_f64(a.init);
+  P::merge(total, acc);
+  nat n = (nat)P::to_f64(total);
+  if (a.final_op == RMI_FIN_SQRT) n = sqrt(n);
+  return n;
+}
+
+// lane-load `v` of a row, scaled by 1/norm and written to the same place of `orow`
+template <class P, bool VEC16>
+__device__ __forceinline__ void write_scaled(const NormArgs& a,
+                                             char* orow,
+                                             const typename Held<P, VEC16>::type& x,
+                                             i64 v,
+                                             typename P::nat norm)
+{
+  using in_t = typename P::in_t;
+  if constexpr (VEC16) {
+    if (v < a.nvec) {
+      u32x4 y = x;
+      static_for<P::VEC>([&](auto j) {
+        Put<in_t>::template at<decltype(j)::value>(y, In<in_t>::template get<decltype(j)::value>(x) / norm);
+      });
+      store16(orow + v * 16, y);
+    } else {
+      // the overlapping last vector: only its last `tail` elements are new
+      in_t* o        = reinterpret_cast<in_t*>(orow) + (a.len - P::VEC);
+      const int skip = P::VEC - a.tail;
+      static_for<P::VEC>([&](auto j) {
+        if (j >= skip) Put<in_t>::st(o + j, In<in_t>::template get<decltype(j)::value>(x) / norm);
+      });
+    }
+  } else {
+    Put<in_t>::st(reinterpret_cast<in_t*>(orow) + v, x / norm);
+  }
+}
+
+// G lanes of one wave per row, at most kUnroll lane-loads per lane: the row stays in
+// registers from the reduction to the scaling.
+template <class P, bool VEC16>
+__global__ __launch_bounds__(kBlock) void normalize_wave_kernel(NormArgs a)
+{
+  using acc_t    = typename P::acc_t;
+  using H        = Held<P, VEC16>;
+  const int lane = threadIdx.x & (kWave - 1);
+  const i64 wid  = (i64)blockIdx.x * (kBlock / kWave) + (threadIdx.x >> 6);
+  const int G    = a.G;
+  const int c    = lane & (G - 1);
+  const i64 row  = wid * (kWave >> a.logG) + (lane >> a.logG);
+  const i64 nload = a.nvec + (a.tail > 0 ? 1 : 0);
+  const bool live = row < a.n_rows;
+  const char* rp  = static_cast<const char*>(a.in) + row * a.row_bytes;
+
+  typename H::type x[kUnroll];
+  acc_t acc = P::neutral();
+  if (live) {
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u)
+      if (c + u * G < nload) x[u] = H::load_any(rp, c + u * G, a.nvec, a.len);
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u)
+      if (c + u * G < nload) H::push_any(acc, x[u], c + u * G, a.nvec, a.len, a.tail);
+  }
+  group_allreduce<P>(acc, G);
+  if (!live) return;
+  const auto norm = row_norm<P>(a, acc);
+  if (!(norm > (typename P::nat)a.eps)) return;  // also leaves NaN norms untouched
+  char* orow = static_cast<char*>(a.out) + row * a.row_bytes;
+#pragma unroll
+  for (int u = 0; u < kUnroll; ++u)
+    if (c + u * G < nload) write_scaled<P, VEC16>(a, orow, x[u], c + u * G, norm);
+}
+
+// One team of 64 << logT threads per row, two sweeps.
+template <class P, bool VEC16>
+__global__ __launch_bounds__(1024) void normalize_team_kernel(NormArgs a)
+{
+  using acc_t = typename P::acc_t;
+  using H     = Held<P, VEC16>;
+  using nat   = typename P::nat;
+  __shared__ acc_t sm[16];
+  __shared__ nat sm_norm;
+
+  const int T     = blockDim.x;
+  const int t     = threadIdx.x;
+  const i64 row   = blockIdx.x;
+  const i64 nload = a.nvec + (a.tail > 0 ? 1 : 0);
+  const char* rp  = static_cast<const char*>(a.in) + row * a.row_bytes;
+
+  acc_t acc = P::neutral();
+  for (i64 v = t; v < nload; v += (i64)kUnroll * T) {
+    typename H::type x[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u)
+      if (v + (i64)u * T < nload) x[u] = H::load_any(rp, v + (i64)u * T, a.nvec, a.len);
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u)
+      if (v + (i64)u * T < nload) H::push_any(acc, x[u], v + (i64)u * T, a.nvec, a.len, a.tail);
+  }
+  wave_allreduce<P>(acc);
+  if ((t & (kWave - 1)) == 0) sm[t >> 6] = acc;
+  __syncthreads();
+  if (t == 0) {
+    for (int w = 1; w < (T >> 6); ++w)
+      P::merge(acc, sm[w]);
+    sm_norm = row_norm<P>(a, acc);
+  }
+  __syncthreads();
+  const nat norm = sm_norm;
+  if (!(norm > (nat)a.eps)) return;
+  char* orow = static_cast<char*>(a.out) + row * a.row_bytes;
+  for (i64 v = t; v < nload; v += (i64)kUnroll * T) {
+    typename H::type x[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u)
+      if (v + (i64)u * T < nload) x[u] = H::load_any(rp, v + (i64)u * T, a.nvec, a.len);
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u)
+      if (v + (i64)u * T < nload) write_scaled<P, VEC16>(a, orow, x[u], v + (i64)u * T, norm);
+  }
+}
+
+}  // namespace rmi

@@ -13,6 +13,7 @@
 #include <raft/linalg/map_reduce.cuh>
 #include <raft/linalg/map_then_reduce.cuh>
 #include <raft/linalg/norm.cuh>
+#include <raft/linalg/normalize.cuh>
 #include <raft/linalg/reduce.cuh>
 #include <raft/linalg/strided_reduction.cuh>
 #include <raft/matrix/argmax.cuh>
@@ -573,8 +574,48 @@ void handle_workspace_reuse()
   RAFT_HIP_TRY(hipStreamDestroy(s));
 }
 
+// cpp/tests/linalg/normalize.cu:40-135: row_normalize against rowNorm followed by a
+// per-row division, rows {11,101,12345} x cols {2,3,7,12,33,125,254} x {L1,L2,Linf}
+template <typename T, typename Idx>
+void row_normalize_cases(double tol)
+{
+  using namespace raft::linalg;
+  raft::resources handle;
+  auto stream = raft::resource::get_cuda_stream(handle);
+  for (int rows : {11, 101, 12345})
+    for (int cols : {2, 3, 7, 12, 33, 125, 254}) {
+      auto h   = uniform<T>((size_t)rows * cols, -10.0, 10.0, 1234);
+      auto in  = raft::make_device_matrix<T, Idx, raft::row_major>(handle, (Idx)rows, (Idx)cols);
+      auto out = raft::make_device_matrix<T, Idx, raft::row_major>(handle, (Idx)rows, (Idx)cols);
+      raft::update_device(in.data_handle(), h.data(), h.size(), stream);
+      auto in_v = raft::make_device_matrix_view<const T, Idx, raft::row_major>(in.data_handle(),
+                                                                               (Idx)rows, (Idx)cols);
+      for (int nt = 0; nt < 3; ++nt) {
+        if (nt == 0) row_normalize<L1Norm>(handle, in_v, out.view());
+        if (nt == 1) row_normalize<L2Norm>(handle, in_v, out.view());
+        if (nt == 2) row_normalize<LinfNorm>(handle, in_v, out.view());
+        auto got = to_host(out.data_handle(), h.size(), stream);
+        std::vector<double> want(h.size());
+        for (int i = 0; i < rows; ++i) {
+          double n = 0;
+          for (int j = 0; j < cols; ++j) {
+            const double x = (double)h[(size_t)i * cols + j];
+            n = nt == 0 ? n + std::fabs(x) : nt == 1 ? n + x * x : std::max(n, std::fabs(x));
+          }
+          if (nt == 1) n = std::sqrt(n);
+          for (int j = 0; j < cols; ++j)
+            want[(size_t)i * cols + j] = (double)h[(size_t)i * cols + j] / n;
+        }
+        CHECK(all_close(got, want, tol));
+      }
+    }
+}
+
 }  // namespace
 
+TEST_CASE(RowNormalizeFI32) { row_normalize_cases<float, int>(1e-5); }
+TEST_CASE(RowNormalizeDI32) { row_normalize_cases<double, int>(1e-8); }
+TEST_CASE(RowNormalizeFU32) { row_normalize_cases<float, std::uint32_t>(1e-5); }
 TEST_CASE(ReduceSimpleF) { simple_max<float>(); }
 TEST_CASE(ReduceSimpleD) { simple_max<double>(); }
 TEST_CASE(ReduceTestFFI32) { reduce_full<float, float, int>(2e-6, {11, 1234}, {7, 33, 128, 500}); }

@@ -148,6 +148,15 @@ def test_null_and_workspace_errors_without_a_launch():
     assert lib.rmi_reduce(C.byref(d), 0x1000, 0x2000, None, 0, None) == api.ERR_WORKSPACE
     assert lib.rmi_reduce(C.byref(d), 0x1000, 0x2000, 0x3000, 16, None) == api.ERR_WORKSPACE
     assert lib.rmi_map_reduce(C.byref(d), -1, None, None, None, 0, None) == api.ERR_BAD_SHAPE
+    dn = api.make_desc(api.I8, api.I8, 10, 10)
+    assert lib.rmi_row_normalize(C.byref(dn), 0x1000, 0x2000, 1e-8, None) == api.ERR_UNSUPPORTED
+    dn = api.make_desc(api.F32, api.F32, 10, 10, final_op=api.FIN_SQ)
+    assert lib.rmi_row_normalize(C.byref(dn), 0x1000, 0x2000, 1e-8, None) == api.ERR_UNSUPPORTED
+    dn = api.make_desc(api.F32, api.F32, 10, 10)
+    assert lib.rmi_row_normalize(C.byref(dn), None, 0x2000, 1e-8, None) == api.ERR_NULL
+    assert lib.rmi_row_normalize(C.byref(dn), 0x1002, 0x2000, 1e-8, None) == api.ERR_ALIGNMENT
+    dn = api.make_desc(api.F32, api.F32, 0, 10)
+    assert lib.rmi_row_normalize(C.byref(dn), None, None, 1e-8, None) == api.OK
     # zero outputs: success, nothing to do
     d = api.make_desc(api.F32, api.F32, 0, 100)
     assert lib.rmi_reduce(C.byref(d), None, None, None, 0, None) == api.OK

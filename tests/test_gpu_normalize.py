@@ -1,0 +1,133 @@
+"""Row normalisation (rmi_row_normalize) on the GPU against the fp64 oracle: the shape
+grid of the reference's test (cpp/tests/linalg/normalize.cu:111-135), long rows, half
+types, rows below eps left untouched, in-place use."""
+import ctypes as C
+import itertools
+
+import numpy as np
+import pytest
+
+from raft_amd import _capi as api
+from tests import _util as u
+
+pytestmark = pytest.mark.gpu
+
+NORMS = {
+    "l1": (api.MAIN_ABS, api.RED_ADD, api.FIN_IDENTITY),
+    "l2": (api.MAIN_SQ, api.RED_ADD, api.FIN_SQRT),
+    "linf": (api.MAIN_ABS, api.RED_MAX, api.FIN_IDENTITY),
+}
+
+
+def _oracle(desc, data, prev, eps):
+    out = np.ascontiguousarray(prev, dtype=np.float64).copy()
+    rc = u.load_oracle().orc_row_normalize(C.byref(desc), data.ctypes.data, out.ctypes.data, eps)
+    assert rc == 0
+    return out
+
+
+def _gpu(desc, data, prev_raw, eps, inplace=False):
+    import torch
+    from raft_amd import device as dev
+    x = torch.from_numpy(data.view(np.uint8).reshape(-1)).cuda()
+    o = x if inplace else torch.from_numpy(prev_raw.view(np.uint8).reshape(-1).copy()).cuda()
+    rc = api.load().rmi_row_normalize(C.byref(desc), x.data_ptr(), o.data_ptr(), eps,
+                                      dev.current_stream_ptr())
+    assert rc == 0, api.status_string(rc)
+    torch.cuda.synchronize()
+    return o.cpu().numpy().view(data.dtype).copy()
+
+
+def _as_f64(dt, raw):
+    return u.from_bf16(raw).astype(np.float64) if dt == api.BF16 else raw.astype(np.float64)
+
+
+@pytest.mark.parametrize("dt,npdt,tol", [(api.F32, np.float32, 1e-5), (api.F64, np.float64, 1e-8)])
+@pytest.mark.parametrize("norm", list(NORMS))
+@pytest.mark.parametrize("rows,cols", itertools.product([11, 101, 12345],
+                                                        [2, 3, 7, 12, 33, 125, 254]))
+def test_reference_grid(gpu, dt, npdt, tol, norm, rows, cols):
+    rng = np.random.default_rng(1234)
+    data = rng.uniform(-10, 10, rows * cols).astype(npdt)
+    main, red, fin = NORMS[norm]
+    d = api.make_desc(dt, dt, rows, cols, main_op=main, reduce_op=red, final_op=fin)
+    prev = np.full(rows * cols, 7.0, dtype=npdt)
+    got = _gpu(d, data, prev, 1e-8)
+    exp = _oracle(d, data, prev, 1e-8)
+    assert u.approx_ok(got, exp, tol).all(), u.worst_rel(got, exp)
+
+
+@pytest.mark.parametrize("rows,cols", [(37, 1024), (9, 5000), (5, 70001), (3, 1 << 18), (2000, 1000)])
+@pytest.mark.parametrize("norm", ["l1", "l2", "linf"])
+def test_long_rows(gpu, rows, cols, norm):
+    rng = np.random.default_rng(cols)
+    data = rng.standard_normal(rows * cols).astype(np.float32)
+    main, red, fin = NORMS[norm]
+    d = api.make_desc(api.F32, api.F32, rows, cols, main_op=main, reduce_op=red, final_op=fin)
+    prev = np.zeros(rows * cols, dtype=np.float32)
+    got = _gpu(d, data, prev, 1e-8)
+    exp = _oracle(d, data, prev, 1e-8)
+    assert u.approx_ok(got, exp, 1e-5).all(), u.worst_rel(got, exp)
+    if norm == "l2":  # unit rows
+        n = np.linalg.norm(got.reshape(rows, cols).astype(np.float64), axis=1)
+        assert np.allclose(n, 1.0, atol=1e-5)
+
+
+@pytest.mark.parametrize("dt", [api.F16, api.BF16])
+@pytest.mark.parametrize("rows,cols", [(100, 64), (1000, 100), (33, 7), (7, 9000)])
+def test_half_types(gpu, dt, rows, cols):
+    rng = np.random.default_rng(3)
+    f = rng.uniform(-4, 4, rows * cols).astype(np.float32)
+    data = f.astype(np.float16) if dt == api.F16 else u.to_bf16(f)
+    d = api.make_desc(dt, dt, rows, cols, main_op=api.MAIN_SQ, final_op=api.FIN_SQRT)
+    prev = np.zeros(rows * cols, dtype=data.dtype)
+    got = _as_f64(dt, _gpu(d, data, prev, 1e-8))
+    exp = _oracle(d, data, _as_f64(dt, prev), 1e-8)
+    assert u.approx_ok(got, exp, u.OUT_TOL[dt]).all(), u.worst_rel(got, exp)
+
+
+def test_rows_below_eps_are_left_untouched(gpu):
+    rows, cols = 64, 96
+    rng = np.random.default_rng(8)
+    m = rng.standard_normal((rows, cols)).astype(np.float32)
+    m[::4] = 0.0          # norm 0
+    m[1::8] *= 1e-12      # norm far below eps
+    d = api.make_desc(api.F32, api.F32, rows, cols, main_op=api.MAIN_SQ, final_op=api.FIN_SQRT)
+    prev = np.full(rows * cols, -3.0, dtype=np.float32)
+    got = _gpu(d, m.reshape(-1), prev, 1e-6).reshape(rows, cols)
+    exp = _oracle(d, m.reshape(-1), prev, 1e-6).reshape(rows, cols)
+    assert (got[::4] == -3.0).all() and (got[1::8] == -3.0).all()
+    assert u.approx_ok(got, exp, 1e-5).all()
+
+
+@pytest.mark.parametrize("rows,cols", [(1000, 128), (50, 33), (4, 20000)])
+def test_in_place(gpu, rows, cols):
+    rng = np.random.default_rng(rows)
+    data = rng.standard_normal(rows * cols).astype(np.float32)
+    d = api.make_desc(api.F32, api.F32, rows, cols, main_op=api.MAIN_SQ, final_op=api.FIN_SQRT)
+    got = _gpu(d, data, None, 1e-8, inplace=True)
+    exp = _oracle(d, data, data, 1e-8)
+    assert u.approx_ok(got, exp, 1e-5).all(), u.worst_rel(got, exp)
+
+
+def test_full_size_embedding_shape(gpu):
+    """1,000,000 x 128 fp32 (the shape of benchmark config 2): unit L2 rows, and the
+    oracle on a slice."""
+    import torch
+    from raft_amd import device as dev
+    rows, cols = 1000000, 128
+    g = torch.Generator(device="cuda")
+    g.manual_seed(2)
+    x = torch.randn(rows * cols, generator=g, device="cuda")
+    o = torch.empty_like(x)
+    d = api.make_desc(api.F32, api.F32, rows, cols, main_op=api.MAIN_SQ, final_op=api.FIN_SQRT)
+    rc = api.load().rmi_row_normalize(C.byref(d), x.data_ptr(), o.data_ptr(), 1e-8,
+                                      dev.current_stream_ptr())
+    assert rc == 0
+    n = torch.linalg.vector_norm(o.view(rows, cols).double(), dim=1)
+    assert torch.allclose(n, torch.ones_like(n), atol=1e-6)
+    ns = 5000
+    sub = x[: ns * cols].cpu().numpy()
+    ds = api.make_desc(api.F32, api.F32, ns, cols, main_op=api.MAIN_SQ, final_op=api.FIN_SQRT)
+    exp = _oracle(ds, sub, np.zeros(ns * cols), 1e-8)
+    assert u.approx_ok(o[: ns * cols].cpu().numpy(), exp, 1e-5).all()

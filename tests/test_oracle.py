@@ -273,3 +273,25 @@ def test_typed_matches_sequential(oracle):
     d = api.make_desc(api.BF16, api.F32, 2, 100000)
     out = np.zeros(2, dtype=np.float32)
     assert u.fp_close(u.oracle_typed(d, xb, out), u.oracle_reduce(d, xb)).all()
+
+
+# row normalisation against numpy: x / ||x|| per row for the three norms, rows below
+# eps keep their previous contents (cpp/include/raft/linalg/detail/normalize.cuh:52-56)
+def test_row_normalize_against_numpy(oracle):
+    import ctypes as C
+    rng = np.random.default_rng(21)
+    rows, cols = 17, 29
+    m = rng.standard_normal((rows, cols))
+    m[5] = 0.0
+    cases = [(api.MAIN_ABS, api.RED_ADD, api.FIN_IDENTITY, np.abs(m).sum(axis=1)),
+             (api.MAIN_SQ, api.RED_ADD, api.FIN_SQRT, np.linalg.norm(m, axis=1)),
+             (api.MAIN_ABS, api.RED_MAX, api.FIN_IDENTITY, np.abs(m).max(axis=1))]
+    for main, red, fin, norms in cases:
+        d = api.make_desc(api.F64, api.F64, rows, cols, main_op=main, reduce_op=red, final_op=fin)
+        out = np.full(rows * cols, -1.0)
+        rc = oracle.orc_row_normalize(C.byref(d), m.ctypes.data, out.ctypes.data, 1e-8)
+        assert rc == 0
+        out = out.reshape(rows, cols)
+        want = np.where(norms[:, None] > 1e-8, m / np.where(norms > 0, norms, 1.0)[:, None], -1.0)
+        assert np.allclose(out, want, rtol=1e-14, atol=0)
+        assert (out[5] == -1.0).all()
