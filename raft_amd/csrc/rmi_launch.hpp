@@ -139,9 +139,11 @@ int run(const PlanX& pl, const Problem& pr, hipStream_t st)
 // ---- row normalisation -----------------------------------------------------------
 struct NormPlan {
   bool vec16   = false;
-  bool team    = false;
+  int kind     = 0;  // 0: lanes of a wave per row, 1: register-resident team, 2: two sweeps
   int G        = 1;
   int logG     = 0;
+  int L        = 4;  // wave kernel: lane-loads per lane and row
+  int hold     = 4;  // team kernel: lane-loads held per thread
   int threads  = kBlock;
   int64_t grid = 0;
   int64_t nvec = 0;
@@ -158,14 +160,27 @@ inline NormPlan make_norm_plan(int64_t n_rows, int64_t len, int elem_bytes)
   p.tail                  = (int)(len % step);
   const int64_t nload     = p.nvec + (p.tail > 0 ? 1 : 0);
   if (nload <= (int64_t)kUnroll * kWave) {
-    const int64_t g = ceildiv(nload, kUnroll);
-    p.G             = g >= 64 ? 64 : pow2ceil(g < 1 ? 1 : g);
-    p.logG          = ilog2(p.G);
-    p.grid          = ceildiv(n_rows, (int64_t)(kWave / p.G) * (kBlock / kWave));
+    // at least 8 lanes (128 contiguous bytes) per row and load instruction where the
+    // row is that long; shorter rows take one lane-load per lane and several rows
+    p.L    = nload <= 8 ? 1 : (nload <= 16 ? 2 : 4);
+    p.G    = pow2ceil(ceildiv(nload, p.L));
+    p.logG = ilog2(p.G);
+    p.grid = ceildiv(n_rows, (int64_t)(kWave / p.G) * (kUnroll / p.L) * (kBlock / kWave));
   } else {
-    p.team    = true;
-    p.threads = nload >= (int64_t)4 * 1024 * kUnroll ? 1024 : kBlock;
-    p.grid    = n_rows;
+    p.grid = n_rows;
+    if (nload <= 256 * 4) {
+      p.kind = 1, p.threads = 256, p.hold = 4;
+    } else if (nload <= 256 * 8) {
+      p.kind = 1, p.threads = 256, p.hold = 8;
+    } else if (nload <= 1024 * 4) {
+      p.kind = 1, p.threads = 1024, p.hold = 4;
+    } else if (nload <= 1024 * 8) {
+      p.kind = 1, p.threads = 1024, p.hold = 8;
+    } else if (nload <= 1024 * 16) {
+      p.kind = 1, p.threads = 1024, p.hold = 16;
+    } else {
+      p.kind = 2, p.threads = 1024;
+    }
   }
   return p;
 }
@@ -180,16 +195,25 @@ int run_normalize(const NormPlan& pl, const NormArgs& args, hipStream_t st)
   a.tail     = pl.tail;
   a.G        = pl.G;
   a.logG     = pl.logG;
+  a.L        = pl.L;
   if (pl.grid > 0x7fffffffLL) return RMI_ERR_BAD_SHAPE;
   const dim3 grid((unsigned)pl.grid);
-  if (!pl.team) {
+  if (pl.kind == 0) {
     if (pl.vec16)
       hipLaunchKernelGGL((normalize_wave_kernel<P, true>), grid, dim3(kBlock), 0, st, a);
     else
       hipLaunchKernelGGL((normalize_wave_kernel<P, false>), grid, dim3(kBlock), 0, st, a);
-  } else {
+  } else if (pl.kind == 1) {
     // rows of 4 KB and more always hold whole vectors
-    hipLaunchKernelGGL((normalize_team_kernel<P, true>), grid, dim3(pl.threads), 0, st, a);
+    const dim3 block((unsigned)pl.threads);
+    if (pl.hold == 4)
+      hipLaunchKernelGGL((normalize_team_kernel<P, 4>), grid, block, 0, st, a);
+    else if (pl.hold == 8)
+      hipLaunchKernelGGL((normalize_team_kernel<P, 8>), grid, block, 0, st, a);
+    else
+      hipLaunchKernelGGL((normalize_team_kernel<P, 16>), grid, block, 0, st, a);
+  } else {
+    hipLaunchKernelGGL((normalize_sweep_kernel<P>), grid, dim3(pl.threads), 0, st, a);
   }
   return hipGetLastError() == hipSuccess ? RMI_OK : RMI_ERR_LAUNCH;
 }

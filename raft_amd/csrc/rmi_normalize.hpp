@@ -20,7 +20,7 @@ struct NormArgs {
   int tail;    // elements after the last whole vector
   int G;       // lanes per row (wave kernel)
   int logG;
-  int logT;    // team kernel: 64 << logT threads per row
+  int L;       // wave kernel: lane-loads per lane and row (1, 2 or 4)
   int final_op;
   double init;
   double eps;
@@ -129,48 +129,123 @@ __device__ __forceinline__ void write_scaled(const NormArgs& a,
   }
 }
 
-// G lanes of one wave per row, at most kUnroll lane-loads per lane: the row stays in
-// registers from the reduction to the scaling.
+// G lanes of one wave per row, L lane-loads per lane and row, kUnroll / L rows per
+// lane group and step: kUnroll loads in flight per lane whatever the row length, and
+// the rows stay in registers from the reduction to the scaling.
+template <class P, bool VEC16, int L>
+__device__ __forceinline__ void normalize_wave_body(const NormArgs& a)
+{
+  using acc_t         = typename P::acc_t;
+  using H             = Held<P, VEC16>;
+  constexpr int TILES = kUnroll / L;
+  const int lane      = threadIdx.x & (kWave - 1);
+  const i64 wid       = (i64)blockIdx.x * (kBlock / kWave) + (threadIdx.x >> 6);
+  const int G         = a.G;
+  const int R         = kWave >> a.logG;
+  const int c         = lane & (G - 1);
+  const int g         = lane >> a.logG;
+  const i64 nload     = a.nvec + (a.tail > 0 ? 1 : 0);
+
+  typename H::type x[kUnroll];
+  i64 row[TILES];
+#pragma unroll
+  for (int t = 0; t < TILES; ++t) {
+    row[t] = (wid * TILES + t) * R + g;
+    if (row[t] < a.n_rows) {
+      const char* rp = static_cast<const char*>(a.in) + row[t] * a.row_bytes;
+#pragma unroll
+      for (int u = 0; u < L; ++u)
+        if (c + u * G < nload) x[t * L + u] = H::load_any(rp, c + u * G, a.nvec, a.len);
+    }
+  }
+  acc_t acc[TILES];
+#pragma unroll
+  for (int t = 0; t < TILES; ++t) {
+    acc[t] = P::neutral();
+    if (row[t] < a.n_rows) {
+#pragma unroll
+      for (int u = 0; u < L; ++u)
+        if (c + u * G < nload) H::push_any(acc[t], x[t * L + u], c + u * G, a.nvec, a.len, a.tail);
+    }
+  }
+#pragma unroll
+  for (int t = 0; t < TILES; ++t)
+    group_allreduce<P>(acc[t], G);
+#pragma unroll
+  for (int t = 0; t < TILES; ++t) {
+    if (row[t] < a.n_rows) {
+      const auto norm = row_norm<P>(a, acc[t]);
+      if (norm > (typename P::nat)a.eps) {  // false for NaN norms too
+        char* orow = static_cast<char*>(a.out) + row[t] * a.row_bytes;
+#pragma unroll
+        for (int u = 0; u < L; ++u)
+          if (c + u * G < nload) write_scaled<P, VEC16>(a, orow, x[t * L + u], c + u * G, norm);
+      }
+    }
+  }
+}
+
 template <class P, bool VEC16>
 __global__ __launch_bounds__(kBlock) void normalize_wave_kernel(NormArgs a)
 {
-  using acc_t    = typename P::acc_t;
-  using H        = Held<P, VEC16>;
-  const int lane = threadIdx.x & (kWave - 1);
-  const i64 wid  = (i64)blockIdx.x * (kBlock / kWave) + (threadIdx.x >> 6);
-  const int G    = a.G;
-  const int c    = lane & (G - 1);
-  const i64 row  = wid * (kWave >> a.logG) + (lane >> a.logG);
-  const i64 nload = a.nvec + (a.tail > 0 ? 1 : 0);
-  const bool live = row < a.n_rows;
-  const char* rp  = static_cast<const char*>(a.in) + row * a.row_bytes;
-
-  typename H::type x[kUnroll];
-  acc_t acc = P::neutral();
-  if (live) {
-#pragma unroll
-    for (int u = 0; u < kUnroll; ++u)
-      if (c + u * G < nload) x[u] = H::load_any(rp, c + u * G, a.nvec, a.len);
-#pragma unroll
-    for (int u = 0; u < kUnroll; ++u)
-      if (c + u * G < nload) H::push_any(acc, x[u], c + u * G, a.nvec, a.len, a.tail);
+  if (a.L == 1) {
+    normalize_wave_body<P, VEC16, 1>(a);
+  } else if (a.L == 2) {
+    normalize_wave_body<P, VEC16, 2>(a);
+  } else {
+    normalize_wave_body<P, VEC16, 4>(a);
   }
-  group_allreduce<P>(acc, G);
-  if (!live) return;
-  const auto norm = row_norm<P>(a, acc);
-  if (!(norm > (typename P::nat)a.eps)) return;  // also leaves NaN norms untouched
-  char* orow = static_cast<char*>(a.out) + row * a.row_bytes;
-#pragma unroll
-  for (int u = 0; u < kUnroll; ++u)
-    if (c + u * G < nload) write_scaled<P, VEC16>(a, orow, x[u], c + u * G, norm);
 }
 
-// One team of 64 << logT threads per row, two sweeps.
-template <class P, bool VEC16>
+// One team of blockDim.x threads per row; the row (at most UH lane-loads per thread)
+// stays in registers from the reduction to the scaling.
+template <class P, int UH>
 __global__ __launch_bounds__(1024) void normalize_team_kernel(NormArgs a)
 {
   using acc_t = typename P::acc_t;
-  using H     = Held<P, VEC16>;
+  using H     = Held<P, true>;
+  using nat   = typename P::nat;
+  __shared__ acc_t sm[16];
+  __shared__ nat sm_norm;
+
+  const int T     = blockDim.x;
+  const int t     = threadIdx.x;
+  const i64 row   = blockIdx.x;
+  const i64 nload = a.nvec + (a.tail > 0 ? 1 : 0);
+  const char* rp  = static_cast<const char*>(a.in) + row * a.row_bytes;
+
+  typename H::type x[UH];
+#pragma unroll
+  for (int u = 0; u < UH; ++u)
+    if (t + (i64)u * T < nload) x[u] = H::load_any(rp, t + (i64)u * T, a.nvec, a.len);
+  acc_t acc = P::neutral();
+#pragma unroll
+  for (int u = 0; u < UH; ++u)
+    if (t + (i64)u * T < nload) H::push_any(acc, x[u], t + (i64)u * T, a.nvec, a.len, a.tail);
+  wave_allreduce<P>(acc);
+  if ((t & (kWave - 1)) == 0) sm[t >> 6] = acc;
+  __syncthreads();
+  if (t == 0) {
+    for (int w = 1; w < (T >> 6); ++w)
+      P::merge(acc, sm[w]);
+    sm_norm = row_norm<P>(a, acc);
+  }
+  __syncthreads();
+  const nat norm = sm_norm;
+  if (!(norm > (nat)a.eps)) return;
+  char* orow = static_cast<char*>(a.out) + row * a.row_bytes;
+#pragma unroll
+  for (int u = 0; u < UH; ++u)
+    if (t + (i64)u * T < nload) write_scaled<P, true>(a, orow, x[u], t + (i64)u * T, norm);
+}
+
+// Rows too long for a team's registers: one team of 1024 threads sweeps the row
+// twice (the second sweep finds most of it in the caches).
+template <class P>
+__global__ __launch_bounds__(1024) void normalize_sweep_kernel(NormArgs a)
+{
+  using acc_t = typename P::acc_t;
+  using H     = Held<P, true>;
   using nat   = typename P::nat;
   __shared__ acc_t sm[16];
   __shared__ nat sm_norm;
@@ -210,7 +285,7 @@ __global__ __launch_bounds__(1024) void normalize_team_kernel(NormArgs a)
       if (v + (i64)u * T < nload) x[u] = H::load_any(rp, v + (i64)u * T, a.nvec, a.len);
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u)
-      if (v + (i64)u * T < nload) write_scaled<P, VEC16>(a, orow, x[u], v + (i64)u * T, norm);
+      if (v + (i64)u * T < nload) write_scaled<P, true>(a, orow, x[u], v + (i64)u * T, norm);
   }
 }
 

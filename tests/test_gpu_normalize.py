@@ -57,7 +57,8 @@ def test_reference_grid(gpu, dt, npdt, tol, norm, rows, cols):
     assert u.approx_ok(got, exp, tol).all(), u.worst_rel(got, exp)
 
 
-@pytest.mark.parametrize("rows,cols", [(37, 1024), (9, 5000), (5, 70001), (3, 1 << 18), (2000, 1000)])
+@pytest.mark.parametrize("rows,cols", [(37, 1024), (9, 5000), (5, 70001), (3, 1 << 18), (2000, 1000),
+                                       (21, 4001), (13, 16003), (7, 30000), (6, 60002), (40, 65536)])
 @pytest.mark.parametrize("norm", ["l1", "l2", "linf"])
 def test_long_rows(gpu, rows, cols, norm):
     rng = np.random.default_rng(cols)
