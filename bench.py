@@ -425,6 +425,35 @@ def main():
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) / 200 * 1e3
 
+    def extra_row_normalize():
+        # the step after config 2 in an embedding pipeline: x / ||x||_2 per row, same
+        # matrix shape; algorithmic bytes = matrix read once + written once
+        rows, cols = 1000000, 128
+        xs = [mk_normal(rows, cols, 2 + 7919 * i) for i in range(3)]
+        os_ = [torch.empty_like(x) for x in xs]
+        d = api.make_desc(api.F32, api.F32, rows, cols, main_op=api.MAIN_SQ, final_op=api.FIN_SQRT)
+        ref = C.byref(d)
+        call = lib.rmi_row_normalize
+        for i in range(5):
+            rc = call(ref, xs[i % 3].data_ptr(), os_[i % 3].data_ptr(), 1e-8, sptr)
+            assert rc == 0, api.status_string(rc)
+        torch.cuda.synchronize()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        n = max(10, args.steps // 4)
+        e0.record(stream)
+        for i in range(n):
+            call(ref, xs[i % 3].data_ptr(), os_[i % 3].data_ptr(), 1e-8, sptr)
+        e1.record(stream)
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / n
+        nb = 2 * rows * cols * 4
+        norms = torch.linalg.vector_norm(os_[0].view(rows, cols).double(), dim=1)
+        return dict(workload="row_normalize L2 fp32 1000000x128 (read + write)", ms_per_step=ms,
+                    alg_bytes=nb, GBps=nb / (ms * 1e-3) / 1e9,
+                    pct_of_peak=100.0 * nb / (ms * 1e-3) / 1e9 / PEAK_HBM_GBPS,
+                    check={"unit_rows": bool(torch.allclose(norms, torch.ones_like(norms), atol=1e-6))})
+
     results = {}
     cpu = {}
     for name in names:
@@ -459,6 +488,7 @@ def main():
                      "traffic": MEASURED_TRAFFIC.get(HEADLINE)},
         "cpu_baseline": cpu.get(HEADLINE),
         "launch_floor_us": launch_floor_us(),
+        "extras": {"row_normalize": extra_row_normalize()} if args.configs == "all" else {},
         "configs": results,
         "cpu_baselines": cpu,
         "device": torch.cuda.get_device_name(0),
