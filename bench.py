@@ -454,6 +454,41 @@ def main():
                     pct_of_peak=100.0 * nb / (ms * 1e-3) / 1e9 / PEAK_HBM_GBPS,
                     check={"unit_rows": bool(torch.allclose(norms, torch.ones_like(norms), atol=1e-6))})
 
+    def extra_meanvar():
+        # config 3's mean followed by stddev reads the matrix twice; meanvar gives the mean
+        # and the variance in one read of the same 10000000x64 matrix
+        rows, cols = 10000000, 64
+        xs = [mk_normal(rows, cols, 3 + 7919 * i) for i in range(3)]
+        mean = torch.empty(cols, dtype=torch.float32, device="cuda")
+        var = torch.empty(cols, dtype=torch.float32, device="cuda")
+        nws = lib.rmi_meanvar_workspace_bytes(api.F32, api.ROW_MAJOR, rows, cols)
+        ws = torch.empty(max(nws, 16), dtype=torch.uint8, device="cuda")
+
+        def call(i):
+            return lib.rmi_meanvar(api.F32, api.ROW_MAJOR, rows, cols, 1, xs[i % 3].data_ptr(),
+                                   mean.data_ptr(), var.data_ptr(), ws.data_ptr(), nws, sptr)
+        for i in range(5):
+            rc = call(i)
+            assert rc == 0, api.status_string(rc)
+        torch.cuda.synchronize()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        n = max(10, args.steps // 4)
+        e0.record(stream)
+        for i in range(n):
+            call(i)
+        e1.record(stream)
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / n
+        nb = rows * cols * 4
+        x = xs[(n - 1) % 3].view(rows, cols)
+        ok = bool(torch.allclose(mean.double(), x.double().mean(dim=0), rtol=1e-5, atol=1e-5) and
+                  torch.allclose(var.double(), x.double().var(dim=0, unbiased=True), rtol=1e-5))
+        return dict(workload="meanvar fp32 10000000x64 row-major (one read)", ms_per_step=ms,
+                    alg_bytes=nb, GBps=nb / (ms * 1e-3) / 1e9,
+                    pct_of_peak=100.0 * nb / (ms * 1e-3) / 1e9 / PEAK_HBM_GBPS,
+                    check={"torch_fp64": ok})
+
     results = {}
     cpu = {}
     for name in names:
@@ -488,7 +523,8 @@ def main():
                      "traffic": MEASURED_TRAFFIC.get(HEADLINE)},
         "cpu_baseline": cpu.get(HEADLINE),
         "launch_floor_us": launch_floor_us(),
-        "extras": {"row_normalize": extra_row_normalize()} if args.configs == "all" else {},
+        "extras": ({"row_normalize": extra_row_normalize(), "meanvar": extra_meanvar()}
+                   if args.configs == "all" else {}),
         "configs": results,
         "cpu_baselines": cpu,
         "device": torch.cuda.get_device_name(0),

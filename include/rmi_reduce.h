@@ -243,6 +243,27 @@ RMI_API int rmi_row_normalize(const rmi_reduce_desc* desc,
                               double eps,
                               void* stream);
 
+/* Mean and variance of every column of an [n_rows, n_cols] matrix in one pass over
+ * the data: mean[j] = sum_i x[i, j] / n_rows, var[j] = sum_i (x[i, j] - mean[j])^2 /
+ * max(1, sample ? n_rows - 1 : n_rows).  Replaces detail::meanvar
+ * (stats/detail/meanvar.cuh:187-236) behind raft::stats::meanvar
+ * (stats/meanvar.cuh:38-49 pointer form, :74-98 mdspan form).  `dtype` is F32 or F64
+ * (data, mean and var share it), `layout` an rmi_layout.  The arithmetic is f64
+ * throughout.  An empty column set is a no-op; n_rows == 0 writes zeros.  The workspace
+ * follows the rules of rmi_reduce. */
+RMI_API size_t rmi_meanvar_workspace_bytes(int dtype, int layout, int64_t n_rows, int64_t n_cols);
+RMI_API int rmi_meanvar(int dtype,
+                        int layout,
+                        int64_t n_rows,
+                        int64_t n_cols,
+                        int sample,
+                        const void* data,
+                        void* mean,
+                        void* var,
+                        void* workspace,
+                        size_t workspace_bytes,
+                        void* stream);
+
 #ifdef __cplusplus
 } /* extern "C" */
 #endif

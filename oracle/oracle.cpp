@@ -34,13 +34,15 @@
 //       include/raft/matrix/detail/math.cuh:292-352
 //   row normalisation: include/raft/linalg/detail/normalize.cuh:36-57,
 //       include/raft/linalg/normalize.cuh:91-107
+//   one-pass mean and variance: include/raft/stats/detail/meanvar.cuh:16-99
 //
 // Pinned by (tests/test_oracle.py): the closed-form fixtures of
 // tests/linalg/reduce.cu:108-177, tests/matrix/argmax.cu:71-75,
 // tests/matrix/argmin.cu:71-75, tests/util/reduction.cu:167-181,
 // tests/core/operators_host.cpp:134-172, tests/stats/sum.cu:50-98,
 // tests/stats/stddev.cu:139-150, tests/linalg/map_then_reduce.cu:140-169, and
-// by numpy closed forms on random inputs.  The summation ORDER of the
+// by numpy closed forms on random inputs (orc_meanvar: numpy's two-pass mean / var
+// and the statistical tolerances of tests/stats/meanvar.cu:27-33).  The summation ORDER of the
 // reference's device kernels (CUB block reductions, float atomics) is not
 // recoverable from its sources and is not pinned by its own tests either; both
 // implementations here fix an order of their own.
@@ -729,6 +731,43 @@ ORC_API int orc_row_normalize(const rmi_reduce_desc* d, const void* in, double* 
     case RMI_BF16: return normalize_seq(*d, (const bf16*)in, out, eps);
     case RMI_F32: return normalize_seq(*d, (const float*)in, out, eps);
     case RMI_F64: return normalize_seq(*d, (const double*)in, out, eps);
+    default: return RMI_ERR_UNSUPPORTED;
+  }
+}
+
+// Mean and variance of every column in one pass, fp64: the reference's mean_var
+// monoid (cpp/include/raft/stats/detail/meanvar.cuh:16-99) applied element by element
+// in row order.  Merging a state {w, m, s} with the singleton {1, x, 0} by its
+// operator+= (:60-74): cw = w + 1; d = m - x; s += cw * (d * w/cw) * (d * 1/cw);
+// m = m * w/cw + x * 1/cw.  var = s / max(1, sample ? w - 1 : w) (:88-98).
+template <class T>
+static int meanvar_seq(int layout, int64_t n_rows, int64_t n_cols, int sample, const T* in,
+                       double* mean, double* var)
+{
+  for (int64_t j = 0; j < n_cols; ++j) {
+    double w = 0.0, m = 0.0, s = 0.0;
+    for (int64_t i = 0; i < n_rows; ++i) {
+      const double x  = (double)(layout == RMI_ROW_MAJOR ? in[i * n_cols + j] : in[j * n_rows + i]);
+      const double cw = w + 1.0;
+      const double fa = w / cw, fb = 1.0 / cw;
+      const double d  = m - x;
+      s += cw * (d * fa) * (d * fb);
+      m = m * fa + x * fb;
+      w = cw;
+    }
+    mean[j] = m;
+    var[j]  = s / std::max(1.0, sample ? w - 1.0 : w);
+  }
+  return RMI_OK;
+}
+
+ORC_API int orc_meanvar(int dtype, int layout, int64_t n_rows, int64_t n_cols, int sample,
+                        const void* in, double* mean, double* var)
+{
+  if (layout != RMI_ROW_MAJOR && layout != RMI_COL_MAJOR) return RMI_ERR_BAD_ENUM;
+  switch (dtype) {
+    case RMI_F32: return meanvar_seq(layout, n_rows, n_cols, sample, (const float*)in, mean, var);
+    case RMI_F64: return meanvar_seq(layout, n_rows, n_cols, sample, (const double*)in, mean, var);
     default: return RMI_ERR_UNSUPPORTED;
   }
 }

@@ -79,6 +79,9 @@ SYMBOLS = {
                                     C.c_void_p]),
     "rmi_map_reduce": (C.c_int, [C.POINTER(ReduceDesc), C.c_int64, C.c_void_p, C.c_void_p,
                                  C.c_void_p, C.c_size_t, C.c_void_p]),
+    "rmi_meanvar_workspace_bytes": (C.c_size_t, [C.c_int, C.c_int, C.c_int64, C.c_int64]),
+    "rmi_meanvar": (C.c_int, [C.c_int, C.c_int, C.c_int64, C.c_int64, C.c_int, C.c_void_p,
+                              C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
 }
 
 _lib = None

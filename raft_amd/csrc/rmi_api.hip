@@ -119,6 +119,29 @@ rmi_reduce_desc as_single_row(const rmi_reduce_desc& d, int64_t len)
   return r;
 }
 
+// meanvar: one output pair per column, whatever the layout.
+int meanvar_plan(int dtype, int layout, int64_t n_rows, int64_t n_cols, PlanX& pl, run_fn& fn)
+{
+  if (dtype < 0 || dtype >= RMI_DTYPE_COUNT_) return RMI_ERR_BAD_ENUM;
+  if (layout != RMI_ROW_MAJOR && layout != RMI_COL_MAJOR) return RMI_ERR_BAD_ENUM;
+  if (n_rows < 0 || n_cols < 0) return RMI_ERR_BAD_SHAPE;
+  if (dtype == RMI_F32) fn = lookup_meanvar_f32();
+  else if (dtype == RMI_F64) fn = lookup_meanvar_f64();
+  else return RMI_ERR_UNSUPPORTED;
+  rmi_reduce_desc d{};
+  d.in_dtype  = dtype;
+  d.out_dtype = dtype;
+  d.layout    = layout;
+  d.apply     = RMI_ALONG_COLUMNS;
+  d.n_rows    = n_rows;
+  d.n_cols    = n_cols;
+  d.plan_hint = RMI_PLAN_AUTO;
+  PolicyKey key;
+  key.in_dtype = dtype;
+  key.family   = kFamMeanVar;
+  return make_plan(d, key, (int)sizeof(mv_t), cu_count(), pl);
+}
+
 }  // namespace
 }  // namespace rmi
 
@@ -231,6 +254,50 @@ int rmi_row_normalize(const rmi_reduce_desc* desc,
   a.init      = d.init.f;
   a.eps       = eps;
   return fn(pl, a, static_cast<hipStream_t>(stream));
+}
+
+size_t rmi_meanvar_workspace_bytes(int dtype, int layout, int64_t n_rows, int64_t n_cols)
+{
+  rmi::PlanX pl;
+  rmi::run_fn fn = nullptr;
+  if (rmi::meanvar_plan(dtype, layout, n_rows, n_cols, pl, fn) != RMI_OK) return 0;
+  return pl.ws_bytes;
+}
+
+int rmi_meanvar(int dtype,
+                int layout,
+                int64_t n_rows,
+                int64_t n_cols,
+                int sample,
+                const void* data,
+                void* mean,
+                void* var,
+                void* workspace,
+                size_t workspace_bytes,
+                void* stream)
+{
+  using namespace rmi;
+  PlanX pl;
+  run_fn fn    = nullptr;
+  const int rc = meanvar_plan(dtype, layout, n_rows, n_cols, pl, fn);
+  if (rc != RMI_OK) return rc;
+  if (pl.n_out == 0) return RMI_OK;
+  if (mean == nullptr || var == nullptr) return RMI_ERR_NULL;
+  if (pl.len > 0 && data == nullptr) return RMI_ERR_NULL;
+  const int es = dtype_size(dtype);
+  if (!aligned(data, es) || !aligned(mean, es) || !aligned(var, es)) return RMI_ERR_ALIGNMENT;
+  if (pl.ws_bytes > 0) {
+    if (workspace == nullptr || workspace_bytes < pl.ws_bytes) return RMI_ERR_WORKSPACE;
+    if (!aligned(workspace, 16)) return RMI_ERR_WORKSPACE;
+  }
+  Problem pr{};
+  pr.in            = data;
+  pr.ws            = workspace;
+  pr.epi.out       = mean;
+  pr.epi.aux       = var;
+  pr.epi.s1        = sample ? 1.0 : 0.0;
+  pr.epi.out_dtype = dtype;
+  return fn(pl, pr, static_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"

@@ -223,9 +223,11 @@ __device__ __forceinline__ T xchg(T v)
 //   merge(acc, other)              acc = reduce_op(acc, other)
 //   exchange<SEL>(acc)             acc of the partner lane
 //   from_scalar(f, i), from_out(p, dtype, k), result/store: see Epilogue.
-// merge must be exactly commutative (bitwise), which the butterfly relies on.
+// merge must be exactly commutative (bitwise) for results to be independent of the
+// lane a result is read from (PolMeanVar is commutative up to rounding only: its
+// results are valid from any lane but not bitwise equal across lanes).
 
-enum : int { kClsFloat = 0, kClsInt = 1, kClsKvp = 2 };
+enum : int { kClsFloat = 0, kClsInt = 1, kClsKvp = 2, kClsMeanVar = 3 };
 
 template <int MAIN>
 __device__ __forceinline__ double main_f64(double d)
@@ -526,6 +528,75 @@ struct PolKvp {
   }
 };
 
+// ---- mean and variance in one pass ---------------------------------------------
+// State of a set of w values: their mean is k + sd / w and their sum of squared
+// deviations from the mean is sdd - sd * sd / w, where sd and sdd are the sums of
+// (x - k) and (x - k)^2 and the shift k is the first value the lane saw.  With the
+// shift inside the data's range the subtraction loses a few bits at most, and an
+// element costs three f64 operations and no division.  Two states merge by the
+// pairwise update of Chan et al. that the reference's mean_var monoid uses
+// (stats/detail/meanvar.cuh:16-99); the merged state is stored with k = mean, sd = 0.
+struct mv_t {
+  double w;
+  double k;
+  double sd;
+  double sdd;
+};
+
+__device__ __forceinline__ double mv_mean(const mv_t& a)
+{
+  return a.w > 0.0 ? a.k + a.sd / a.w : 0.0;
+}
+__device__ __forceinline__ double mv_m2(const mv_t& a)
+{
+  return a.w > 0.0 ? fmax(a.sdd - a.sd * a.sd / a.w, 0.0) : 0.0;
+}
+
+template <class InT>
+struct PolMeanVar {
+  using in_t               = InT;
+  using nat                = typename In<InT>::nat;
+  using acc_t              = mv_t;
+  static constexpr int VEC = In<InT>::VEC;
+  static constexpr int CLS = kClsMeanVar;
+
+  static __device__ __forceinline__ acc_t neutral() { return mv_t{0.0, 0.0, 0.0, 0.0}; }
+  static __device__ __forceinline__ void push(acc_t& a, nat x, i64)
+  {
+    const double xd = (double)x;
+    a.k             = a.w == 0.0 ? xd : a.k;
+    const double d  = xd - a.k;
+    a.sd += d;
+    a.sdd = fma(d, d, a.sdd);
+    a.w += 1.0;
+  }
+  static __device__ __forceinline__ void push_vec(acc_t& a, const u32x4& v, i64)
+  {
+    static_for<VEC>([&](auto j) { push(a, In<InT>::template get<j>(v), 0); });
+  }
+  static __device__ __forceinline__ void push_cols(acc_t (&a)[VEC], const u32x4& v, i64)
+  {
+    static_for<VEC>([&](auto j) { push(a[j], In<InT>::template get<j>(v), 0); });
+  }
+  static __device__ __forceinline__ void merge(acc_t& a, const acc_t& b)
+  {
+    const double cw = a.w + b.w;
+    const double ma = mv_mean(a), mb = mv_mean(b);
+    const double sa = mv_m2(a), sb = mv_m2(b);
+    const double fb = cw > 0.0 ? b.w / cw : 0.0;
+    const double d  = mb - ma;
+    a.k             = ma + d * fb;
+    a.sdd           = (sa + sb) + d * d * (a.w * fb);
+    a.sd            = 0.0;
+    a.w             = cw;
+  }
+  template <int SEL>
+  static __device__ __forceinline__ acc_t exchange(const acc_t& a)
+  {
+    return mv_t{xchg<SEL>(a.w), xchg<SEL>(a.k), xchg<SEL>(a.sd), xchg<SEL>(a.sdd)};
+  }
+};
+
 // ---------------------------------------------------------------------------
 // The last, overlapping vector of a row whose length is not a multiple of VEC:
 // it ends exactly at the row's end, so its first `skip` elements were already
@@ -748,6 +819,20 @@ __device__ __forceinline__ void finish(const Epilogue& e, i64 k, typename P::acc
       a = o;
     }
     store_int(e, k, a);
+  } else if constexpr (P::CLS == kClsMeanVar) {
+    // out: means, aux: variances (written here), s1: 1 for the sample variance.
+    // stats/detail/meanvar.cuh:88-98: var = M2 / max(1, sample ? w - 1 : w)
+    const double mean = mv_mean(acc);
+    const double den  = fmax(1.0, e.s1 != 0.0 ? acc.w - 1.0 : acc.w);
+    const double var  = mv_m2(acc) / den;
+    void* vp          = const_cast<void*>(e.aux);
+    if (e.out_dtype == RMI_F64) {
+      static_cast<double*>(e.out)[k] = mean;
+      static_cast<double*>(vp)[k]    = var;
+    } else {
+      static_cast<float*>(e.out)[k] = (float)mean;
+      static_cast<float*>(vp)[k]    = (float)var;
+    }
   } else {
     using key_t = decltype(acc.key);
     using val_t = decltype(acc.value);

@@ -86,7 +86,7 @@ inline bool is_int_dtype(int dt)
 inline bool is_kvp_dtype(int dt) { return dt >= RMI_KVP_I32_F32 && dt <= RMI_KVP_I64_F64; }
 
 // Which accumulator family serves a descriptor.
-enum : int { kFamFloat = 0, kFamKbn = 1, kFamInt = 2, kFamKvp = 3 };
+enum : int { kFamFloat = 0, kFamKbn = 1, kFamInt = 2, kFamKvp = 3, kFamMeanVar = 4 };
 
 struct PolicyKey {
   int in_dtype = 0;

@@ -54,3 +54,16 @@ def map_reduce(desc: api.ReduceDesc, length: int, inp: torch.Tensor, out: torch.
                             ws.data_ptr(), n, current_stream_ptr())
     if rc != api.OK:
         raise RmiError(rc, "rmi_map_reduce")
+
+
+def meanvar(dtype: int, layout: int, n_rows: int, n_cols: int, sample: bool,
+            data: torch.Tensor, mean: torch.Tensor, var: torch.Tensor) -> None:
+    """Run rmi_meanvar on the current torch stream."""
+    lib = api.load()
+    n = lib.rmi_meanvar_workspace_bytes(dtype, layout, n_rows, n_cols)
+    ws = torch.empty(n, dtype=torch.uint8, device=data.device) if n else None
+    rc = lib.rmi_meanvar(dtype, layout, n_rows, n_cols, 1 if sample else 0, data.data_ptr(),
+                         mean.data_ptr(), var.data_ptr(), ws.data_ptr() if n else None, n,
+                         current_stream_ptr())
+    if rc != api.OK:
+        raise RmiError(rc, "rmi_meanvar")

@@ -19,6 +19,7 @@
 #include <raft/matrix/argmax.cuh>
 #include <raft/matrix/argmin.cuh>
 #include <raft/stats/mean.cuh>
+#include <raft/stats/meanvar.cuh>
 #include <raft/stats/stddev.cuh>
 #include <raft/stats/sum.cuh>
 #include <raft/util/cudart_utils.hpp>
@@ -417,6 +418,97 @@ void mean_stddev(double tol)
     }
 }
 
+// ---------------------------------------------------------------------------
+// cpp/tests/stats/meanvar.cu:20-150: normal data, both layouts, sample and population
+// variance, checked by the reference's statistical bounds (mean_tol, var_tol with
+// N_SIGMAS = 6) and against a two-pass fp64 evaluation
+// ---------------------------------------------------------------------------
+template <typename T>
+void meanvar_cases(double tol)
+{
+  raft::resources handle;
+  auto stream = raft::resource::get_cuda_stream(handle);
+  struct Case { double mean, stddev; int rows, cols; bool sample, row_major; };
+  std::vector<Case> cases;
+  for (bool rm : {false, true})
+    for (int cols : {32, 64, 128, 256, 257}) {
+      cases.push_back({1.0, 2.0, 1024, cols, true, rm});
+      cases.push_back({-1.0, 2.0, 1024, cols, false, rm});
+    }
+  cases.push_back({-1.0, 2.0, 700, 13, false, true});
+  cases.push_back({10.0, 2.0, 50000, 811, false, true});
+  cases.push_back({3.0, 1.0, 1, 9, true, true});
+  for (const auto& c : cases) {
+    const size_t n = (size_t)c.rows * c.cols;
+    auto data_h    = normal<T>(n, c.mean, c.stddev, 1234);
+    auto data_d    = raft::make_device_vector<T, int>(handle, (int)n);
+    raft::update_device(data_d.data_handle(), data_h.data(), n, stream);
+    auto mean = raft::make_device_vector<T, int>(handle, c.cols);
+    auto var  = raft::make_device_vector<T, int>(handle, c.cols);
+    if (c.row_major) {
+      raft::stats::meanvar(handle,
+                           raft::make_device_matrix_view<const T, int, raft::row_major>(
+                             data_d.data_handle(), c.rows, c.cols),
+                           mean.view(), var.view(), c.sample);
+    } else {
+      raft::stats::meanvar(handle,
+                           raft::make_device_matrix_view<const T, int, raft::col_major>(
+                             data_d.data_handle(), c.rows, c.cols),
+                           mean.view(), var.view(), c.sample);
+    }
+    auto mean_h = to_host(mean.data_handle(), (size_t)c.cols, stream);
+    auto var_h  = to_host(var.data_handle(), (size_t)c.cols, stream);
+    std::vector<double> want_m(c.cols), want_v(c.cols);
+    for (int j = 0; j < c.cols; ++j) {
+      double s = 0;
+      for (int i = 0; i < c.rows; ++i)
+        s += (double)data_h[at(c.row_major, c.rows, c.cols, i, j)];
+      const double m = s / c.rows;
+      double ss      = 0;
+      for (int i = 0; i < c.rows; ++i) {
+        const double d = (double)data_h[at(c.row_major, c.rows, c.cols, i, j)] - m;
+        ss += d * d;
+      }
+      want_m[j] = m;
+      want_v[j] = ss / std::max(1, c.sample ? c.rows - 1 : c.rows);
+    }
+    CHECK(all_close(mean_h, want_m, tol));
+    CHECK(all_close(var_h, want_v, tol));
+    if (c.rows > 1) {
+      const double mean_tol = 6.0 * c.stddev / std::sqrt((double)c.rows);
+      const double var_tol =
+        6.0 * c.stddev * c.stddev * std::sqrt(2.0 / std::max(1, c.rows - 1));
+      bool ok = true;
+      for (int j = 0; j < c.cols; ++j) {
+        ok &= std::fabs((double)mean_h[j] - c.mean) <= mean_tol;
+        ok &= std::fabs((double)var_h[j] - c.stddev * c.stddev) <= var_tol;
+      }
+      CHECK(ok);
+    }
+    // the pointer form gives the same results
+    auto mean2 = raft::make_device_vector<T, int>(handle, c.cols);
+    auto var2  = raft::make_device_vector<T, int>(handle, c.cols);
+    raft::stats::meanvar(mean2.data_handle(), var2.data_handle(), data_d.data_handle(), c.cols,
+                         c.rows, c.sample, c.row_major, stream);
+    CHECK(to_host(mean2.data_handle(), (size_t)c.cols, stream) == mean_h);
+    CHECK(to_host(var2.data_handle(), (size_t)c.cols, stream) == var_h);
+  }
+  // size mismatch between data and var is rejected (stats/meanvar.cuh:84)
+  auto data = raft::make_device_matrix<T, int, raft::row_major>(handle, 4, 5);
+  auto m5   = raft::make_device_vector<T, int>(handle, 5);
+  auto v4   = raft::make_device_vector<T, int>(handle, 4);
+  bool threw = false;
+  try {
+    raft::stats::meanvar(handle,
+                         raft::make_device_matrix_view<const T, int, raft::row_major>(
+                           data.data_handle(), 4, 5),
+                         m5.view(), v4.view(), false);
+  } catch (const raft::logic_error&) {
+    threw = true;
+  }
+  CHECK(threw);
+}
+
 // cpp/tests/stats/mean.cu:177-185: int8 -> half
 void mean_int8_to_half()
 {
@@ -633,6 +725,8 @@ TEST_CASE(NormF) { norms<float, float>(1e-5); }
 TEST_CASE(NormD) { norms<double, double>(1e-9); }
 TEST_CASE(MeanStddevF) { mean_stddev<float>(1e-5); }
 TEST_CASE(MeanStddevD) { mean_stddev<double>(1e-9); }
+TEST_CASE(MeanVarF) { meanvar_cases<float>(1e-5); }
+TEST_CASE(MeanVarD) { meanvar_cases<double>(1e-9); }
 TEST_CASE(MeanInt8ToHalf) { mean_int8_to_half(); }
 TEST_CASE(SumAccuracyF) { sum_accuracy<float>(0.0001f, 1e7, 0.001); }
 TEST_CASE(SumAccuracyD) { sum_accuracy<double>(0.000001, 1e12, 0.0001); }

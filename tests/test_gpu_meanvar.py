@@ -1,0 +1,139 @@
+"""One-pass mean and variance (rmi_meanvar) on the GPU against the fp64 oracle: the
+parameter grid of the reference's test (cpp/tests/stats/meanvar.cu:89-124) with its
+statistical tolerances, both layouts, ragged shapes, shifted data, empty inputs."""
+import numpy as np
+import pytest
+
+from raft_amd import _capi as api
+from tests import _util as u
+
+pytestmark = pytest.mark.gpu
+
+NP = {api.F32: np.float32, api.F64: np.float64}
+
+
+def _oracle(dt, layout, rows, cols, sample, stored):
+    mean = np.zeros(cols)
+    var = np.zeros(cols)
+    rc = u.load_oracle().orc_meanvar(dt, layout, rows, cols, int(sample), stored.ctypes.data,
+                                     mean.ctypes.data, var.ctypes.data)
+    assert rc == 0
+    return mean, var
+
+
+def _gpu(dt, layout, rows, cols, sample, stored):
+    import torch
+    from raft_amd import device as dev
+    x = torch.from_numpy(stored.reshape(-1)).cuda()
+    tdt = torch.float32 if dt == api.F32 else torch.float64
+    mean = torch.full((max(cols, 1),), 77.0, dtype=tdt, device="cuda")
+    var = torch.full((max(cols, 1),), 77.0, dtype=tdt, device="cuda")
+    dev.meanvar(dt, layout, rows, cols, sample, x, mean, var)
+    torch.cuda.synchronize()
+    return mean.cpu().numpy()[:cols], var.cpu().numpy()[:cols]
+
+
+def _make(rng, dt, layout, rows, cols, mu, sd):
+    m = rng.normal(mu, sd, (rows, cols)).astype(NP[dt])
+    return np.ascontiguousarray(m if layout == api.ROW_MAJOR else m.T)
+
+
+def _check(dt, layout, rows, cols, sample, stored, tol=1e-5):
+    got_m, got_v = _gpu(dt, layout, rows, cols, sample, stored)
+    exp_m, exp_v = _oracle(dt, layout, rows, cols, sample, stored)
+    assert u.fp_close(got_m, exp_m, tol).all(), u.worst_rel(got_m, exp_m)
+    assert u.fp_close(got_v, exp_v, tol).all(), u.worst_rel(got_v, exp_v)
+    return got_m, got_v
+
+
+# (mean, stddev, rows, cols, sample, row_major): cpp/tests/stats/meanvar.cu:89-124
+REF_F = [(1.0, 2.0, 1024, c, True, False) for c in (32, 64, 128, 256)] + \
+        [(-1.0, 2.0, 1024, c, False, False) for c in (32, 64, 128, 256, 257)] + \
+        [(1.0, 2.0, 1024, c, True, True) for c in (32, 64, 128, 256)] + \
+        [(-1.0, 2.0, 1024, c, False, True) for c in (32, 64, 128, 256, 257)] + \
+        [(-1.0, 2.0, 700, 13, False, True)]
+REF_D = [(1.0, 2.0, 1024, c, True, rm) for rm in (False, True) for c in (32, 64, 128, 256)] + \
+        [(-1.0, 2.0, 1024, c, False, rm) for rm in (False, True) for c in (32, 64, 128, 256)]
+
+
+@pytest.mark.parametrize("dt,case", [(api.F32, c) for c in REF_F] + [(api.F64, c) for c in REF_D])
+def test_reference_grid(gpu, dt, case):
+    mu, sd, rows, cols, sample, row_major = case
+    layout = api.ROW_MAJOR if row_major else api.COL_MAJOR
+    stored = _make(np.random.default_rng(1234), dt, layout, rows, cols, mu, sd)
+    got_m, got_v = _check(dt, layout, rows, cols, sample, stored)
+    # the reference's own acceptance bounds on normal data
+    assert np.all(np.abs(got_m - mu) <= 6 * sd / np.sqrt(rows))
+    assert np.all(np.abs(got_v - sd * sd) <= 6 * sd * sd * np.sqrt(2.0 / max(1, rows - 1)))
+
+
+@pytest.mark.parametrize("dt", [api.F32, api.F64])
+@pytest.mark.parametrize("layout", [api.ROW_MAJOR, api.COL_MAJOR])
+@pytest.mark.parametrize("rows,cols", [(1, 1), (1, 7), (2, 3), (3, 1), (5, 2), (17, 5), (64, 3),
+                                       (100, 33), (1000, 1), (4097, 19), (333, 1023),
+                                       (20000, 6), (7, 4099), (300000, 4), (3, 100000),
+                                       (150001, 37)])
+def test_ragged_shapes(gpu, dt, layout, rows, cols):
+    stored = _make(np.random.default_rng(rows * 31 + cols), dt, layout, rows, cols, 3.0, 2.0)
+    for sample in (False, True):
+        _check(dt, layout, rows, cols, sample, stored)
+
+
+@pytest.mark.parametrize("layout", [api.ROW_MAJOR, api.COL_MAJOR])
+def test_shifted_data(gpu, layout):
+    """A mean far above the spread: sums of raw squares would cancel, the shifted sums
+    and the pairwise merge do not."""
+    rows, cols = 50000, 24
+    stored = _make(np.random.default_rng(7), api.F64, layout, rows, cols, 1e6, 1e-2)
+    _check(api.F64, layout, rows, cols, True, stored, tol=1e-7)
+    stored = _make(np.random.default_rng(8), api.F32, layout, rows, cols, 1e3, 1.0)
+    _check(api.F32, layout, rows, cols, True, stored)
+
+
+def test_constant_columns(gpu):
+    rows, cols = 10000, 40
+    stored = np.full((rows, cols), 3.25, dtype=np.float32)
+    got_m, got_v = _gpu(api.F32, api.ROW_MAJOR, rows, cols, True, stored)
+    assert np.all(got_m == 3.25) and np.all(got_v == 0.0)
+
+
+@pytest.mark.parametrize("layout", [api.ROW_MAJOR, api.COL_MAJOR])
+def test_empty(gpu, layout):
+    # no columns: nothing is written; no rows: zeros
+    got_m, got_v = _gpu(api.F32, layout, 5, 0, False, np.zeros(1, dtype=np.float32))
+    assert got_m.size == 0 and got_v.size == 0
+    got_m, got_v = _gpu(api.F32, layout, 0, 6, True, np.zeros(1, dtype=np.float32))
+    assert np.all(got_m == 0) and np.all(got_v == 0)
+
+
+def test_reference_large_case(gpu):
+    """{10, 2, 500000 x 811, population variance, row-major}
+    (cpp/tests/stats/meanvar.cu:109), checked against the oracle on a column sample and by
+    the reference's statistical bound on every column."""
+    import torch
+    from raft_amd import device as dev
+    rows, cols, mu, sd = 500000, 811, 10.0, 2.0
+    g = torch.Generator(device="cuda").manual_seed(1234)
+    x = torch.empty((rows, cols), dtype=torch.float32, device="cuda").normal_(mu, sd, generator=g)
+    mean = torch.empty(cols, dtype=torch.float32, device="cuda")
+    var = torch.empty(cols, dtype=torch.float32, device="cuda")
+    dev.meanvar(api.F32, api.ROW_MAJOR, rows, cols, False, x, mean, var)
+    torch.cuda.synchronize()
+    got_m, got_v = mean.cpu().numpy(), var.cpu().numpy()
+    assert np.all(np.abs(got_m - mu) <= 6 * sd / np.sqrt(rows))
+    assert np.all(np.abs(got_v - sd * sd) <= 6 * sd * sd * np.sqrt(2.0 / (rows - 1)))
+    pick = [0, 1, 405, 809, 810]
+    sub = np.ascontiguousarray(x[:, pick].cpu().numpy())
+    exp_m, exp_v = _oracle(api.F32, api.ROW_MAJOR, rows, len(pick), False, sub)
+    assert u.fp_close(got_m[pick], exp_m).all() and u.fp_close(got_v[pick], exp_v).all()
+
+
+def test_validation(gpu):
+    lib = api.load()
+    assert lib.rmi_meanvar(api.F16, api.ROW_MAJOR, 4, 4, 0, None, None, None, None, 0, None) \
+        == api.ERR_UNSUPPORTED
+    assert lib.rmi_meanvar(api.F32, 9, 4, 4, 0, None, None, None, None, 0, None) == api.ERR_BAD_ENUM
+    assert lib.rmi_meanvar(api.F32, api.ROW_MAJOR, -1, 4, 0, None, None, None, None, 0, None) \
+        == api.ERR_BAD_SHAPE
+    assert lib.rmi_meanvar(api.F32, api.ROW_MAJOR, 4, 4, 0, None, None, None, None, 0, None) \
+        == api.ERR_NULL

@@ -295,3 +295,32 @@ def test_row_normalize_against_numpy(oracle):
         want = np.where(norms[:, None] > 1e-8, m / np.where(norms > 0, norms, 1.0)[:, None], -1.0)
         assert np.allclose(out, want, rtol=1e-14, atol=0)
         assert (out[5] == -1.0).all()
+
+
+# ---- one-pass mean and variance -------------------------------------------------------
+# orc_meanvar restates the reference's running merge; numpy's two-pass mean / var fix
+# what it must produce.  A wrong merge weight, a missing cross term or N instead of N-1
+# each fail the 1e-12 bar; the reference's own statistical bound on normal data
+# (cpp/tests/stats/meanvar.cu:27-33,127-150) is checked beside it.
+@pytest.mark.parametrize("npdt,dt", [(np.float32, api.F32), (np.float64, api.F64)])
+@pytest.mark.parametrize("layout", [api.ROW_MAJOR, api.COL_MAJOR])
+@pytest.mark.parametrize("sample", [False, True])
+def test_meanvar_against_numpy(oracle, npdt, dt, layout, sample):
+    rng = np.random.default_rng(1234)
+    for rows, cols, mu, sd in [(1024, 32, 1.0, 2.0), (700, 13, -1.0, 2.0), (1, 5, 3.0, 1.0),
+                               (2, 3, 1e4, 1e-2), (257, 1, 0.0, 1.0)]:
+        m = rng.normal(mu, sd, (rows, cols)).astype(npdt)
+        stored = np.ascontiguousarray(m if layout == api.ROW_MAJOR else m.T)
+        mean = np.zeros(cols)
+        var = np.zeros(cols)
+        rc = oracle.orc_meanvar(dt, layout, rows, cols, int(sample), stored.ctypes.data,
+                                mean.ctypes.data, var.ctypes.data)
+        assert rc == 0
+        m64 = m.astype(np.float64)
+        exp_mean = m64.mean(axis=0)
+        exp_var = m64.var(axis=0, ddof=1 if sample and rows > 1 else 0)
+        np.testing.assert_allclose(mean, exp_mean, rtol=1e-12, atol=1e-12)
+        np.testing.assert_allclose(var, exp_var, rtol=1e-9, atol=1e-12)
+        if rows >= 700 and sd == 2.0:
+            assert np.all(np.abs(mean - mu) <= 6 * sd / np.sqrt(rows))
+            assert np.all(np.abs(var - sd * sd) <= 6 * sd * sd * np.sqrt(2.0 / (rows - 1)))
