@@ -1,0 +1,302 @@
+// Benchmarks of the reduction primitives over the shape grids of the reference's own
+// benchmark programs, timed the way its fixture times them: before every timed call a
+// scratch buffer is overwritten to evict the caches, then one call is bracketed by two
+// events on the stream (cpp/bench/prims/common/benchmark.hpp:59-158).  Grids:
+//   reduce            cpp/bench/prims/linalg/reduce.cu:44-55
+//   rowNorm           cpp/bench/prims/linalg/norm.cu:57-69
+//   rowNormalize      cpp/bench/prims/linalg/normalize.cu:57-69
+//   map_then_reduce   cpp/bench/prims/linalg/map_then_reduce.cu:41-56
+//   Argmin            cpp/bench/prims/matrix/argmin.cu:55-60
+// One line per case: name, shape, mean time per call, algorithmic GB/s.
+//
+// usage: prims_bench [--filter substring] [--min-iters N] [--max-bytes B] [--no-flush]
+#include <raft/core/device_mdarray.hpp>
+#include <raft/core/device_mdspan.hpp>
+#include <raft/core/resources.hpp>
+#include <raft/linalg/map_then_reduce.cuh>
+#include <raft/linalg/norm.cuh>
+#include <raft/linalg/normalize.cuh>
+#include <raft/linalg/reduce.cuh>
+#include <raft/matrix/argmin.cuh>
+#include <raft/util/cudart_utils.hpp>
+
+#include <algorithm>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <string>
+#include <vector>
+
+namespace {
+
+// uniform values in [lo, hi) from a counter hash: cheap, reproducible, no state
+template <typename T>
+__global__ void fill_uniform(T* p, size_t n, double lo, double hi, unsigned long long seed)
+{
+  size_t i            = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (; i < n; i += stride) {
+    unsigned long long z = (i + seed) * 0x9E3779B97F4A7C15ull;
+    z ^= z >> 30;
+    z *= 0xBF58476D1CE4E5B9ull;
+    z ^= z >> 27;
+    z *= 0x94D049BB133111EBull;
+    z ^= z >> 31;
+    const double u = (double)(z >> 11) * (1.0 / 9007199254740992.0);
+    p[i]           = (T)(lo + (hi - lo) * u);
+  }
+}
+
+__global__ void fill_words(unsigned* p, size_t n, unsigned v)
+{
+  size_t i            = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (; i < n; i += stride)
+    p[i] = v;
+}
+
+struct Options {
+  std::string filter;
+  int min_iters    = 10;
+  size_t max_bytes = (size_t)96 << 30;
+  bool flush       = true;
+};
+
+template <typename T>
+struct Identity {  // the reference benchmark's own functor: takes the header-template path
+  __host__ __device__ T operator()(T a) const { return a; }
+};
+
+class Harness {
+ public:
+  explicit Harness(const Options& o) : opt_(o)
+  {
+    stream_ = raft::resource::get_cuda_stream(handle_);
+    // three times the last-level cache, as the reference flushes three times its L2; the
+    // 256 MB memory-side cache of this GPU is the level that matters here
+    int l2 = 0;
+    RAFT_HIP_TRY(hipDeviceGetAttribute(&l2, hipDeviceAttributeL2CacheSize, 0));
+    flush_bytes_ = 3 * std::max<size_t>((size_t)l2, (size_t)256 << 20);
+    RAFT_HIP_TRY(hipMalloc(&flush_buf_, flush_bytes_));
+    RAFT_HIP_TRY(hipEventCreate(&e0_));
+    RAFT_HIP_TRY(hipEventCreate(&e1_));
+  }
+  ~Harness()
+  {
+    (void)hipFree(flush_buf_);
+    (void)hipEventDestroy(e0_);
+    (void)hipEventDestroy(e1_);
+  }
+  raft::resources& handle() { return handle_; }
+  hipStream_t stream() const { return stream_; }
+  bool wanted(const std::string& name) const
+  {
+    return opt_.filter.empty() || name.find(opt_.filter) != std::string::npos;
+  }
+  bool fits(size_t bytes) const { return bytes <= opt_.max_bytes; }
+
+  template <typename F>
+  void run(const std::string& name, const std::string& shape, size_t alg_bytes, F&& call)
+  {
+    call();  // warm-up: code objects, workspace
+    RAFT_HIP_TRY(hipStreamSynchronize(stream_));
+    double total_ms = 0.0;
+    int iters       = 0;
+    // at least min_iters calls and 20 ms of kernel time, at most 200 calls
+    while (iters < opt_.min_iters || (total_ms < 20.0 && iters < 200)) {
+      if (opt_.flush)
+        fill_words<<<2048, 256, 0, stream_>>>(static_cast<unsigned*>(flush_buf_),
+                                              flush_bytes_ / 4, (unsigned)iters);
+      RAFT_HIP_TRY(hipEventRecord(e0_, stream_));
+      call();
+      RAFT_HIP_TRY(hipEventRecord(e1_, stream_));
+      RAFT_HIP_TRY(hipEventSynchronize(e1_));
+      float ms = 0.f;
+      RAFT_HIP_TRY(hipEventElapsedTime(&ms, e0_, e1_));
+      total_ms += ms;
+      ++iters;
+    }
+    const double us = total_ms * 1e3 / iters;
+    std::printf("%-34s %-22s %10.2f us %9.1f GB/s  iters=%d\n", name.c_str(), shape.c_str(), us,
+                (double)alg_bytes / (us * 1e-6) / 1e9, iters);
+    std::fflush(stdout);
+  }
+
+ private:
+  Options opt_;
+  raft::resources handle_;
+  hipStream_t stream_ = nullptr;
+  void* flush_buf_    = nullptr;
+  size_t flush_bytes_ = 0;
+  hipEvent_t e0_{}, e1_{};
+};
+
+template <typename T>
+struct DeviceBuf {
+  T* p     = nullptr;
+  size_t n = 0;
+  explicit DeviceBuf(size_t count) : n(count) { RAFT_HIP_TRY(hipMalloc(&p, std::max<size_t>(n, 1) * sizeof(T))); }
+  ~DeviceBuf() { (void)hipFree(p); }
+  DeviceBuf(const DeviceBuf&)            = delete;
+  DeviceBuf& operator=(const DeviceBuf&) = delete;
+  void uniform(double lo, double hi, hipStream_t s)
+  {
+    if (n) fill_uniform<<<4096, 256, 0, s>>>(p, n, lo, hi, 1234ull);
+  }
+};
+
+template <typename T>
+const char* tname()
+{
+  return sizeof(T) == 4 ? "float" : "double";
+}
+
+std::string shape2(long long r, long long c) { return std::to_string(r) + "x" + std::to_string(c); }
+
+template <typename T>
+void bench_reduce(Harness& h)
+{
+  const std::vector<std::pair<int, int>> sizes{{8 * 1024, 1024},  {1024, 8 * 1024},
+                                               {8 * 1024, 8 * 1024}, {32 * 1024, 1024},
+                                               {1024, 32 * 1024},  {32 * 1024, 32 * 1024}};
+  for (bool along_rows : {false, true})
+    for (auto size : sizes) {
+      const int rows = size.first, cols = size.second;
+      const std::string name =
+        std::string("reduce<") + tname<T>() + ">/" + (along_rows ? "along_rows" : "along_cols");
+      const size_t n = (size_t)rows * cols;
+      if (!h.wanted(name) || !h.fits(n * sizeof(T))) continue;
+      DeviceBuf<T> in(n), out((size_t)std::max(rows, cols));
+      in.uniform(-1.0, 1.0, h.stream());
+      h.run(name, shape2(rows, cols), n * sizeof(T), [&] {
+        if (along_rows)
+          raft::linalg::reduce<true, true>(out.p, in.p, cols, rows, T(0), h.stream());
+        else
+          raft::linalg::reduce<true, false>(out.p, in.p, cols, rows, T(0), h.stream());
+      });
+    }
+}
+
+template <typename T, typename IdxT>
+void bench_row_norm(Harness& h)
+{
+  const std::string name = std::string("rowNorm<") + tname<T>() + "," +
+                           (sizeof(IdxT) == 4 ? "int" : "int64_t") + ">";
+  if (!h.wanted(name)) return;
+  for (IdxT rows : {10, 100, 1000, 10000, 100000})
+    for (IdxT cols : {16, 32, 64, 128, 256, 512, 1024}) {
+      const size_t n = (size_t)rows * cols;
+      DeviceBuf<T> in(n), dots((size_t)rows);
+      in.uniform(-10.0, 10.0, h.stream());
+      h.run(name, shape2(rows, cols), n * sizeof(T), [&] {
+        auto iv = raft::make_device_matrix_view<const T, IdxT, raft::row_major>(in.p, rows, cols);
+        auto ov = raft::make_device_vector_view<T, IdxT>(dots.p, rows);
+        raft::linalg::norm<raft::linalg::L2Norm, raft::Apply::ALONG_ROWS>(h.handle(), iv, ov,
+                                                                          raft::sqrt_op());
+      });
+    }
+}
+
+template <typename T, typename IdxT>
+void bench_row_normalize(Harness& h)
+{
+  const std::string name = std::string("rowNormalize<") + tname<T>() + "," +
+                           (sizeof(IdxT) == 4 ? "int" : "int64_t") + ">";
+  if (!h.wanted(name)) return;
+  for (IdxT rows : {10, 100, 1000, 10000, 100000})
+    for (IdxT cols : {8, 16, 32, 64, 128, 256, 512, 1024, 2048, 4096, 8192, 16384}) {
+      const size_t n = (size_t)rows * cols;
+      DeviceBuf<T> in(n), out(n);
+      in.uniform(-10.0, 10.0, h.stream());
+      h.run(name, shape2(rows, cols), 2 * n * sizeof(T), [&] {
+        auto iv = raft::make_device_matrix_view<const T, IdxT, raft::row_major>(in.p, rows, cols);
+        auto ov = raft::make_device_matrix_view<T, IdxT, raft::row_major>(out.p, rows, cols);
+        raft::linalg::row_normalize<raft::linalg::L2Norm>(h.handle(), iv, ov);
+      });
+    }
+}
+
+template <typename T>
+void bench_map_then_reduce(Harness& h)
+{
+  const std::vector<int> lens{1024 * 1024,     32 * 1024 * 1024,     1024 * 1024 * 1024,
+                              1024 * 1024 + 2, 32 * 1024 * 1024 + 2, 1024 * 1024 * 1024 + 2,
+                              1024 * 1024 + 1, 32 * 1024 * 1024 + 1, 1024 * 1024 * 1024 + 1};
+  for (int len : lens) {
+    const size_t n = (size_t)len;
+    if (!h.fits(n * sizeof(T))) continue;
+    const std::string user = std::string("map_then_reduce<") + tname<T>() + ">/user_functor";
+    const std::string lib  = std::string("map_then_reduce<") + tname<T>() + ">/identity_op";
+    if (!h.wanted(user) && !h.wanted(lib)) continue;
+    DeviceBuf<T> in(n), out(1);
+    in.uniform(-1.0, 1.0, h.stream());
+    if (h.wanted(user))
+      h.run(user, std::to_string(len), n * sizeof(T), [&] {
+        raft::linalg::mapThenSumReduce(out.p, len, Identity<T>(), h.stream(), in.p);
+      });
+    if (h.wanted(lib))
+      h.run(lib, std::to_string(len), n * sizeof(T), [&] {
+        raft::linalg::mapThenSumReduce(out.p, len, raft::identity_op(), h.stream(), in.p);
+      });
+  }
+}
+
+template <typename T>
+void bench_argmin(Harness& h)
+{
+  const std::string name = std::string("Argmin<") + tname<T>() + ",uint32_t,int64_t>";
+  if (!h.wanted(name)) return;
+  for (std::int64_t rows : {1000, 10000, 100000, 1000000, 10000000})
+    for (std::int64_t cols : {64, 128, 256, 512, 1024}) {
+      const size_t n = (size_t)rows * cols;
+      if (!h.fits(n * sizeof(T))) continue;
+      DeviceBuf<T> matrix(n);
+      DeviceBuf<std::uint32_t> indices((size_t)rows);
+      matrix.uniform(-1.0, 1.0, h.stream());
+      h.run(name, shape2(rows, cols), n * sizeof(T), [&] {
+        auto mv =
+          raft::make_device_matrix_view<const T, std::int64_t, raft::row_major>(matrix.p, rows, cols);
+        auto iv = raft::make_device_vector_view<std::uint32_t, std::int64_t>(indices.p, rows);
+        raft::matrix::argmin(h.handle(), mv, iv);
+      });
+    }
+}
+
+}  // namespace
+
+int main(int argc, char** argv)
+{
+  Options opt;
+  for (int i = 1; i < argc; ++i) {
+    if (!std::strcmp(argv[i], "--filter") && i + 1 < argc) opt.filter = argv[++i];
+    else if (!std::strcmp(argv[i], "--min-iters") && i + 1 < argc) opt.min_iters = std::atoi(argv[++i]);
+    else if (!std::strcmp(argv[i], "--max-bytes") && i + 1 < argc) opt.max_bytes = std::strtoull(argv[++i], nullptr, 10);
+    else if (!std::strcmp(argv[i], "--no-flush")) opt.flush = false;
+    else {
+      std::fprintf(stderr, "usage: %s [--filter s] [--min-iters n] [--max-bytes b] [--no-flush]\n", argv[0]);
+      return 2;
+    }
+  }
+  int n = 0;
+  if (hipGetDeviceCount(&n) != hipSuccess || n == 0) {
+    std::fprintf(stderr, "no GPU visible\n");
+    return 2;
+  }
+  Harness h(opt);
+  bench_reduce<float>(h);
+  bench_reduce<double>(h);
+  bench_row_norm<float, int>(h);
+  bench_row_norm<double, int>(h);
+  bench_row_norm<float, std::int64_t>(h);
+  bench_row_norm<double, std::int64_t>(h);
+  bench_row_normalize<float, int>(h);
+  bench_row_normalize<double, int>(h);
+  bench_row_normalize<float, std::int64_t>(h);
+  bench_row_normalize<double, std::int64_t>(h);
+  bench_map_then_reduce<float>(h);
+  bench_map_then_reduce<double>(h);
+  bench_argmin<float>(h);
+  bench_argmin<double>(h);
+  return 0;
+}

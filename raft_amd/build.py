@@ -86,10 +86,18 @@ def build_cpp_tests() -> list[Path]:
     return sorted((tdir / "bin").glob("*"))
 
 
+def build_bench() -> list[Path]:
+    """Compile the benchmark program over the reference's shape grids (hipcc)."""
+    bdir = ROOT / "raft_amd" / "bench"
+    _run(["make", "-s", "-C", str(bdir)])
+    return sorted((bdir / "bin").glob("*"))
+
+
 def build_all(force: bool = True) -> None:
     build_library(force=force)
     build_oracle()
     build_cpp_tests()
+    build_bench()
 
 
 if __name__ == "__main__":

@@ -68,7 +68,8 @@ struct In<double> {
   template <int J>
   static __device__ __forceinline__ nat get(const u32x4& v)
   {
-    return __hiloint2double((int)v[2 * J + 1], (int)v[2 * J]);
+    typedef double f64x2 __attribute__((ext_vector_type(2)));
+    return __builtin_bit_cast(f64x2, v)[J];
   }
   static __device__ __forceinline__ nat ld(const double* p)
   {
@@ -152,7 +153,8 @@ struct In<int64_t> {
   template <int J>
   static __device__ __forceinline__ nat get(const u32x4& v)
   {
-    return (int64_t)(((u64)v[2 * J + 1] << 32) | (u64)v[2 * J]);
+    typedef int64_t i64x2 __attribute__((ext_vector_type(2)));
+    return __builtin_bit_cast(i64x2, v)[J];
   }
   static __device__ __forceinline__ nat ld(const int64_t* p) { return *p; }
 };

@@ -74,27 +74,48 @@ constexpr int vec_width()
   }
 }
 
-// acc = fold of main_op(row[j], j) for j = first, first + stride, ... over whole
-// 16-byte vectors, then the tail elements
+// acc = fold of main_op(row[j], j0 + j) over the D elements at `row`: whole 16-byte
+// vectors first + k * stride (four lane loads in flight), then the tail elements.
+// j0 is the position of row[0] along the reduced axis.
 template <typename In, typename Out, typename Idx, typename Main, typename Red>
 __device__ __forceinline__ Out sweep_row(const In* row, Idx D, int first, int stride, Out acc,
-                                         Main& main_op, Red& red)
+                                         Main& main_op, Red& red, Idx j0 = 0)
 {
   constexpr int V = vec_width<In>();
   if constexpr (V > 1) {
-    const Idx nvec = D / V;
-    for (Idx v = first; v < nvec; v += stride) {
+    constexpr int U = 4;
+    struct alignas(1) pack {
+      char b[16];
+    };
+    const Idx nvec  = D / V;
+    const char* base = reinterpret_cast<const char*>(row);
+    auto take = [&](const pack& raw, Idx v) {
       In x[V];  // one 16-byte lane load at any element-aligned address
-      __builtin_memcpy(x, reinterpret_cast<const char*>(row) + (std::size_t)v * 16, 16);
+      __builtin_memcpy(x, raw.b, 16);
 #pragma unroll
       for (int j = 0; j < V; ++j)
-        acc = red(acc, static_cast<Out>(main_op(x[j], static_cast<Idx>(v * V + j))));
+        acc = red(acc, static_cast<Out>(main_op(x[j], static_cast<Idx>(j0 + v * V + j))));
+    };
+    Idx v = first;
+    for (; v + (Idx)(U - 1) * stride < nvec; v += (Idx)U * stride) {
+      pack raw[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        __builtin_memcpy(raw[u].b, base + (std::size_t)(v + (Idx)u * stride) * 16, 16);
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        take(raw[u], v + (Idx)u * stride);
+    }
+    for (; v < nvec; v += stride) {
+      pack raw;
+      __builtin_memcpy(raw.b, base + (std::size_t)v * 16, 16);
+      take(raw, v);
     }
     for (Idx j = nvec * V + first; j < D; j += stride)
-      acc = red(acc, static_cast<Out>(main_op(row[j], j)));
+      acc = red(acc, static_cast<Out>(main_op(row[j], static_cast<Idx>(j0 + j))));
   } else {
     for (Idx j = first; j < D; j += stride)
-      acc = red(acc, static_cast<Out>(main_op(row[j], j)));
+      acc = red(acc, static_cast<Out>(main_op(row[j], static_cast<Idx>(j0 + j))));
   }
   return acc;
 }
@@ -130,8 +151,9 @@ __global__ __launch_bounds__(kBlock) void rows_block_kernel(Out* dots, Out* part
   const std::int64_t j0  = (std::int64_t)b * chunk;
   const std::int64_t j1  = j0 + chunk < (std::int64_t)D ? j0 + chunk : (std::int64_t)D;
   Out acc                = init;
-  for (std::int64_t j = j0 + threadIdx.x; j < j1; j += kBlock)
-    acc = red(acc, static_cast<Out>(main_op(data[row * D + j], static_cast<Idx>(j))));
+  if (j1 > j0)
+    acc = sweep_row<In, Out, Idx>(data + row * D + j0, (Idx)(j1 - j0), (int)threadIdx.x, kBlock,
+                                  acc, main_op, red, (Idx)j0);
   acc = group_reduce(acc, kWave, red);
   if ((threadIdx.x & (kWave - 1)) == 0) sm[threadIdx.x >> 6] = acc;
   __syncthreads();
@@ -180,18 +202,35 @@ __global__ __launch_bounds__(kBlock) void cols_kernel(Out* dots, Out* partial, c
   }
 }
 
-// second pass over partials[n_out][B], one thread per output, fixed order
+// second pass over partials[n_out][B]: LB lanes of a wave per output (LB a power of
+// two <= 64), each folding every LB-th partial, then a butterfly: a fixed order
 template <typename Out, typename Red, typename Fin>
 __global__ __launch_bounds__(kBlock) void fold_kernel(Out* dots, const Out* partial,
                                                       std::int64_t n_out, int B, Out init,
-                                                      bool inplace, Red red, Fin fin)
+                                                      bool inplace, Red red, Fin fin, int LB,
+                                                      int logLB)
 {
-  const std::int64_t o = (std::int64_t)blockIdx.x * kBlock + threadIdx.x;
-  if (o >= n_out) return;
-  Out acc = init;
-  for (int b = 0; b < B; ++b)
-    acc = red(acc, partial[o * B + b]);
-  dots[o] = fin(inplace ? red(dots[o], acc) : acc);
+  const std::int64_t gtid = (std::int64_t)blockIdx.x * kBlock + threadIdx.x;
+  const std::int64_t o    = gtid >> logLB;
+  const int lb            = (int)(gtid & (LB - 1));
+  Out acc                 = init;
+  if (o < n_out) {
+    const Out* p = partial + o * B;
+    int b        = lb;
+    for (; b + 7 * LB < B; b += 8 * LB) {  // eight loads in flight, folded in order
+      Out x[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        x[u] = p[b + u * LB];
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        acc = red(acc, x[u]);
+    }
+    for (; b < B; b += LB)
+      acc = red(acc, p[b]);
+  }
+  acc = group_reduce(acc, LB, red);
+  if (lb == 0 && o < n_out) dots[o] = fin(inplace ? red(dots[o], acc) : acc);
 }
 
 inline int pow2ceil(std::int64_t x)
@@ -217,6 +256,16 @@ inline void check_launch(const char* what)
                           hipGetErrorString(e));
 }
 
+template <typename Out, typename Red, typename Fin>
+void launch_fold(Out* dots, const Out* partial, std::int64_t n_out, int B, Out init, bool inplace,
+                 Red red, Fin fin, hipStream_t stream)
+{
+  const int LB             = B >= 64 ? 64 : pow2ceil(B);
+  const std::int64_t grid  = (n_out * LB + kBlock - 1) / kBlock;
+  hipLaunchKernelGGL((fold_kernel<Out, Red, Fin>), dim3((unsigned)grid), dim3(kBlock), 0, stream,
+                     dots, partial, n_out, B, init, inplace, red, fin, LB, ilog2(LB));
+}
+
 // dots[N] from N contiguous rows of D elements
 template <typename In, typename Out, typename Idx, typename Main, typename Red, typename Fin>
 void coalesced(Out* dots, const In* data, Idx D, Idx N, Out init, hipStream_t stream, bool inplace,
@@ -238,12 +287,16 @@ void coalesced(Out* dots, const In* data, Idx D, Idx N, Out init, hipStream_t st
     return;
   }
   // few long rows: split each into B chunks so that the grid fills the device
-  std::int64_t B = (2048 + (std::int64_t)N - 1) / (std::int64_t)N;
-  const std::int64_t max_b = ((std::int64_t)D + 4 * kBlock - 1) / (4 * kBlock);
+  // chunks are whole multiples of one block sweep (256 lanes x 4 loads x V elements), so
+  // every chunk starts on a vector boundary of its row
+  constexpr std::int64_t quantum = (std::int64_t)kBlock * 4 * V;
+  std::int64_t B = (1024 + (std::int64_t)N - 1) / (std::int64_t)N;
+  const std::int64_t max_b = ((std::int64_t)D + quantum - 1) / quantum;
   if (B > max_b) B = max_b;
   if (B < 1) B = 1;
-  const std::int64_t chunk = ((std::int64_t)D + B - 1) / B;
-  B                        = ((std::int64_t)D + chunk - 1) / chunk;
+  std::int64_t chunk = ((std::int64_t)D + B - 1) / B;
+  chunk              = (chunk + quantum - 1) / quantum * quantum;
+  B                  = ((std::int64_t)D + chunk - 1) / chunk;
   Out* partial             = nullptr;
   if (B > 1) RAFT_HIP_TRY(hipMallocAsync((void**)&partial, sizeof(Out) * (std::size_t)N * B, stream));
   hipLaunchKernelGGL((rows_block_kernel<In, Out, Idx, Main, Red, Fin>),
@@ -251,9 +304,7 @@ void coalesced(Out* dots, const In* data, Idx D, Idx N, Out init, hipStream_t st
                      data, D, N, init, inplace, main_op, red, fin, (int)B, chunk);
   check_launch("rows_block_kernel");
   if (B > 1) {
-    hipLaunchKernelGGL((fold_kernel<Out, Red, Fin>),
-                       dim3((unsigned)(((std::int64_t)N + kBlock - 1) / kBlock)), dim3(kBlock), 0,
-                       stream, dots, partial, (std::int64_t)N, (int)B, init, inplace, red, fin);
+    launch_fold(dots, partial, (std::int64_t)N, (int)B, init, inplace, red, fin, stream);
     check_launch("fold_kernel");
     RAFT_HIP_TRY(hipFreeAsync(partial, stream));
   }
@@ -280,9 +331,7 @@ void strided(Out* dots, const In* data, Idx D, Idx N, Out init, hipStream_t stre
                      data, D, N, init, inplace, main_op, red, fin, TX, ilog2(TX), (int)B);
   check_launch("cols_kernel");
   if (B > 1) {
-    hipLaunchKernelGGL((fold_kernel<Out, Red, Fin>),
-                       dim3((unsigned)(((std::int64_t)D + kBlock - 1) / kBlock)), dim3(kBlock), 0,
-                       stream, dots, partial, (std::int64_t)D, (int)B, init, inplace, red, fin);
+    launch_fold(dots, partial, (std::int64_t)D, (int)B, init, inplace, red, fin, stream);
     check_launch("fold_kernel");
     RAFT_HIP_TRY(hipFreeAsync(partial, stream));
   }

@@ -9,6 +9,19 @@
 
 namespace raft::linalg {
 namespace detail {
+// The reference calls map(in[i]) (linalg/detail/map_then_reduce.cuh:58-61); the
+// reduction's main_op is called with (value, index).  A map functor of the caller's
+// own is wrapped so that it sees the value alone.
+template <typename MapOp>
+struct unary_map_adapter {
+  MapOp map;
+  template <typename T, typename I>
+  constexpr RAFT_INLINE_FUNCTION auto operator()(const T& x, I) const
+  {
+    return map(x);
+  }
+};
+
 template <typename InType, typename OutType, typename MapOp, typename ReduceLambda,
           typename... Args>
 void map_reduce_call(const resources* res, OutType* out, size_t len, OutType neutral, MapOp map,
@@ -17,8 +30,14 @@ void map_reduce_call(const resources* res, OutType* out, size_t len, OutType neu
   static_assert(sizeof...(Args) == 0,
                 "map-then-reduce over several input arrays is not lowered to the reduction "
                 "library; only map(in[i]) is");
-  raft::detail::rmi::reduce(res, stream, out, in, std::int64_t(1), (std::int64_t)len, true, true,
-                            neutral, false, map, op, raft::identity_op());
+  if constexpr (raft::detail::rmi::main_tag<MapOp>::value >= 0) {
+    raft::detail::rmi::reduce(res, stream, out, in, std::int64_t(1), (std::int64_t)len, true,
+                              true, neutral, false, map, op, raft::identity_op());
+  } else {
+    raft::detail::rmi::reduce(res, stream, out, in, std::int64_t(1), (std::int64_t)len, true,
+                              true, neutral, false, unary_map_adapter<MapOp>{map}, op,
+                              raft::identity_op());
+  }
 }
 }  // namespace detail
 

@@ -254,7 +254,8 @@ TEST_CASE(VocabularyStillLowered)
   CHECK(ok);
 }
 
-// map_reduce with a device lambda
+// map_reduce with a device lambda: the map sees the value alone
+// (linalg/detail/map_then_reduce.cuh:58-61)
 TEST_CASE(MapReduceLambda)
 {
   raft::resources handle;
@@ -266,7 +267,7 @@ TEST_CASE(MapReduceLambda)
   raft::update_device(in.data_handle(), h.data(), h.size(), stream);
   auto in_c = raft::make_device_vector_view<const float, int>(in.data_handle(), len);
   raft::linalg::map_reduce(handle, in_c, out.view(), 0.0f,
-                           [] __device__(float x, int) { return x > 0.0f ? x : 0.0f; },
+                           [] __device__(float x) { return x > 0.0f ? x : 0.0f; },
                            raft::add_op());
   double want = 0;
   for (float x : h)
