@@ -14,6 +14,7 @@
 #include <raft/core/kvp.hpp>
 #include <raft/core/operators.hpp>
 #include <raft/core/resources.hpp>
+#include <raft/linalg/detail/rmi_scratch.hpp>
 
 #include "rmi_reduce.h"
 
@@ -205,7 +206,7 @@ class workspace_lease {
     if (res != nullptr) {
       ptr_ = res->workspace(bytes);
     } else {
-      RAFT_HIP_TRY(hipMallocAsync(&ptr_, bytes, stream));
+      ptr_   = scratch_alloc(bytes, stream);
       owned_ = true;
     }
   }
@@ -213,7 +214,7 @@ class workspace_lease {
   workspace_lease& operator=(const workspace_lease&) = delete;
   ~workspace_lease()
   {
-    if (owned_ && ptr_ != nullptr) (void)hipFreeAsync(ptr_, stream_);
+    if (owned_) scratch_free(ptr_, stream_);
   }
   void* data() const { return ptr_; }
   size_t size() const { return bytes_; }

@@ -29,6 +29,7 @@
 #include <type_traits>
 
 #include <raft/core/error.hpp>
+#include <raft/linalg/detail/rmi_scratch.hpp>
 
 namespace raft::detail::rmi::generic {
 
@@ -298,7 +299,7 @@ void coalesced(Out* dots, const In* data, Idx D, Idx N, Out init, hipStream_t st
   chunk              = (chunk + quantum - 1) / quantum * quantum;
   B                  = ((std::int64_t)D + chunk - 1) / chunk;
   Out* partial             = nullptr;
-  if (B > 1) RAFT_HIP_TRY(hipMallocAsync((void**)&partial, sizeof(Out) * (std::size_t)N * B, stream));
+  if (B > 1) partial = static_cast<Out*>(scratch_alloc(sizeof(Out) * (std::size_t)N * B, stream));
   hipLaunchKernelGGL((rows_block_kernel<In, Out, Idx, Main, Red, Fin>),
                      dim3((unsigned)((std::int64_t)N * B)), dim3(kBlock), 0, stream, dots, partial,
                      data, D, N, init, inplace, main_op, red, fin, (int)B, chunk);
@@ -306,7 +307,7 @@ void coalesced(Out* dots, const In* data, Idx D, Idx N, Out init, hipStream_t st
   if (B > 1) {
     launch_fold(dots, partial, (std::int64_t)N, (int)B, init, inplace, red, fin, stream);
     check_launch("fold_kernel");
-    RAFT_HIP_TRY(hipFreeAsync(partial, stream));
+    scratch_free(partial, stream);
   }
 }
 
@@ -325,7 +326,7 @@ void strided(Out* dots, const In* data, Idx D, Idx N, Out init, hipStream_t stre
   if (B < 1) B = 1;
   if (B > 4096) B = 4096;
   Out* partial = nullptr;
-  if (B > 1) RAFT_HIP_TRY(hipMallocAsync((void**)&partial, sizeof(Out) * (std::size_t)D * B, stream));
+  if (B > 1) partial = static_cast<Out*>(scratch_alloc(sizeof(Out) * (std::size_t)D * B, stream));
   hipLaunchKernelGGL((cols_kernel<In, Out, Idx, Main, Red, Fin>),
                      dim3((unsigned)gridx, (unsigned)B), dim3(kBlock), 0, stream, dots, partial,
                      data, D, N, init, inplace, main_op, red, fin, TX, ilog2(TX), (int)B);
@@ -333,7 +334,7 @@ void strided(Out* dots, const In* data, Idx D, Idx N, Out init, hipStream_t stre
   if (B > 1) {
     launch_fold(dots, partial, (std::int64_t)D, (int)B, init, inplace, red, fin, stream);
     check_launch("fold_kernel");
-    RAFT_HIP_TRY(hipFreeAsync(partial, stream));
+    scratch_free(partial, stream);
   }
 }
 

@@ -11,6 +11,7 @@
 #include <raft/linalg/map_reduce.cuh>
 #include <raft/linalg/reduce.cuh>
 #include <raft/linalg/strided_reduction.cuh>
+#include <raft/stats/weighted_mean.cuh>
 #include <raft/util/cudart_utils.hpp>
 
 #include <cstdint>
@@ -274,6 +275,68 @@ TEST_CASE(MapReduceLambda)
     want += x > 0 ? x : 0;
   CHECK(close(to_host(out.data_handle(), 1, stream)[0], want, 1e-4));
 }
+
+// cpp/tests/stats/weighted_mean.cu:24-300: weighted means along rows and columns, both
+// layouts, against the naive host evaluation with the reference's tolerance (tol * N)
+template <typename T>
+void weighted_mean_cases(double tol)
+{
+  raft::resources handle;
+  auto stream = raft::resource::get_cuda_stream(handle);
+  struct Case { int M, N; bool along_rows, row_major; };
+  const std::vector<Case> cases{{4, 4, true, true},      {32, 32, true, false},
+                                {32, 64, false, false},  {32, 256, true, true},
+                                {32, 256, false, false}, {1024, 32, true, false},
+                                {1024, 64, true, true},  {1024, 128, true, false},
+                                {1024, 256, true, true}, {1024, 32, false, false},
+                                {1024, 64, false, true}, {1024, 128, false, false},
+                                {1024, 256, false, true}, {3, 100000, true, true},
+                                {100000, 5, false, true}};
+  for (const auto& c : cases) {
+    const int rows = c.M, cols = c.N;
+    const int wlen = c.along_rows ? cols : rows, olen = c.along_rows ? rows : cols;
+    auto hd = uniform<T>((size_t)rows * cols, -1.0, 1.0, 1234);
+    auto hw = uniform<T>((size_t)wlen, -1.0, 1.0, 4321);
+    auto dd = raft::make_device_vector<T, int>(handle, rows * cols);
+    auto dw = raft::make_device_vector<T, int>(handle, wlen);
+    auto mu = raft::make_device_vector<T, int>(handle, olen);
+    raft::update_device(dd.data_handle(), hd.data(), hd.size(), stream);
+    raft::update_device(dw.data_handle(), hw.data(), hw.size(), stream);
+    auto wv = raft::make_device_vector_view<const T, int>(dw.data_handle(), wlen);
+    auto run = [&](auto layout) {
+      using layout_t = decltype(layout);
+      auto in = raft::make_device_matrix_view<const T, int, layout_t>(dd.data_handle(), rows, cols);
+      if (c.along_rows)
+        raft::stats::row_weighted_mean(handle, in, wv, mu.view());
+      else
+        raft::stats::col_weighted_mean(handle, in, wv, mu.view());
+    };
+    if (c.row_major) run(raft::row_major{}); else run(raft::col_major{});
+    double ws = 0;
+    for (T w : hw)
+      ws += (double)w;
+    // the device sums the weights in T; divide by that sum as the reference does
+    std::vector<double> want(olen, 0.0);
+    for (int k = 0; k < olen; ++k) {
+      double s = 0;
+      for (int r = 0; r < wlen; ++r) {
+        const size_t idx = c.along_rows ? at(c.row_major, rows, cols, k, r)
+                                        : at(c.row_major, rows, cols, r, k);
+        s += (double)hd[idx] * (double)hw[r];
+      }
+      want[k] = s / ws;
+    }
+    auto got = to_host(mu.data_handle(), (size_t)olen, stream);
+    bool ok  = true;
+    const double bound = tol * wlen / std::fabs(ws) + tol;
+    for (int k = 0; k < olen; ++k)
+      ok &= std::fabs((double)got[k] - want[k]) <= bound * (1.0 + std::fabs(want[k]));
+    if (!ok) std::printf("  weighted mean %dx%d along_rows=%d row_major=%d\n", rows, cols, c.along_rows, c.row_major);
+    CHECK(ok);
+  }
+}
+TEST_CASE(WeightedMeanF) { weighted_mean_cases<float>(1e-6); }
+TEST_CASE(WeightedMeanD) { weighted_mean_cases<double>(1e-14); }
 
 int main()
 {
