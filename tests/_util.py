@@ -3,6 +3,7 @@ comparators and a one-call "run on the GPU through the C ABI" helper."""
 from __future__ import annotations
 
 import ctypes as C
+import os
 from pathlib import Path
 
 import numpy as np
@@ -244,3 +245,22 @@ def check_against_oracle(desc, data, *, old_raw=None, aux_raw=None, misalign_ele
                           f"worst rel {worst_rel(got, exp):.3e}, first bad "
                           f"{np.flatnonzero(~ok)[:5]} got {got[~ok][:5]} want {exp[~ok][:5]}")
     return got_raw
+
+
+def golden():
+    """The reference's known-answer vectors (tests/golden/reference_fixtures.json)."""
+    import json
+    global _golden
+    try:
+        return _golden
+    except NameError:
+        pass
+    with open(os.path.join(os.path.dirname(__file__), "golden", "reference_fixtures.json")) as f:
+        _golden = json.load(f)
+    return _golden
+
+
+LAYOUT_AXIS = {"row_major/along_rows": (api.ROW_MAJOR, api.ALONG_ROWS),
+               "row_major/along_columns": (api.ROW_MAJOR, api.ALONG_COLUMNS),
+               "col_major/along_rows": (api.COL_MAJOR, api.ALONG_ROWS),
+               "col_major/along_columns": (api.COL_MAJOR, api.ALONG_COLUMNS)}

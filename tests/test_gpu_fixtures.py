@@ -8,24 +8,26 @@ from tests import _util as u
 
 pytestmark = pytest.mark.gpu
 
+GOLD = u.golden()
+
 
 # cpp/tests/linalg/reduce.cu:108-177 (simpleTest): data 1..12 as 3x4, max_op, init 0.
-@pytest.mark.parametrize("layout,apply,expected", [
-    (api.ROW_MAJOR, api.ALONG_ROWS, [4, 8, 12]),
-    (api.ROW_MAJOR, api.ALONG_COLUMNS, [9, 10, 11, 12]),
-    (api.COL_MAJOR, api.ALONG_ROWS, [10, 11, 12]),
-    (api.COL_MAJOR, api.ALONG_COLUMNS, [3, 6, 9, 12]),
-])
+@pytest.mark.parametrize("case", list(GOLD["reduce_simple_max"]["expected"]))
 @pytest.mark.parametrize("dt,npdt", [(api.F32, np.float32), (api.F64, np.float64)])
-def test_reduce_simple_max(gpu, layout, apply, expected, dt, npdt):
-    data = np.arange(1, 13, dtype=npdt)
-    d = api.make_desc(dt, dt, 3, 4, layout=layout, apply=apply, reduce_op=api.RED_MAX)
+def test_reduce_simple_max(gpu, case, dt, npdt):
+    g = GOLD["reduce_simple_max"]
+    layout, apply = u.LAYOUT_AXIS[case]
+    expected = g["expected"][case]
+    data = np.array(g["data"], dtype=npdt)
+    d = api.make_desc(dt, dt, g["rows"], g["cols"], layout=layout, apply=apply,
+                      reduce_op=api.RED_MAX)
     got = u.gpu_reduce(d, data)
     assert got.tolist() == [float(e) for e in expected]
 
 
 # cpp/tests/matrix/argmax.cu:71-75 and argmin.cu:71-75: 3x4 literal, key-only output.
-ARG_DATA = [0.1, 0.2, 0.3, 0.4, 0.4, 0.3, 0.2, 0.1, 0.2, 0.3, 0.5, 0.0]
+ARG = GOLD["matrix_arg"]
+ARG_DATA = ARG["data"]
 
 
 @pytest.mark.parametrize("dt,npdt", [(api.F32, np.float32), (api.F64, np.float64)])
@@ -33,33 +35,32 @@ def test_matrix_argmax_argmin_fixture(gpu, dt, npdt):
     data = np.array(ARG_DATA, dtype=npdt)
     dmax = api.make_desc(dt, api.I32, 3, 4, main_op=api.MAIN_KVP, reduce_op=api.RED_ARGMAX,
                          final_op=api.FIN_KEY, init_i=0, init_f=-np.inf)
-    assert u.gpu_reduce(dmax, data).tolist() == [3, 0, 2]
+    assert u.gpu_reduce(dmax, data).tolist() == ARG["argmax"]
     dmin = api.make_desc(dt, api.I32, 3, 4, main_op=api.MAIN_KVP, reduce_op=api.RED_ARGMIN,
                          final_op=api.FIN_KEY, init_i=0, init_f=np.inf)
-    assert u.gpu_reduce(dmin, data).tolist() == [0, 3, 3]
+    assert u.gpu_reduce(dmin, data).tolist() == ARG["argmin"]
 
 
 # cpp/tests/util/reduction.cu:167-171,179-181: the literal 64-vector.
-VEC64 = [1, 2, 3, 4, 1, 2, 3, 4, 1, 2, 3, 4, 1, 2, 3, 5, 1, 2, 3, 4, 1, 2,
-         3, 4, 1, 2, 0, 4, 1, 2, 3, 4, 1, 2, 3, 4, 1, 2, 3, 4, 1, 2, 3, 4,
-         1, 2, 3, 4, 1, 2, 3, 4, 1, 2, 3, 4, 1, 2, 3, 4, 1, 2, 3, 4]
+W64 = GOLD["wave_vector64"]
+VEC64 = W64["data"]
 
 
 def test_wave_reduction_vector(gpu):
     x = np.array(VEC64, dtype=np.int32)
-    for red, init, want in [(api.RED_MIN, 2**62, 0), (api.RED_MAX, -2**62, 5),
-                            (api.RED_ADD, 0, 158)]:
+    for red, init, want in [(api.RED_MIN, 2**62, W64["min"]), (api.RED_MAX, -2**62, W64["max"]),
+                            (api.RED_ADD, 0, W64["sum"])]:
         d = api.make_desc(api.I32, api.I64, 1, 64, reduce_op=red, init_i=init)
         assert u.gpu_reduce(d, x).tolist() == [want]
     xf = x.astype(np.float32)
     d = api.make_desc(api.F32, api.KVP_I32_F32, 1, 64, main_op=api.MAIN_KVP,
                       reduce_op=api.RED_ARGMAX, init_i=0, init_f=-np.inf)
     r = u.gpu_reduce(d, xf)
-    assert (int(r["key"][0]), float(r["value"][0])) == (15, 5.0)
+    assert [int(r["key"][0]), float(r["value"][0])] == W64["argmax"]
     d = api.make_desc(api.F32, api.KVP_I32_F32, 1, 64, main_op=api.MAIN_KVP,
                       reduce_op=api.RED_ARGMIN, init_i=0, init_f=np.inf)
     r = u.gpu_reduce(d, xf)
-    assert (int(r["key"][0]), float(r["value"][0])) == (26, 0.0)
+    assert [int(r["key"][0]), float(r["value"][0])] == W64["argmin"]
 
 
 # cpp/tests/stats/sum.cu:50-98,139-140 ("Accuracy"): per column, every third row holds

@@ -10,16 +10,18 @@ from raft_amd import _capi as api
 from tests import _util as u
 
 
+GOLD = u.golden()
+
+
 # cpp/tests/linalg/reduce.cu:108-177
-@pytest.mark.parametrize("layout,apply,expected", [
-    (api.ROW_MAJOR, api.ALONG_ROWS, [4, 8, 12]),
-    (api.ROW_MAJOR, api.ALONG_COLUMNS, [9, 10, 11, 12]),
-    (api.COL_MAJOR, api.ALONG_ROWS, [10, 11, 12]),
-    (api.COL_MAJOR, api.ALONG_COLUMNS, [3, 6, 9, 12]),
-])
-def test_simple_max_fixture(oracle, layout, apply, expected):
-    data = np.arange(1, 13, dtype=np.float32)
-    d = api.make_desc(api.F32, api.F32, 3, 4, layout=layout, apply=apply, reduce_op=api.RED_MAX)
+@pytest.mark.parametrize("case", list(GOLD["reduce_simple_max"]["expected"]))
+def test_simple_max_fixture(oracle, case):
+    g = GOLD["reduce_simple_max"]
+    layout, apply = u.LAYOUT_AXIS[case]
+    expected = g["expected"][case]
+    data = np.array(g["data"], dtype=np.float32)
+    d = api.make_desc(api.F32, api.F32, g["rows"], g["cols"], layout=layout, apply=apply,
+                      reduce_op=api.RED_MAX)
     assert u.oracle_reduce(d, data).tolist() == expected
     out = np.zeros(len(expected), dtype=np.float32)
     assert u.oracle_typed(d, data, out).tolist() == expected
@@ -27,35 +29,36 @@ def test_simple_max_fixture(oracle, layout, apply, expected):
 
 # cpp/tests/matrix/argmax.cu:71-75, argmin.cu:71-75
 def test_argmax_argmin_fixture(oracle):
-    data = np.array([0.1, 0.2, 0.3, 0.4, 0.4, 0.3, 0.2, 0.1, 0.2, 0.3, 0.5, 0.0], np.float32)
-    d = api.make_desc(api.F32, api.I32, 3, 4, main_op=api.MAIN_KVP, reduce_op=api.RED_ARGMAX,
-                      final_op=api.FIN_KEY, init_f=-np.inf)
-    assert u.oracle_reduce(d, data)[0].tolist() == [3, 0, 2]
-    out = np.zeros(3, dtype=np.int32)
-    assert u.oracle_typed(d, data, out).tolist() == [3, 0, 2]
-    d = api.make_desc(api.F32, api.I32, 3, 4, main_op=api.MAIN_KVP, reduce_op=api.RED_ARGMIN,
-                      final_op=api.FIN_KEY, init_f=np.inf)
-    assert u.oracle_reduce(d, data)[0].tolist() == [0, 3, 3]
-    assert u.oracle_typed(d, data, out).tolist() == [0, 3, 3]
+    g = GOLD["matrix_arg"]
+    data = np.array(g["data"], np.float32)
+    d = api.make_desc(api.F32, api.I32, g["rows"], g["cols"], main_op=api.MAIN_KVP,
+                      reduce_op=api.RED_ARGMAX, final_op=api.FIN_KEY, init_f=-np.inf)
+    assert u.oracle_reduce(d, data)[0].tolist() == g["argmax"]
+    out = np.zeros(g["rows"], dtype=np.int32)
+    assert u.oracle_typed(d, data, out).tolist() == g["argmax"]
+    d = api.make_desc(api.F32, api.I32, g["rows"], g["cols"], main_op=api.MAIN_KVP,
+                      reduce_op=api.RED_ARGMIN, final_op=api.FIN_KEY, init_f=np.inf)
+    assert u.oracle_reduce(d, data)[0].tolist() == g["argmin"]
+    assert u.oracle_typed(d, data, out).tolist() == g["argmin"]
 
 
 # cpp/tests/util/reduction.cu:167-171,179-181
 def test_vector64_fixture(oracle):
-    from tests.test_gpu_fixtures import VEC64
-    x = np.array(VEC64, dtype=np.int32)
-    for red, init, want in [(api.RED_MIN, 2**62, 0), (api.RED_MAX, -2**62, 5),
-                            (api.RED_ADD, 0, 158)]:
+    g = GOLD["wave_vector64"]
+    x = np.array(g["data"], dtype=np.int32)
+    for red, init, want in [(api.RED_MIN, 2**62, g["min"]), (api.RED_MAX, -2**62, g["max"]),
+                            (api.RED_ADD, 0, g["sum"])]:
         d = api.make_desc(api.I32, api.I64, 1, 64, reduce_op=red, init_i=init)
         assert u.oracle_reduce(d, x).tolist() == [want]
     xf = x.astype(np.float32)
     d = api.make_desc(api.F32, api.KVP_I32_F32, 1, 64, main_op=api.MAIN_KVP,
                       reduce_op=api.RED_ARGMAX, init_f=-np.inf)
     k, v = u.oracle_reduce(d, xf)
-    assert (k[0], v[0]) == (15, 5.0)
+    assert [k[0], v[0]] == g["argmax"]
     d = api.make_desc(api.F32, api.KVP_I32_F32, 1, 64, main_op=api.MAIN_KVP,
                       reduce_op=api.RED_ARGMIN, init_f=np.inf)
     k, v = u.oracle_reduce(d, xf)
-    assert (k[0], v[0]) == (26, 0.0)
+    assert [k[0], v[0]] == g["argmin"]
 
 
 # cpp/tests/core/operators_host.cpp:134-172: truth table of argmin_op / argmax_op on
@@ -75,21 +78,20 @@ def _arg2(red, first, second):
 
 
 def test_arg_op_truth_table(oracle):
-    a, b, c = (0, np.float32(1.2)), (0, np.float32(3.4)), (1, np.float32(1.2))
+    g = GOLD["arg_op_truth_table"]
+    pair = {n: (kv[0], np.float32(kv[1])) for n, kv in g["pairs"].items()}
     f = lambda kv: (kv[0], float(kv[1]))
-    for red, table in [
-        (api.RED_ARGMIN, [(a, b, a), (b, a, a), (a, c, a), (c, a, a), (b, c, c), (c, b, c)]),
-        (api.RED_ARGMAX, [(a, b, b), (b, a, b), (a, c, a), (c, a, a), (b, c, b), (c, b, b)]),
-    ]:
+    for red, table in [(api.RED_ARGMIN, g["argmin"]), (api.RED_ARGMAX, g["argmax"])]:
         for x, y, want in table:
-            assert _arg2(red, x, y) == f(want), (red, x, y)
+            assert _arg2(red, pair[x], pair[y]) == f(pair[want]), (red, x, y)
 
 
 # cpp/tests/stats/sum.cu:50-98: triples (3v, -vL, +vL) must still sum to rows*v.
-@pytest.mark.parametrize("npdt,dt,v,L", [(np.float32, api.F32, 1e-4, 1e7),
-                                         (np.float64, api.F64, 1e-6, 1e12)])
-def test_sum_compensation_fixture(oracle, npdt, dt, v, L):
-    rows, cols = 1024, 32
+@pytest.mark.parametrize("case", GOLD["sum_accuracy"]["cases"],
+                         ids=lambda c: f"{c['dtype']}-{c['rows']}x{c['cols']}")
+def test_sum_compensation_fixture(oracle, case):
+    npdt, dt = (np.float32, api.F32) if case["dtype"] == "f32" else (np.float64, api.F64)
+    v, L, rows, cols = case["value"], case["large"], case["rows"], case["cols"]
     m = np.full((rows, cols), v, dtype=np.float64)
     for r in range(2, rows, 3):
         m[r], m[r - 1], m[r - 2] = v * L, -v * L, 3 * v
@@ -108,9 +110,10 @@ def test_sum_compensation_fixture(oracle, npdt, dt, v, L):
 
 # cpp/tests/stats/stddev.cu:139-150,187-190,198-202
 def test_stddev_fixtures(oracle):
-    rows, cols = 4096, 2
-    data = np.full(rows * cols, 1.25, dtype=np.float32)
-    mu = np.full(cols, 1.25)
+    g = GOLD["stddev_constant"]
+    rows, cols = g["rows"], g["cols"]
+    data = np.full(rows * cols, g["value"], dtype=np.float32)
+    mu = np.full(cols, g["value"])
     for sample in (False, True):
         r = 1.0 / (rows - 1 if sample else rows)
         rm = r * rows if sample else 1.0
@@ -126,13 +129,15 @@ def test_stddev_fixtures(oracle):
 
 # cpp/tests/linalg/map_then_reduce.cu:140-169
 def test_map_reduce_planted(oracle):
+    g = GOLD["map_reduce_planted"]
     rng = np.random.default_rng(1234)
-    x = rng.uniform(2.0, 3.0, 1237).astype(np.float32)
-    x[42], x[337] = 1.0, 5.0
+    x = rng.uniform(g["lo"], g["hi"], g["len"]).astype(np.float32)
+    for pos, val in g["planted"].items():
+        x[int(pos)] = val
     d = api.make_desc(api.F32, api.F32, 1, x.size, reduce_op=api.RED_MIN, init_f=np.inf)
-    assert u.oracle_reduce(d, x).tolist() == [1.0]
+    assert u.oracle_reduce(d, x).tolist() == [g["min"]]
     d = api.make_desc(api.F32, api.F32, 1, x.size, reduce_op=api.RED_MAX, init_f=-np.inf)
-    assert u.oracle_reduce(d, x).tolist() == [5.0]
+    assert u.oracle_reduce(d, x).tolist() == [g["max"]]
 
 
 # What the mathematics fixes: numpy's own reductions on a non-square random matrix for
