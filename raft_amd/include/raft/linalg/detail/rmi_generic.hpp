@@ -29,6 +29,8 @@
 #include <type_traits>
 
 #include <raft/core/error.hpp>
+#include <raft/core/operators.hpp>
+#include <raft/linalg/detail/map.cuh>
 #include <raft/linalg/detail/rmi_scratch.hpp>
 
 namespace raft::detail::rmi::generic {
@@ -353,6 +355,94 @@ void reduce(hipStream_t stream, Out* dots, const In* data, std::int64_t n_rows,
     const Idx D = row_major ? n_cols : n_rows, N = row_major ? n_rows : n_cols;
     strided<In, Out, Idx>(dots, data, D, N, init, stream, inplace, main_op, red, fin);
   }
+}
+
+// ---- map over several equally long arrays, then reduce to one value -------------------
+// out = fold over i of map(in[i], args[i]...) starting from `neutral`
+// (linalg/detail/map_then_reduce.cuh:47-95 in the reference, whose blocks accumulate
+// into the output with atomics; here partials are folded in a fixed order).  Lanes move
+// packs of R elements per array as the elementwise map does.
+template <int R, typename Out, typename Map, typename Red, typename... Done>
+__device__ __forceinline__ void fold_pack_set(Out& acc, Map& map, Red& red,
+                                              const raft::linalg::detail::map_pack_set<R>&,
+                                              const raft::linalg::detail::map_pack<Done, R>&... xs)
+{
+#pragma unroll
+  for (int j = 0; j < R; ++j)
+    acc = red(acc, static_cast<Out>(map(xs.v[j]...)));
+}
+template <int R, typename Out, typename Map, typename Red, typename T, typename... Rest,
+          typename... Done>
+__device__ __forceinline__ void fold_pack_set(
+  Out& acc, Map& map, Red& red, const raft::linalg::detail::map_pack_set<R, T, Rest...>& s,
+  const raft::linalg::detail::map_pack<Done, R>&... xs)
+{
+  fold_pack_set<R>(acc, map, red, s.tail, xs..., s.head);
+}
+
+template <int R, typename Out, typename Map, typename Red, typename... InTs>
+__global__ __launch_bounds__(kBlock) void map_reduce_multi_kernel(Out* partial, std::int64_t len,
+                                                                  std::int64_t packs_per_block,
+                                                                  Out neutral, Map map, Red red,
+                                                                  const InTs*... ins)
+{
+  constexpr int U = 4;
+  __shared__ Out sm[kBlock / kWave];
+  const std::int64_t npack = len / R;
+  const std::int64_t begin = (std::int64_t)blockIdx.x * packs_per_block;
+  const std::int64_t end   = begin + packs_per_block < npack ? begin + packs_per_block : npack;
+  Out acc                  = neutral;
+  for (std::int64_t p0 = begin + threadIdx.x; p0 < end; p0 += (std::int64_t)kBlock * U) {
+    raft::linalg::detail::map_pack_set<R, InTs...> held[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const std::int64_t p = p0 + (std::int64_t)u * kBlock;
+      if (p < end) raft::linalg::detail::map_load_set(held[u], p * R, ins...);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const std::int64_t p = p0 + (std::int64_t)u * kBlock;
+      if (p < end) fold_pack_set<R>(acc, map, red, held[u]);
+    }
+  }
+  // the last len % R elements, on the first workgroup
+  const std::int64_t i = npack * R + (std::int64_t)threadIdx.x;
+  if (blockIdx.x == 0 && i < len) acc = red(acc, static_cast<Out>(map(ins[i]...)));
+  acc = group_reduce(acc, kWave, red);
+  if ((threadIdx.x & (kWave - 1)) == 0) sm[threadIdx.x >> 6] = acc;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < kBlock / kWave; ++w)
+      acc = red(acc, sm[w]);
+    partial[blockIdx.x] = acc;
+  }
+}
+
+template <typename Out, typename Map, typename Red, typename... InTs>
+void map_reduce_multi(hipStream_t stream, Out* out, std::int64_t len, Out neutral, Map map, Red red,
+                      const InTs*... ins)
+{
+  using raft::linalg::detail::map_min;
+  using raft::linalg::detail::map_ratio_of;
+  constexpr int R                = map_min(16, map_ratio_of<InTs>()...);
+  constexpr std::int64_t quantum = (std::int64_t)kBlock * 4;  // packs per block sweep
+  const std::int64_t npack       = len / R;
+  std::int64_t B                 = (npack + quantum - 1) / quantum;
+  if (B > 1024) B = 1024;
+  if (B < 1) B = 1;
+  std::int64_t per = (npack + B - 1) / B;
+  per              = (per + quantum - 1) / quantum * quantum;
+  if (per < quantum) per = quantum;
+  B = (npack + per - 1) / per;
+  if (B < 1) B = 1;
+  Out* partial = static_cast<Out*>(scratch_alloc(sizeof(Out) * (std::size_t)B, stream));
+  hipLaunchKernelGGL((map_reduce_multi_kernel<R, Out, Map, Red, InTs...>), dim3((unsigned)B),
+                     dim3(kBlock), 0, stream, partial, len, per, neutral, map, red, ins...);
+  check_launch("map_reduce_multi_kernel");
+  launch_fold(out, partial, (std::int64_t)1, (int)B, neutral, false, red, raft::identity_op(),
+              stream);
+  check_launch("fold_kernel");
+  scratch_free(partial, stream);
 }
 
 }  // namespace raft::detail::rmi::generic

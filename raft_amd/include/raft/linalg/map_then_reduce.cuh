@@ -25,12 +25,20 @@ struct unary_map_adapter {
 template <typename InType, typename OutType, typename MapOp, typename ReduceLambda,
           typename... Args>
 void map_reduce_call(const resources* res, OutType* out, size_t len, OutType neutral, MapOp map,
-                     ReduceLambda op, hipStream_t stream, const InType* in, Args...)
+                     ReduceLambda op, hipStream_t stream, const InType* in, Args... args)
 {
-  static_assert(sizeof...(Args) == 0,
-                "map-then-reduce over several input arrays is not lowered to the reduction "
-                "library; only map(in[i]) is");
-  if constexpr (raft::detail::rmi::main_tag<MapOp>::value >= 0) {
+  if constexpr (sizeof...(Args) > 0) {
+    // map(in[i], args[i]...) over several arrays: arbitrary device code by nature
+#if defined(__HIPCC__)
+    (void)res;
+    raft::detail::rmi::generic::map_reduce_multi(stream, out, (std::int64_t)len, neutral, map, op,
+                                                 in, args...);
+#else
+    static_assert(sizeof...(Args) == 0,
+                  "map-then-reduce over several input arrays runs device code of the caller: "
+                  "compile this translation unit with hipcc");
+#endif
+  } else if constexpr (raft::detail::rmi::main_tag<MapOp>::value >= 0) {
     raft::detail::rmi::reduce(res, stream, out, in, std::int64_t(1), (std::int64_t)len, true,
                               true, neutral, false, map, op, raft::identity_op());
   } else {

@@ -338,6 +338,51 @@ void weighted_mean_cases(double tol)
 TEST_CASE(WeightedMeanF) { weighted_mean_cases<float>(1e-6); }
 TEST_CASE(WeightedMeanD) { weighted_mean_cases<double>(1e-14); }
 
+// map over two arrays, then sum: the call shape of linalg/detail/mean_squared_error.cuh:18-24
+// (sq_diff(a, b) summed over two arrays) and stats/detail/kl_divergence.cuh:62
+TEST_CASE(MapReduceTwoArrays)
+{
+  raft::resources handle;
+  auto stream = raft::resource::get_cuda_stream(handle);
+  for (int len : {0, 1, 3, 1000, 4099, (1 << 20) + 5, (1 << 24) + 1}) {
+    auto ha = uniform<float>((size_t)len, -1.0, 1.0, 31);
+    auto hb = uniform<float>((size_t)len, -1.0, 1.0, 32);
+    auto da = raft::make_device_vector<float, int>(handle, len + 1);
+    auto db = raft::make_device_vector<float, int>(handle, len + 1);
+    auto out = raft::make_device_scalar<double>(handle);
+    // one element of slack in front: element-aligned, not 16-byte aligned
+    raft::update_device(da.data_handle() + 1, ha.data(), ha.size(), stream);
+    raft::update_device(db.data_handle() + 1, hb.data(), hb.size(), stream);
+    const float weight = 0.5f;
+    auto sq_diff       = [weight] __device__(float a, float b) {
+      const double d = (double)a - (double)b;
+      return d * d * weight;
+    };
+    raft::linalg::mapThenSumReduce<float, decltype(sq_diff), std::uint32_t, 256, const float*>(
+      out.data_handle(), (std::uint32_t)len, sq_diff, stream, da.data_handle() + 1,
+      (const float*)(db.data_handle() + 1));
+    double want = 0;
+    for (int i = 0; i < len; ++i) {
+      const double d = (double)ha[i] - (double)hb[i];
+      want += d * d * 0.5;
+    }
+    CHECK(close(to_host(out.data_handle(), 1, stream)[0], want, 1e-9));
+    // a maximum over three arrays through mapReduce
+    auto dc = raft::make_device_vector<float, int>(handle, len + 1);
+    raft::update_device(dc.data_handle(), ha.data(), ha.size(), stream);
+    auto outf = raft::make_device_scalar<float>(handle);
+    raft::linalg::mapReduce<float>(
+      outf.data_handle(), (size_t)len, -1e30f,
+      [] __device__(float a, float b, float c) { return a * b + c; }, raft::max_op(), stream,
+      (const float*)(da.data_handle() + 1), (const float*)(db.data_handle() + 1),
+      (const float*)dc.data_handle());
+    float wantf = -1e30f;
+    for (int i = 0; i < len; ++i)
+      wantf = std::max(wantf, ha[i] * hb[i] + ha[i]);
+    CHECK(close(to_host(outf.data_handle(), 1, stream)[0], wantf, 1e-6));
+  }
+}
+
 int main()
 {
   int n = 0;

@@ -40,3 +40,11 @@ def test_cpp_generic_functors_on_gpu(gpu):
     a hipcc translation unit by the header fallback (tests/cpp/test_raft_generic.hip)."""
     out = _run("test_raft_generic", 600)
     assert "0 failed" in out
+
+
+@pytest.mark.gpu
+def test_cpp_map_family_on_gpu(gpu):
+    """raft::linalg::map / map_offset / unaryOp / writeOnlyUnaryOp / binaryOp
+    (tests/cpp/test_raft_map.hip, compiled by hipcc)."""
+    out = _run("test_raft_map", 600)
+    assert "0 failed" in out
