@@ -22,7 +22,7 @@ namespace rmi {
 constexpr int kBlock      = 256;  // threads per workgroup (the team kernel may use up to 1024)
 constexpr int kUnroll     = 4;    // independent 16-byte loads in flight per lane
 constexpr int kColUnroll  = 4;    // rows per lane and tile in the column kernel
-constexpr int kTeamUnroll = 8;    // loads in flight per lane in the team-per-row kernel
+constexpr int kTeamUnroll = 4;    // lane-loads per batch in the team-per-row kernel
 
 struct RowArgs {
   const void* in;
@@ -311,7 +311,7 @@ __global__ __launch_bounds__(kBlock) void row_wave_kernel(RowArgs a)
 
 // ---------------------------------------------------------------------------
 // Teams of T = 64 << logT threads (1..16 waves); each team sweeps one chunk of
-// one row with kTeamUnroll loads in flight per lane.  A workgroup holds
+// one row in batches of kTeamUnroll loads per lane.  A workgroup holds
 // blockDim.x / T teams.  B chunks per row: B == 1 writes outputs, B > 1 writes
 // partials for the second pass.
 // ---------------------------------------------------------------------------
@@ -343,14 +343,47 @@ __global__ __launch_bounds__(1024) void row_block_kernel(RowArgs a)
     const i64 v1   = (v0 + a.chunk < a.nvec) ? (v0 + a.chunk) : a.nvec;
     const char* rp = static_cast<const char*>(a.in) + row * a.row_bytes;
     i64 v          = v0 + t;
-    for (; v + (U - 1) * (i64)T < v1; v += (i64)U * T) {
+    // A chunk of fewer than three batches per thread is read 2 * U lane-loads at a
+    // time: all of it is in flight at once and the accumulate step starts as the first
+    // vectors arrive.
+    if (a.chunk < (i64)3 * U * T) {
+      constexpr int W = 2 * U;
+      for (; v + (W - 1) * (i64)T < v1; v += (i64)W * T) {
+        typename H::type x[W];
+#pragma unroll
+        for (int u = 0; u < W; ++u)
+          x[u] = H::load(rp, v + (i64)u * T);
+#pragma unroll
+        for (int u = 0; u < W; ++u)
+          H::push(acc, x[u], (v + (i64)u * T) * S);
+      }
+    }
+    // Whole batches of U lane-loads; the next batch is issued before the current one is
+    // accumulated, so its latency overlaps the arithmetic (the loop holds no stores:
+    // gfx9 counts loads and stores in one in-order counter).
+    if (v + (U - 1) * (i64)T < v1) {
       typename H::type x[U];
 #pragma unroll
       for (int u = 0; u < U; ++u)
         x[u] = H::load(rp, v + (i64)u * T);
+      for (;;) {
+        const i64 vn    = v + (i64)U * T;
+        const bool more = vn + (U - 1) * (i64)T < v1;
+        typename H::type y[U];
+        if (more) {
 #pragma unroll
-      for (int u = 0; u < U; ++u)
-        H::push(acc, x[u], (v + (i64)u * T) * S);
+          for (int u = 0; u < U; ++u)
+            y[u] = H::load(rp, vn + (i64)u * T);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+          H::push(acc, x[u], (v + (i64)u * T) * S);
+        v = vn;
+        if (!more) break;
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+          x[u] = y[u];
+      }
     }
     if (v < v1) {  // fewer than U lane-loads left for this lane
       typename H::type x[U - 1];

@@ -102,7 +102,7 @@ int run(const PlanX& pl, const Problem& pr, hipStream_t st)
       } else {
         const dim3 block((unsigned)(pl.threads < kBlock ? kBlock : pl.threads));
         if (pl.vec16)
-          hipLaunchKernelGGL((row_block_kernel<P, true>), grid, block, 0, st, a);
+          hipLaunchKernelGGL((row_block_kernel<P, true>), grid, block, lds, st, a);
         else
           hipLaunchKernelGGL((row_block_kernel<P, false>), grid, block, 0, st, a);
         if (pl.kind == RMI_PLAN_ROW_SPLIT) rc = launch_fold<P>(pl, pr, pl.B, st);

@@ -19,7 +19,8 @@ namespace rmi {
 
 constexpr int kPlanBlock  = 256;
 constexpr int kPlanUnroll = 4;      // lane-loads in flight: sub-wave and column kernels
-constexpr int kPlanTeamUnroll = 8;  // lane-loads in flight: team-per-row kernel
+constexpr int kPlanTeamUnroll = 4;  // lane-loads per batch: team-per-row kernel
+constexpr int kTeamMinLoads   = 16; // a thread of a widened team keeps at least this many loads
 constexpr int kWavesPerCu = 32;  // 8 resident waves on each of the 4 SIMDs
 // Workgroups per CU of the persistent column kernel.  Measured on MI355X: with two
 // tiles in flight per workgroup, 2 per CU (8 waves) sustains ~7.1 TB/s; 4 and 8 per CU
@@ -279,12 +280,24 @@ inline int make_plan(const rmi_reduce_desc& d,
       kind = RMI_PLAN_ROW_WAVE;
     } else {
       // widen the team on a row until the machine's wave slots are filled, as long
-      // as every thread keeps a full batch of lane-loads
+      // as every thread keeps kTeamMinLoads lane-loads
       while (threads < 1024 && p.n_out * (threads / 64) < slots &&
-             p.nvec >= (int64_t)2 * threads * kPlanTeamUnroll)
+             p.nvec >= (int64_t)kTeamMinLoads * threads)
         threads *= 2;
+      // Long rows: a team wide enough that a thread sees two to four batches (sums) or
+      // four to eight (arg-reductions, whose accumulate step is longer).  One wave
+      // streaming a long row alone leaves thousands of row streams open at once, which
+      // measured 3-7 points slower than 128- or 256-thread teams.
+      {
+        const bool kvp     = key.family == kFamKvp;
+        const int64_t want = p.nvec / (kvp ? 16 : 8);
+        int wide           = kvp ? 64 : 128;
+        while (wide < 256 && wide * 2 <= want)
+          wide *= 2;
+        if (wide > threads) threads = wide;
+      }
       if (threads == 1024 && p.n_out * 16 < slots &&
-          p.nvec >= (int64_t)2 * kPlanBlock * kPlanTeamUnroll) {
+          p.nvec >= (int64_t)kTeamMinLoads * kPlanBlock) {
         kind = RMI_PLAN_ROW_SPLIT;
       } else {
         kind = RMI_PLAN_ROW_BLOCK;
@@ -330,11 +343,21 @@ inline int make_plan(const rmi_reduce_desc& d,
     p.chunk       = p.nvec;
     const int teams = threads >= kPlanBlock ? 1 : kPlanBlock / threads;
     p.grid_blocks   = ceildiv(p.n_out, teams);
+    if (threads <= kPlanBlock && p.vec16 && p.grid_blocks > (int64_t)8 * n_cu) {
+      // More workgroups than fit at once: the resident 256-thread workgroups per CU are
+      // capped by a dynamic LDS reservation the kernel never touches.  4 keep 64-128 KB
+      // in flight per CU, which measured best across row lengths and accumulators; 3
+      // gain another 3 points for sums over rows of 128 KB and more (eight or more
+      // batches per thread) and lose 20 on arg-reductions.
+      const bool deep = threads == kPlanBlock && key.family != kFamKvp &&
+                        p.nvec >= (int64_t)8 * kPlanTeamUnroll * kPlanBlock;
+      p.lds_reserve   = kLdsPerCu / (deep ? 3 : 4) - 768;
+    }
   } else {
     p.kind        = RMI_PLAN_ROW_SPLIT;
     p.team_kernel = true;
     p.threads     = kPlanBlock;
-    const int64_t quantum = (int64_t)kPlanBlock * kPlanTeamUnroll;
+    const int64_t quantum = (int64_t)kPlanBlock * 8;
     int64_t B             = ceildiv(slots, p.n_out * (kPlanBlock / 64));
     const int64_t maxB    = p.nvec / quantum > 1 ? p.nvec / quantum : 1;
     if (B > maxB) B = maxB;

@@ -152,7 +152,7 @@ TEST_CASE(plan_selector)
   p = plan(RMI_F32, RMI_F32, 10000000, 64, RMI_ALONG_COLUMNS);
   CHECK(p.kind == RMI_PLAN_COL_TILE && p.n_outputs == 64 && p.reduce_len == 10000000);
   p = plan(RMI_F32, RMI_KVP_I32_F32, 65536, 32000, RMI_ALONG_ROWS, RMI_RED_ARGMAX, RMI_MAIN_KVP);
-  CHECK(p.kind == RMI_PLAN_ROW_WAVE && p.lanes_per_row == 64);
+  CHECK(p.kind == RMI_PLAN_ROW_BLOCK && p.block_threads == 256 && p.passes == 1);
   p = plan(RMI_F32, RMI_F32, 100, 7);
   CHECK(p.vec_bytes == 16);  // 28-byte rows: one 16-byte lane load and three tail elements
   p = plan(RMI_F32, RMI_F32, 100, 3);

@@ -65,7 +65,7 @@ BENCH_SHAPES = [
      api.PLAN_ROW_WAVE, 1),
     (api.F32, api.F32, 10000000, 64, dict(apply=api.ALONG_COLUMNS), api.PLAN_COL_TILE, 2),
     (api.F32, api.KVP_I32_F32, 65536, 32000,
-     dict(main_op=api.MAIN_KVP, reduce_op=api.RED_ARGMAX), api.PLAN_ROW_WAVE, 1),
+     dict(main_op=api.MAIN_KVP, reduce_op=api.RED_ARGMAX), api.PLAN_ROW_BLOCK, 1),
     (api.I8, api.I64, 4096, 16384, {}, api.PLAN_ROW_BLOCK, 1),
     (api.I8, api.I64, 16777216, 8, {}, api.PLAN_ROW_LANES, 1),
     (api.BF16, api.F32, 8, 4194304, {}, api.PLAN_ROW_SPLIT, 2),
