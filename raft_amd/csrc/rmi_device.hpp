@@ -616,18 +616,6 @@ __device__ __forceinline__ void push_vec_from(typename P::acc_t& a,
   });
 }
 
-template <class P>
-__device__ __forceinline__ void push_cols_from(typename P::acc_t (&a)[P::VEC],
-                                               const u32x4& v,
-                                               i64 idx,
-                                               int skip)
-{
-  using in_t = typename P::in_t;
-  static_for<P::VEC>([&](auto j) {
-    if (j >= skip) P::push(a[j], In<in_t>::template get<j>(v), idx);
-  });
-}
-
 // ---------------------------------------------------------------------------
 // Wave-level all-reduce over groups of G lanes (G a power of two, 1..64).
 // G is wave-uniform at run time; every lane of the wave must call this.

@@ -457,19 +457,13 @@ __global__ __launch_bounds__(kBlock) void col_kernel(ColArgs a)
     acc[j] = P::neutral();
 
   if constexpr (VEC16) {
-    // MASKED: the row length is not a multiple of the vector width.  The partial
-    // group's vector ends at the row's end and its first `skip` columns belong to the
-    // group before it; all lanes then run the masked accumulate (skip == 0 for whole
-    // groups) so that a wave stays on one instruction stream.
-    auto sweep = [&](const char* p, int skip, auto masked) {
-      auto take = [&](const u32x4& v, i64 r) {
-        if constexpr (decltype(masked)::value) {
-          push_cols_from<P>(acc, v, r, skip);
-        } else {
-          P::push_cols(acc, v, r);
-        }
-      };
-      i64 tile = blockIdx.y;
+    // The row length need not be a multiple of the vector width: the last, partial
+    // group of columns reads the vector that ends at the row's end.  Its first
+    // S - tail columns belong to the group before it; they are accumulated here a
+    // second time and dropped at the end, which is cheaper than masking every step.
+    if (whole || part) {
+      const char* p = whole ? inb + cv * 16 : inb + (a.n_out - S) * (i64)sizeof(in_t);
+      i64 tile      = blockIdx.y;
       u32x4 x[kColUnroll];
       if (tile < n_full) {
 #pragma unroll
@@ -486,7 +480,7 @@ __global__ __launch_bounds__(kBlock) void col_kernel(ColArgs a)
         }
 #pragma unroll
         for (int u = 0; u < kColUnroll; ++u)
-          take(x[u], tile * RT + ty + (i64)u * TY);
+          P::push_cols(acc, x[u], tile * RT + ty + (i64)u * TY);
 #pragma unroll
         for (int u = 0; u < kColUnroll; ++u)
           x[u] = y[u];
@@ -494,14 +488,8 @@ __global__ __launch_bounds__(kBlock) void col_kernel(ColArgs a)
       }
       if ((i64)blockIdx.y == n_full % a.B) {  // the rows past the last whole tile
         for (i64 r = n_full * RT + ty; r < a.len; r += TY)
-          take(load16(p + r * a.row_bytes), r);
+          P::push_cols(acc, load16(p + r * a.row_bytes), r);
       }
-    };
-    if (a.tail == 0) {
-      if (whole) sweep(inb + cv * 16, 0, std::false_type{});
-    } else if (whole || part) {
-      const char* p = whole ? inb + cv * 16 : inb + (a.n_out - S) * (i64)sizeof(in_t);
-      sweep(p, whole ? 0 : S - a.tail, std::true_type{});
     }
   } else if (whole) {
     const in_t* p = reinterpret_cast<const in_t*>(inb) + cv;
