@@ -572,12 +572,23 @@ struct PolMeanVar {
     a.sdd = fma(d, d, a.sdd);
     a.w += 1.0;
   }
+  // One shifted step without the first-value test (the caller has set a.k).
+  static __device__ __forceinline__ void step(acc_t& a, double xd)
+  {
+    const double d = xd - a.k;
+    a.sd += d;
+    a.sdd = fma(d, d, a.sdd);
+  }
   static __device__ __forceinline__ void push_vec(acc_t& a, const u32x4& v, i64)
   {
-    static_for<VEC>([&](auto j) { push(a, In<InT>::template get<j>(v), 0); });
+    // the shift is tested once per vector, behind a branch that is taken once per lane
+    if (a.w == 0.0) a.k = (double)In<InT>::template get<0>(v);
+    static_for<VEC>([&](auto j) { step(a, (double)In<InT>::template get<j>(v)); });
+    a.w += (double)VEC;
   }
   static __device__ __forceinline__ void push_cols(acc_t (&a)[VEC], const u32x4& v, i64)
   {
+    // per-column selects: a branch here measured slower on ragged widths
     static_for<VEC>([&](auto j) { push(a[j], In<InT>::template get<j>(v), 0); });
   }
   static __device__ __forceinline__ void merge(acc_t& a, const acc_t& b)
