@@ -48,3 +48,18 @@ def test_cpp_map_family_on_gpu(gpu):
     (tests/cpp/test_raft_map.hip, compiled by hipcc)."""
     out = _run("test_raft_map", 600)
     assert "0 failed" in out
+
+
+@pytest.mark.gpu
+def test_bench_program_runs_on_gpu(gpu):
+    """The benchmark program over the reference's shape grids starts, runs one small grid
+    and prints one line per case (raft_amd/bench/prims_bench.hip)."""
+    exe = BIN.parent.parent.parent / "raft_amd" / "bench" / "bin" / "prims_bench"
+    if not exe.exists():
+        from raft_amd import build
+        build.build_bench()
+    proc = subprocess.run([str(exe), "--filter", "rowNorm<float,int>", "--min-iters", "2"],
+                          capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stdout[-2000:] + proc.stderr[-2000:]
+    lines = [l for l in proc.stdout.splitlines() if l.startswith("rowNorm<float,int>")]
+    assert len(lines) == 35 and all("GB/s" in l for l in lines)
