@@ -1,0 +1,167 @@
+// Host-only property test of the launch-plan selector (raft_amd/csrc/rmi_plan.hpp), built
+// with -fsanitize=address,undefined: random and extreme shapes, every dtype and hint, and the
+// invariants the kernels and the host checks rely on (coverage of the row by the chunks,
+// lane groups that hold the whole row, grid and workspace sizes, LDS reservations).
+#include <cstdio>
+#include <cstdlib>
+#include <random>
+
+#include "../../raft_amd/csrc/rmi_plan.hpp"
+
+namespace {
+int failures = 0;
+long planned[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+#define REQUIRE(cond)                                                              \
+  do {                                                                             \
+    if (!(cond)) {                                                                 \
+      if (++failures < 20)                                                         \
+        std::printf("  %s:%d: %s  [dtype %d layout %d apply %d rows %lld cols %lld hint %d]\n", \
+                    __FILE__, __LINE__, #cond, d.in_dtype, d.layout, d.apply,      \
+                    (long long)d.n_rows, (long long)d.n_cols, d.plan_hint);        \
+    }                                                                              \
+  } while (0)
+
+void check(const rmi_reduce_desc& d, int n_cu)
+{
+  using namespace rmi;
+  PolicyKey key;
+  int acc_bytes = 0;
+  const int rc  = classify(d, key, acc_bytes);
+  if (rc != RMI_OK) return;
+  PlanX p;
+  const int prc = make_plan(d, key, acc_bytes, n_cu, p);
+  if (prc != RMI_OK) {
+    REQUIRE(prc == RMI_ERR_BAD_SHAPE);
+    return;
+  }
+  ++planned[p.kind];
+  const bool row_major  = d.layout == RMI_ROW_MAJOR;
+  const bool along_rows = d.apply == RMI_ALONG_ROWS;
+  const int64_t contiguous = row_major ? d.n_cols : d.n_rows;
+  const int64_t other      = row_major ? d.n_rows : d.n_cols;
+  REQUIRE(p.strided == (row_major != along_rows));
+  REQUIRE(p.n_out == (p.strided ? contiguous : other));
+  REQUIRE(p.len == (p.strided ? other : contiguous));
+  if (p.n_out == 0) {
+    REQUIRE(p.kind == RMI_PLAN_EMPTY && p.passes == 0);
+    return;
+  }
+  if (p.len == 0) {
+    REQUIRE(p.kind == RMI_PLAN_EMPTY && p.grid_blocks >= 1);
+    return;
+  }
+  REQUIRE(p.grid_blocks >= 1 && p.grid_blocks <= 0x7fffffffLL);
+  REQUIRE(p.lds_reserve >= 0 && p.lds_reserve <= 64 * 1024);
+  REQUIRE((p.ws_bytes > 0) == (p.passes == 2));
+  REQUIRE(p.B >= 1 && p.B <= 4096);
+  if (p.passes == 2) REQUIRE(p.ws_bytes == (size_t)p.n_out * p.B * acc_bytes);
+  const int es = dtype_size(d.in_dtype);
+  if (p.kind != RMI_PLAN_ROW_LANES) {
+    REQUIRE(p.row_bytes == contiguous * es);
+    REQUIRE(p.vec16 == (p.row_bytes >= 16));
+    REQUIRE(p.nvec * p.step + p.tail == contiguous);
+    REQUIRE(p.tail >= 0 && p.tail < p.step);
+  }
+  const int64_t nload = p.nvec + (p.tail > 0 ? 1 : 0);
+  switch (p.kind) {
+    case RMI_PLAN_ROW_LANES:
+      REQUIRE(!p.strided && p.K >= 2 && p.K <= 16 && p.K * contiguous * es == 16);
+      break;
+    case RMI_PLAN_ROW_WAVE:
+      REQUIRE(!p.strided);
+      if (p.team_kernel) {
+        REQUIRE(p.threads == 64 && p.B == 1 && p.chunk == p.nvec);
+      } else {
+        REQUIRE(p.G >= 1 && p.G <= 64 && (p.G & (p.G - 1)) == 0 && (1 << p.logG) == p.G);
+        // the lanes of a row hold all of its lane-loads, kPlanUnroll apiece (one for short rows)
+        REQUIRE((int64_t)p.G * (p.short_rows ? 1 : kPlanUnroll) >= nload);
+      }
+      break;
+    case RMI_PLAN_ROW_BLOCK:
+      REQUIRE(!p.strided && p.team_kernel && p.B == 1 && p.chunk == p.nvec);
+      REQUIRE(p.threads >= 64 && p.threads <= 1024 && (p.threads & (p.threads - 1)) == 0);
+      break;
+    case RMI_PLAN_ROW_SPLIT:
+      REQUIRE(!p.strided && p.team_kernel && p.B >= 2 && p.threads == kPlanBlock);
+      REQUIRE(p.chunk > 0 && (int64_t)p.B * p.chunk >= p.nvec && (int64_t)(p.B - 1) * p.chunk < p.nvec);
+      REQUIRE(p.grid_blocks == p.n_out * p.B);
+      break;
+    case RMI_PLAN_COL_TILE:
+      REQUIRE(p.strided);
+      REQUIRE(p.TX >= 1 && p.TX <= 64 && (p.TX & (p.TX - 1)) == 0 && (1 << p.logTX) == p.TX);
+      REQUIRE(p.gridx * p.TX >= nload && (p.gridx - 1) * p.TX < nload);
+      REQUIRE(p.grid_blocks == p.gridx * p.B);
+      break;
+    default: REQUIRE(false);
+  }
+  rmi_plan out{};
+  export_plan(p, out);
+  REQUIRE(out.n_outputs == p.n_out && out.reduce_len == p.len && out.workspace_bytes == p.ws_bytes);
+}
+}  // namespace
+
+int main()
+{
+  std::mt19937_64 g(20240607);
+  auto pick = [&](std::initializer_list<int64_t> v) {
+    return *(v.begin() + (size_t)(g() % v.size()));
+  };
+  long cases = 0;
+  for (int it = 0; it < 400000; ++it) {
+    rmi_reduce_desc d{};
+    d.in_dtype  = (int)(g() % 8);
+    d.layout    = (int)(g() % 2);
+    d.apply     = (int)(g() % 2);
+    d.plan_hint = (int)(g() % 7);
+    const int kind = (int)(g() % 4);
+    if (kind == 0) {  // sums
+      d.out_dtype = d.in_dtype >= RMI_F16 ? RMI_F32 : (g() % 2 ? RMI_I64 : RMI_F32);
+      d.reduce_op = RMI_RED_ADD;
+    } else if (kind == 1) {  // min / max
+      d.out_dtype = d.in_dtype >= RMI_F16 ? RMI_F64 : RMI_I64;
+      d.reduce_op = g() % 2 ? RMI_RED_MAX : RMI_RED_MIN;
+    } else {  // arg reductions
+      d.main_op   = RMI_MAIN_KVP;
+      d.reduce_op = g() % 2 ? RMI_RED_ARGMAX : RMI_RED_ARGMIN;
+      d.out_dtype = d.in_dtype == RMI_F64 ? (g() % 2 ? RMI_KVP_I32_F64 : RMI_KVP_I64_F64)
+                                          : (g() % 2 ? RMI_KVP_I32_F32 : RMI_KVP_I64_F32);
+    }
+    // log-uniform extents with the edge values mixed in
+    auto extent = [&]() -> int64_t {
+      if (g() % 8 == 0) return pick({0, 1, 2, 3, 7, 15, 16, 17, 63, 64, 65, 255, 256, 257, 1023, 1024, 1025, 4095, 4096, 4097});
+      const int bits = (int)(g() % 34);
+      return (int64_t)(g() & ((1ull << bits) - 1)) + (g() % 2);
+    };
+    d.n_rows = extent();
+    d.n_cols = extent();
+    // keep the element count within what one GPU could hold (2^38), larger ones are
+    // rejected or planned just the same but are not interesting
+    if ((long double)d.n_rows * (long double)d.n_cols > 274877906944.0L) d.n_cols = d.n_cols % 4096;
+    for (int n_cu : {256, 1, 304})
+      check(d, n_cu);
+    ++cases;
+  }
+  // the extremes the header promises to reject
+  {
+    rmi_reduce_desc d{};
+    d.in_dtype = RMI_F32, d.out_dtype = RMI_F32;
+    d.n_rows = ((int64_t)1 << 41), d.n_cols = 1;
+    rmi::PolicyKey key;
+    int acc = 0;
+    rmi::PlanX p;
+    if (rmi::classify(d, key, acc) == RMI_OK && rmi::make_plan(d, key, acc, 256, p) != RMI_ERR_BAD_SHAPE) {
+      std::printf("  2^41 rows accepted\n");
+      ++failures;
+    }
+  }
+  std::printf("plans checked: lanes %ld wave %ld block %ld split %ld col %ld empty %ld\n",
+              planned[RMI_PLAN_ROW_LANES], planned[RMI_PLAN_ROW_WAVE], planned[RMI_PLAN_ROW_BLOCK],
+              planned[RMI_PLAN_ROW_SPLIT], planned[RMI_PLAN_COL_TILE], planned[RMI_PLAN_EMPTY]);
+  for (int k = RMI_PLAN_ROW_LANES; k <= RMI_PLAN_EMPTY; ++k)
+    if (planned[k] < 1000) {
+      std::printf("  plan kind %d was hardly exercised\n", k);
+      ++failures;
+    }
+  std::printf("%ld descriptors, %d failed\n", cases, failures);
+  return failures == 0 ? 0 : 1;
+}

@@ -28,6 +28,13 @@ def test_cpp_host_layer():
     assert "0 failed" in out
 
 
+def test_plan_selector_properties():
+    """400000 random and extreme descriptors through the plan selector under ASan / UBSan
+    (tests/cpp/test_plan_fuzz.cpp): the invariants kernels and host checks rely on."""
+    out = _run("test_plan_fuzz", 120)
+    assert "0 failed" in out
+
+
 @pytest.mark.gpu
 def test_cpp_api_on_gpu(gpu):
     out = _run("test_raft_api", 600)
