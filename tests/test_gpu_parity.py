@@ -64,6 +64,29 @@ def test_reduce_thick(gpu, rows, cols):
         u.check_against_oracle(d, data, label=f"thick {rows}x{cols} l{layout} a{apply}")
 
 
+# Many long rows: the automatic plan gives each row a team of 64, 128 or 256 threads
+# depending on the row's length and the accumulator; lengths straddle the team sizes and
+# leave ragged last batches and tail elements.
+@pytest.mark.parametrize("in_dt,out_dt,kw", [
+    (api.F32, api.F32, dict(main_op=api.MAIN_SQ)),
+    (api.F64, api.F64, {}),
+    (api.BF16, api.F32, dict(main_op=api.MAIN_ABS)),
+    (api.I8, api.I64, {}),
+    (api.F32, api.KVP_I32_F32, dict(main_op=api.MAIN_KVP, reduce_op=api.RED_ARGMAX, init_f=-np.inf)),
+    (api.F64, api.I64, dict(main_op=api.MAIN_KVP, reduce_op=api.RED_ARGMIN, final_op=api.FIN_KEY,
+                            init_f=np.inf)),
+])
+@pytest.mark.parametrize("rows,cols", [(3000, 1029), (3000, 2051), (2500, 4099), (2100, 8197),
+                                       (2100, 16390), (1100, 33001)])
+def test_many_long_rows(gpu, in_dt, out_dt, kw, rows, cols):
+    rng = np.random.default_rng(rows + cols)
+    data = _rand(rng, in_dt, rows * cols)
+    d = api.make_desc(in_dt, out_dt, rows, cols, **kw)
+    p = api.plan_query(d)
+    assert p.kind in (api.PLAN_ROW_WAVE, api.PLAN_ROW_BLOCK) and p.passes == 1
+    u.check_against_oracle(d, data, label=f"long rows {rows}x{cols} dt{in_dt}")
+
+
 # cpp/tests/linalg/coalesced_reduction.cu:109-139: 10000 x {3..270}, 10 x 25000, ...
 @pytest.mark.parametrize("rows,cols", [(10000, c) for c in
                                        (3, 5, 7, 9, 17, 31, 32, 33, 55, 63, 64, 65, 128, 270)]
