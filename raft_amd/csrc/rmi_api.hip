@@ -45,14 +45,16 @@ run_fn lookup(const PolicyKey& k)
 
 bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 
-int plan_for(const rmi_reduce_desc* desc, PlanX& pl, PolicyKey& key)
+// `in` is the input pointer when the plan is made for a launch (its position within a
+// 128-byte line decides whether rows are staged through LDS), nullptr for queries.
+int plan_for(const rmi_reduce_desc* desc, PlanX& pl, PolicyKey& key, const void* in = nullptr)
 {
   if (desc == nullptr) return RMI_ERR_NULL;
   int acc_bytes = 8;
   int rc        = classify(*desc, key, acc_bytes);
   if (rc != RMI_OK) return rc;
   if (lookup(key) == nullptr) return RMI_ERR_UNSUPPORTED;
-  return make_plan(*desc, key, acc_bytes, cu_count(), pl);
+  return make_plan(*desc, key, acc_bytes, cu_count(), pl, reinterpret_cast<uintptr_t>(in) % 128);
 }
 
 int reduce_impl(const rmi_reduce_desc& d,
@@ -64,7 +66,7 @@ int reduce_impl(const rmi_reduce_desc& d,
 {
   PlanX pl;
   PolicyKey key;
-  int rc = plan_for(&d, pl, key);
+  int rc = plan_for(&d, pl, key, in);
   if (rc != RMI_OK) return rc;
   if (pl.n_out == 0) return RMI_OK;
   if (out == nullptr) return RMI_ERR_NULL;
@@ -120,7 +122,8 @@ rmi_reduce_desc as_single_row(const rmi_reduce_desc& d, int64_t len)
 }
 
 // meanvar: one output pair per column, whatever the layout.
-int meanvar_plan(int dtype, int layout, int64_t n_rows, int64_t n_cols, PlanX& pl, run_fn& fn)
+int meanvar_plan(int dtype, int layout, int64_t n_rows, int64_t n_cols, PlanX& pl, run_fn& fn,
+                 uintptr_t in_misalign = 0)
 {
   if (dtype < 0 || dtype >= RMI_DTYPE_COUNT_) return RMI_ERR_BAD_ENUM;
   if (layout != RMI_ROW_MAJOR && layout != RMI_COL_MAJOR) return RMI_ERR_BAD_ENUM;
@@ -139,7 +142,7 @@ int meanvar_plan(int dtype, int layout, int64_t n_rows, int64_t n_cols, PlanX& p
   PolicyKey key;
   key.in_dtype = dtype;
   key.family   = kFamMeanVar;
-  return make_plan(d, key, (int)sizeof(mv_t), cu_count(), pl);
+  return make_plan(d, key, (int)sizeof(mv_t), cu_count(), pl, in_misalign);
 }
 
 }  // namespace
@@ -279,7 +282,8 @@ int rmi_meanvar(int dtype,
   using namespace rmi;
   PlanX pl;
   run_fn fn    = nullptr;
-  const int rc = meanvar_plan(dtype, layout, n_rows, n_cols, pl, fn);
+  const int rc = meanvar_plan(dtype, layout, n_rows, n_cols, pl, fn,
+                              reinterpret_cast<uintptr_t>(data) % 128);
   if (rc != RMI_OK) return rc;
   if (pl.n_out == 0) return RMI_OK;
   if (mean == nullptr || var == nullptr) return RMI_ERR_NULL;

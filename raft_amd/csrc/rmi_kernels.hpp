@@ -22,6 +22,8 @@ namespace rmi {
 constexpr int kBlock      = 256;  // threads per workgroup (the team kernel may use up to 1024)
 constexpr int kUnroll     = 4;    // independent 16-byte loads in flight per lane
 constexpr int kColUnroll  = 4;    // rows per lane and tile in the column kernel
+constexpr int kStageBytes  = 4096 + 128 + 16;  // LDS staging area of one wave (row_wave_kernel)
+constexpr int kStageLoads  = 5;  // lane-loads that cover 4096 + 112 bytes
 constexpr int kTeamUnroll = 4;    // lane-loads per batch in the team-per-row kernel
 
 struct RowArgs {
@@ -267,7 +269,7 @@ __global__ __launch_bounds__(kBlock) void row_short_kernel(RowArgs a)
 // gives every lane at most kUnroll lane-loads per row (nvec <= kUnroll*G); the
 // loop is there for forced plans.
 // ---------------------------------------------------------------------------
-template <class P, bool VEC16>
+template <class P, bool VEC16, bool STAGED = false>
 __global__ __launch_bounds__(kBlock) void row_wave_kernel(RowArgs a)
 {
   using acc_t     = typename P::acc_t;
@@ -282,10 +284,66 @@ __global__ __launch_bounds__(kBlock) void row_wave_kernel(RowArgs a)
   const i64 nvec  = a.nvec;
 
   acc_t acc = P::neutral();
-  if (row < a.n_out) {
+  if constexpr (STAGED) {
+    // Rows are whole 16-byte vectors (tail == 0) at 16-byte aligned addresses, but their
+    // lane-group pieces would straddle 128-byte lines.  The wave reads its R rows as one
+    // contiguous span that starts on a line, lane after lane, into its LDS area (every
+    // line is requested once), and the lane groups then take their vectors from LDS.
+    static_assert(VEC16, "staging moves 16-byte vectors");
+    extern __shared__ __attribute__((aligned(16))) char stage_lds[];
+    char* lw        = stage_lds + (threadIdx.x >> 6) * kStageBytes;
+    const char* inb = static_cast<const char*>(a.in);
+    const i64 row0  = wid * R;
+    const i64 rows_here = a.n_out - row0 < R ? a.n_out - row0 : R;
+    if (rows_here > 0) {
+      const i64 s0   = row0 * a.row_bytes;            // the span, in bytes from a.in
+      const i64 s1   = s0 + rows_here * a.row_bytes;
+      const int lead = (int)((reinterpret_cast<uintptr_t>(inb) + (uintptr_t)s0) & 127);  // multiple of 16
+      const i64 w0   = s0 - lead;                     // line-aligned start (may precede a.in)
+      // Every lane loads and stores unconditionally: a position outside the span is
+      // clamped to the span's first or last vector, which some lane moves anyway (the
+      // same line, the same LDS bytes, the same data).  Loads under a lane mask would be
+      // conditional definitions, after which the compiler copies registers and waits for
+      // each load in turn.
+      u32x4 x[kStageLoads];
+      i64 off[kStageLoads];
+#pragma unroll
+      for (int u = 0; u < kStageLoads; ++u) {
+        off[u] = w0 + ((i64)u * kWave + lane) * 16;
+        off[u] = off[u] < s0 ? s0 : (off[u] > s1 - 16 ? s1 - 16 : off[u]);
+        x[u]   = load16(inb + off[u]);
+      }
+#pragma unroll
+      for (int u = 0; u < kStageLoads; ++u)
+        *reinterpret_cast<u32x4*>(lw + (off[u] - w0)) = x[u];
+    }
+    // LDS operations of one wave complete in order; keep the compiler from moving the
+    // reads of other lanes' data above the writes
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    if (row < a.n_out) {
+      const int lead = (int)((reinterpret_cast<uintptr_t>(inb) + (uintptr_t)(row0 * a.row_bytes)) & 127);
+      const char* rp = lw + lead + (row - row0) * a.row_bytes;
+      u32x4 x[kUnroll];
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        const i64 v = c + u * G < nvec ? c + u * G : nvec - 1;  // clamped, not masked: see above
+        x[u]        = *reinterpret_cast<const u32x4*>(rp + v * 16);
+      }
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u)
+        if (c + u * G < nvec) P::push_vec(acc, x[u], (i64)(c + u * G) * S);
+    }
+  } else if (row < a.n_out) {
     const char* rp = static_cast<const char*>(a.in) + row * a.row_bytes;
     i64 v          = c;
-    for (; v + (kUnroll - 1) * G < nvec; v += kUnroll * G) {
+    // Whole batches that every lane of the group takes part in (forced plans only: the
+    // automatic plan leaves at most kUnroll lane-loads per lane).  The condition is the
+    // same for all lanes of a group: were it per lane, the lanes with one more whole
+    // vector would run this loop and the others the masked batch below, one after the
+    // other, and the row would take two trips to memory.
+    for (; (v - c) + (i64)kUnroll * G <= nvec; v += kUnroll * G) {
       typename H::type x[kUnroll];
 #pragma unroll
       for (int u = 0; u < kUnroll; ++u)
@@ -295,7 +353,7 @@ __global__ __launch_bounds__(kBlock) void row_wave_kernel(RowArgs a)
         H::push(acc, x[u], (v + u * G) * S);
     }
     const i64 nload = nvec + (a.tail > 0 ? 1 : 0);  // the tail is one more lane-load
-    if (v < nload) {  // fewer than kUnroll lane-loads left for this lane
+    if (v < nload) {  // the last, masked batch: up to kUnroll lane-loads per lane
       typename H::type x[kUnroll];
 #pragma unroll
       for (int u = 0; u < kUnroll; ++u)

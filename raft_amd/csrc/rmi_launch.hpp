@@ -52,7 +52,7 @@ template <class P>
 int run(const PlanX& pl, const Problem& pr, hipStream_t st)
 {
   static_assert(kBlock == kPlanBlock && kUnroll == kPlanUnroll && kColUnroll == kPlanUnroll &&
-                  kTeamUnroll == kPlanTeamUnroll,
+                  kTeamUnroll == kPlanTeamUnroll && kStageBytes == kStageBytesPerWave,
                 "plan selector and kernels must agree on block size and unroll");
   int rc = RMI_OK;
   switch (pl.kind) {
@@ -94,7 +94,9 @@ int run(const PlanX& pl, const Problem& pr, hipStream_t st)
           else
             hipLaunchKernelGGL((row_short_kernel<P, false>), grid, dim3(kBlock), 0, st, a);
         } else {
-          if (pl.vec16)
+          if (pl.vec16 && pl.staged)
+            hipLaunchKernelGGL((row_wave_kernel<P, true, true>), grid, dim3(kBlock), lds, st, a);
+          else if (pl.vec16)
             hipLaunchKernelGGL((row_wave_kernel<P, true>), grid, dim3(kBlock), lds, st, a);
           else
             hipLaunchKernelGGL((row_wave_kernel<P, false>), grid, dim3(kBlock), 0, st, a);

@@ -27,6 +27,10 @@ constexpr int kWavesPerCu = 32;  // 8 resident waves on each of the 4 SIMDs
 // lose 2 and 8 points to queueing in the memory system.
 constexpr int kColBlocksPerCu = 2;
 constexpr int kLdsPerCu       = 160 * 1024;  // LDS bytes of one gfx950 CU
+constexpr int64_t kBytesInFlightPerCu = 80 * 1024;  // target of the wave-per-row plan
+// LDS staging area of one wave: its rows (at most 64 lanes x 4 loads x 16 B) plus the
+// lead-in of a line-aligned start and one vector of slack
+constexpr int kStageBytesPerWave = 4096 + 128 + 16;
 
 struct PlanX {
   int kind        = RMI_PLAN_EMPTY;
@@ -34,6 +38,8 @@ struct PlanX {
   bool vec16      = false;  // 16-byte lane loads
   bool short_rows = false;  // ROW_WAVE served by the one-load-per-lane kernel
   bool team_kernel = false; // served by the team-per-row kernel
+  bool stage_ok    = false; // ROW_WAVE: rows could be staged through LDS
+  bool staged      = false; // ROW_WAVE: rows are staged through LDS (line-aligned span reads)
   int elem_bytes  = 0;
   int step        = 1;  // elements per lane-load
   int64_t n_out   = 0;
@@ -190,7 +196,8 @@ inline int make_plan(const rmi_reduce_desc& d,
                      const PolicyKey& key,
                      int acc_bytes,
                      int n_cu,
-                     PlanX& p)
+                     PlanX& p,
+                     uintptr_t in_misalign = 0)  // the input pointer modulo 128, when known
 {
   p            = PlanX{};
   p.acc_bytes  = acc_bytes;
@@ -327,18 +334,29 @@ inline int make_plan(const rmi_reduce_desc& d,
     p.grid_blocks        = ceildiv(p.n_out, rows_w * (kPlanBlock / 64));
     if (!p.short_rows && p.vec16) {
       // Bytes in flight per CU are what the memory system is sensitive to: about
-      // 80 KB (5 workgroups of 256 lanes x 4 loads x 16 B) sustains the most; the
+      // 80 KB sustains the most (5 workgroups when 256 lanes hold 4 loads of 16 B); the
       // default 8 resident workgroups lose 3-4 points to queueing.  A dynamic LDS
-      // reservation the kernel never touches caps the resident workgroups.
-      const int64_t loads_per_lane = ceildiv(nload, p.G);
-      if (key.family == kFamKvp) {
-        // the arg-reductions' longer accumulate step wants more waves to hide behind:
-        // 7 workgroups measured 86 % where 5 give 77 %
-        if (loads_per_lane >= 3) p.lds_reserve = kLdsPerCu / 7 - 768;
-      } else if (loads_per_lane >= 4) {
-        p.lds_reserve = kLdsPerCu / 5 - 768;
-      } else if (loads_per_lane == 3) {
-        p.lds_reserve = kLdsPerCu / 6 - 768;
+      // reservation caps the resident workgroups: as many as bring the bytes in flight
+      // closest to 80 KB, at least 4.  Arg-reductions, whose accumulate step is longer,
+      // want more waves to hide behind: at least 7 (86 % where 5 give 77 %).
+      const int64_t wg_bytes = (int64_t)(kPlanBlock / p.G) * nload * 16;
+      int64_t cap            = (kBytesInFlightPerCu + wg_bytes / 2) / wg_bytes;
+      if (key.family == kFamKvp && cap < 7) cap = 7;
+      if (cap < 4) cap = 4;
+      p.lds_reserve = cap >= 8 ? 0 : kLdsPerCu / (int)cap - 768;
+      // Rows whose length is a multiple of 16 bytes but not of a 128-byte line, or that
+      // start off a line: every 128- or 256-byte piece a lane group reads straddles
+      // lines, and the L1 sends a request per line and instruction (twice the requests
+      // to L2, a third more misses).  Such rows are staged: the wave reads its rows as
+      // one line-aligned contiguous span into LDS and the lane groups read from there.
+      // (a wave's rows have to fill at least half of its staging area: below that the
+      // fixed five loads and stores per lane cost more than the lines saved)
+      p.stage_ok = p.tail == 0 && (row_bytes % 16) == 0 && (64 / p.G) * row_bytes >= 2048;
+      if (p.stage_ok && ((row_bytes % 128) != 0 || (in_misalign % 128) != 0) &&
+          (in_misalign % 16) == 0) {
+        p.staged = true;
+        if (p.lds_reserve < kStageBytesPerWave * (kPlanBlock / 64))
+          p.lds_reserve = kStageBytesPerWave * (kPlanBlock / 64);
       }
     }
   } else if (kind == RMI_PLAN_ROW_BLOCK) {

@@ -11,6 +11,7 @@
 namespace {
 int failures = 0;
 long planned[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+long staged_plans = 0;
 #define REQUIRE(cond)                                                              \
   do {                                                                             \
     if (!(cond)) {                                                                 \
@@ -21,7 +22,7 @@ long planned[8] = {0, 0, 0, 0, 0, 0, 0, 0};
     }                                                                              \
   } while (0)
 
-void check(const rmi_reduce_desc& d, int n_cu)
+void check(const rmi_reduce_desc& d, int n_cu, uintptr_t in_misalign)
 {
   using namespace rmi;
   PolicyKey key;
@@ -29,7 +30,7 @@ void check(const rmi_reduce_desc& d, int n_cu)
   const int rc  = classify(d, key, acc_bytes);
   if (rc != RMI_OK) return;
   PlanX p;
-  const int prc = make_plan(d, key, acc_bytes, n_cu, p);
+  const int prc = make_plan(d, key, acc_bytes, n_cu, p, in_misalign);
   if (prc != RMI_OK) {
     REQUIRE(prc == RMI_ERR_BAD_SHAPE);
     return;
@@ -75,6 +76,16 @@ void check(const rmi_reduce_desc& d, int n_cu)
         REQUIRE(p.G >= 1 && p.G <= 64 && (p.G & (p.G - 1)) == 0 && (1 << p.logG) == p.G);
         // the lanes of a row hold all of its lane-loads, kPlanUnroll apiece (one for short rows)
         REQUIRE((int64_t)p.G * (p.short_rows ? 1 : kPlanUnroll) >= nload);
+        if (p.staged) {
+          ++staged_plans;
+          // whole vectors at 16-byte aligned addresses; the wave's rows and the lead-in of a
+          // line-aligned start fit its LDS area, which the launch reserves for four waves
+          REQUIRE(p.stage_ok && !p.short_rows && p.vec16 && p.tail == 0);
+          REQUIRE(p.row_bytes % 16 == 0 && in_misalign % 16 == 0);
+          REQUIRE((64 / p.G) * p.row_bytes + 112 + 16 <= kStageBytesPerWave);
+          REQUIRE(p.lds_reserve >= 4 * kStageBytesPerWave);
+          REQUIRE(p.row_bytes % 128 != 0 || in_misalign % 128 != 0);
+        }
       }
       break;
     case RMI_PLAN_ROW_BLOCK:
@@ -137,8 +148,9 @@ int main()
     // keep the element count within what one GPU could hold (2^38), larger ones are
     // rejected or planned just the same but are not interesting
     if ((long double)d.n_rows * (long double)d.n_cols > 274877906944.0L) d.n_cols = d.n_cols % 4096;
+    const uintptr_t mis = (uintptr_t)pick({0, 0, 0, 16, 32, 64, 112, 4, 8, 2, 1});
     for (int n_cu : {256, 1, 304})
-      check(d, n_cu);
+      check(d, n_cu, mis);
     ++cases;
   }
   // the extremes the header promises to reject
@@ -162,6 +174,10 @@ int main()
       std::printf("  plan kind %d was hardly exercised\n", k);
       ++failures;
     }
+  if (staged_plans < 1000) {
+    std::printf("  staged plans were hardly exercised (%ld)\n", staged_plans);
+    ++failures;
+  }
   std::printf("%ld descriptors, %d failed\n", cases, failures);
   return failures == 0 ? 0 : 1;
 }

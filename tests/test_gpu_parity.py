@@ -87,6 +87,28 @@ def test_many_long_rows(gpu, in_dt, out_dt, kw, rows, cols):
     u.check_against_oracle(d, data, label=f"long rows {rows}x{cols} dt{in_dt}")
 
 
+# Rows of whole 16-byte vectors that do not fill 128-byte lines, or that start off a line:
+# the wave-per-row plan stages them through LDS (a line-aligned contiguous read of the
+# wave's rows).  Row counts leave partial last waves; shifts move the input by 16..112 bytes.
+@pytest.mark.parametrize("in_dt,out_dt,kw,es", [
+    (api.F32, api.F32, dict(main_op=api.MAIN_SQ, final_op=api.FIN_SQRT), 4),
+    (api.F64, api.F64, {}, 8),
+    (api.BF16, api.F32, {}, 2),
+    (api.I8, api.I64, dict(main_op=api.MAIN_ABS), 1),
+    (api.F32, api.KVP_I32_F32, dict(main_op=api.MAIN_KVP, reduce_op=api.RED_ARGMIN, init_f=np.inf), 4),
+])
+@pytest.mark.parametrize("row_bytes", [272, 400, 528, 800, 1200, 2064, 4000, 4080])
+@pytest.mark.parametrize("rows,shift", [(1, 0), (7, 16), (1000, 0), (1000, 112), (5003, 48)])
+def test_staged_rows(gpu, in_dt, out_dt, kw, es, row_bytes, rows, shift):
+    cols = row_bytes // es
+    rng = np.random.default_rng(row_bytes + rows + shift)
+    data = _rand(rng, in_dt, rows * cols)
+    d = api.make_desc(in_dt, out_dt, rows, cols, **kw)
+    assert api.plan_query(d).kind == api.PLAN_ROW_WAVE
+    u.check_against_oracle(d, data, misalign_elems=shift // es,
+                           label=f"staged {rows}x{cols} dt{in_dt} +{shift}")
+
+
 # cpp/tests/linalg/coalesced_reduction.cu:109-139: 10000 x {3..270}, 10 x 25000, ...
 @pytest.mark.parametrize("rows,cols", [(10000, c) for c in
                                        (3, 5, 7, 9, 17, 31, 32, 33, 55, 63, 64, 65, 128, 270)]
