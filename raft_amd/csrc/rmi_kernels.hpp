@@ -196,6 +196,45 @@ __global__ __launch_bounds__(kBlock) void row_lanes_kernel(RowArgs a)
 }
 
 // ---------------------------------------------------------------------------
+// The last batch of a row (or chunk): N lane-loads per lane at v, v + stride, ...,
+// of which those below `end` exist.  N is the same for the whole wave (the caller
+// derives it from wave-uniform values and dispatches on it), so no load instruction
+// is spent on positions no lane has; within the batch loads are unconditional (a
+// position past `end` re-reads the last one) and only the accumulation is masked.
+// Loads under a lane mask are conditional definitions, after which the compiler
+// copies registers and waits for every load in turn.
+// ---------------------------------------------------------------------------
+template <class P, bool VEC16, int N, class IdxT>
+__device__ __forceinline__ void last_batch(typename P::acc_t& acc, const char* rp, IdxT v,
+                                           IdxT stride, IdxT end, i64 nvec, i64 len, int tail)
+{
+  using H = Held<P, VEC16>;
+  typename H::type x[N];
+#pragma unroll
+  for (int u = 0; u < N; ++u) {
+    const IdxT vl = v + u * stride < end ? v + u * stride : end - 1;
+    x[u]          = H::load_any(rp, vl, nvec, len);
+  }
+#pragma unroll
+  for (int u = 0; u < N; ++u)
+    if (v + u * stride < end) H::push_any(acc, x[u], v + u * stride, nvec, len, tail);
+}
+
+// n = 1 .. 4 lane-loads per lane, wave-uniform
+template <class P, bool VEC16, class IdxT>
+__device__ __forceinline__ void last_batch_n(int n, typename P::acc_t& acc, const char* rp,
+                                             IdxT v, IdxT stride, IdxT end, i64 nvec, i64 len,
+                                             int tail)
+{
+  switch (n) {
+    case 1: last_batch<P, VEC16, 1, IdxT>(acc, rp, v, stride, end, nvec, len, tail); break;
+    case 2: last_batch<P, VEC16, 2, IdxT>(acc, rp, v, stride, end, nvec, len, tail); break;
+    case 3: last_batch<P, VEC16, 3, IdxT>(acc, rp, v, stride, end, nvec, len, tail); break;
+    default: last_batch<P, VEC16, 4, IdxT>(acc, rp, v, stride, end, nvec, len, tail); break;
+  }
+}
+
+// ---------------------------------------------------------------------------
 // Short rows: nvec <= G, one lane-load per lane per row, kUnroll tiles of
 // 64/G rows in flight per wave.
 // ---------------------------------------------------------------------------
@@ -214,13 +253,18 @@ __global__ __launch_bounds__(kBlock) void row_short_kernel(RowArgs a)
   const i64 nload  = a.nvec + (a.tail > 0 ? 1 : 0);  // the tail is one more lane-load
   const bool incol = c < nload;
 
+  // Loads are unconditional: a lane without work (past the row's last lane-load, or a
+  // row past the matrix) re-reads the nearest vector that has some.  Loads under a lane
+  // mask are conditional definitions, after which the compiler copies registers and
+  // waits for every load in turn.
   typename H::type x[kUnroll];
   i64 row[kUnroll];
+  const i64 cl = incol ? (i64)c : nload - 1;
 #pragma unroll
   for (int t = 0; t < kUnroll; ++t) {
-    row[t] = (wid * kUnroll + t) * R + g;
-    if (incol && row[t] < a.n_out)
-      x[t] = H::load_any(inb + row[t] * a.row_bytes, c, a.nvec, a.len);
+    row[t]       = (wid * kUnroll + t) * R + g;
+    const i64 rl = row[t] < a.n_out ? row[t] : a.n_out - 1;
+    x[t]         = H::load_any(inb + rl * a.row_bytes, cl, a.nvec, a.len);
   }
   acc_t acc[kUnroll];
 #pragma unroll
@@ -353,15 +397,12 @@ __global__ __launch_bounds__(kBlock) void row_wave_kernel(RowArgs a)
         H::push(acc, x[u], (v + u * G) * S);
     }
     const i64 nload = nvec + (a.tail > 0 ? 1 : 0);  // the tail is one more lane-load
-    if (v < nload) {  // the last, masked batch: up to kUnroll lane-loads per lane
-      typename H::type x[kUnroll];
-#pragma unroll
-      for (int u = 0; u < kUnroll; ++u)
-        if (v + u * G < nload) x[u] = H::load_any(rp, v + u * G, nvec, a.len);
-#pragma unroll
-      for (int u = 0; u < kUnroll; ++u)
-        if (v + u * G < nload) H::push_any(acc, x[u], v + u * G, nvec, a.len, a.tail);
-    }
+    // the last batch: what is left of the row, up to kUnroll lane-loads per lane; the
+    // count is the same for every lane of the wave
+    const i64 left = nload - (v - c);
+    if (left > 0)  // G is a power of two: no 64-bit division on the device
+      last_batch_n<P, VEC16, i64>((int)((left + G - 1) >> a.logG), acc, rp, v, (i64)G, nload, nvec,
+                                  a.len, a.tail);
   }
   group_allreduce<P>(acc, G);
   if (c == 0 && row < a.n_out) finish<P>(a.epi, row, acc);
@@ -400,58 +441,57 @@ __global__ __launch_bounds__(1024) void row_block_kernel(RowArgs a)
     const i64 v0   = (i64)b * a.chunk;
     const i64 v1   = (v0 + a.chunk < a.nvec) ? (v0 + a.chunk) : a.nvec;
     const char* rp = static_cast<const char*>(a.in) + row * a.row_bytes;
-    i64 v          = v0 + t;
+    // `vb` is the first lane-load of the team's next batch: every loop condition below
+    // is the same for all lanes of the team, so a wave follows one path (a per-lane
+    // condition would send the lanes with one more whole batch through a loop and the
+    // others through the last batch, one after the other).
+    i64 vb = v0;
     // A chunk of fewer than three batches per thread is read 2 * U lane-loads at a
     // time: all of it is in flight at once and the accumulate step starts as the first
     // vectors arrive.
     if (a.chunk < (i64)3 * U * T) {
       constexpr int W = 2 * U;
-      for (; v + (W - 1) * (i64)T < v1; v += (i64)W * T) {
+      for (; vb + (i64)W * T <= v1; vb += (i64)W * T) {
         typename H::type x[W];
 #pragma unroll
         for (int u = 0; u < W; ++u)
-          x[u] = H::load(rp, v + (i64)u * T);
+          x[u] = H::load(rp, vb + t + (i64)u * T);
 #pragma unroll
         for (int u = 0; u < W; ++u)
-          H::push(acc, x[u], (v + (i64)u * T) * S);
+          H::push(acc, x[u], (vb + t + (i64)u * T) * S);
       }
     }
     // Whole batches of U lane-loads; the next batch is issued before the current one is
     // accumulated, so its latency overlaps the arithmetic (the loop holds no stores:
     // gfx9 counts loads and stores in one in-order counter).
-    if (v + (U - 1) * (i64)T < v1) {
+    if (vb + (i64)U * T <= v1) {
       typename H::type x[U];
 #pragma unroll
       for (int u = 0; u < U; ++u)
-        x[u] = H::load(rp, v + (i64)u * T);
+        x[u] = H::load(rp, vb + t + (i64)u * T);
       for (;;) {
-        const i64 vn    = v + (i64)U * T;
-        const bool more = vn + (U - 1) * (i64)T < v1;
+        const i64 vn    = vb + (i64)U * T;
+        const bool more = vn + (i64)U * T <= v1;
         typename H::type y[U];
         if (more) {
 #pragma unroll
           for (int u = 0; u < U; ++u)
-            y[u] = H::load(rp, vn + (i64)u * T);
+            y[u] = H::load(rp, vn + t + (i64)u * T);
         }
 #pragma unroll
         for (int u = 0; u < U; ++u)
-          H::push(acc, x[u], (v + (i64)u * T) * S);
-        v = vn;
+          H::push(acc, x[u], (vb + t + (i64)u * T) * S);
+        vb = vn;
         if (!more) break;
 #pragma unroll
         for (int u = 0; u < U; ++u)
           x[u] = y[u];
       }
     }
-    if (v < v1) {  // fewer than U lane-loads left for this lane
-      typename H::type x[U - 1];
-#pragma unroll
-      for (int u = 0; u < U - 1; ++u)
-        if (v + (i64)u * T < v1) x[u] = H::load(rp, v + (i64)u * T);
-#pragma unroll
-      for (int u = 0; u < U - 1; ++u)
-        if (v + (i64)u * T < v1) H::push(acc, x[u], (v + (i64)u * T) * S);
-    }
+    // what is left: fewer than U * T lane-loads, at most U per lane
+    if (vb < v1)
+      last_batch_n<P, VEC16, i64>((int)((v1 - vb + T - 1) >> (6 + a.logT)), acc, rp, vb + t, (i64)T,
+                                  v1, a.nvec, a.len, 0);
     // the overlapping last vector of the row goes to the team that owns the last chunk
     if (a.tail > 0 && b == a.B - 1 && t == 0)
       H::push_any(acc, H::load_any(rp, a.nvec, a.nvec, a.len), a.nvec, a.nvec, a.len, a.tail);

@@ -150,12 +150,17 @@ __device__ __forceinline__ void normalize_wave_body(const NormArgs& a)
   i64 row[TILES];
 #pragma unroll
   for (int t = 0; t < TILES; ++t) {
-    row[t] = (wid * TILES + t) * R + g;
-    if (row[t] < a.n_rows) {
-      const char* rp = static_cast<const char*>(a.in) + row[t] * a.row_bytes;
+    // Unconditional loads: a lane-load past the row's end re-reads the last one, a row
+    // past the matrix the last row.  Loads under a lane mask are conditional
+    // definitions, after which the compiler copies registers and waits for every load
+    // in turn; the accumulation and the stores below stay masked.
+    row[t]         = (wid * TILES + t) * R + g;
+    const i64 rl   = row[t] < a.n_rows ? row[t] : a.n_rows - 1;
+    const char* rp = static_cast<const char*>(a.in) + rl * a.row_bytes;
 #pragma unroll
-      for (int u = 0; u < L; ++u)
-        if (c + u * G < nload) x[t * L + u] = H::load_any(rp, c + u * G, a.nvec, a.len);
+    for (int u = 0; u < L; ++u) {
+      const i64 vl   = c + u * G < nload ? (i64)(c + u * G) : nload - 1;
+      x[t * L + u]   = H::load_any(rp, vl, a.nvec, a.len);
     }
   }
   acc_t acc[TILES];
@@ -216,8 +221,10 @@ __global__ __launch_bounds__(1024) void normalize_team_kernel(NormArgs a)
 
   typename H::type x[UH];
 #pragma unroll
-  for (int u = 0; u < UH; ++u)
-    if (t + (i64)u * T < nload) x[u] = H::load_any(rp, t + (i64)u * T, a.nvec, a.len);
+  for (int u = 0; u < UH; ++u) {  // unconditional, clamped: see normalize_wave_body
+    const i64 vl = t + (i64)u * T < nload ? t + (i64)u * T : nload - 1;
+    x[u]         = H::load_any(rp, vl, a.nvec, a.len);
+  }
   acc_t acc = P::neutral();
 #pragma unroll
   for (int u = 0; u < UH; ++u)
@@ -260,8 +267,10 @@ __global__ __launch_bounds__(1024) void normalize_sweep_kernel(NormArgs a)
   for (i64 v = t; v < nload; v += (i64)kUnroll * T) {
     typename H::type x[kUnroll];
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u)
-      if (v + (i64)u * T < nload) x[u] = H::load_any(rp, v + (i64)u * T, a.nvec, a.len);
+    for (int u = 0; u < kUnroll; ++u) {  // unconditional, clamped: see normalize_wave_body
+      const i64 vl = v + (i64)u * T < nload ? v + (i64)u * T : nload - 1;
+      x[u]         = H::load_any(rp, vl, a.nvec, a.len);
+    }
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u)
       if (v + (i64)u * T < nload) H::push_any(acc, x[u], v + (i64)u * T, a.nvec, a.len, a.tail);
@@ -281,8 +290,10 @@ __global__ __launch_bounds__(1024) void normalize_sweep_kernel(NormArgs a)
   for (i64 v = t; v < nload; v += (i64)kUnroll * T) {
     typename H::type x[kUnroll];
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u)
-      if (v + (i64)u * T < nload) x[u] = H::load_any(rp, v + (i64)u * T, a.nvec, a.len);
+    for (int u = 0; u < kUnroll; ++u) {  // unconditional, clamped: see normalize_wave_body
+      const i64 vl = v + (i64)u * T < nload ? v + (i64)u * T : nload - 1;
+      x[u]         = H::load_any(rp, vl, a.nvec, a.len);
+    }
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u)
       if (v + (i64)u * T < nload) write_scaled<P, true>(a, orow, x[u], v + (i64)u * T, norm);
