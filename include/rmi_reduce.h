@@ -154,7 +154,7 @@ typedef enum rmi_plan_kind {
   RMI_PLAN_AUTO       = 0,
   RMI_PLAN_ROW_LANES  = 1, /* several whole rows per lane-load (rows <= 8 B..16 B)  */
   RMI_PLAN_ROW_WAVE   = 2, /* 1..64 lanes of one wavefront per row                  */
-  RMI_PLAN_ROW_BLOCK  = 3, /* one 256-thread block per row, LDS tree                */
+  RMI_PLAN_ROW_BLOCK  = 3, /* a team of 128..1024 threads per row, LDS combine       */
   RMI_PLAN_ROW_SPLIT  = 4, /* several blocks per row + second pass over partials    */
   RMI_PLAN_COL_TILE   = 5, /* column reduction: column-contiguous lanes, row ranges
                               per block, LDS combine, second pass over partials    */
