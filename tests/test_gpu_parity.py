@@ -87,9 +87,11 @@ def test_many_long_rows(gpu, in_dt, out_dt, kw, rows, cols):
     u.check_against_oracle(d, data, label=f"long rows {rows}x{cols} dt{in_dt}")
 
 
-# Rows of whole 16-byte vectors that do not fill 128-byte lines, or that start off a line:
-# the wave-per-row plan stages them through LDS (a line-aligned contiguous read of the
-# wave's rows).  Row counts leave partial last waves; shifts move the input by 16..112 bytes.
+# Rows that do not fill 128-byte lines, or that start off a line: the wave-per-row plan
+# stages rows of whole 16-byte vectors through LDS (a line-aligned contiguous read of the
+# wave's rows).  Row lengths that are multiples of 8 and 4 bytes only (they end in tail
+# elements and take the direct path) sit beside them, so both sides of the plan's choice are
+# covered.  Row counts leave partial last waves; shifts move the input by 16..112 bytes.
 @pytest.mark.parametrize("in_dt,out_dt,kw,es", [
     (api.F32, api.F32, dict(main_op=api.MAIN_SQ, final_op=api.FIN_SQRT), 4),
     (api.F64, api.F64, {}, 8),
@@ -97,9 +99,12 @@ def test_many_long_rows(gpu, in_dt, out_dt, kw, rows, cols):
     (api.I8, api.I64, dict(main_op=api.MAIN_ABS), 1),
     (api.F32, api.KVP_I32_F32, dict(main_op=api.MAIN_KVP, reduce_op=api.RED_ARGMIN, init_f=np.inf), 4),
 ])
-@pytest.mark.parametrize("row_bytes", [272, 400, 528, 800, 1200, 2064, 4000, 4080])
+@pytest.mark.parametrize("row_bytes", [272, 400, 516, 520, 528, 796, 800, 1000, 1200, 2052, 2064,
+                                       4000, 4080, 4088, 4092])
 @pytest.mark.parametrize("rows,shift", [(1, 0), (7, 16), (1000, 0), (1000, 112), (5003, 48)])
 def test_staged_rows(gpu, in_dt, out_dt, kw, es, row_bytes, rows, shift):
+    if row_bytes % es:
+        pytest.skip("not a whole number of elements")
     cols = row_bytes // es
     rng = np.random.default_rng(row_bytes + rows + shift)
     data = _rand(rng, in_dt, rows * cols)
