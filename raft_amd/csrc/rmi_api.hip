@@ -181,12 +181,15 @@ int rmi_plan_query(const rmi_reduce_desc* desc, rmi_plan* plan)
   return RMI_OK;
 }
 
+// The plan, and with it the workspace, can depend on where the input starts (rows read in
+// groups need a 16-byte aligned start): a query answers for the larger of the two.
 size_t rmi_reduce_workspace_bytes(const rmi_reduce_desc* desc)
 {
-  rmi::PlanX pl;
+  rmi::PlanX pl, pu;
   rmi::PolicyKey key;
   if (rmi::plan_for(desc, pl, key) != RMI_OK) return 0;
-  return pl.ws_bytes;
+  if (rmi::plan_for(desc, pu, key, reinterpret_cast<const void*>(uintptr_t{1})) != RMI_OK) return 0;
+  return pl.ws_bytes > pu.ws_bytes ? pl.ws_bytes : pu.ws_bytes;
 }
 
 int rmi_reduce(const rmi_reduce_desc* desc,
@@ -261,10 +264,11 @@ int rmi_row_normalize(const rmi_reduce_desc* desc,
 
 size_t rmi_meanvar_workspace_bytes(int dtype, int layout, int64_t n_rows, int64_t n_cols)
 {
-  rmi::PlanX pl;
+  rmi::PlanX pl, pu;
   rmi::run_fn fn = nullptr;
   if (rmi::meanvar_plan(dtype, layout, n_rows, n_cols, pl, fn) != RMI_OK) return 0;
-  return pl.ws_bytes;
+  if (rmi::meanvar_plan(dtype, layout, n_rows, n_cols, pu, fn, 1) != RMI_OK) return 0;
+  return pl.ws_bytes > pu.ws_bytes ? pl.ws_bytes : pu.ws_bytes;
 }
 
 int rmi_meanvar(int dtype,

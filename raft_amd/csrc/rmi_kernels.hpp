@@ -50,9 +50,20 @@ struct ColArgs {
   i64 row_bytes;   // D * sizeof(element)
   i64 nvec;        // whole lane-loads per row: D / VEC (VEC16) or D (element-wise)
   int tail;        // VEC16: columns after the last whole vector (D % VEC)
-  int TX;          // lanes along the contiguous dimension (power of two <= 64)
-  int logTX;
+  int TX;          // lanes along the contiguous dimension (<= 64)
+  int TY;          // rows per step: kBlock / TX, rounded down
+  int logTX;       // log2(TX) when TX is a power of two
+  int dense;       // TX is not a power of two: thread t is lane t % TX of row t / TX, the
+                   // last kBlock - TX * TY threads idle, rows are combined through LDS
+  int treeTY;      // dense: TY rounded up to a power of two
   int B;           // gridDim.y
+  // Rows read in groups (group > 0): `in` is taken as a [len][group * cols] matrix of whole
+  // 16-byte vectors, column c of which is real column c % cols; the `rem` elements after
+  // the last whole group are added one by one, and every real column gets group * B
+  // partials, ordered [cols][group][B].
+  int group;
+  i64 cols;
+  i64 rem;
   Epilogue epi;
 };
 
@@ -539,12 +550,13 @@ __global__ __launch_bounds__(kBlock) void col_kernel(ColArgs a)
 
   const int t      = threadIdx.x;
   const int TX     = a.TX;
-  const int TY     = kBlock >> a.logTX;
-  const int tx     = t & (TX - 1);
-  const int ty     = t >> a.logTX;
+  const int TY     = a.TY;
+  const int ty     = a.dense ? (int)((unsigned)t / (unsigned)TX) : t >> a.logTX;
+  const int tx     = t - ty * TX;
+  const bool live  = ty < TY;
   const i64 cv     = (i64)blockIdx.x * TX + tx;
-  const bool whole = cv < a.nvec;                          // a full lane-load of columns
-  const bool part  = VEC16 && cv == a.nvec && a.tail > 0;  // the last, partial group
+  const bool whole = live && cv < a.nvec;                          // a full lane-load of columns
+  const bool part  = live && VEC16 && cv == a.nvec && a.tail > 0;  // the last, partial group
   const i64 RT     = (i64)TY * kColUnroll;
   const i64 n_full = a.len / RT;
   const char* inb  = static_cast<const char*>(a.in);
@@ -587,6 +599,12 @@ __global__ __launch_bounds__(kBlock) void col_kernel(ColArgs a)
       if ((i64)blockIdx.y == n_full % a.B) {  // the rows past the last whole tile
         for (i64 r = n_full * RT + ty; r < a.len; r += TY)
           P::push_cols(acc, load16(p + r * a.row_bytes), r);
+        if (a.group > 0 && ty == 0) {  // the real rows past the last whole group
+          const in_t* e = reinterpret_cast<const in_t*>(inb + a.len * a.row_bytes) + cv * S;
+#pragma unroll
+          for (int j = 0; j < S; ++j)
+            if (cv * S + j < a.rem) P::push(acc[j], In<in_t>::ld(e + j), 0);
+        }
       }
     }
   } else if (whole) {
@@ -607,21 +625,38 @@ __global__ __launch_bounds__(kBlock) void col_kernel(ColArgs a)
     }
   }
 
-  // lanes of one wave that share tx sit TX, 2*TX, ... apart
-  for (int m = TX; m < kWave; m <<= 1) {
+  if (a.dense) {
+    // rows of the step sit TX threads apart: a tree over them in LDS, rows 0..TY-1 of
+    // every lane into row 0 (idle threads hold the neutral element)
 #pragma unroll
     for (int j = 0; j < S; ++j)
-      P::merge(acc[j], bperm_acc<P>(acc[j], m));
-  }
-  // one value per (wave, tx, j) through LDS, folded by the block's first TX threads
-  const int lane = t & (kWave - 1);
-  const int wave = t >> 6;
-  if (lane < TX) {
+      sm[t * S + j] = acc[j];
+    __syncthreads();
+    for (int s = a.treeTY >> 1; s >= 1; s >>= 1) {
+      if (ty < s && ty + s < TY) {
 #pragma unroll
-    for (int j = 0; j < S; ++j)
-      sm[(wave * kWave + lane) * S + j] = acc[j];
+        for (int j = 0; j < S; ++j)
+          P::merge(sm[t * S + j], sm[(t + s * TX) * S + j]);
+      }
+      __syncthreads();
+    }
+  } else {
+    // lanes of one wave that share tx sit TX, 2*TX, ... apart
+    for (int m = TX; m < kWave; m <<= 1) {
+#pragma unroll
+      for (int j = 0; j < S; ++j)
+        P::merge(acc[j], bperm_acc<P>(acc[j], m));
+    }
+    // one value per (wave, tx, j) through LDS, folded by the block's first TX threads
+    const int lane = t & (kWave - 1);
+    const int wave = t >> 6;
+    if (lane < TX) {
+#pragma unroll
+      for (int j = 0; j < S; ++j)
+        sm[(wave * kWave + lane) * S + j] = acc[j];
+    }
+    __syncthreads();
   }
-  __syncthreads();
   if (t < TX && (whole || part)) {
     // the partial group holds the row's last S columns; its first S - tail are
     // already covered by the group before it
@@ -630,11 +665,17 @@ __global__ __launch_bounds__(kBlock) void col_kernel(ColArgs a)
 #pragma unroll
     for (int j = 0; j < S; ++j) {
       if (j >= first) {
-        acc_t r = sm[(0 * kWave + t) * S + j];
-        for (int w = 1; w < W; ++w)
-          P::merge(r, sm[(w * kWave + t) * S + j]);
+        acc_t r = sm[t * S + j];
+        if (!a.dense) {
+          for (int w = 1; w < W; ++w)
+            P::merge(r, sm[(w * kWave + t) * S + j]);
+        }
         const i64 col = col0 + j;
-        if (a.B == 1) {
+        if (a.group > 0) {
+          const unsigned rg = (unsigned)col / (unsigned)a.cols;
+          const unsigned c  = (unsigned)col - rg * (unsigned)a.cols;
+          static_cast<acc_t*>(a.partial)[((i64)c * a.group + rg) * a.B + blockIdx.y] = r;
+        } else if (a.B == 1) {
           finish<P>(a.epi, col, r);
         } else {
           static_cast<acc_t*>(a.partial)[col * a.B + blockIdx.y] = r;

@@ -121,15 +121,31 @@ int run(const PlanX& pl, const Problem& pr, hipStream_t st)
       a.nvec           = pl.nvec;
       a.tail           = pl.tail;
       a.TX             = pl.TX;
+      a.TY             = pl.TY;
       a.logTX          = pl.logTX;
+      a.dense          = pl.dense ? 1 : 0;
+      a.treeTY         = pow2ceil(pl.TY);
       a.B              = pl.B;
       a.epi            = pr.epi;
+      if (pl.group > 0) {  // rows read in groups: a [group_len][group * n_out] matrix
+        a.n_out     = pl.n_out * pl.group;
+        a.len       = pl.group_len;
+        a.row_bytes = pl.row_bytes * pl.group;
+        a.nvec      = pl.group_nvec;
+        a.tail      = 0;
+        a.group     = pl.group;
+        a.cols      = pl.n_out;
+        a.rem       = (pl.len - pl.group_len * pl.group) * pl.n_out;
+      }
       const dim3 grid((unsigned)pl.gridx, (unsigned)pl.B);
       if (pl.vec16)
         hipLaunchKernelGGL((col_kernel<P, true>), grid, dim3(kBlock), 0, st, a);
       else
         hipLaunchKernelGGL((col_kernel<P, false>), grid, dim3(kBlock), 0, st, a);
-      if (pl.B > 1) rc = launch_fold<P>(pl, pr, pl.B, st);
+      if (pl.group > 0)
+        rc = launch_fold<P>(pl, pr, pl.B * pl.group, st);
+      else if (pl.B > 1)
+        rc = launch_fold<P>(pl, pr, pl.B, st);
       break;
     }
     default: rc = RMI_ERR_BAD_ENUM;

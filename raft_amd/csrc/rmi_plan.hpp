@@ -26,6 +26,7 @@ constexpr int kWavesPerCu = 32;  // 8 resident waves on each of the 4 SIMDs
 // tiles in flight per workgroup, 2 per CU (8 waves) sustains ~7.1 TB/s; 4 and 8 per CU
 // lose 2 and 8 points to queueing in the memory system.
 constexpr int kColBlocksPerCu = 2;
+constexpr int64_t kGroupMinLen = 256;  // COL_TILE: fewest row groups worth reading rows in groups
 constexpr int kLdsPerCu       = 160 * 1024;  // LDS bytes of one gfx950 CU
 constexpr int64_t kBytesInFlightPerCu = 80 * 1024;  // target of the wave-per-row plan
 // LDS staging area of one wave: its rows (at most 64 lanes x 4 loads x 16 B) plus the
@@ -53,9 +54,14 @@ struct PlanX {
   int threads     = kPlanBlock;  // ROW_BLOCK / ROW_SPLIT block size
   int B           = 1;           // partials per output
   int64_t chunk   = 0;           // ROW_SPLIT: lane-loads per block
-  int TX          = 1;           // COL_TILE
-  int logTX       = 0;
+  int TX          = 1;           // COL_TILE: lanes along a row per workgroup
+  int TY          = 1;           // COL_TILE: rows per workgroup step (TX * TY <= block)
+  int logTX       = 0;           // COL_TILE: log2(TX) when TX is a power of two
+  bool dense      = false;       // COL_TILE: TX is not a power of two
   int64_t gridx   = 0;  // COL_TILE: blocks along the contiguous dimension
+  int group       = 0;  // COL_TILE: > 0 when `group` consecutive rows are read as one row
+  int64_t group_len  = 0;  // COL_TILE, grouped: whole groups (rows of the widened matrix)
+  int64_t group_nvec = 0;  // COL_TILE, grouped: 16-byte vectors per group
   int64_t grid_blocks    = 0;
   int passes             = 1;
   int lds_reserve        = 0;  // dynamic LDS bytes reserved only to cap occupancy
@@ -242,26 +248,64 @@ inline int make_plan(const rmi_reduce_desc& d,
   const int64_t nload = p.nvec + (p.tail > 0 ? 1 : 0);
 
   if (p.strided) {
-    p.kind  = RMI_PLAN_COL_TILE;
-    p.TX    = (int)(nload < 64 ? pow2ceil(nload) : 64);
-    p.logTX = ilog2(p.TX);
-    const int TY = kPlanBlock / p.TX;
-    p.gridx      = ceildiv(nload, p.TX);
+    p.kind = RMI_PLAN_COL_TILE;
+    // Rows shorter than one 16-byte vector would be read element by element.  The matrix is
+    // one contiguous array, so `group` consecutive rows whose bytes add up to whole vectors
+    // are read as ONE row of a matrix with len / group rows.  A thread's columns of the
+    // widened row are fixed real columns (widened column c is real column c % n_out of row
+    // c / n_out within the group), so each real column ends up with group * B partials,
+    // which the second pass folds; the rows after the last whole group are added element by
+    // element.  Reductions that need the row index (arg-reductions) stay on the plain path,
+    // as do inputs that do not start on a 16-byte boundary and matrices with fewer than
+    // kGroupMinLen groups.
+    int64_t lanes = nload, rows = p.len;
+    if (key.family != kFamKvp && row_bytes < 16 && (in_misalign % 16) == 0) {
+      const int64_t low = row_bytes & -row_bytes;  // largest power of two in row_bytes
+      if (p.len / (16 / low) >= kGroupMinLen) {
+        p.group      = (int)(16 / low);
+        p.group_len  = p.len / p.group;
+        p.group_nvec = row_bytes / low;
+        p.vec16      = true;
+        lanes        = p.group_nvec;
+        rows         = p.group_len;
+      }
+    }
+    // A workgroup covers TX lane-loads of a row (TX columns groups) times TY rows per step.
+    // Rows of up to 64 lane-loads take exactly that many lanes, and as many rows as fit the
+    // workgroup: 33 lane-loads on 64 lanes would leave every other lane idle, 7 rows of 33
+    // leave 25 of 256.  Longer rows are cut into the fewest pieces of at most 64 lanes that
+    // keep four lanes in five busy (or the best of four cuts).
+    {
+      const int64_t g0 = ceildiv(lanes, 64);
+      int64_t best_g = g0, best_num = -1, best_den = 1;
+      for (int64_t g = g0; g < g0 + 4; ++g) {
+        const int64_t tx = ceildiv(lanes, g), ty = kPlanBlock / tx;
+        const int64_t num = lanes * ty, den = g * kPlanBlock;  // busy lanes / lanes
+        if (best_num < 0 || num * best_den > best_num * den) best_g = g, best_num = num, best_den = den;
+        if (num * 5 >= den * 4) break;
+      }
+      p.TX    = (int)ceildiv(lanes, best_g);
+      p.TY    = kPlanBlock / p.TX;
+      p.gridx = ceildiv(lanes, p.TX);
+      p.dense = (p.TX & (p.TX - 1)) != 0;
+      p.logTX = p.dense ? 0 : ilog2(p.TX);
+    }
     // row tiles of TY*unroll rows are dealt round-robin to B blocks: kColBlocksPerCu
     // blocks per CU, but at least two tiles per block
-    const int64_t tile_rows = (int64_t)TY * kPlanUnroll;
+    const int64_t tile_rows = (int64_t)p.TY * kPlanUnroll;
     // arg-reductions spend longer in their accumulate step: 3 workgroups per CU measured
     // 84 % where 2 give 78 % (sums lose a point or two at 3)
     const int per_cu = key.family == kFamKvp ? kColBlocksPerCu + 1 : kColBlocksPerCu;
     int64_t B               = ceildiv((int64_t)n_cu * per_cu, p.gridx);
-    const int64_t maxB      = ceildiv(p.len, tile_rows * 2);
+    const int64_t maxB      = ceildiv(rows, tile_rows * 2);
     if (B > maxB) B = maxB;
     if (B < 1) B = 1;
     if (B > 4096) B = 4096;
     p.B = (int)B;
     p.grid_blocks         = p.gridx * p.B;
-    p.passes              = p.B > 1 ? 2 : 1;
-    p.ws_bytes            = p.B > 1 ? (size_t)p.n_out * p.B * acc_bytes : 0;
+    const int64_t fold_b  = p.group > 0 ? (int64_t)p.B * p.group : p.B;
+    p.passes              = fold_b > 1 ? 2 : 1;
+    p.ws_bytes            = fold_b > 1 ? (size_t)p.n_out * fold_b * acc_bytes : 0;
     if (p.gridx > 0x7fffffffLL) return RMI_ERR_BAD_SHAPE;
     return RMI_OK;
   }
@@ -416,7 +460,7 @@ inline void export_plan(const PlanX& p, rmi_plan& o)
   o.kind            = p.kind;
   o.vec_bytes       = p.vec16 ? 16 : p.elem_bytes;
   o.lanes_per_row   = p.kind == RMI_PLAN_ROW_WAVE ? p.G : 0;
-  o.blocks_per_out  = p.B;
+  o.blocks_per_out  = p.group > 0 ? p.B * p.group : p.B;
   o.block_threads   = (p.team_kernel && p.threads > kPlanBlock) ? p.threads : kPlanBlock;
   o.passes          = p.passes;
   o.grid_blocks     = p.grid_blocks;

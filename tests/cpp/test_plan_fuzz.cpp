@@ -12,6 +12,7 @@ namespace {
 int failures = 0;
 long planned[8] = {0, 0, 0, 0, 0, 0, 0, 0};
 long staged_plans = 0;
+long grouped_plans = 0;
 #define REQUIRE(cond)                                                              \
   do {                                                                             \
     if (!(cond)) {                                                                 \
@@ -55,11 +56,12 @@ void check(const rmi_reduce_desc& d, int n_cu, uintptr_t in_misalign)
   REQUIRE(p.lds_reserve >= 0 && p.lds_reserve <= 64 * 1024);
   REQUIRE((p.ws_bytes > 0) == (p.passes == 2));
   REQUIRE(p.B >= 1 && p.B <= 4096);
-  if (p.passes == 2) REQUIRE(p.ws_bytes == (size_t)p.n_out * p.B * acc_bytes);
+  if (p.passes == 2)
+    REQUIRE(p.ws_bytes == (size_t)p.n_out * p.B * (p.group > 0 ? p.group : 1) * acc_bytes);
   const int es = dtype_size(d.in_dtype);
   if (p.kind != RMI_PLAN_ROW_LANES) {
     REQUIRE(p.row_bytes == contiguous * es);
-    REQUIRE(p.vec16 == (p.row_bytes >= 16));
+    REQUIRE(p.vec16 == (p.row_bytes >= 16 || p.group > 0));
     REQUIRE(p.nvec * p.step + p.tail == contiguous);
     REQUIRE(p.tail >= 0 && p.tail < p.step);
   }
@@ -99,9 +101,26 @@ void check(const rmi_reduce_desc& d, int n_cu, uintptr_t in_misalign)
       break;
     case RMI_PLAN_COL_TILE:
       REQUIRE(p.strided);
-      REQUIRE(p.TX >= 1 && p.TX <= 64 && (p.TX & (p.TX - 1)) == 0 && (1 << p.logTX) == p.TX);
-      REQUIRE(p.gridx * p.TX >= nload && (p.gridx - 1) * p.TX < nload);
+      REQUIRE(p.TX >= 1 && p.TX <= 64 && p.TY == kPlanBlock / p.TX && p.TY >= 4);
+      REQUIRE(p.dense == ((p.TX & (p.TX - 1)) != 0));
+      if (!p.dense) REQUIRE((1 << p.logTX) == p.TX);
       REQUIRE(p.grid_blocks == p.gridx * p.B);
+      {
+        const int64_t lanes = p.group > 0 ? p.group_nvec : nload;
+        REQUIRE(p.gridx * p.TX >= lanes && (p.gridx - 1) * p.TX < lanes);
+        // at least three lanes in five carry data (cuts of a row are chosen for four in five)
+        REQUIRE(lanes * p.TY * 5 >= p.gridx * kPlanBlock * 3 || lanes < 4);
+      }
+      if (p.group > 0) {
+        ++grouped_plans;
+        // rows shorter than a 16-byte vector, in groups that are whole vectors at aligned
+        // addresses, enough of them, no index-dependent reduction
+        REQUIRE(key.family != rmi::kFamKvp && in_misalign % 16 == 0 && p.row_bytes < 16);
+        REQUIRE(p.group >= 2 && p.group <= 16 && (p.group * p.row_bytes) % 16 == 0);
+        REQUIRE(p.group_nvec * 16 == p.group * p.row_bytes && p.group_nvec <= 15);
+        REQUIRE(p.group_len == p.len / p.group && p.group_len >= rmi::kGroupMinLen);
+        REQUIRE(p.passes == 2);
+      }
       break;
     default: REQUIRE(false);
   }
@@ -174,6 +193,10 @@ int main()
       std::printf("  plan kind %d was hardly exercised\n", k);
       ++failures;
     }
+  if (grouped_plans < 1000) {
+    std::printf("  grouped column plans were hardly exercised (%ld)\n", grouped_plans);
+    ++failures;
+  }
   if (staged_plans < 1000) {
     std::printf("  staged plans were hardly exercised (%ld)\n", staged_plans);
     ++failures;

@@ -351,3 +351,39 @@ def test_bitwise_repeatable(gpu):
         a = u.gpu_reduce(d, data)
         for _ in range(3):
             assert np.array_equal(a, u.gpu_reduce(d, data))
+
+
+# Column reductions over rows that are not a power-of-two number of lane-loads: a workgroup
+# takes as many whole rows as fit its 256 threads and combines them through LDS.  Rows shorter
+# than a 16-byte vector are read in groups of 2..16 consecutive rows that make whole vectors
+# (each real column then gets group x blocks partials, and the rows after the last whole
+# group are added element by element); a start off a 16-byte boundary and arg-reductions
+# read such rows element by element instead, with the same result.
+@pytest.mark.parametrize("in_dt,out_dt,kw", [
+    (api.F32, api.F32, {}),
+    (api.F32, api.F32, dict(main_op=api.MAIN_SQ, final_op=api.FIN_SQRT)),
+    (api.F32, api.F32, dict(reduce_op=api.RED_MAX, init_f=-np.inf)),
+    (api.F64, api.F64, {}),
+    (api.BF16, api.F32, {}),
+    (api.F16, api.F32, dict(main_op=api.MAIN_ABS)),
+    (api.I8, api.I64, {}),
+    (api.I32, api.I64, dict(reduce_op=api.RED_MIN, init_i=2**62)),
+    (api.F32, api.KVP_I32_F32, dict(main_op=api.MAIN_KVP, reduce_op=api.RED_ARGMAX, init_f=-np.inf)),
+])
+@pytest.mark.parametrize("rows,cols", [(1024, 3), (70001, 3), (1027, 5), (300000, 7), (4099, 63),
+                                       (70001, 129), (5000, 130), (2051, 1001), (66000, 33),
+                                       (530, 4097), (255, 63), (40000, 1), (33333, 2),
+                                       (9000, 100), (3000, 260), (2500, 517), (77, 37)])
+@pytest.mark.parametrize("shift", [0, 1])
+def test_grouped_columns(gpu, in_dt, out_dt, kw, rows, cols, shift):
+    es = api.load().rmi_dtype_size(in_dt)
+    rng = np.random.default_rng(rows * 7 + cols + shift)
+    data = _rand(rng, in_dt, rows * cols)
+    d = api.make_desc(in_dt, out_dt, rows, cols, apply=api.ALONG_COLUMNS, **kw)
+    pl = api.plan_query(d)
+    assert pl.kind == api.PLAN_COL_TILE
+    if cols * es < 16 and kw.get("main_op") != api.MAIN_KVP and rows >= 4096:
+        group = 16 // np.gcd(16, cols * es)
+        assert pl.passes == 2 and pl.blocks_per_out % group == 0
+    u.check_against_oracle(d, data, misalign_elems=shift,
+                           label=f"grouped {rows}x{cols} dt{in_dt} +{shift}")
