@@ -50,11 +50,12 @@ struct ColArgs {
   i64 row_bytes;   // D * sizeof(element)
   i64 nvec;        // whole lane-loads per row: D / VEC (VEC16) or D (element-wise)
   int tail;        // VEC16: columns after the last whole vector (D % VEC)
-  int TX;          // lanes along the contiguous dimension (<= 64)
+  int TX;          // lanes along the contiguous dimension (<= 128)
   int TY;          // rows per step: kBlock / TX, rounded down
   int logTX;       // log2(TX) when TX is a power of two
-  int dense;       // TX is not a power of two: thread t is lane t % TX of row t / TX, the
-                   // last kBlock - TX * TY threads idle, rows are combined through LDS
+  int dense;       // TX is not a power of two or exceeds a wave: thread t is lane t % TX of
+                   // row t / TX, the last kBlock - TX * TY threads idle, and the rows of a
+                   // step are combined through LDS instead of lane exchanges
   int treeTY;      // dense: TY rounded up to a power of two
   int B;           // gridDim.y
   // Rows read in groups (group > 0): `in` is taken as a [len][group * cols] matrix of whole
@@ -532,6 +533,8 @@ __global__ __launch_bounds__(1024) void row_block_kernel(RowArgs a)
 // Reduction along the strided dimension of a [len][n_out] row-major array.
 // Thread (tx, ty): tx owns one lane-load wide group of adjacent columns for
 // the whole kernel, ty strides over the rows of the tiles dealt to this block.
+// TX is the row's lane-load count itself when that is at most 128 (TY whole rows
+// per step, one contiguous span), else an equal cut of it.
 // Persistent: kColBlocksPerCu workgroups per CU; row tiles of TY*kColUnroll rows
 // are dealt round-robin over blockIdx.y, so at any moment the grid reads one
 // compact, advancing window of the matrix, and a workgroup's next tile is in

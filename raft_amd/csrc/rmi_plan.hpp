@@ -26,6 +26,7 @@ constexpr int kWavesPerCu = 32;  // 8 resident waves on each of the 4 SIMDs
 // tiles in flight per workgroup, 2 per CU (8 waves) sustains ~7.1 TB/s; 4 and 8 per CU
 // lose 2 and 8 points to queueing in the memory system.
 constexpr int kColBlocksPerCu = 2;
+constexpr int kColMaxLanes = 128;     // COL_TILE: most lanes of a workgroup along one row
 constexpr int64_t kGroupMinLen = 256;  // COL_TILE: fewest row groups worth reading rows in groups
 constexpr int kLdsPerCu       = 160 * 1024;  // LDS bytes of one gfx950 CU
 constexpr int64_t kBytesInFlightPerCu = 80 * 1024;  // target of the wave-per-row plan
@@ -270,24 +271,19 @@ inline int make_plan(const rmi_reduce_desc& d,
         rows         = p.group_len;
       }
     }
-    // A workgroup covers TX lane-loads of a row (TX columns groups) times TY rows per step.
-    // Rows of up to 64 lane-loads take exactly that many lanes, and as many rows as fit the
-    // workgroup: 33 lane-loads on 64 lanes would leave every other lane idle, 7 rows of 33
-    // leave 25 of 256.  Longer rows are cut into the fewest pieces of at most 64 lanes that
-    // keep four lanes in five busy (or the best of four cuts).
+    // A workgroup covers TX lane-loads of a row times TY rows per step.  Rows of up to
+    // kColMaxLanes lane-loads take exactly that many lanes, and as many whole rows as fit the
+    // workgroup: its step then reads one contiguous span, and 33 lane-loads keep 231 of 256
+    // lanes busy where a power-of-two 64 would idle every other lane.  Longer rows are cut
+    // into the fewest equal pieces of at most kColMaxLanes lanes.  (Measured at 512 MB fp32,
+    // D = 260 / 300 / 517 / 4097: 83 / 82 / 77 / 67 % this way, 70 / 71 / 61 / 54 % with
+    // pieces of at most 64 lanes; reading such rows in aligned groups did not help.)
     {
-      const int64_t g0 = ceildiv(lanes, 64);
-      int64_t best_g = g0, best_num = -1, best_den = 1;
-      for (int64_t g = g0; g < g0 + 4; ++g) {
-        const int64_t tx = ceildiv(lanes, g), ty = kPlanBlock / tx;
-        const int64_t num = lanes * ty, den = g * kPlanBlock;  // busy lanes / lanes
-        if (best_num < 0 || num * best_den > best_num * den) best_g = g, best_num = num, best_den = den;
-        if (num * 5 >= den * 4) break;
-      }
-      p.TX    = (int)ceildiv(lanes, best_g);
+      const int64_t cuts = ceildiv(lanes, kColMaxLanes);
+      p.TX    = (int)ceildiv(lanes, cuts);
       p.TY    = kPlanBlock / p.TX;
       p.gridx = ceildiv(lanes, p.TX);
-      p.dense = (p.TX & (p.TX - 1)) != 0;
+      p.dense = (p.TX & (p.TX - 1)) != 0 || p.TX > 64;
       p.logTX = p.dense ? 0 : ilog2(p.TX);
     }
     // row tiles of TY*unroll rows are dealt round-robin to B blocks: kColBlocksPerCu

@@ -101,14 +101,14 @@ void check(const rmi_reduce_desc& d, int n_cu, uintptr_t in_misalign)
       break;
     case RMI_PLAN_COL_TILE:
       REQUIRE(p.strided);
-      REQUIRE(p.TX >= 1 && p.TX <= 64 && p.TY == kPlanBlock / p.TX && p.TY >= 4);
-      REQUIRE(p.dense == ((p.TX & (p.TX - 1)) != 0));
+      REQUIRE(p.TX >= 1 && p.TX <= 128 && p.TY == kPlanBlock / p.TX && p.TY >= 2);
+      REQUIRE(p.dense == ((p.TX & (p.TX - 1)) != 0 || p.TX > 64));
       if (!p.dense) REQUIRE((1 << p.logTX) == p.TX);
       REQUIRE(p.grid_blocks == p.gridx * p.B);
       {
         const int64_t lanes = p.group > 0 ? p.group_nvec : nload;
         REQUIRE(p.gridx * p.TX >= lanes && (p.gridx - 1) * p.TX < lanes);
-        // at least three lanes in five carry data (cuts of a row are chosen for four in five)
+        // at least three lanes in five carry data
         REQUIRE(lanes * p.TY * 5 >= p.gridx * kPlanBlock * 3 || lanes < 4);
       }
       if (p.group > 0) {
