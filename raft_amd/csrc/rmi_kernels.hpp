@@ -39,6 +39,9 @@ struct RowArgs {
   int logG;
   int B;           // chunks per row (row_block_kernel)
   int logT;        // row_block_kernel: a team is 64 << logT threads
+  int R;           // row_short_kernel, any G: 64 / G rows per wave step
+  u32 invG;        // row_short_kernel, any G: 65536 / G + 1, so that (x * invG) >> 16 == x / G
+  u32 invR;        // likewise for R                              for every x < 64
   Epilogue epi;
 };
 
@@ -248,9 +251,12 @@ __device__ __forceinline__ void last_batch_n(int n, typename P::acc_t& acc, cons
 
 // ---------------------------------------------------------------------------
 // Short rows: nvec <= G, one lane-load per lane per row, kUnroll tiles of
-// 64/G rows in flight per wave.
+// 64/G rows in flight per wave.  ANYG = false: G is a power of two.  true: G is
+// the row's lane-load count itself (4..32), 64 / G whole rows share the wave and
+// its last 64 % G lanes idle; 9 lane-loads then keep 63 lanes busy where 16
+// lanes per row would idle 7 of every 16.
 // ---------------------------------------------------------------------------
-template <class P, bool VEC16>
+template <class P, bool VEC16, bool ANYG = false>
 __global__ __launch_bounds__(kBlock) void row_short_kernel(RowArgs a)
 {
   using acc_t     = typename P::acc_t;
@@ -259,11 +265,11 @@ __global__ __launch_bounds__(kBlock) void row_short_kernel(RowArgs a)
   const int lane  = threadIdx.x & (kWave - 1);
   const i64 wid   = (i64)blockIdx.x * (kBlock / kWave) + (threadIdx.x >> 6);
   const int G     = a.G;
-  const int R     = kWave >> a.logG;
-  const int c     = lane & (G - 1);
-  const int g     = lane >> a.logG;
+  const int R     = ANYG ? a.R : kWave >> a.logG;
+  const int g     = ANYG ? (int)(((u32)lane * a.invG) >> 16) : lane >> a.logG;
+  const int c     = ANYG ? lane - g * G : lane & (G - 1);
   const i64 nload  = a.nvec + (a.tail > 0 ? 1 : 0);  // the tail is one more lane-load
-  const bool incol = c < nload;
+  const bool incol = ANYG ? g < R : c < nload;
 
   // Loads are unconditional: a lane without work (past the row's last lane-load, or a
   // row past the matrix) re-reads the nearest vector that has some.  Loads under a lane
@@ -284,6 +290,29 @@ __global__ __launch_bounds__(kBlock) void row_short_kernel(RowArgs a)
     acc[t] = P::neutral();
     if (incol && row[t] < a.n_out) H::push_any(acc[t], x[t], c, a.nvec, a.len, a.tail);
   }
+  const i64 wave_row0 = wid * kUnroll * R;
+  if constexpr (ANYG) {
+    // fold each row's lanes into its first one: lane c takes lane c + s for s = 1, 2, 4 ...
+    for (int s = 1; s < G; s <<= 1) {
+#pragma unroll
+      for (int t = 0; t < kUnroll; ++t) {
+        const acc_t v = shfl_acc<P>(acc[t], lane + s);
+        if (c + s < G) P::merge(acc[t], v);
+      }
+    }
+    // lane q takes the wave's q-th output (tile q / R, row q % R of it): one contiguous
+    // run of kUnroll * R <= 64 outputs per wave
+    const int tq  = (int)(((u32)lane * a.invR) >> 16);
+    const int src = (lane - tq * R) * G;
+    acc_t mine    = acc[0];
+#pragma unroll
+    for (int t = 0; t < kUnroll; ++t) {
+      const acc_t v = shfl_acc<P>(acc[t], src);
+      if (tq == t) mine = v;
+    }
+    if (lane < kUnroll * R && wave_row0 + lane < a.n_out) finish<P>(a.epi, wave_row0 + lane, mine);
+    return;
+  }
 #pragma unroll
   for (int t = 0; t < kUnroll; ++t)
     group_allreduce<P>(acc[t], G);
@@ -291,7 +320,6 @@ __global__ __launch_bounds__(kBlock) void row_short_kernel(RowArgs a)
   // Every lane of a group now holds its row's result.  Hand the results to lanes
   // so that consecutive lanes own consecutive rows: the wave's kUnroll*R outputs
   // then leave as one contiguous run per store instead of R-element pieces.
-  const i64 wave_row0 = wid * kUnroll * R;
   if (G == 1) {
 #pragma unroll
     for (int t = 0; t < kUnroll; ++t)

@@ -89,7 +89,12 @@ int run(const PlanX& pl, const Problem& pr, hipStream_t st)
         }
       } else if (pl.kind == RMI_PLAN_ROW_WAVE && !pl.team_kernel) {
         if (pl.short_rows) {
-          if (pl.vec16)
+          if (pl.any_g) {
+            a.R    = 64 / pl.G;
+            a.invG = 65536u / (unsigned)pl.G + 1;
+            a.invR = 65536u / (unsigned)a.R + 1;
+            hipLaunchKernelGGL((row_short_kernel<P, true, true>), grid, dim3(kBlock), 0, st, a);
+          } else if (pl.vec16)
             hipLaunchKernelGGL((row_short_kernel<P, true>), grid, dim3(kBlock), 0, st, a);
           else
             hipLaunchKernelGGL((row_short_kernel<P, false>), grid, dim3(kBlock), 0, st, a);

@@ -39,6 +39,7 @@ struct PlanX {
   bool strided    = false;  // reduce along the strided dimension
   bool vec16      = false;  // 16-byte lane loads
   bool short_rows = false;  // ROW_WAVE served by the one-load-per-lane kernel
+  bool any_g      = false;  // short_rows with G = the row's lane-load count (not a power of two)
   bool team_kernel = false; // served by the team-per-row kernel
   bool stage_ok    = false; // ROW_WAVE: rows could be staged through LDS
   bool staged      = false; // ROW_WAVE: rows are staged through LDS (line-aligned span reads)
@@ -373,7 +374,20 @@ inline int make_plan(const rmi_reduce_desc& d,
       // at 16 vectors, 8 lanes measured better).
       if (p.G < 8 && !(p.tail == 0 && nload < 16)) p.G = 8;
     }
-    p.logG               = ilog2(p.G);
+    // Lane-load counts that are not close to a power of two (times 1..4 loads per lane)
+    // leave lanes without work: 9 lane-loads on 8 lanes x 2 loads use 9 slots of 16.  The
+    // one-load-per-lane kernel also runs with G = the lane-load count itself, 64 / G whole
+    // rows per wave step.  Its cross-lane steps cost more, so it is taken only where the
+    // power-of-two plans fill fewer than seven slots in ten: 5 lane-loads, and 9 to 12 with
+    // tail elements (1M x 20 / 33 / 35 / 41 / 45 floats: 69 / 52 / 53 / 59 / 62 % -> 78 / 74 /
+    // 76 / 70 / 75 %; at 6, 7, 19 or 21 lane-loads it measured 2 to 10 points slower).
+    if (p.vec16 && (nload == 5 || (p.tail > 0 && nload >= 9 && nload <= 12)) &&
+        (hint == RMI_PLAN_AUTO || hint == RMI_PLAN_ROW_WAVE)) {
+      p.short_rows = true;
+      p.any_g      = true;
+      p.G          = (int)nload;
+    }
+    p.logG               = p.any_g ? 0 : ilog2(p.G);
     const int64_t rows_w = (int64_t)(64 / p.G) * (p.short_rows ? kPlanUnroll : 1);
     p.grid_blocks        = ceildiv(p.n_out, rows_w * (kPlanBlock / 64));
     if (!p.short_rows && p.vec16) {

@@ -75,7 +75,13 @@ void check(const rmi_reduce_desc& d, int n_cu, uintptr_t in_misalign)
       if (p.team_kernel) {
         REQUIRE(p.threads == 64 && p.B == 1 && p.chunk == p.nvec);
       } else {
-        REQUIRE(p.G >= 1 && p.G <= 64 && (p.G & (p.G - 1)) == 0 && (1 << p.logG) == p.G);
+        if (p.any_g) {
+          // one lane per lane-load, whole rows per wave, one run of at most 64 outputs
+          REQUIRE(p.short_rows && p.vec16 && p.G == nload && p.G >= 4 && p.G <= 32);
+          REQUIRE((64 / p.G) * kPlanUnroll <= 64);
+        } else {
+          REQUIRE(p.G >= 1 && p.G <= 64 && (p.G & (p.G - 1)) == 0 && (1 << p.logG) == p.G);
+        }
         // the lanes of a row hold all of its lane-loads, kPlanUnroll apiece (one for short rows)
         REQUIRE((int64_t)p.G * (p.short_rows ? 1 : kPlanUnroll) >= nload);
         if (p.staged) {

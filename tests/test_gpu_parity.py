@@ -387,3 +387,29 @@ def test_grouped_columns(gpu, in_dt, out_dt, kw, rows, cols, shift):
         assert pl.passes == 2 and pl.blocks_per_out % group == 0
     u.check_against_oracle(d, data, misalign_elems=shift,
                            label=f"grouped {rows}x{cols} dt{in_dt} +{shift}")
+
+
+# Rows of 5 lane-loads, or of 9..12 with tail elements: one lane per lane-load, 64 / G whole
+# rows per wave step (G is not a power of two, the wave's last lanes idle).  Row counts around
+# one wave's 4 * (64 / G) rows, and starts off a 16-byte boundary.
+@pytest.mark.parametrize("in_dt,out_dt,kw,cols_list", [
+    (api.F32, api.F32, {}, (17, 20, 33, 35, 38, 41, 45, 47)),
+    (api.F32, api.F32, dict(main_op=api.MAIN_SQ, final_op=api.FIN_SQRT), (19, 34, 46)),
+    (api.F64, api.F64, {}, (9, 10, 17, 19, 21, 23)),
+    (api.BF16, api.F32, {}, (36, 70, 77, 85, 95)),
+    (api.I8, api.I64, {}, (70, 80, 131, 150, 170, 191)),
+    (api.F32, api.KVP_I32_F32, dict(main_op=api.MAIN_KVP, reduce_op=api.RED_ARGMAX, init_f=-np.inf),
+     (20, 33, 47)),
+    (api.F32, api.F32, dict(reduce_op=api.RED_MIN, init_f=np.inf), (18, 43)),
+])
+@pytest.mark.parametrize("rows,shift", [(1, 0), (6, 1), (28, 0), (29, 3), (49, 0), (1000, 1), (5003, 0)])
+def test_any_lane_count_rows(gpu, in_dt, out_dt, kw, cols_list, rows, shift):
+    for cols in cols_list:
+        rng = np.random.default_rng(rows * 11 + cols + shift)
+        data = _rand(rng, in_dt, rows * cols)
+        d = api.make_desc(in_dt, out_dt, rows, cols, **kw)
+        pl = api.plan_query(d)
+        assert pl.kind == api.PLAN_ROW_WAVE
+        assert pl.lanes_per_row in (5, 9, 10, 11, 12), (cols, pl.lanes_per_row)
+        u.check_against_oracle(d, data, misalign_elems=shift,
+                               label=f"any-G {rows}x{cols} dt{in_dt} +{shift}")
