@@ -230,6 +230,7 @@ __device__ __forceinline__ T xchg(T v)
 // results are valid from any lane but not bitwise equal across lanes).
 
 enum : int { kClsFloat = 0, kClsInt = 1, kClsKvp = 2, kClsMeanVar = 3 };
+enum : int { kTailEach = 0, kTailZero = 1, kTailDup = 2 };
 
 template <int MAIN>
 __device__ __forceinline__ double main_f64(double d)
@@ -280,6 +281,12 @@ struct PolF {
   using acc_t              = double;
   static constexpr int VEC = In<InT>::VEC;
   static constexpr int CLS = kClsFloat;
+  // How the overlapping last vector of a row (its first VEC - tail elements were already
+  // counted) is folded: kTailZero: those elements are zeroed and the vector is pushed whole
+  // (sums: every main op maps 0 to 0); kTailDup: the vector is pushed whole as it is (min,
+  // max and arg-reductions do not change when an element is seen twice); kTailEach: element
+  // by element.
+  static constexpr int kTail = RED == RMI_RED_ADD ? kTailZero : kTailDup;
 
   static __device__ __forceinline__ acc_t neutral()
   {
@@ -360,6 +367,7 @@ struct PolKbn {
   using acc_t              = kbn_t;
   static constexpr int VEC = In<InT>::VEC;
   static constexpr int CLS = kClsFloat;
+  static constexpr int kTail = kTailZero;
 
   static __device__ __forceinline__ acc_t neutral() { return kbn_t{0.0, 0.0}; }
   static __device__ __forceinline__ void push(acc_t& a, nat x, i64)
@@ -398,6 +406,7 @@ struct PolI {
   using acc_t              = i64;
   static constexpr int VEC = In<InT>::VEC;
   static constexpr int CLS = kClsInt;
+  static constexpr int kTail = RED == RMI_RED_ADD ? kTailZero : kTailDup;
   // 8-bit inputs: fold a whole vector in 32 bits first (16 terms of at most
   // 2^14 cannot overflow), then widen once.
   static constexpr bool kNarrow = sizeof(InT) == 1;
@@ -499,6 +508,7 @@ struct PolKvp {
   using acc_t              = kvp_t<KeyT, val_t>;
   static constexpr int VEC = In<InT>::VEC;
   static constexpr int CLS = kClsKvp;
+  static constexpr int kTail = kTailDup;
   static constexpr KeyT kKeyMax = sizeof(KeyT) == 4 ? (KeyT)INT32_MAX : (KeyT)INT64_MAX;
 
   static __device__ __forceinline__ acc_t neutral()
@@ -561,6 +571,7 @@ struct PolMeanVar {
   using acc_t              = mv_t;
   static constexpr int VEC = In<InT>::VEC;
   static constexpr int CLS = kClsMeanVar;
+  static constexpr int kTail = kTailEach;
 
   static __device__ __forceinline__ acc_t neutral() { return mv_t{0.0, 0.0, 0.0, 0.0}; }
   static __device__ __forceinline__ void push(acc_t& a, nat x, i64)

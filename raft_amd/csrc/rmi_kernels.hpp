@@ -121,7 +121,20 @@ struct Held {
                                                   i64 len,
                                                   int tail)
   {
-    if constexpr (VEC16) {
+    if constexpr (VEC16 && P::kTail == kTailDup) {
+      P::push_vec(a, x, v < nvec ? v * P::VEC : len - P::VEC);
+    } else if constexpr (VEC16 && P::kTail == kTailZero) {
+      // bytes [0, skip) of the overlapping vector are cleared; the masks are wave-uniform
+      const int skip = (P::VEC - tail) * (int)sizeof(in_t);
+      u32x4 y;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        const int s = skip - 4 * w;
+        const u32 m = s >= 4 ? 0u : s <= 0 ? ~0u : ~0u << (8 * s);
+        y[w]        = v < nvec ? x[w] : x[w] & m;
+      }
+      P::push_vec(a, y, v * P::VEC);
+    } else if constexpr (VEC16) {
       if (v < nvec) {
         P::push_vec(a, x, v * P::VEC);
       } else {
