@@ -15,6 +15,7 @@
 #include <raft/util/cudart_utils.hpp>
 
 #include <cstdint>
+#include <limits>
 #include <random>
 
 #include "check.hpp"
@@ -226,6 +227,70 @@ TEST_CASE(UnknownTypesAndReduceOps)
       for (int j = 0; j < cols; ++j)
         p *= h[(size_t)r * cols + j];
       ok &= close(got[r], p, 1e-12);
+    }
+    CHECK(ok);
+  }
+}
+
+// Column reductions of the template path over element types of 1, 2 and 8 bytes: rows
+// shorter than one 16-byte lane load, rows that end in a partial one, wide rows; the main_op
+// uses the row index, so a thread that owned a wrong column or row would show.
+template <typename T>
+void strided_index_cases()
+{
+  raft::resources handle;
+  auto stream = raft::resource::get_cuda_stream(handle);
+  for (auto [rows, cols] : std::vector<std::pair<int, int>>{
+         {9, 1}, {2000, 3}, {1501, 5}, {4099, 20}, {777, 33}, {3000, 129}, {300, 1030}, {40001, 16}}) {
+    std::mt19937 g(rows + cols);
+    std::uniform_int_distribution<int> di(-100, 100);
+    std::vector<T> h((size_t)rows * cols);
+    for (auto& x : h)
+      x = (T)di(g);
+    auto d   = raft::make_device_matrix<T, int, raft::row_major>(handle, rows, cols);
+    auto out = raft::make_device_vector<long long, int>(handle, cols);
+    raft::update_device(d.data_handle(), h.data(), h.size(), stream);
+    raft::linalg::strided_reduction(
+      handle, raft::make_const_mdspan(d.view()), out.view(), 0LL, false,
+      [] __device__(T a, int i) { return (long long)a * (long long)(1 + i % 5); }, raft::add_op());
+    auto got = to_host(out.data_handle(), (size_t)cols, stream);
+    bool ok  = true;
+    for (int j = 0; j < cols; ++j) {
+      long long s = 0;
+      for (int i = 0; i < rows; ++i)
+        s += (long long)h[(size_t)i * cols + j] * (1 + i % 5);
+      ok &= got[j] == s;
+    }
+    if (!ok) std::printf("  strided %dx%d, %zu-byte elements\n", rows, cols, sizeof(T));
+    CHECK(ok);
+  }
+}
+TEST_CASE(StridedIndexInt8) { strided_index_cases<std::int8_t>(); }
+TEST_CASE(StridedIndexInt16) { strided_index_cases<std::int16_t>(); }
+TEST_CASE(StridedIndexDouble) { strided_index_cases<double>(); }
+
+// arg-max along the columns with the test-local functors (the reference's own kernels
+// reject KeyValuePair outputs there, linalg/strided_reduction.cuh:70-77)
+TEST_CASE(KvpColumnsCustomFunctors)
+{
+  raft::resources handle;
+  auto stream = raft::resource::get_cuda_stream(handle);
+  using KVP   = raft::KeyValuePair<int, float>;
+  for (auto [rows, cols] : std::vector<std::pair<int, int>>{{5000, 7}, {3001, 64}, {901, 130}}) {
+    auto h   = uniform<float>((size_t)rows * cols, -1.0, 1.0, 99 + cols);
+    auto d   = raft::make_device_matrix<float, int, raft::row_major>(handle, rows, cols);
+    auto out = raft::make_device_vector<KVP, int>(handle, cols);
+    raft::update_device(d.data_handle(), h.data(), h.size(), stream);
+    raft::linalg::strided_reduction(handle, raft::make_const_mdspan(d.view()), out.view(),
+                                    KVP{0, -std::numeric_limits<float>::infinity()}, false,
+                                    ValueToKVP<float, int>{}, ArgMaxOp<int, float>{});
+    auto got = to_host(out.data_handle(), (size_t)cols, stream);
+    bool ok  = true;
+    for (int j = 0; j < cols; ++j) {
+      int best = 0;
+      for (int i = 1; i < rows; ++i)
+        if (h[(size_t)i * cols + j] > h[(size_t)best * cols + j]) best = i;
+      ok &= got[j].key == best && got[j].value == h[(size_t)best * cols + j];
     }
     CHECK(ok);
   }
