@@ -375,13 +375,16 @@ inline int make_plan(const rmi_reduce_desc& d,
       if (p.G < 8 && !(p.tail == 0 && nload < 16)) p.G = 8;
     }
     // Lane-load counts that are not close to a power of two (times 1..4 loads per lane)
-    // leave lanes without work: 9 lane-loads on 8 lanes x 2 loads use 9 slots of 16.  The
-    // one-load-per-lane kernel also runs with G = the lane-load count itself, 64 / G whole
-    // rows per wave step.  Its cross-lane steps cost more, so it is taken only where the
-    // power-of-two plans fill fewer than seven slots in ten: 5 lane-loads, and 9 to 12 with
-    // tail elements (1M x 20 / 33 / 35 / 41 / 45 floats: 69 / 52 / 53 / 59 / 62 % -> 78 / 74 /
-    // 76 / 70 / 75 %; at 6, 7, 19 or 21 lane-loads it measured 2 to 10 points slower).
-    if (p.vec16 && (nload == 5 || (p.tail > 0 && nload >= 9 && nload <= 12)) &&
+    // leave lanes without work: 9 lane-loads on 8 lanes x 2 loads use 9 slots of 16, and a
+    // row cut over two load instructions is fetched as two pieces.  The one-load-per-lane
+    // kernel also runs with G = the lane-load count itself, 64 / G whole rows per wave step
+    // (one contiguous span per load instruction).  Its cross-lane steps cost more, so the
+    // rule follows what was measured on 1M-row fp32 matrices: 5 lane-loads, and 6 or 9 to 17
+    // when the row ends in tail elements (D = 20 / 21 / 33 / 41 / 45 / 54 / 62: 69 / 66 / 52 /
+    // 59 / 62 / 69 / 72 % -> 78 / 77 / 74 / 70 / 75 / 79 / 80 %); at 7 lane-loads with a tail, or
+    // at 6, 7, 19, 21 without one, it measured 2 to 10 points slower.
+    if (p.vec16 &&
+        (nload == 5 || (p.tail > 0 && (nload == 6 || (nload >= 9 && nload <= 17)))) &&
         (hint == RMI_PLAN_AUTO || hint == RMI_PLAN_ROW_WAVE)) {
       p.short_rows = true;
       p.any_g      = true;
