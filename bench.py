@@ -535,8 +535,8 @@ def main():
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs (see
 # profiles/), scaled by the same counters' reading for a copy kernel of known size.
 MEASURED_TRAFFIC: dict[str, float | None] = {
-    "cfg1": 10.36e6, "cfg2": 516.03e6, "cfg3_mean": 2561.34e6, "cfg3_stddev": 2561.34e6,
-    "cfg4": 8394.17e6, "cfg5a": 67.28e6, "cfg5b": 268.58e6, "cfg5c": 67.34e6,
+    "cfg1": 10.36e6, "cfg2": 516.04e6, "cfg3_mean": 2561.39e6, "cfg3_stddev": 2561.38e6,
+    "cfg4": 8394.27e6, "cfg5a": 67.28e6, "cfg5b": 268.58e6, "cfg5c": 67.33e6,
 }
 
 
