@@ -6,8 +6,9 @@
 // lane-load, used for rows shorter than 16 bytes.
 //
 //   row_lanes_kernel  K whole rows inside one 16-byte vector: no cross-lane step
-//   row_short_kernel  rows of at most G<=8 vectors: one vector per lane, G lanes
-//                     per row, 4 row-tiles in flight per wave
+//   row_short_kernel  one vector per lane, G lanes per row (a power of two up to 8,
+//                     or the row's own lane-load count up to 32), 4 row-tiles in
+//                     flight per wave
 //   row_wave_kernel   G<=64 lanes of one wave per row, at most 4 loads per lane
 //   row_block_kernel  teams of 64..1024 threads per row chunk, B chunks per row;
 //                     B == 1 writes outputs, B > 1 writes partials

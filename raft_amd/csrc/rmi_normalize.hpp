@@ -20,7 +20,9 @@ struct NormArgs {
   int tail;    // elements after the last whole vector
   int G;       // lanes per row (wave kernel)
   int logG;
-  int L;       // wave kernel: lane-loads per lane and row (1, 2 or 4)
+  int L;       // wave kernel: lane-loads per lane and row (1 to 4); 0: one per lane with
+               // G = the row's lane-load count itself (not a power of two)
+  u32 invG;    // L == 0: 65536 / G + 1, so that (lane * invG) >> 16 == lane / G
   int final_op;
   double init;
   double eps;
@@ -110,20 +112,13 @@ __device__ __forceinline__ void write_scaled(const NormArgs& a,
 {
   using in_t = typename P::in_t;
   if constexpr (VEC16) {
-    if (v < a.nvec) {
-      u32x4 y = x;
-      static_for<P::VEC>([&](auto j) {
-        Put<in_t>::template at<decltype(j)::value>(y, In<in_t>::template get<decltype(j)::value>(x) / norm);
-      });
-      store16(orow + v * 16, y);
-    } else {
-      // the overlapping last vector: only its last `tail` elements are new
-      in_t* o        = reinterpret_cast<in_t*>(orow) + (a.len - P::VEC);
-      const int skip = P::VEC - a.tail;
-      static_for<P::VEC>([&](auto j) {
-        if (j >= skip) Put<in_t>::st(o + j, In<in_t>::template get<decltype(j)::value>(x) / norm);
-      });
-    }
+    // The overlapping last vector (v == nvec) is stored whole where it was read: its first
+    // VEC - tail elements repeat what the lane before it stores, bit for bit.
+    u32x4 y = x;
+    static_for<P::VEC>([&](auto j) {
+      Put<in_t>::template at<decltype(j)::value>(y, In<in_t>::template get<decltype(j)::value>(x) / norm);
+    });
+    store16(v < a.nvec ? orow + v * 16 : orow + (a.len - P::VEC) * (i64)sizeof(in_t), y);
   } else {
     Put<in_t>::st(reinterpret_cast<in_t*>(orow) + v, x / norm);
   }
@@ -190,13 +185,73 @@ __device__ __forceinline__ void normalize_wave_body(const NormArgs& a)
   }
 }
 
+// Rows of G lane-loads, G not a power of two: one lane per lane-load, 64 / G whole rows per
+// wave step and kUnroll steps in flight, so every load and store instruction covers one
+// contiguous span of the matrix; the wave's last 64 % G lanes idle.  The row's lanes are
+// folded into its first one (lane c takes lane c + s for s = 1, 2, 4 ...), which hands the
+// norm back to all of them.
+template <class P>
+__device__ __forceinline__ void normalize_anyg_body(const NormArgs& a)
+{
+  using acc_t     = typename P::acc_t;
+  using H         = Held<P, true>;
+  const int lane  = threadIdx.x & (kWave - 1);
+  const i64 wid   = (i64)blockIdx.x * (kBlock / kWave) + (threadIdx.x >> 6);
+  const int G     = a.G;
+  const int R     = kWave / G;
+  const int g     = (int)(((u32)lane * a.invG) >> 16);
+  const int c     = lane - g * G;
+  const bool live = g < R;
+
+  typename H::type x[kUnroll];
+  i64 row[kUnroll];
+  const i64 cl = live ? (i64)c : (i64)G - 1;
+#pragma unroll
+  for (int t = 0; t < kUnroll; ++t) {  // unconditional, clamped: see normalize_wave_body
+    row[t]       = (wid * kUnroll + t) * R + g;
+    const i64 rl = row[t] < a.n_rows ? row[t] : a.n_rows - 1;
+    x[t] = H::load_any(static_cast<const char*>(a.in) + rl * a.row_bytes, cl, a.nvec, a.len);
+  }
+  acc_t acc[kUnroll];
+#pragma unroll
+  for (int t = 0; t < kUnroll; ++t) {
+    acc[t] = P::neutral();
+    if (live && row[t] < a.n_rows) H::push_any(acc[t], x[t], c, a.nvec, a.len, a.tail);
+  }
+  for (int s = 1; s < G; s <<= 1) {
+#pragma unroll
+    for (int t = 0; t < kUnroll; ++t) {
+      const acc_t v = shfl_acc<P>(acc[t], lane + s);
+      if (c + s < G) P::merge(acc[t], v);
+    }
+  }
+  const int first = live ? g * G : lane;
+#pragma unroll
+  for (int t = 0; t < kUnroll; ++t) {
+    const acc_t total = shfl_acc<P>(acc[t], first);
+    if (live && row[t] < a.n_rows) {
+      const auto norm = row_norm<P>(a, total);
+      if (norm > (typename P::nat)a.eps)  // false for NaN norms too
+        write_scaled<P, true>(a, static_cast<char*>(a.out) + row[t] * a.row_bytes, x[t], c, norm);
+    }
+  }
+}
+
 template <class P, bool VEC16>
 __global__ __launch_bounds__(kBlock) void normalize_wave_kernel(NormArgs a)
 {
+  if constexpr (VEC16) {
+    if (a.L == 0) {
+      normalize_anyg_body<P>(a);
+      return;
+    }
+  }
   if (a.L == 1) {
     normalize_wave_body<P, VEC16, 1>(a);
   } else if (a.L == 2) {
     normalize_wave_body<P, VEC16, 2>(a);
+  } else if (a.L == 3) {
+    normalize_wave_body<P, VEC16, 3>(a);
   } else {
     normalize_wave_body<P, VEC16, 4>(a);
   }

@@ -74,8 +74,24 @@ def test_long_rows(gpu, rows, cols, norm):
         assert np.allclose(n, 1.0, atol=1e-5)
 
 
+# Rows whose lane-load count is not a power of two take one lane per lane-load (3..32 and
+# 48..63 lane-loads, whole rows per wave step) or three loads per lane; row counts around
+# one wave's and one workgroup's share.
+@pytest.mark.parametrize("cols", [10, 20, 21, 45, 50, 67, 100, 127, 129, 190, 200, 222, 250, 255, 300])
+@pytest.mark.parametrize("rows", [1, 5, 29, 257, 4099])
+def test_lane_counts(gpu, rows, cols):
+    rng = np.random.default_rng(rows * 1000 + cols)
+    data = rng.uniform(-3, 3, rows * cols).astype(np.float32)
+    d = api.make_desc(api.F32, api.F32, rows, cols, main_op=api.MAIN_SQ, final_op=api.FIN_SQRT)
+    prev = np.full(rows * cols, 9.0, dtype=np.float32)
+    got = _gpu(d, data, prev, 1e-8)
+    exp = _oracle(d, data, prev, 1e-8)
+    assert u.approx_ok(got, exp, 1e-5).all(), u.worst_rel(got, exp)
+
+
 @pytest.mark.parametrize("dt", [api.F16, api.BF16])
-@pytest.mark.parametrize("rows,cols", [(100, 64), (1000, 100), (33, 7), (7, 9000)])
+@pytest.mark.parametrize("rows,cols", [(100, 64), (1000, 100), (33, 7), (7, 9000), (500, 33), (301, 108),
+                                       (64, 450)])
 def test_half_types(gpu, dt, rows, cols):
     rng = np.random.default_rng(3)
     f = rng.uniform(-4, 4, rows * cols).astype(np.float32)
