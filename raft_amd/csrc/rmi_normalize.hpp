@@ -115,9 +115,19 @@ __device__ __forceinline__ void write_scaled(const NormArgs& a,
     // The overlapping last vector (v == nvec) is stored whole where it was read: its first
     // VEC - tail elements repeat what the lane before it stores, bit for bit.
     u32x4 y = x;
-    static_for<P::VEC>([&](auto j) {
-      Put<in_t>::template at<decltype(j)::value>(y, In<in_t>::template get<decltype(j)::value>(x) / norm);
-    });
+    if constexpr (sizeof(in_t) == 2) {
+      // 16-bit elements: one division per lane-load, then products in fp32 that are rounded
+      // to 11 or 8 significant bits anyway (eight divisions per lane-load made these rows
+      // ALU-bound); fp32 and fp64 rows divide element by element as the reference does
+      const typename P::nat inv = (typename P::nat)1 / norm;
+      static_for<P::VEC>([&](auto j) {
+        Put<in_t>::template at<decltype(j)::value>(y, In<in_t>::template get<decltype(j)::value>(x) * inv);
+      });
+    } else {
+      static_for<P::VEC>([&](auto j) {
+        Put<in_t>::template at<decltype(j)::value>(y, In<in_t>::template get<decltype(j)::value>(x) / norm);
+      });
+    }
     store16(v < a.nvec ? orow + v * 16 : orow + (a.len - P::VEC) * (i64)sizeof(in_t), y);
   } else {
     Put<in_t>::st(reinterpret_cast<in_t*>(orow) + v, x / norm);
