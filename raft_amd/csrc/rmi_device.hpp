@@ -482,6 +482,16 @@ struct PolI {
   {
     static_for<VEC>([&](auto j) { push(a[j], In<InT>::template get<j>(v), 0); });
   }
+  // Column sums of 8-bit elements gather in 32-bit accumulators (one add per byte where a
+  // 64-bit one costs three) and are emptied into the 64-bit ones every kColFlush lane-loads
+  // (2 % more instructions): a term is at most 2^14 (a squared byte), so 128 of them stay far
+  // below 2^31, and matrices of a few hundred MB already pass through the emptying step.
+  static constexpr bool kColNarrow = kNarrow && RED == RMI_RED_ADD;
+  static constexpr int kColFlush   = 128;
+  static __device__ __forceinline__ void push_cols_narrow(int32_t (&a)[VEC], const u32x4& v)
+  {
+    static_for<VEC>([&](auto j) { a[j] += main_i32<MAIN>((int32_t)In<InT>::template get<j>(v)); });
+  }
   static __device__ __forceinline__ void merge(acc_t& a, const acc_t& b) { a = red<i64>(a, b); }
   template <int SEL>
   static __device__ __forceinline__ acc_t exchange(const acc_t& a)

@@ -584,12 +584,19 @@ __global__ __launch_bounds__(1024) void row_block_kernel(RowArgs a)
 // is what lets loads stay in flight across iterations: gfx9 counts loads and
 // stores in one in-order counter.)
 // ---------------------------------------------------------------------------
+// policies that gather column terms in 32-bit accumulators first (P::kColNarrow)
+template <class P, class = void>
+struct col_narrow : std::false_type {};
+template <class P>
+struct col_narrow<P, std::void_t<decltype(P::kColNarrow)>> : std::bool_constant<P::kColNarrow> {};
+
 template <class P, bool VEC16>
 __global__ __launch_bounds__(kBlock) void col_kernel(ColArgs a)
 {
   using acc_t     = typename P::acc_t;
   using in_t      = typename P::in_t;
   constexpr int S = VEC16 ? P::VEC : 1;
+  constexpr bool NARROW = VEC16 && col_narrow<P>::value;
   constexpr int W = kBlock / kWave;
   __shared__ acc_t sm[W * kWave * S];
 
@@ -620,6 +627,18 @@ __global__ __launch_bounds__(kBlock) void col_kernel(ColArgs a)
       const char* p = whole ? inb + cv * 16 : inb + (a.n_out - S) * (i64)sizeof(in_t);
       i64 tile      = blockIdx.y;
       u32x4 x[kColUnroll];
+      int32_t narrow[NARROW ? S : 1] = {};
+      int gathered                   = 0;  // lane-loads in `narrow`
+      auto flush = [&]() {
+        if constexpr (NARROW) {
+#pragma unroll
+          for (int j = 0; j < S; ++j) {
+            acc[j] += narrow[j];
+            narrow[j] = 0;
+          }
+          gathered = 0;
+        }
+      };
       if (tile < n_full) {
 #pragma unroll
         for (int u = 0; u < kColUnroll; ++u)
@@ -633,14 +652,23 @@ __global__ __launch_bounds__(kBlock) void col_kernel(ColArgs a)
           for (int u = 0; u < kColUnroll; ++u)
             y[u] = load16(p + (next * RT + ty + (i64)u * TY) * a.row_bytes);
         }
+        if constexpr (NARROW) {
 #pragma unroll
-        for (int u = 0; u < kColUnroll; ++u)
-          P::push_cols(acc, x[u], tile * RT + ty + (i64)u * TY);
+          for (int u = 0; u < kColUnroll; ++u)
+            P::push_cols_narrow(narrow, x[u]);
+          gathered += kColUnroll;
+          if (gathered >= P::kColFlush) flush();
+        } else {
+#pragma unroll
+          for (int u = 0; u < kColUnroll; ++u)
+            P::push_cols(acc, x[u], tile * RT + ty + (i64)u * TY);
+        }
 #pragma unroll
         for (int u = 0; u < kColUnroll; ++u)
           x[u] = y[u];
         tile = next;
       }
+      flush();
       if ((i64)blockIdx.y == n_full % a.B) {  // the rows past the last whole tile
         for (i64 r = n_full * RT + ty; r < a.len; r += TY)
           P::push_cols(acc, load16(p + r * a.row_bytes), r);

@@ -413,3 +413,26 @@ def test_any_lane_count_rows(gpu, in_dt, out_dt, kw, cols_list, rows, shift):
         assert pl.lanes_per_row in (5, 6, 9, 10, 11, 12, 13, 14, 15, 16, 17), (cols, pl.lanes_per_row)
         u.check_against_oracle(d, data, misalign_elems=shift,
                                label=f"any-G {rows}x{cols} dt{in_dt} +{shift}")
+
+
+# Column sums of 8-bit elements gather in 32-bit accumulators that are emptied into the
+# 64-bit ones every 128 lane-loads: 17M rows give every thread of the 512 workgroups more
+# than that.  Extreme values (all -128, squared) would overflow 32 bits within 2^17 terms.
+@pytest.mark.parametrize("in_dt,kw", [(api.I8, dict(main_op=api.MAIN_SQ)), (api.U8, {}),
+                                      (api.I8, dict(main_op=api.MAIN_ABS))])
+def test_narrow_column_sums_many_rows(gpu, in_dt, kw):
+    rows, cols = 17_000_001, 16
+    npdt = np.int8 if in_dt == api.I8 else np.uint8
+    data = np.full(rows * cols, -128 if in_dt == api.I8 else 255, dtype=npdt)
+    rng = np.random.default_rng(5)
+    idx = rng.integers(0, rows * cols, 1_000_000)
+    data[idx] = rng.integers(-128 if in_dt == api.I8 else 0, 128 if in_dt == api.I8 else 256,
+                             idx.size).astype(npdt)
+    d = api.make_desc(in_dt, api.I64, rows, cols, apply=api.ALONG_COLUMNS, **kw)
+    got = u.decode_out(api.I64, u.gpu_reduce(d, data))
+    m = data.reshape(rows, cols).astype(np.int64)
+    if kw.get("main_op") == api.MAIN_SQ:
+        m = m * m
+    elif kw.get("main_op") == api.MAIN_ABS:
+        m = np.abs(m)
+    assert np.array_equal(got, m.sum(axis=0))
