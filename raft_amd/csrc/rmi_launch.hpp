@@ -236,10 +236,16 @@ int run_normalize(const NormPlan& pl, const NormArgs& args, hipStream_t st)
   if (pl.grid > 0x7fffffffLL) return RMI_ERR_BAD_SHAPE;
   const dim3 grid((unsigned)pl.grid);
   if (pl.kind == 0) {
-    if (pl.vec16)
-      hipLaunchKernelGGL((normalize_wave_kernel<P, true>), grid, dim3(kBlock), 0, st, a);
-    else
+    if (!pl.vec16) {
       hipLaunchKernelGGL((normalize_wave_kernel<P, false>), grid, dim3(kBlock), 0, st, a);
+    } else if ((a.row_bytes % 128 == 0 || (pl.L == 1 && ((kWave / pl.G) * a.row_bytes) % 128 == 0)) &&
+               reinterpret_cast<uintptr_t>(a.out) % 128 == 0) {
+      // every store instruction writes whole cache lines (rows of whole lines, or the rows
+      // of one wave step together) at an aligned address: streamed stores
+      hipLaunchKernelGGL((normalize_wave_kernel<P, true, true>), grid, dim3(kBlock), 0, st, a);
+    } else {
+      hipLaunchKernelGGL((normalize_wave_kernel<P, true>), grid, dim3(kBlock), 0, st, a);
+    }
   } else if (pl.kind == 1) {
     // rows of 4 KB and more always hold whole vectors
     const dim3 block((unsigned)pl.threads);

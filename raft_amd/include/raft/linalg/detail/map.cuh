@@ -48,12 +48,52 @@ struct map_pack {
   T v[R];
 };
 
+// Packs of 4, 8 or 16 bytes move as one non-temporal access (every element is read and
+// written once); other sizes element by element.
+template <int BYTES>
+struct map_word {
+  using type = void;
+};
+template <>
+struct map_word<4> {
+  using type = std::uint32_t;
+};
+template <>
+struct map_word<8> {
+  typedef std::uint32_t type __attribute__((ext_vector_type(2)));
+};
+template <>
+struct map_word<16> {
+  typedef std::uint32_t type __attribute__((ext_vector_type(4)));
+};
+
 template <typename T, int R>
 __device__ __forceinline__ map_pack<T, R> map_load(const T* p, std::int64_t off)
 {
   map_pack<T, R> x;
-  __builtin_memcpy(&x, p + off, sizeof(x));
+  using W = typename map_word<(int)sizeof(map_pack<T, R>)>::type;
+  if constexpr (!std::is_void_v<W> && std::is_trivially_copyable_v<T>) {
+    typedef W W_unaligned __attribute__((aligned(1)));
+    const W w = __builtin_nontemporal_load(reinterpret_cast<const W_unaligned*>(p + off));
+    __builtin_memcpy(&x, &w, sizeof(x));
+  } else {
+    __builtin_memcpy(&x, p + off, sizeof(x));
+  }
   return x;
+}
+
+template <typename T, int R>
+__device__ __forceinline__ void map_store(T* p, std::int64_t off, const map_pack<T, R>& x)
+{
+  using W = typename map_word<(int)sizeof(map_pack<T, R>)>::type;
+  if constexpr (!std::is_void_v<W> && std::is_trivially_copyable_v<T>) {
+    typedef W W_unaligned __attribute__((aligned(1)));
+    W w;
+    __builtin_memcpy(&w, &x, sizeof(x));
+    __builtin_nontemporal_store(w, reinterpret_cast<W_unaligned*>(p + off));
+  } else {
+    __builtin_memcpy(p + off, &x, sizeof(x));
+  }
 }
 
 template <int R, bool PassOffset, typename IdxT>
@@ -91,7 +131,7 @@ __device__ __forceinline__ void map_store_set(map_cfg<R, PassOffset, IdxT>, OutT
   for (int j = 0; j < R; ++j)
     o.v[j] = map_apply<PassOffset, OutT, IdxT, Func, Done...>(f, static_cast<IdxT>(off + j),
                                                               xs.v[j]...);
-  __builtin_memcpy(out + off, &o, sizeof(o));
+  map_store<OutT, R>(out, off, o);
 }
 template <int R, bool PassOffset, typename IdxT, typename OutT, typename Func, typename T,
           typename... Rest, typename... Done>
