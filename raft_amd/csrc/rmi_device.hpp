@@ -903,6 +903,60 @@ __device__ __forceinline__ void finish_run(const Epilogue& e, i64 k0, typename P
       return;
     }
   }
+  if constexpr (P::CLS == kClsFloat && (K % 2 == 0)) {
+    // the same for floating results: four f32 or two f64 per 16-byte store, two f32 per
+    // 8-byte store (k0 is a multiple of K, so the stores are aligned when the output is)
+    if (e.plain && e.out_aligned16) {
+      auto value = [&](int r) {
+        typename P::acc_t a = P::from_f64(e.init_f);
+        P::merge(a, acc[r]);
+        return P::to_f64(a);
+      };
+      if (e.out_dtype == RMI_F32) {
+        float y[K];
+#pragma unroll
+        for (int r = 0; r < K; ++r) {
+          y[r] = (float)value(r);
+          if (e.final_op == RMI_FIN_SQRT) y[r] = sqrt(y[r]);
+          if (e.final_op == RMI_FIN_MUL_CONST) y[r] = y[r] * (float)e.s1;
+        }
+        float* o = static_cast<float*>(e.out) + k0;
+        if constexpr (K % 4 == 0) {
+#pragma unroll
+          for (int r = 0; r < K; r += 4) {
+            u32x4 v;
+            v[0] = as_u32(y[r]), v[1] = as_u32(y[r + 1]), v[2] = as_u32(y[r + 2]), v[3] = as_u32(y[r + 3]);
+            __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(o + r));
+          }
+        } else {
+          typedef u32 u32x2 __attribute__((ext_vector_type(2)));
+#pragma unroll
+          for (int r = 0; r < K; r += 2) {
+            u32x2 v;
+            v[0] = as_u32(y[r]), v[1] = as_u32(y[r + 1]);
+            __builtin_nontemporal_store(v, reinterpret_cast<u32x2*>(o + r));
+          }
+        }
+        return;
+      }
+      if (e.out_dtype == RMI_F64) {
+        typedef double f64x2 __attribute__((ext_vector_type(2)));
+#pragma unroll
+        for (int r = 0; r < K; r += 2) {
+          f64x2 v;
+#pragma unroll
+          for (int q = 0; q < 2; ++q) {
+            double y = value(r + q);
+            if (e.final_op == RMI_FIN_SQRT) y = sqrt(y);
+            if (e.final_op == RMI_FIN_MUL_CONST) y = y * e.s1;
+            v[q] = y;
+          }
+          __builtin_nontemporal_store(v, reinterpret_cast<f64x2*>(static_cast<double*>(e.out) + k0 + r));
+        }
+        return;
+      }
+    }
+  }
 #pragma unroll
   for (int r = 0; r < K; ++r)
     finish<P>(e, k0 + r, acc[r]);

@@ -194,11 +194,15 @@ __global__ __launch_bounds__(kBlock) void row_lanes_kernel(RowArgs a)
   const char* inb = static_cast<const char*>(a.in);
 
   u32x4 x[kUnroll];
+  if (nfull > 0) {
 #pragma unroll
-  for (int u = 0; u < kUnroll; ++u) {
-    // consecutive lanes take consecutive vectors within each unroll slot
-    const i64 v = ((i64)blockIdx.x * kUnroll + u) * kBlock + threadIdx.x;
-    if (v < nfull) x[u] = load16(inb + v * 16);
+    for (int u = 0; u < kUnroll; ++u) {
+      // consecutive lanes take consecutive vectors within each unroll slot; the loads are
+      // unconditional (a vector past the end re-reads the last one): loads under a lane
+      // mask make the compiler wait for each of them in turn
+      const i64 v = ((i64)blockIdx.x * kUnroll + u) * kBlock + threadIdx.x;
+      x[u]        = load16(inb + (v < nfull ? v : nfull - 1) * 16);
+    }
   }
 #pragma unroll
   for (int u = 0; u < kUnroll; ++u) {

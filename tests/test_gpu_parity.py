@@ -436,3 +436,36 @@ def test_narrow_column_sums_many_rows(gpu, in_dt, kw):
     elif kw.get("main_op") == api.MAIN_ABS:
         m = np.abs(m)
     assert np.array_equal(got, m.sum(axis=0))
+
+
+# Rows that fit several times into one 16-byte vector (1, 2, 4 or 8 bytes long): lane-local
+# sums, and each lane's results leave as one streamed 8- or 16-byte store when the epilogue is
+# identity, sqrt or a multiplication by a constant and the output is f32, f64 or int64.
+# Row counts that are not a multiple of the rows per vector end with lanes of their own.
+@pytest.mark.parametrize("in_dt,out_dt,cols", [
+    (api.F32, api.F32, 1), (api.F32, api.F32, 2), (api.F64, api.F64, 1), (api.BF16, api.F32, 1),
+    (api.BF16, api.F32, 2), (api.F16, api.F32, 4), (api.F32, api.F64, 1), (api.F16, api.F64, 2),
+    (api.I8, api.I64, 1), (api.I8, api.I64, 4), (api.U8, api.I64, 8), (api.I32, api.I64, 2),
+    (api.I8, api.I32, 2),
+])
+@pytest.mark.parametrize("final", ["identity", "sqrt", "mul", "inplace"])
+@pytest.mark.parametrize("rows", [1, 3, 1025, 70003])
+def test_rows_inside_a_vector(gpu, in_dt, out_dt, cols, final, rows):
+    integer = in_dt in (api.I8, api.U8, api.I32)
+    if integer and final in ("sqrt", "mul"):
+        pytest.skip("floating epilogues")
+    kw = {}
+    if final == "sqrt":
+        kw = dict(main_op=api.MAIN_SQ, final_op=api.FIN_SQRT)
+    elif final == "mul":
+        kw = dict(final_op=api.FIN_MUL_CONST, final_scalar=0.25)
+    elif final == "inplace":
+        kw = dict(inplace=True)
+    rng = np.random.default_rng(rows + cols)
+    data = _rand(rng, in_dt, rows * cols)
+    d = api.make_desc(in_dt, out_dt, rows, cols, **kw)
+    assert api.plan_query(d).kind == api.PLAN_ROW_LANES
+    old = None
+    if final == "inplace":
+        old = u.encode_out(out_dt, rng.integers(-5, 5, rows).astype(np.float64))
+    u.check_against_oracle(d, data, old_raw=old, label=f"lanes {rows}x{cols} {final}")
