@@ -151,10 +151,14 @@ __global__ __launch_bounds__(kMapBlock) void map_kernel(OutT* out, std::int64_t 
   const std::int64_t p0 =
     (std::int64_t)blockIdx.x * (kMapBlock * kMapUnroll) + (std::int64_t)threadIdx.x;
   map_pack_set<R, InTs...> held[kMapUnroll];
+  if (npack > 0) {
+    // unconditional loads (a pack past the end re-reads the last one): under a lane mask
+    // the compiler waits for every load in turn
 #pragma unroll
-  for (int u = 0; u < kMapUnroll; ++u) {
-    const std::int64_t p = p0 + (std::int64_t)u * kMapBlock;
-    if (p < npack) map_load_set(held[u], p * R, ins...);
+    for (int u = 0; u < kMapUnroll; ++u) {
+      const std::int64_t p = p0 + (std::int64_t)u * kMapBlock;
+      map_load_set(held[u], (p < npack ? p : npack - 1) * R, ins...);
+    }
   }
 #pragma unroll
   for (int u = 0; u < kMapUnroll; ++u) {

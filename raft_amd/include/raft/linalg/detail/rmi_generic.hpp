@@ -508,9 +508,9 @@ __global__ __launch_bounds__(kBlock) void map_reduce_multi_kernel(Out* partial, 
   for (std::int64_t p0 = begin + threadIdx.x; p0 < end; p0 += (std::int64_t)kBlock * U) {
     raft::linalg::detail::map_pack_set<R, InTs...> held[U];
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
+    for (int u = 0; u < U; ++u) {  // unconditional, clamped: see map_kernel
       const std::int64_t p = p0 + (std::int64_t)u * kBlock;
-      if (p < end) raft::linalg::detail::map_load_set(held[u], p * R, ins...);
+      raft::linalg::detail::map_load_set(held[u], (p < end ? p : end - 1) * R, ins...);
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
