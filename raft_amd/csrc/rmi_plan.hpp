@@ -279,8 +279,11 @@ inline int make_plan(const rmi_reduce_desc& d,
     // into the fewest equal pieces of at most kColMaxLanes lanes.  (Measured at 512 MB fp32,
     // D = 260 / 300 / 517 / 4097: 83 / 82 / 77 / 67 % this way, 70 / 71 / 61 / 54 % with
     // pieces of at most 64 lanes; reading such rows in aligned groups did not help.)
+    // Rows that are whole multiples of 64 lane-loads keep pieces of exactly 64 lanes (1 KB
+    // at a 1 KB stride within the row, four rows per step): 32768 x 32768 floats read 86 %
+    // that way and 70 % in 128-lane pieces.
     {
-      const int64_t cuts = ceildiv(lanes, kColMaxLanes);
+      const int64_t cuts = lanes % 64 == 0 ? lanes / 64 : ceildiv(lanes, kColMaxLanes);
       p.TX    = (int)ceildiv(lanes, cuts);
       p.TY    = kPlanBlock / p.TX;
       p.gridx = ceildiv(lanes, p.TX);
