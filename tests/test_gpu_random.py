@@ -1,0 +1,123 @@
+"""Randomised parity: seeded random shapes, layouts, axes, element types and functor
+triples through the C ABI against the oracle.  The shape distribution is log-uniform in
+both extents (up to a few million elements) and mixes in the values around which the plans
+change (powers of two, one more, one less), so every plan and its edge cases are drawn."""
+import os
+
+import numpy as np
+import pytest
+
+from raft_amd import _capi as api
+from tests import _util as u
+from tests.test_gpu_parity import _rand
+
+pytestmark = pytest.mark.gpu
+
+SUM_TYPES = [(api.F32, api.F32), (api.F64, api.F64), (api.BF16, api.F32), (api.F16, api.F32),
+             (api.I8, api.I64), (api.U8, api.I64), (api.I32, api.I64), (api.F32, api.F64),
+             (api.I64, api.I64)]
+MINMAX_TYPES = [(api.F32, api.F32), (api.F64, api.F64), (api.F16, api.F32), (api.I8, api.I64),
+                (api.I32, api.I64)]
+ARG_TYPES = [(api.F32, api.KVP_I32_F32), (api.F64, api.KVP_I32_F64), (api.F32, api.KVP_I64_F32),
+             (api.BF16, api.KVP_I32_F32)]
+EDGES = [1, 2, 3, 4, 5, 7, 8, 9, 15, 16, 17, 31, 32, 33, 63, 64, 65, 127, 128, 129, 255, 256, 257,
+         511, 513, 1023, 1025, 4095, 4097]
+
+
+def _extent(rng, cap):
+    if rng.random() < 0.35:
+        return int(min(cap, rng.choice(EDGES)))
+    return int(min(cap, np.exp(rng.uniform(0, np.log(cap)))))
+
+
+def _case(seed):
+    rng = np.random.default_rng(seed)
+    kind = rng.choice(["sum", "sum", "minmax", "arg"])
+    total = 3_000_000
+    a = _extent(rng, 300_000)
+    b = _extent(rng, max(1, total // a))
+    rows, cols = (a, b) if rng.random() < 0.5 else (b, a)
+    layout = int(rng.choice([api.ROW_MAJOR, api.COL_MAJOR]))
+    apply = int(rng.choice([api.ALONG_ROWS, api.ALONG_COLUMNS]))
+    kw = dict(layout=layout, apply=apply)
+    if kind == "sum":
+        in_dt, out_dt = SUM_TYPES[rng.integers(len(SUM_TYPES))]
+        kw["main_op"] = int(rng.choice([api.MAIN_IDENTITY, api.MAIN_SQ, api.MAIN_ABS, api.MAIN_NZ]))
+        if out_dt in (api.F32, api.F64):
+            fin = rng.choice(["id", "sqrt", "mul"])
+            if fin == "sqrt" and kw["main_op"] in (api.MAIN_SQ, api.MAIN_ABS, api.MAIN_NZ):
+                kw["final_op"] = api.FIN_SQRT
+            elif fin == "mul":
+                kw["final_op"], kw["final_scalar"] = api.FIN_MUL_CONST, 0.125
+        if rng.random() < 0.25:
+            kw["inplace"] = True
+    elif kind == "minmax":
+        in_dt, out_dt = MINMAX_TYPES[rng.integers(len(MINMAX_TYPES))]
+        mx = rng.random() < 0.5
+        kw["reduce_op"] = api.RED_MAX if mx else api.RED_MIN
+        kw["main_op"] = int(rng.choice([api.MAIN_IDENTITY, api.MAIN_ABS]))
+        kw["init_f"], kw["init_i"] = (-np.inf, -2**62) if mx else (np.inf, 2**62)
+    else:
+        in_dt, out_dt = ARG_TYPES[rng.integers(len(ARG_TYPES))]
+        mx = rng.random() < 0.5
+        kw.update(main_op=api.MAIN_KVP, reduce_op=api.RED_ARGMAX if mx else api.RED_ARGMIN,
+                  init_f=-np.inf if mx else np.inf)
+    es = api.DTYPE_SIZE[in_dt]
+    shift = int(rng.choice([0, 0, 1, 2, 3, 16 // es if es < 16 else 1]))
+    return kind, in_dt, out_dt, rows, cols, kw, shift, rng
+
+
+# RMI_RANDOM_CASES widens the draw for a longer run
+@pytest.mark.parametrize("seed", range(int(os.environ.get("RMI_RANDOM_CASES", "400"))))
+def test_random_case(gpu, seed):
+    kind, in_dt, out_dt, rows, cols, kw, shift, rng = _case(seed)
+    data = _rand(rng, in_dt, rows * cols)
+    if kind == "arg" and rows * cols > 8:
+        # plant ties: copies of the extreme value at random places
+        flat = data.reshape(-1)
+        flat[rng.integers(0, flat.size, 6)] = flat.max() if kw["reduce_op"] == api.RED_ARGMAX \
+            else flat.min()
+    d = api.make_desc(in_dt, out_dt, rows, cols, **kw)
+    old = None
+    if kw.get("inplace"):
+        n = u.n_outputs(d)
+        old = u.encode_out(out_dt, rng.integers(-3, 4, n).astype(np.float64))
+    label = (f"seed {seed}: {kind} {api.DTYPE_NAME[in_dt]}->{api.DTYPE_NAME[out_dt]} {rows}x{cols} "
+             f"layout {kw['layout']} apply {kw['apply']} +{shift} {kw}")
+    u.check_against_oracle(d, data, old_raw=old, misalign_elems=shift, label=label)
+
+
+# The same for row normalisation and the one-pass mean / variance.
+@pytest.mark.parametrize("seed", range(int(os.environ.get("RMI_RANDOM_CASES", "400")) // 4))
+def test_random_normalize(gpu, seed):
+    from tests import test_gpu_normalize as tn
+    rng = np.random.default_rng(10_000 + seed)
+    cols = _extent(rng, 100_000)
+    rows = _extent(rng, max(1, 2_000_000 // cols))
+    dt = int(rng.choice([api.F32, api.F32, api.F64, api.BF16, api.F16]))
+    norm = str(rng.choice(list(tn.NORMS)))
+    main, red, fin = tn.NORMS[norm]
+    f = rng.uniform(-4, 4, rows * cols)
+    if dt == api.BF16:
+        data = u.to_bf16(f.astype(np.float32))
+    else:
+        data = f.astype({api.F32: np.float32, api.F64: np.float64, api.F16: np.float16}[dt])
+    d = api.make_desc(dt, dt, rows, cols, main_op=main, reduce_op=red, final_op=fin)
+    prev = np.zeros(rows * cols, dtype=data.dtype)
+    got = tn._as_f64(dt, tn._gpu(d, data, prev, 1e-8))
+    exp = tn._oracle(d, data, tn._as_f64(dt, prev), 1e-8)
+    tol = {api.F32: 1e-5, api.F64: 1e-8}.get(dt, u.OUT_TOL[dt])
+    assert u.approx_ok(got, exp, tol).all(), (seed, dt, rows, cols, norm, u.worst_rel(got, exp))
+
+
+@pytest.mark.parametrize("seed", range(int(os.environ.get("RMI_RANDOM_CASES", "400")) // 4))
+def test_random_meanvar(gpu, seed):
+    from tests import test_gpu_meanvar as tm
+    rng = np.random.default_rng(20_000 + seed)
+    a = _extent(rng, 200_000)
+    b = _extent(rng, max(1, 2_000_000 // a))
+    rows, cols = (a, b) if rng.random() < 0.5 else (b, a)
+    dt = int(rng.choice([api.F32, api.F64]))
+    layout = int(rng.choice([api.ROW_MAJOR, api.COL_MAJOR]))
+    stored = tm._make(rng, dt, layout, rows, cols, float(rng.uniform(-50, 50)), float(rng.uniform(0.1, 5)))
+    tm._check(dt, layout, rows, cols, bool(rng.random() < 0.5), stored)
