@@ -14,6 +14,7 @@
 #include <raft/stats/weighted_mean.cuh>
 #include <raft/util/cudart_utils.hpp>
 
+#include <cmath>
 #include <cstdint>
 #include <limits>
 #include <random>
@@ -293,6 +294,89 @@ TEST_CASE(KvpColumnsCustomFunctors)
       ok &= got[j].key == best && got[j].value == h[(size_t)best * cols + j];
     }
     CHECK(ok);
+  }
+}
+
+// util/detail/popc.cuh:30-65: a bit count over packed words as a coalesced reduction of an
+// N x 1 column-major view, whose lambda masks the last word by its index
+template <typename value_t, typename index_t>
+void popc_caller_case(index_t n_words, index_t max_len)
+{
+  raft::resources handle;
+  auto stream = raft::resource::get_cuda_stream(handle);
+  std::mt19937_64 g(n_words + max_len);
+  std::vector<value_t> h((size_t)n_words);
+  for (auto& x : h)
+    x = (value_t)g();
+  auto d       = raft::make_device_vector<value_t, index_t>(handle, n_words);
+  auto counter = raft::make_device_vector<index_t, index_t>(handle, 1);
+  raft::update_device(d.data_handle(), h.data(), h.size(), stream);
+  constexpr index_t bits  = sizeof(value_t) * 8;
+  const value_t tail_len  = (value_t)(max_len % bits);
+  const value_t tail_mask = tail_len ? (value_t)((value_t{1} << tail_len) - value_t{1}) : (value_t) ~value_t{0};
+  auto values = raft::make_device_matrix_view<const value_t, index_t, raft::col_major>(
+    d.data_handle(), n_words, 1);
+  raft::linalg::coalesced_reduction(
+    handle, values, counter.view(), index_t{0}, false,
+    [tail_mask, n_words] __device__(value_t value, index_t index) {
+      const value_t v = index == n_words - 1 ? (value_t)(value & tail_mask) : value;
+      return (index_t)__popcll((unsigned long long)v);
+    });
+  auto got = to_host(counter.data_handle(), 1, stream);
+  index_t want = 0;
+  for (index_t i = 0; i < n_words; ++i) {
+    const value_t v = i == n_words - 1 ? (value_t)(h[(size_t)i] & tail_mask) : h[(size_t)i];
+    want += (index_t)__builtin_popcountll((unsigned long long)v);
+  }
+  if (got[0] != want) std::printf("  popc %lld words: %lld != %lld\n", (long long)n_words, (long long)got[0], (long long)want);
+  CHECK(got[0] == want);
+}
+TEST_CASE(PopcCaller)
+{
+  popc_caller_case<std::uint32_t, std::int64_t>(1, 7);
+  popc_caller_case<std::uint32_t, std::int64_t>(1000, 1000 * 32 - 5);
+  popc_caller_case<std::uint32_t, std::int64_t>(3000001, 3000001LL * 32 - 31);
+  popc_caller_case<std::uint64_t, std::int64_t>(777777, 777777LL * 64 - 1);
+  popc_caller_case<std::uint8_t, std::int64_t>(100003, 100003LL * 8 - 3);
+}
+
+// linalg/detail/tsvd.cuh:213-245: the signed value of largest magnitude per column or per
+// row, with the caller's own reduce lambda (sign flip of the singular vectors)
+TEST_CASE(SignedAbsMaxCaller)
+{
+  raft::resources handle;
+  auto stream = raft::resource::get_cuda_stream(handle);
+  for (auto [N, D] : std::vector<std::pair<int, int>>{{1000, 7}, {20000, 33}, {64, 5000}, {3, 200000}}) {
+    auto h   = uniform<float>((size_t)N * D, -1.0, 1.0, N + D);
+    auto d   = raft::make_device_vector<float, int>(handle, N * D);
+    raft::update_device(d.data_handle(), h.data(), h.size(), stream);
+    auto absmax = [] __device__(float a, float b) {
+      const float abs_a = a >= 0.f ? a : -a;
+      const float abs_b = b >= 0.f ? b : -b;
+      return abs_a >= abs_b ? a : b;
+    };
+    for (int along_rows = 0; along_rows < 2; ++along_rows) {
+      const int n_out = along_rows ? N : D, len = along_rows ? D : N;
+      auto out = raft::make_device_vector<float, int>(handle, n_out);
+      if (along_rows)
+        raft::linalg::reduce<true, true>(out.data_handle(), d.data_handle(), D, N, 0.f, stream, false,
+                                         raft::identity_op(), absmax, raft::identity_op());
+      else
+        raft::linalg::reduce<true, false>(out.data_handle(), d.data_handle(), D, N, 0.f, stream, false,
+                                          raft::identity_op(), absmax, raft::identity_op());
+      auto got = to_host(out.data_handle(), (size_t)n_out, stream);
+      bool ok  = true;
+      for (int k = 0; k < n_out; ++k) {
+        float best = 0.f;
+        for (int r = 0; r < len; ++r) {
+          const float x = along_rows ? h[(size_t)k * D + r] : h[(size_t)r * D + k];
+          if (std::fabs(x) > std::fabs(best)) best = x;
+        }
+        ok &= got[k] == best;
+      }
+      if (!ok) std::printf("  signed abs-max %dx%d along_rows=%d\n", N, D, along_rows);
+      CHECK(ok);
+    }
   }
 }
 
