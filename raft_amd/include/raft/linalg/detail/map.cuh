@@ -67,14 +67,19 @@ struct map_word<16> {
   typedef std::uint32_t type __attribute__((ext_vector_type(4)));
 };
 
-template <typename T, int R>
+template <typename T, int R, bool NT = true>
 __device__ __forceinline__ map_pack<T, R> map_load(const T* p, std::int64_t off)
 {
   map_pack<T, R> x;
   using W = typename map_word<(int)sizeof(map_pack<T, R>)>::type;
   if constexpr (!std::is_void_v<W> && std::is_trivially_copyable_v<T>) {
     typedef W W_unaligned __attribute__((aligned(1)));
-    const W w = __builtin_nontemporal_load(reinterpret_cast<const W_unaligned*>(p + off));
+    W w;
+    if constexpr (NT) {
+      w = __builtin_nontemporal_load(reinterpret_cast<const W_unaligned*>(p + off));
+    } else {
+      w = *reinterpret_cast<const W_unaligned*>(p + off);
+    }
     __builtin_memcpy(&x, &w, sizeof(x));
   } else {
     __builtin_memcpy(&x, p + off, sizeof(x));
@@ -82,7 +87,7 @@ __device__ __forceinline__ map_pack<T, R> map_load(const T* p, std::int64_t off)
   return x;
 }
 
-template <typename T, int R>
+template <typename T, int R, bool NT = true>
 __device__ __forceinline__ void map_store(T* p, std::int64_t off, const map_pack<T, R>& x)
 {
   using W = typename map_word<(int)sizeof(map_pack<T, R>)>::type;
@@ -90,7 +95,11 @@ __device__ __forceinline__ void map_store(T* p, std::int64_t off, const map_pack
     typedef W W_unaligned __attribute__((aligned(1)));
     W w;
     __builtin_memcpy(&w, &x, sizeof(x));
-    __builtin_nontemporal_store(w, reinterpret_cast<W_unaligned*>(p + off));
+    if constexpr (NT) {
+      __builtin_nontemporal_store(w, reinterpret_cast<W_unaligned*>(p + off));
+    } else {
+      *reinterpret_cast<W_unaligned*>(p + off) = w;
+    }
   } else {
     __builtin_memcpy(p + off, &x, sizeof(x));
   }

@@ -8,9 +8,12 @@
 #include <raft/core/kvp.hpp>
 #include <raft/linalg/binary_op.cuh>
 #include <raft/linalg/map.cuh>
+#include <raft/linalg/matrix_vector_op.cuh>
 #include <raft/linalg/unary_op.cuh>
+#include <raft/stats/mean_center.cuh>
 #include <raft/util/cudart_utils.hpp>
 
+#include <cmath>
 #include <cstdint>
 #include <random>
 
@@ -269,6 +272,134 @@ TEST_CASE(MapShapeMismatchThrows)
   }
   CHECK(threw);
 }
+
+// linalg::matrixVectorOp with one and two vectors: the grid of
+// cpp/tests/linalg/matrix_vector_op.cu:213-218 (1024 x {32, 64}, both layouts, both
+// broadcast directions, input and output pointers 0..2 elements off), the naive kernels of
+// cpp/tests/linalg/matrix_vector_op.cuh:15-105 as the check, plus ragged shapes.
+template <typename T, typename IdxT>
+void matvec_grid(double tol)
+{
+  raft::resources handle;
+  auto stream = raft::resource::get_cuda_stream(handle);
+  struct Shape { IdxT rows, cols; };
+  std::vector<Shape> shapes = {{1024, 32}, {1024, 64}, {2500, 250}, {1000, 33}, {7, 5}, {3, 100003},
+                               {4099, 1}, {1, 777}, {300, 1028}};
+  for (auto sh : shapes)
+    for (int rm = 0; rm < 2; ++rm)
+      for (int bcast = 0; bcast < 2; ++bcast)
+        for (int in_off = 0; in_off < 3; ++in_off)
+          for (int out_off = 0; out_off < 3; out_off += 2) {
+            const size_t len = (size_t)sh.rows * sh.cols;
+            const size_t vlen = bcast ? sh.cols : sh.rows;
+            std::mt19937_64 g(len + rm * 7 + bcast * 3 + in_off);
+            std::uniform_real_distribution<double> u(-1.0, 1.0);
+            std::vector<T> hm(len), hv1(vlen), hv2(vlen);
+            for (auto& x : hm) x = (T)u(g);
+            for (auto& x : hv1) x = (T)u(g);
+            for (auto& x : hv2) x = (T)u(g);
+            auto dm  = raft::make_device_vector<T, size_t>(handle, len + 4);
+            auto dv1 = raft::make_device_vector<T, size_t>(handle, vlen);
+            auto dv2 = raft::make_device_vector<T, size_t>(handle, vlen);
+            auto dout = raft::make_device_vector<T, size_t>(handle, len + 4);
+            raft::update_device(dm.data_handle() + in_off, hm.data(), len, stream);
+            raft::update_device(dv1.data_handle(), hv1.data(), vlen, stream);
+            raft::update_device(dv2.data_handle(), hv2.data(), vlen, stream);
+            const T* in = dm.data_handle() + in_off;
+            T* out      = dout.data_handle() + out_off;
+            auto vec_of = [&](size_t idx) {
+              const size_t D = sh.cols, N = sh.rows;
+              if (rm && bcast) return idx % D;
+              if (!rm && !bcast) return idx % N;
+              if (rm && !bcast) return idx / D;
+              return idx / N;
+            };
+            for (int two = 0; two < 2; ++two) {
+              auto add1 = [] __device__(T a, T b) { return a + b; };
+              auto add2 = [] __device__(T a, T b, T c) { return a + b + c; };
+              if (rm && bcast) {
+                if (two) raft::linalg::matrixVectorOp<true, true>(out, in, dv1.data_handle(), dv2.data_handle(), sh.cols, sh.rows, add2, stream);
+                else raft::linalg::matrixVectorOp<true, true>(out, in, dv1.data_handle(), sh.cols, sh.rows, add1, stream);
+              } else if (rm && !bcast) {
+                if (two) raft::linalg::matrixVectorOp<true, false>(out, in, dv1.data_handle(), dv2.data_handle(), sh.cols, sh.rows, add2, stream);
+                else raft::linalg::matrixVectorOp<true, false>(out, in, dv1.data_handle(), sh.cols, sh.rows, add1, stream);
+              } else if (!rm && bcast) {
+                if (two) raft::linalg::matrixVectorOp<false, true>(out, in, dv1.data_handle(), dv2.data_handle(), sh.cols, sh.rows, add2, stream);
+                else raft::linalg::matrixVectorOp<false, true>(out, in, dv1.data_handle(), sh.cols, sh.rows, add1, stream);
+              } else {
+                if (two) raft::linalg::matrixVectorOp<false, false>(out, in, dv1.data_handle(), dv2.data_handle(), sh.cols, sh.rows, add2, stream);
+                else raft::linalg::matrixVectorOp<false, false>(out, in, dv1.data_handle(), sh.cols, sh.rows, add1, stream);
+              }
+              auto got = to_host(out, len, stream);
+              bool ok  = true;
+              for (size_t i = 0; i < len; ++i) {
+                const size_t k = vec_of(i);
+                const double want = (double)hm[i] + (double)hv1[k] + (two ? (double)hv2[k] : 0.0);
+                ok &= std::fabs((double)got[i] - want) <= tol * (1.0 + std::fabs(want));
+              }
+              if (!ok)
+                std::printf("  matvec %lldx%lld rm=%d bcast=%d in+%d out+%d vecs=%d\n", (long long)sh.rows,
+                            (long long)sh.cols, rm, bcast, in_off, out_off, two + 1);
+              CHECK(ok);
+            }
+          }
+}
+TEST_CASE(MatVecOpFloatI32) { matvec_grid<float, int>(1e-5); }
+TEST_CASE(MatVecOpDoubleI64) { matvec_grid<double, std::int64_t>(1e-7); }
+
+// stats::mean_center / mean_add through the mdspan API: the grid of
+// cpp/tests/stats/mean_center.cu:110-122 (1024 x {32, 64, 128}, both layouts, both
+// directions), in place as well
+template <typename T>
+void mean_center_grid(double tol)
+{
+  raft::resources handle;
+  auto stream = raft::resource::get_cuda_stream(handle);
+  for (int cols : {32, 64, 128, 37})
+    for (int rm = 0; rm < 2; ++rm)
+      for (int bcast = 0; bcast < 2; ++bcast) {
+        const int rows = 1024;
+        const size_t len = (size_t)rows * cols, vlen = bcast ? cols : rows;
+        std::mt19937_64 g(cols + rm + bcast);
+        std::normal_distribution<double> nd(-1.0, 1.0);
+        std::vector<T> hm(len), hmu(vlen);
+        for (auto& x : hm) x = (T)nd(g);
+        for (auto& x : hmu) x = (T)nd(g);
+        auto dm  = raft::make_device_vector<T, int>(handle, (int)len);
+        auto dmu = raft::make_device_vector<T, int>(handle, (int)vlen);
+        auto dout = raft::make_device_vector<T, int>(handle, (int)len);
+        raft::update_device(dm.data_handle(), hm.data(), len, stream);
+        raft::update_device(dmu.data_handle(), hmu.data(), vlen, stream);
+        auto mu = raft::make_device_vector_view<const T, int>(dmu.data_handle(), (int)vlen);
+        auto run = [&](auto layout, bool add) {
+          using L = decltype(layout);
+          auto in  = raft::make_device_matrix_view<const T, int, L>(dm.data_handle(), rows, cols);
+          auto out = raft::make_device_matrix_view<T, int, L>(dout.data_handle(), rows, cols);
+          if (bcast) {
+            if (add) raft::stats::mean_add<raft::Apply::ALONG_ROWS>(handle, in, mu, out);
+            else raft::stats::mean_center<raft::Apply::ALONG_ROWS>(handle, in, mu, out);
+          } else {
+            if (add) raft::stats::mean_add<raft::Apply::ALONG_COLUMNS>(handle, in, mu, out);
+            else raft::stats::mean_center<raft::Apply::ALONG_COLUMNS>(handle, in, mu, out);
+          }
+        };
+        for (int add = 0; add < 2; ++add) {
+          if (rm) run(raft::row_major{}, add); else run(raft::col_major{}, add);
+          auto got = to_host(dout.data_handle(), len, stream);
+          bool ok  = true;
+          for (size_t i = 0; i < len; ++i) {
+            const size_t r = rm ? i / cols : i % rows, c = rm ? i % cols : i / rows;
+            const double m = (double)hmu[bcast ? c : r];
+            const double want = (double)hm[i] + (add ? m : -m);
+            ok &= std::fabs((double)got[i] - want) <= tol * (1.0 + std::fabs(want));
+          }
+          if (!ok) std::printf("  mean_%s 1024x%d rm=%d bcast=%d\n", add ? "add" : "center", cols, rm, bcast);
+          CHECK(ok);
+        }
+      }
+}
+TEST_CASE(MeanCenterF) { mean_center_grid<float>(1e-6); }
+TEST_CASE(MeanCenterD) { mean_center_grid<double>(1e-14); }
 
 int main()
 {
