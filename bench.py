@@ -536,7 +536,7 @@ def main():
 # profiles/), scaled by the same counters' reading for a copy kernel of known size.
 MEASURED_TRAFFIC: dict[str, float | None] = {
     "cfg1": 10.36e6, "cfg2": 516.04e6, "cfg3_mean": 2561.39e6, "cfg3_stddev": 2561.38e6,
-    "cfg4": 8394.27e6, "cfg5a": 67.28e6, "cfg5b": 268.58e6, "cfg5c": 67.33e6,
+    "cfg4": 8394.23e6, "cfg5a": 67.26e6, "cfg5b": 268.53e6, "cfg5c": 67.33e6,
 }
 
 
