@@ -398,6 +398,39 @@ void mean_center_grid(double tol)
         }
       }
 }
+// out == matrix (linalg/matrix_vector_op.cuh:38 allows it), on row lengths with and without
+// elements after the last whole 16-byte pack
+TEST_CASE(MatVecOpInPlace)
+{
+  raft::resources handle;
+  auto stream = raft::resource::get_cuda_stream(handle);
+  for (auto [rows, cols] : std::vector<std::pair<int, int>>{{3000, 13}, {1000, 129}, {513, 64}, {20000, 3}, {7, 4099}})
+    for (int bcast = 0; bcast < 2; ++bcast) {
+      const size_t len = (size_t)rows * cols, vlen = bcast ? cols : rows;
+      auto hm = std::vector<float>(len);
+      auto hv = std::vector<float>(vlen);
+      std::mt19937 g(rows + cols);
+      std::uniform_real_distribution<float> u(-1.f, 1.f);
+      for (auto& x : hm) x = u(g);
+      for (auto& x : hv) x = u(g);
+      auto dm = raft::make_device_vector<float, int>(handle, (int)len);
+      auto dv = raft::make_device_vector<float, int>(handle, (int)vlen);
+      raft::update_device(dm.data_handle(), hm.data(), len, stream);
+      raft::update_device(dv.data_handle(), hv.data(), vlen, stream);
+      auto op = [] __device__(float a, float b) { return 2.f * a - b; };
+      if (bcast)
+        raft::linalg::matrixVectorOp<true, true>(dm.data_handle(), dm.data_handle(), dv.data_handle(), cols, rows, op, stream);
+      else
+        raft::linalg::matrixVectorOp<true, false>(dm.data_handle(), dm.data_handle(), dv.data_handle(), cols, rows, op, stream);
+      auto got = to_host(dm.data_handle(), len, stream);
+      bool ok  = true;
+      for (size_t i = 0; i < len; ++i)
+        ok &= got[i] == 2.f * hm[i] - hv[bcast ? i % cols : i / cols];
+      if (!ok) std::printf("  in place %dx%d bcast=%d\n", rows, cols, bcast);
+      CHECK(ok);
+    }
+}
+
 TEST_CASE(MeanCenterF) { mean_center_grid<float>(1e-6); }
 TEST_CASE(MeanCenterD) { mean_center_grid<double>(1e-14); }
 
