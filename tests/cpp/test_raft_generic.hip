@@ -13,6 +13,7 @@
 #include <raft/linalg/strided_reduction.cuh>
 #include <raft/stats/weighted_mean.cuh>
 #include <raft/util/cudart_utils.hpp>
+#include <raft/util/popc.cuh>
 
 #include <cmath>
 #include <cstdint>
@@ -331,6 +332,31 @@ void popc_caller_case(index_t n_words, index_t max_len)
   if (got[0] != want) std::printf("  popc %lld words: %lld != %lld\n", (long long)n_words, (long long)got[0], (long long)want);
   CHECK(got[0] == want);
 }
+// the same through raft::popc itself (cpp/tests/util/popc.cu: bit arrays whose length is
+// not a multiple of the word size)
+TEST_CASE(PopcHeader)
+{
+  raft::resources handle;
+  auto stream = raft::resource::get_cuda_stream(handle);
+  for (std::int64_t n_bits : std::vector<std::int64_t>{1, 31, 32, 33, 1000, 65537, 10000019}) {
+    const std::int64_t n_words = (n_bits + 31) / 32;
+    std::mt19937 g((unsigned)n_bits);
+    std::vector<std::uint32_t> h((size_t)n_words);
+    for (auto& x : h) x = g();
+    auto d       = raft::make_device_vector<std::uint32_t, std::int64_t>(handle, n_words);
+    auto counter = raft::make_device_vector<std::int64_t, std::int64_t>(handle, 1);
+    raft::update_device(d.data_handle(), h.data(), h.size(), stream);
+    raft::popc(handle, raft::make_device_vector_view<const std::uint32_t, std::int64_t>(d.data_handle(), n_words),
+               raft::make_host_scalar_view<const std::int64_t, std::int64_t>(&n_bits),
+               raft::make_device_scalar_view<std::int64_t>(counter.data_handle()));
+    auto got = to_host(counter.data_handle(), 1, stream);
+    std::int64_t want = 0;
+    for (std::int64_t b = 0; b < n_bits; ++b)
+      want += (h[(size_t)(b / 32)] >> (b % 32)) & 1u;
+    CHECK(got[0] == want);
+  }
+}
+
 TEST_CASE(PopcCaller)
 {
   popc_caller_case<std::uint32_t, std::int64_t>(1, 7);
