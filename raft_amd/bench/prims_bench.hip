@@ -14,6 +14,7 @@
 #include <raft/core/device_mdspan.hpp>
 #include <raft/core/resources.hpp>
 #include <raft/linalg/map_then_reduce.cuh>
+#include <raft/linalg/matrix_vector_op.cuh>
 #include <raft/linalg/norm.cuh>
 #include <raft/linalg/normalize.cuh>
 #include <raft/linalg/reduce.cuh>
@@ -263,6 +264,65 @@ void bench_argmin(Harness& h)
     }
 }
 
+// bench/prims/linalg/matrix_vector_op.cu:136-176: round dimensions in both layouts and
+// broadcast directions, then odd widths with input / output pointers one element off
+struct Add1Vec {
+  template <typename T>
+  __host__ __device__ T operator()(T a, T b) const { return a + b; }
+};
+struct Add2Vec {
+  template <typename T>
+  __host__ __device__ T operator()(T a, T b, T c) const { return a + b + c; }
+};
+
+template <typename T, bool TWO>
+void bench_mat_vec_op(Harness& h)
+{
+  const std::string name = std::string("matrixVectorOp<") + tname<T>() + (TWO ? ",2 vectors>" : ",1 vector>");
+  if (!h.wanted(name)) return;
+  struct Case { long long rows, cols; bool row_major, along_rows; int in_off, out_off; };
+  std::vector<Case> cases;
+  for (bool rm : {true, false})
+    for (bool ar : {true, false})
+      for (long long rows : {1000LL, 100000LL, 1000000LL})
+        for (long long cols : {8LL, 64LL, 256LL, 1024LL})
+          cases.push_back({rows, cols, rm, ar, 0, 0});
+  for (bool rm : {true, false})
+    for (bool ar : {true, false})
+      for (auto rc : std::vector<std::pair<long long, long long>>{{44739207, 7}, {44739207, 15}, {44739207, 16},
+                                                                  {44739207, 17}, {2611236, 256}, {2611236, 257},
+                                                                  {2611236, 263}})
+        for (int io : {0, 1})
+          for (int oo : {0, 1})
+            cases.push_back({rc.first, rc.second, rm, ar, io, oo});
+  for (const auto& c : cases) {
+    const size_t n = (size_t)c.rows * c.cols;
+    if (!h.fits(2 * n * sizeof(T))) continue;
+    DeviceBuf<T> in(n + 1), out(n + 1), v1((size_t)(c.along_rows ? c.cols : c.rows)),
+      v2((size_t)(c.along_rows ? c.cols : c.rows));
+    in.uniform(-1.0, 1.0, h.stream());
+    v1.uniform(-1.0, 1.0, h.stream());
+    v2.uniform(-1.0, 1.0, h.stream());
+    const std::string shape = shape2(c.rows, c.cols) + (c.row_major ? " rm" : " cm") + (c.along_rows ? " ar" : " ac") +
+                              " +" + std::to_string(c.in_off) + "+" + std::to_string(c.out_off);
+    h.run(name, shape, 2 * n * sizeof(T), [&] {
+      T* o       = out.p + c.out_off;
+      const T* i = in.p + c.in_off;
+      const long long D = c.cols, N = c.rows;
+      auto go = [&](auto rm, auto ar) {
+        if constexpr (TWO)
+          raft::linalg::matrixVectorOp<decltype(rm)::value, decltype(ar)::value>(o, i, v1.p, v2.p, D, N, Add2Vec{}, h.stream());
+        else
+          raft::linalg::matrixVectorOp<decltype(rm)::value, decltype(ar)::value>(o, i, v1.p, D, N, Add1Vec{}, h.stream());
+      };
+      if (c.row_major && c.along_rows) go(std::true_type{}, std::true_type{});
+      else if (c.row_major) go(std::true_type{}, std::false_type{});
+      else if (c.along_rows) go(std::false_type{}, std::true_type{});
+      else go(std::false_type{}, std::false_type{});
+    });
+  }
+}
+
 }  // namespace
 
 int main(int argc, char** argv)
@@ -298,5 +358,9 @@ int main(int argc, char** argv)
   bench_map_then_reduce<double>(h);
   bench_argmin<float>(h);
   bench_argmin<double>(h);
+  bench_mat_vec_op<float, false>(h);
+  bench_mat_vec_op<float, true>(h);
+  bench_mat_vec_op<double, false>(h);
+  bench_mat_vec_op<double, true>(h);
   return 0;
 }

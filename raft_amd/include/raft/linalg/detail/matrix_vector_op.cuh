@@ -126,7 +126,9 @@ void launch_matrix_vector(MatT* out, const MatT* matrix, std::int64_t C, std::in
                           hipStream_t stream, const Vec1T* vec1, const Vec2T* vec2)
 {
   const std::int64_t lanes = (C + V - 1) / V;
-  const std::int64_t cuts  = (lanes + 127) / 128;
+  // lines of whole multiples of 64 lanes keep pieces of exactly 64 lanes (1 KB at 1 KB
+  // offsets within the line), others the fewest equal cuts of at most 128
+  const std::int64_t cuts  = lanes % 64 == 0 ? lanes / 64 : (lanes + 127) / 128;
   const int TX             = (int)((lanes + cuts - 1) / cuts);
   const int TY             = kMvBlock / TX;
   const std::int64_t gridx = (lanes + TX - 1) / TX;
