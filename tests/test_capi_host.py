@@ -160,3 +160,45 @@ def test_null_and_workspace_errors_without_a_launch():
     # zero outputs: success, nothing to do
     d = api.make_desc(api.F32, api.F32, 0, 100)
     assert lib.rmi_reduce(C.byref(d), None, None, None, 0, None) == api.OK
+
+
+def test_lane_groups_follow_the_row_length():
+    """Rows whose lane-load count is far from a power of two get one lane per lane-load
+    (5 lane-loads, and 6 or 9..17 with tail elements); the others keep power-of-two groups."""
+    lanes = lambda cols, dt=api.F32, out=api.F32: api.plan_query(
+        api.make_desc(dt, out, 1000000, cols)).lanes_per_row
+    assert lanes(20) == 5 and lanes(17) == 5            # 5 lane-loads, without and with a tail
+    assert lanes(33) == 9 and lanes(45) == 12 and lanes(66) == 17
+    assert lanes(21) == 6                               # 5 whole vectors + one element
+    assert lanes(24) == 8 and lanes(28) == 8            # 6 and 7 whole lane-loads stay on 8 lanes
+    assert lanes(36) == 4                               # 9 whole vectors: 4 lanes x 3 loads
+    assert lanes(128) == 8 and lanes(256) == 16
+    assert lanes(100, api.BF16) == 13                   # 12 whole + 4 elements
+    # arg-reductions follow the same rule
+    d = api.make_desc(api.F32, api.KVP_I32_F32, 1000, 33, main_op=api.MAIN_KVP,
+                      reduce_op=api.RED_ARGMAX)
+    assert api.plan_query(d).lanes_per_row == 9
+
+
+def test_column_plans_of_rows_that_are_not_whole_vectors():
+    """Rows shorter than 16 bytes are folded in groups of rows that make whole vectors (more
+    partials per output, a second pass), unless the reduction needs the row index or the
+    matrix is short; the workspace query covers the plan an unaligned input falls back to."""
+    lib = api.load()
+    d = api.make_desc(api.F32, api.F32, 4_000_000, 3, apply=api.ALONG_COLUMNS)
+    p = api.plan_query(d)
+    assert p.kind == api.PLAN_COL_TILE and p.passes == 2 and p.vec_bytes == 16
+    assert p.blocks_per_out % 4 == 0                    # 4 rows of 12 bytes = 3 vectors
+    assert lib.rmi_reduce_workspace_bytes(C.byref(d)) >= p.workspace_bytes
+    d = api.make_desc(api.I8, api.I64, 4_000_000, 5, apply=api.ALONG_COLUMNS)
+    assert api.plan_query(d).blocks_per_out % 16 == 0   # 16 rows of 5 bytes = 5 vectors
+    d = api.make_desc(api.F32, api.KVP_I32_F32, 4_000_000, 3, apply=api.ALONG_COLUMNS,
+                      main_op=api.MAIN_KVP, reduce_op=api.RED_ARGMIN)
+    assert api.plan_query(d).vec_bytes == 4             # element by element
+    d = api.make_desc(api.F32, api.F32, 500, 3, apply=api.ALONG_COLUMNS)
+    assert api.plan_query(d).vec_bytes == 4             # too few rows to group
+    # wider rows are never grouped: one partial per workgroup row
+    d = api.make_desc(api.F32, api.F32, 1_000_000, 129, apply=api.ALONG_COLUMNS)
+    p = api.plan_query(d)
+    assert p.kind == api.PLAN_COL_TILE and p.vec_bytes == 16 and p.blocks_per_out <= 4096
+    assert p.grid_blocks == p.blocks_per_out            # 33 lane-loads: one workgroup column
