@@ -384,10 +384,13 @@ inline int make_plan(const rmi_reduce_desc& d,
     // (one contiguous span per load instruction).  Its cross-lane steps cost more, so the
     // rule follows what was measured on 1M-row fp32 matrices: 5 lane-loads, and 6 or 9 to 17
     // when the row ends in tail elements (D = 20 / 21 / 33 / 41 / 45 / 54 / 62: 69 / 66 / 52 /
-    // 59 / 62 / 69 / 72 % -> 78 / 77 / 74 / 70 / 75 / 79 / 80 %); at 7 lane-loads with a tail, or
-    // at 6, 7, 19, 21 without one, it measured 2 to 10 points slower.
+    // 59 / 62 / 69 / 72 % -> 78 / 77 / 74 / 70 / 75 / 79 / 80 %), and 18 to 32 with a tail where
+    // the groups fill at least 54 lanes (D = 79 / 83 / 125: 69 / 71 / 72 % -> 77 / 79 / 80 %; at
+    // 23 lane-loads, 46 lanes, it lost 13 points).  At 7 lane-loads with a tail, or at 6, 7,
+    // 19, 21 without one, it measured 2 to 10 points slower.
     if (p.vec16 &&
-        (nload == 5 || (p.tail > 0 && (nload == 6 || (nload >= 9 && nload <= 17)))) &&
+        (nload == 5 || (p.tail > 0 && (nload == 6 || (nload >= 9 && nload <= 17) ||
+                                       (nload >= 18 && nload <= 32 && (64 / nload) * nload >= 54)))) &&
         (hint == RMI_PLAN_AUTO || hint == RMI_PLAN_ROW_WAVE)) {
       p.short_rows = true;
       p.any_g      = true;

@@ -79,6 +79,7 @@ void check(const rmi_reduce_desc& d, int n_cu, uintptr_t in_misalign)
           // one lane per lane-load, whole rows per wave, one run of at most 64 outputs
           REQUIRE(p.short_rows && p.vec16 && p.G == nload && p.G >= 4 && p.G <= 32);
           REQUIRE((64 / p.G) * p.G >= 48);  // at least three lanes in four have a lane-load
+          if (p.G >= 18) REQUIRE((64 / p.G) * p.G >= 54 && p.tail > 0);
           REQUIRE((64 / p.G) * kPlanUnroll <= 64);
         } else {
           REQUIRE(p.G >= 1 && p.G <= 64 && (p.G & (p.G - 1)) == 0 && (1 << p.logG) == p.G);

@@ -169,6 +169,7 @@ def test_lane_groups_follow_the_row_length():
         api.make_desc(dt, out, 1000000, cols)).lanes_per_row
     assert lanes(20) == 5 and lanes(17) == 5            # 5 lane-loads, without and with a tail
     assert lanes(33) == 9 and lanes(45) == 12 and lanes(66) == 17
+    assert lanes(83) == 21 and lanes(125) == 32 and lanes(90) == 8   # 23 lane-loads: 46 lanes, no
     assert lanes(21) == 6                               # 5 whole vectors + one element
     assert lanes(24) == 8 and lanes(28) == 8            # 6 and 7 whole lane-loads stay on 8 lanes
     assert lanes(36) == 4                               # 9 whole vectors: 4 lanes x 3 loads
