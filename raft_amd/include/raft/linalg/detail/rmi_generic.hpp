@@ -177,6 +177,77 @@ __global__ __launch_bounds__(kBlock) void rows_group_kernel(Out* dots, const In*
   if (c == 0 && row < (std::int64_t)N) dots[row] = fin(inplace ? red(dots[row], acc) : acc);
 }
 
+// Rows of G 16-byte lane loads, G not a power of two (3..32, the row's last load may be the
+// pack that ends at the row's end): one lane per load, 64 / G whole rows per wave step, four
+// steps in flight, so every load instruction covers one contiguous span of the matrix; the
+// wave's last 64 % G lanes idle.  Lanes of a row are folded into its first one (lane c takes
+// lane c + s for s = 1, 2, 4 ...).
+template <typename T>
+__device__ __forceinline__ T shfl_any(const T& v, int src)
+{
+  constexpr int NW = (sizeof(T) + 3) / 4;
+  std::uint32_t w[NW] = {};
+  __builtin_memcpy(w, &v, sizeof(T));
+#pragma unroll
+  for (int i = 0; i < NW; ++i)
+    w[i] = (std::uint32_t)__shfl((int)w[i], src, kWave);
+  T r;
+  __builtin_memcpy(&r, w, sizeof(T));
+  return r;
+}
+
+template <typename In, typename Out, typename Idx, typename Main, typename Red, typename Fin>
+__global__ __launch_bounds__(kBlock) void rows_anyg_kernel(Out* dots, const In* data, Idx D, Idx N,
+                                                           Out init, bool inplace, Main main_op,
+                                                           Red red, Fin fin, int G, unsigned invG)
+{
+  constexpr int V = vec_width<In>();
+  constexpr int U = 4;
+  const int lane  = threadIdx.x & (kWave - 1);
+  const std::int64_t wid = (std::int64_t)blockIdx.x * (kBlock / kWave) + (threadIdx.x >> 6);
+  const int R     = kWave / G;
+  const int g     = (int)(((unsigned)lane * invG) >> 16);  // lane / G
+  const int c     = lane - g * G;
+  const bool live = g < R;
+  const std::int64_t nvec = (std::int64_t)D / V;
+  const int tail          = (int)((std::int64_t)D - nvec * V);
+  // element offset of this lane's pack: whole pack c, or the pack that ends at the row's end
+  const bool last_part    = tail > 0 && c == G - 1;
+  const std::int64_t e0   = !live ? 0 : (last_part ? (std::int64_t)D - V : (std::int64_t)c * V);
+  const int first         = last_part ? V - tail : 0;  // elements before it are the neighbour's
+  pack16 x[U];
+  std::int64_t row[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) {  // unconditional loads: a row past the matrix re-reads the last one
+    row[u] = (wid * U + u) * R + g;
+    const std::int64_t rl = row[u] < (std::int64_t)N ? row[u] : (std::int64_t)N - 1;
+    x[u] = load_pack16<false>(data + rl * (std::int64_t)D + e0);
+  }
+  Out acc[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    acc[u] = init;
+    if (live && row[u] < (std::int64_t)N) {
+      In e[V];
+      __builtin_memcpy(e, x[u].w, 16);
+#pragma unroll
+      for (int j = 0; j < V; ++j)
+        if (j >= first) acc[u] = red(acc[u], static_cast<Out>(main_op(e[j], static_cast<Idx>(e0 + j))));
+    }
+  }
+  for (int s = 1; s < G; s <<= 1) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const Out v = shfl_any(acc[u], lane + s);
+      if (c + s < G) acc[u] = red(acc[u], v);
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < U; ++u)
+    if (live && c == 0 && row[u] < (std::int64_t)N)
+      dots[row[u]] = fin(inplace ? red(dots[row[u]], acc[u]) : acc[u]);
+}
+
 // one 256-thread workgroup per chunk of a row; B chunks per row.  B == 1 writes the
 // outputs, B > 1 writes partials[row * B + b].
 template <typename In, typename Out, typename Idx, typename Main, typename Red, typename Fin>
@@ -366,6 +437,20 @@ void coalesced(Out* dots, const In* data, Idx D, Idx N, Out init, hipStream_t st
   if (N <= 0) return;
   constexpr int V           = vec_width<In>();
   const std::int64_t nloads = ((std::int64_t)D + V - 1) / V;
+  if constexpr (V > 1) {
+    // lane-load counts that are not a power of two: one lane per load, whole rows per wave step
+    if (nloads >= 3 && nloads <= 32 && (nloads & (nloads - 1)) != 0 && (std::int64_t)D >= V &&
+        (kWave / nloads) * nloads >= 48) {
+      const int G              = (int)nloads;
+      const int rows_per_block = (kWave / G) * 4 * (kBlock / kWave);
+      const std::int64_t grid  = ((std::int64_t)N + rows_per_block - 1) / rows_per_block;
+      hipLaunchKernelGGL((rows_anyg_kernel<In, Out, Idx, Main, Red, Fin>), dim3((unsigned)grid),
+                         dim3(kBlock), 0, stream, dots, data, D, N, init, inplace, main_op, red, fin,
+                         G, 65536u / (unsigned)G + 1);
+      check_launch("rows_anyg_kernel");
+      return;
+    }
+  }
   if (nloads <= 256 || (std::int64_t)N >= 8192) {
     // lanes per row: about four loads per lane
     std::int64_t g = (nloads + 3) / 4;
