@@ -164,8 +164,10 @@ typedef enum rmi_plan_kind {
 typedef struct rmi_plan {
   int32_t kind;            /* rmi_plan_kind actually chosen                   */
   int32_t vec_bytes;       /* bytes per lane-load (16, or the element size)   */
-  int32_t lanes_per_row;   /* ROW_WAVE: lanes that share one row (1..64)      */
-  int32_t blocks_per_out;  /* ROW_SPLIT / COL_TILE: partials per output       */
+  int32_t lanes_per_row;   /* ROW_WAVE: lanes that share one row (1..64; a    */
+                           /* power of two, or the row's own lane-load count) */
+  int32_t blocks_per_out;  /* ROW_SPLIT / COL_TILE: partials per output (for  */
+                           /* an input that starts on a 16-byte boundary)     */
   int32_t block_threads;   /* threads per workgroup                           */
   int32_t passes;          /* kernel launches (1 or 2)                        */
   int64_t grid_blocks;     /* workgroups of the first launch                  */
@@ -193,7 +195,8 @@ RMI_API size_t rmi_dtype_size(int dtype);
 RMI_API int rmi_plan_query(const rmi_reduce_desc* desc, rmi_plan* plan);
 
 /* Bytes of device workspace rmi_reduce needs for `desc` (0 for single-pass
- * plans).  Replaces the internal rmm::device_uvector of
+ * plans), whatever the alignment of the input pointer (a plan can depend on
+ * it; the larger need is reported).  Replaces the internal rmm::device_uvector of
  * linalg/detail/coalesced_reduction-inl.cuh:560. */
 RMI_API size_t rmi_reduce_workspace_bytes(const rmi_reduce_desc* desc);
 
@@ -235,7 +238,8 @@ RMI_API int rmi_map_reduce(const rmi_reduce_desc* desc,
  * (linalg/normalize.cuh:48-110).  Uses the descriptor fields in_dtype (also the
  * output's type: F16, BF16, F32 or F64), n_rows, n_cols, main_op (IDENTITY, SQ, ABS),
  * reduce_op (ADD, MAX, MIN), final_op (IDENTITY or SQRT) and init.f; the matrix is
- * row-major.  The division happens in the element's arithmetic (f32 for f16 / bf16).
+ * row-major.  F32 / F64 rows are divided element by element in their own arithmetic;
+ * F16 / BF16 rows are multiplied in f32 by one reciprocal of the norm, then rounded.
  * `out` may be `in`.  Needs no workspace. */
 RMI_API int rmi_row_normalize(const rmi_reduce_desc* desc,
                               const void* in,
