@@ -205,3 +205,34 @@ def test_cfg5_mixed_precision_full(gpu):
     d2 = api.make_desc(api.BF16, api.F32, rows, cols, plan_hint=api.PLAN_ROW_BLOCK)
     out2 = _run(d2, xb, torch.zeros(rows, device="cuda"))
     assert u.fp_close(_host(out2), exp).all()
+
+
+# More than 2^31 elements through the plans whose addressing is newest: int8 data keep the
+# memory at 2.3 GB and int64 sums are exact.  The oracle needs minutes for a sequential pass
+# over this much, so the check is torch's own integer sums over the same device buffer, in
+# pieces that stay below 2^31 elements (exact integer arithmetic, no tolerance); the same
+# plans are held to the oracle at sizes it finishes in seconds in test_gpu_parity.py.
+@pytest.mark.parametrize("rows,cols,apply", [
+    (70_001, 32_768, api.ALONG_COLUMNS),     # wide rows cut in 64-lane pieces
+    (17_400_001, 132, api.ALONG_COLUMNS),    # 9 lane-loads: whole rows packed into a workgroup
+    (17_400_001, 132, api.ALONG_ROWS),       # 9 lane-loads with a tail: lane groups of 9
+    (580_000_001, 4, api.ALONG_COLUMNS),     # rows shorter than a vector, read in groups
+    (580_000_001, 4, api.ALONG_ROWS),        # several rows per 16-byte vector
+])
+def test_int8_sums_beyond_2g_elements(gpu, rows, cols, apply):
+    import torch
+    assert rows * cols > 2**31
+    x = torch.randint(-128, 128, (rows * cols,), generator=_gen(rows % 1000 + cols),
+                      device="cuda", dtype=torch.int8)
+    n_out = rows if apply == api.ALONG_ROWS else cols
+    d = api.make_desc(api.I8, api.I64, rows, cols, apply=apply)
+    out = _run(d, x, torch.zeros(n_out, dtype=torch.int64, device="cuda"))
+    m = x.view(rows, cols)
+    step = max(1, (2**30) // cols)
+    if apply == api.ALONG_ROWS:
+        ref = torch.cat([m[r:r + step].sum(dim=1, dtype=torch.int64) for r in range(0, rows, step)])
+    else:
+        ref = torch.zeros(cols, dtype=torch.int64, device="cuda")
+        for r in range(0, rows, step):
+            ref += m[r:r + step].sum(dim=0, dtype=torch.int64)
+    assert torch.equal(out, ref)
