@@ -236,3 +236,52 @@ def test_int8_sums_beyond_2g_elements(gpu, rows, cols, apply):
         for r in range(0, rows, step):
             ref += m[r:r + step].sum(dim=0, dtype=torch.int64)
     assert torch.equal(out, ref)
+
+
+# The same for the one-pass mean / variance (f32, 9 GB) and for row normalisation (bf16,
+# 4.5 GB in and out), against torch in f64 / f32 on the device.
+def test_meanvar_beyond_2g_elements(gpu):
+    import torch
+    from raft_amd import device as dev
+    rows, cols = 35_000_001, 64
+    x = torch.randn(rows * cols, generator=_gen(11), device="cuda") * 2 + 3
+    mean = torch.zeros(cols, device="cuda")
+    var = torch.zeros(cols, device="cuda")
+    dev.meanvar(api.F32, api.ROW_MAJOR, rows, cols, True, x, mean, var)
+    torch.cuda.synchronize()
+    m = x.view(rows, cols)
+    ref_mean = torch.zeros(cols, dtype=torch.float64, device="cuda")
+    step = 4_000_000
+    for r in range(0, rows, step):
+        ref_mean += m[r:r + step].sum(dim=0, dtype=torch.float64)
+    ref_mean /= rows
+    ref_m2 = torch.zeros(cols, dtype=torch.float64, device="cuda")
+    for r in range(0, rows, step):
+        ref_m2 += ((m[r:r + step].double() - ref_mean) ** 2).sum(dim=0)
+    ref_var = ref_m2 / (rows - 1)
+    assert u.fp_close(mean.cpu().numpy(), ref_mean.cpu().numpy()).all()
+    assert u.fp_close(var.cpu().numpy(), ref_var.cpu().numpy()).all()
+
+
+def test_row_normalize_beyond_2g_elements(gpu):
+    import torch
+    from raft_amd import device as dev
+    rows, cols = 17_500_001, 128
+    x = (torch.randn(rows * cols, generator=_gen(12), device="cuda") * 3).to(torch.bfloat16)
+    out = torch.empty_like(x)
+    d = api.make_desc(api.BF16, api.BF16, rows, cols, main_op=api.MAIN_SQ, final_op=api.FIN_SQRT)
+    rc = api.load().rmi_row_normalize(C.byref(d), x.data_ptr(), out.data_ptr(), 1e-8,
+                                      dev.current_stream_ptr())
+    assert rc == api.OK
+    torch.cuda.synchronize()
+    step = 2_000_000
+    for r in (0, rows // 2, rows - step):          # three slices of 2M rows, last one included
+        xs = x.view(rows, cols)[r:r + step].float()
+        ref = xs / torch.linalg.vector_norm(xs, dim=1, keepdim=True)
+        got = out.view(rows, cols)[r:r + step].float()
+        assert torch.allclose(got, ref, rtol=2 ** -7, atol=1e-6)
+    # unit rows everywhere (a checksum over all rows)
+    n = torch.zeros(rows, device="cuda")
+    for r in range(0, rows, step):
+        n[r:r + step] = torch.linalg.vector_norm(out.view(rows, cols)[r:r + step].float(), dim=1)
+    assert (n - 1).abs().max().item() < 2e-2
