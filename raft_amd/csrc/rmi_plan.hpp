@@ -382,14 +382,18 @@ inline int make_plan(const rmi_reduce_desc& d,
     // row cut over two load instructions is fetched as two pieces.  The one-load-per-lane
     // kernel also runs with G = the lane-load count itself, 64 / G whole rows per wave step
     // (one contiguous span per load instruction).  Its cross-lane steps cost more, so the
-    // rule follows what was measured on 1M-row fp32 matrices: 5 lane-loads, and 6 or 9 to 17
+    // rule follows what was measured on 1M-row fp32 matrices: 5 lane-loads, and 6 or 9 to 16
     // when the row ends in tail elements (D = 20 / 21 / 33 / 41 / 45 / 54 / 62: 69 / 66 / 52 /
     // 59 / 62 / 69 / 72 % -> 78 / 77 / 74 / 70 / 75 / 79 / 80 %), and 18 to 32 with a tail where
     // the groups fill at least 54 lanes (D = 79 / 83 / 125: 69 / 71 / 72 % -> 77 / 79 / 80 %; at
     // 23 lane-loads, 46 lanes, it lost 13 points).  At 7 lane-loads with a tail, or at 6, 7,
     // 19, 21 without one, it measured 2 to 10 points slower.
-    if (p.vec16 &&
-        (nload == 5 || (p.tail > 0 && (nload == 6 || (nload >= 9 && nload <= 17) ||
+    // Accumulators of 16 bytes and more (f64 sums, 64-bit keys or values) pay twice as much
+    // per cross-lane step: they keep the variant up to 12 lane-loads only (f64 D = 9 / 17: 48 ->
+    // 61 / 57 %; D = 25 / 33 / 63 lost 12 to 21 points with it).
+    const int64_t any_g_max = acc_bytes > 8 ? 12 : 32;
+    if (p.vec16 && nload <= any_g_max &&
+        (nload == 5 || (p.tail > 0 && (nload == 6 || (nload >= 9 && nload <= 16) ||
                                        (nload >= 18 && nload <= 32 && (64 / nload) * nload >= 54)))) &&
         (hint == RMI_PLAN_AUTO || hint == RMI_PLAN_ROW_WAVE)) {
       p.short_rows = true;
