@@ -439,8 +439,9 @@ void coalesced(Out* dots, const In* data, Idx D, Idx N, Out init, hipStream_t st
   const std::int64_t nloads = ((std::int64_t)D + V - 1) / V;
   if constexpr (V > 1) {
     // lane-load counts that are not a power of two: one lane per load, whole rows per wave step
-    if (nloads >= 3 && nloads <= 32 && (nloads & (nloads - 1)) != 0 && (std::int64_t)D >= V &&
-        (kWave / nloads) * nloads >= 48) {
+    // (accumulators wider than 8 bytes pay twice per cross-lane step: up to 12 loads only)
+    if (nloads >= 3 && nloads <= (sizeof(Out) > 8 ? 12 : 32) && (nloads & (nloads - 1)) != 0 &&
+        (std::int64_t)D >= V && (kWave / nloads) * nloads >= 48) {
       const int G              = (int)nloads;
       const int rows_per_block = (kWave / G) * 4 * (kBlock / kWave);
       const std::int64_t grid  = ((std::int64_t)N + rows_per_block - 1) / rows_per_block;
