@@ -193,11 +193,12 @@ inline NormPlan make_norm_plan(int64_t n_rows, int64_t len, int elem_bytes)
     // Lane-load counts that are not a power of two: one lane per lane-load and 64 / G whole
     // rows per wave step, so that every load and store instruction covers one contiguous
     // span (1M x 33 / 50 / 100 floats: 59 / 60 / 56 % -> 70 / 72 / 71 % of 8 TB/s in + out).
-    // One row per step (33..63 lane-loads) pays from 48 lanes on (D = 200 / 250: 65 / 55 % ->
-    // 71 / 67 %; D = 129 / 160 lose 10 points that way and keep the power-of-two groups).
+    // One row per step (33..63 lane-loads) pays from 54 lanes on (fp32 D = 220 / 250: 62 / 56 %
+    // -> 70 / 67 %, bf16 D = 500: 56 -> 68 %; 50 lanes measured 2 points either way on fp32 and
+    // lost 14 on bf16, D = 129 / 160 lose 10 points that way and keep the power-of-two groups).
     // (f64 rows, whose accumulators are twice as wide, lose 13 points with one row per step.)
     if (p.vec16 && (nload & (nload - 1)) != 0 &&
-        ((nload >= 3 && nload <= 32) || (nload >= 48 && nload < 64 && elem_bytes < 8))) {
+        ((nload >= 3 && nload <= 32) || (nload >= 54 && nload < 64 && elem_bytes < 8))) {
       p.L    = 0;
       p.G    = (int)nload;
       p.logG = 0;

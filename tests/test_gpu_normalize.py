@@ -75,7 +75,7 @@ def test_long_rows(gpu, rows, cols, norm):
 
 
 # Rows whose lane-load count is not a power of two take one lane per lane-load (3..32 and
-# 48..63 lane-loads, whole rows per wave step) or three loads per lane; row counts around
+# 54..63 lane-loads, whole rows per wave step) or three loads per lane; row counts around
 # one wave's and one workgroup's share.
 @pytest.mark.parametrize("cols", [10, 20, 21, 45, 50, 67, 100, 127, 129, 190, 200, 222, 250, 255, 300])
 @pytest.mark.parametrize("rows", [1, 5, 29, 257, 4099])
