@@ -251,9 +251,9 @@ RMI_API int rmi_row_normalize(const rmi_reduce_desc* desc,
  * the data: mean[j] = sum_i x[i, j] / n_rows, var[j] = sum_i (x[i, j] - mean[j])^2 /
  * max(1, sample ? n_rows - 1 : n_rows).  Replaces detail::meanvar
  * (stats/detail/meanvar.cuh:187-236) behind raft::stats::meanvar
- * (stats/meanvar.cuh:38-49 pointer form, :74-98 mdspan form).  `dtype` is F32 or F64
- * (data, mean and var share it), `layout` an rmi_layout.  The arithmetic is f64
- * throughout.  An empty column set is a no-op; n_rows == 0 writes zeros.  The workspace
+ * (stats/meanvar.cuh:38-49 pointer form, :74-98 mdspan form).  `dtype` is F32, F64,
+ * F16 or BF16 (data, mean and var share it), `layout` an rmi_layout.  The arithmetic is
+ * f64 throughout; results are rounded once to `dtype`.  An empty column set is a no-op; n_rows == 0 writes zeros.  The workspace
  * follows the rules of rmi_reduce. */
 RMI_API size_t rmi_meanvar_workspace_bytes(int dtype, int layout, int64_t n_rows, int64_t n_cols);
 RMI_API int rmi_meanvar(int dtype,

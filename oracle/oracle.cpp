@@ -740,6 +740,11 @@ ORC_API int orc_row_normalize(const rmi_reduce_desc* d, const void* in, double* 
 // in row order.  Merging a state {w, m, s} with the singleton {1, x, 0} by its
 // operator+= (:60-74): cw = w + 1; d = m - x; s += cw * (d * w/cw) * (d * 1/cw);
 // m = m * w/cw + x * 1/cw.  var = s / max(1, sample ? w - 1 : w) (:88-98).
+inline double as_double(float x) { return (double)x; }
+inline double as_double(double x) { return x; }
+inline double as_double(f16 x) { return (double)half_to_float(x.b); }
+inline double as_double(bf16 x) { return (double)bf16_to_float(x.b); }
+
 template <class T>
 static int meanvar_seq(int layout, int64_t n_rows, int64_t n_cols, int sample, const T* in,
                        double* mean, double* var)
@@ -747,7 +752,7 @@ static int meanvar_seq(int layout, int64_t n_rows, int64_t n_cols, int sample, c
   for (int64_t j = 0; j < n_cols; ++j) {
     double w = 0.0, m = 0.0, s = 0.0;
     for (int64_t i = 0; i < n_rows; ++i) {
-      const double x  = (double)(layout == RMI_ROW_MAJOR ? in[i * n_cols + j] : in[j * n_rows + i]);
+      const double x  = as_double(layout == RMI_ROW_MAJOR ? in[i * n_cols + j] : in[j * n_rows + i]);
       const double cw = w + 1.0;
       const double fa = w / cw, fb = 1.0 / cw;
       const double d  = m - x;
@@ -768,6 +773,8 @@ ORC_API int orc_meanvar(int dtype, int layout, int64_t n_rows, int64_t n_cols, i
   switch (dtype) {
     case RMI_F32: return meanvar_seq(layout, n_rows, n_cols, sample, (const float*)in, mean, var);
     case RMI_F64: return meanvar_seq(layout, n_rows, n_cols, sample, (const double*)in, mean, var);
+    case RMI_F16: return meanvar_seq(layout, n_rows, n_cols, sample, (const f16*)in, mean, var);
+    case RMI_BF16: return meanvar_seq(layout, n_rows, n_cols, sample, (const bf16*)in, mean, var);
     default: return RMI_ERR_UNSUPPORTED;
   }
 }

@@ -130,6 +130,8 @@ int meanvar_plan(int dtype, int layout, int64_t n_rows, int64_t n_cols, PlanX& p
   if (n_rows < 0 || n_cols < 0) return RMI_ERR_BAD_SHAPE;
   if (dtype == RMI_F32) fn = lookup_meanvar_f32();
   else if (dtype == RMI_F64) fn = lookup_meanvar_f64();
+  else if (dtype == RMI_F16) fn = lookup_meanvar_f16();
+  else if (dtype == RMI_BF16) fn = lookup_meanvar_bf16();
   else return RMI_ERR_UNSUPPORTED;
   rmi_reduce_desc d{};
   d.in_dtype  = dtype;

@@ -848,12 +848,22 @@ __device__ __forceinline__ void finish(const Epilogue& e, i64 k, typename P::acc
     const double den  = fmax(1.0, e.s1 != 0.0 ? acc.w - 1.0 : acc.w);
     const double var  = mv_m2(acc) / den;
     void* vp          = const_cast<void*>(e.aux);
-    if (e.out_dtype == RMI_F64) {
-      static_cast<double*>(e.out)[k] = mean;
-      static_cast<double*>(vp)[k]    = var;
-    } else {
-      static_cast<float*>(e.out)[k] = (float)mean;
-      static_cast<float*>(vp)[k]    = (float)var;
+    switch (e.out_dtype) {
+      case RMI_F64:
+        static_cast<double*>(e.out)[k] = mean;
+        static_cast<double*>(vp)[k]    = var;
+        break;
+      case RMI_F16:
+        static_cast<f16_t*>(e.out)[k] = (f16_t)(float)mean;
+        static_cast<f16_t*>(vp)[k]    = (f16_t)(float)var;
+        break;
+      case RMI_BF16:
+        static_cast<uint16_t*>(e.out)[k] = f32_to_bf16((float)mean);
+        static_cast<uint16_t*>(vp)[k]    = f32_to_bf16((float)var);
+        break;
+      default:
+        static_cast<float*>(e.out)[k] = (float)mean;
+        static_cast<float*>(vp)[k]    = (float)var;
     }
   } else {
     using key_t = decltype(acc.key);

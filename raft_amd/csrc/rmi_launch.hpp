@@ -398,5 +398,7 @@ norm_fn lookup_norm_f32(int main_op, int red_op);
 norm_fn lookup_norm_f64(int main_op, int red_op);
 run_fn lookup_meanvar_f32();
 run_fn lookup_meanvar_f64();
+run_fn lookup_meanvar_f16();
+run_fn lookup_meanvar_bf16();
 
 }  // namespace rmi

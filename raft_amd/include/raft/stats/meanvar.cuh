@@ -17,8 +17,9 @@ template <typename T, typename I>
 void meanvar(const resources* res, T* mean, T* var, const T* data, I D, I N, bool sample,
              bool rowMajor, hipStream_t stream)
 {
-  static_assert(std::is_same_v<T, float> || std::is_same_v<T, double>,
-                "meanvar: float and double data are offered");
+  static_assert(std::is_same_v<T, float> || std::is_same_v<T, double> || std::is_same_v<T, __half> ||
+                  std::is_same_v<T, raft::bfloat16_t>,
+                "meanvar: float, double, half and bfloat16 data are offered");
   const int dtype  = raft::detail::rmi::dtype_of<T>::value;
   const int layout = rowMajor ? RMI_ROW_MAJOR : RMI_COL_MAJOR;
   const size_t ws_bytes =

@@ -128,10 +128,42 @@ def test_reference_large_case(gpu):
 
 def test_validation(gpu):
     lib = api.load()
-    assert lib.rmi_meanvar(api.F16, api.ROW_MAJOR, 4, 4, 0, None, None, None, None, 0, None) \
+    assert lib.rmi_meanvar(api.I32, api.ROW_MAJOR, 4, 4, 0, None, None, None, None, 0, None) \
         == api.ERR_UNSUPPORTED
     assert lib.rmi_meanvar(api.F32, 9, 4, 4, 0, None, None, None, None, 0, None) == api.ERR_BAD_ENUM
     assert lib.rmi_meanvar(api.F32, api.ROW_MAJOR, -1, 4, 0, None, None, None, None, 0, None) \
         == api.ERR_BAD_SHAPE
     assert lib.rmi_meanvar(api.F32, api.ROW_MAJOR, 4, 4, 0, None, None, None, None, 0, None) \
         == api.ERR_NULL
+
+
+# 16-bit data (f16, bf16): the arithmetic is f64, mean and variance are rounded once to the
+# data's type; the oracle reads the same stored bits.
+@pytest.mark.parametrize("dt", [api.F16, api.BF16])
+@pytest.mark.parametrize("layout", [api.ROW_MAJOR, api.COL_MAJOR])
+@pytest.mark.parametrize("rows,cols", [(1, 5), (17, 3), (1000, 64), (4097, 19), (333, 1023),
+                                       (200000, 8), (9, 4100)])
+def test_half_types(gpu, dt, layout, rows, cols):
+    import torch
+    from raft_amd import device as dev
+    rng = np.random.default_rng(rows + cols)
+    f = rng.normal(1.5, 2.0, (rows, cols)).astype(np.float32)
+    f = np.ascontiguousarray(f if layout == api.ROW_MAJOR else f.T)
+    stored = f.astype(np.float16).view(np.uint16) if dt == api.F16 else u.to_bf16(f.reshape(-1))
+    stored = np.ascontiguousarray(stored.reshape(-1))
+    x = torch.from_numpy(stored.view(np.int16)).cuda()
+    mean = torch.zeros(cols, dtype=torch.int16, device="cuda")
+    var = torch.zeros(cols, dtype=torch.int16, device="cuda")
+    for sample in (False, True):
+        dev.meanvar(dt, layout, rows, cols, sample, x, mean, var)
+        torch.cuda.synchronize()
+        raw_m = mean.cpu().numpy().view(np.uint16)
+        raw_v = var.cpu().numpy().view(np.uint16)
+        if dt == api.F16:
+            got_m, got_v = raw_m.view(np.float16).astype(np.float64), raw_v.view(np.float16).astype(np.float64)
+        else:
+            got_m, got_v = u.from_bf16(raw_m).astype(np.float64), u.from_bf16(raw_v).astype(np.float64)
+        exp_m, exp_v = _oracle(dt, layout, rows, cols, sample, stored)
+        tol = u.OUT_TOL[dt]
+        assert u.fp_close(got_m, exp_m, tol).all(), u.worst_rel(got_m, exp_m)
+        assert u.fp_close(got_v, exp_v, tol).all(), u.worst_rel(got_v, exp_v)
