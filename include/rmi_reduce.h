@@ -233,7 +233,8 @@ RMI_API int rmi_map_reduce(const rmi_reduce_desc* desc,
 
 /* Row normalisation fused with its norm: out[i, :] = in[i, :] / norm_i with
  * norm_i = final_op(reduce_op(init, fold over j of main_op(in[i, j]))); rows whose
- * norm is <= eps (or NaN) are left untouched.  Replaces detail::coalesced_normalize
+ * norm is <= eps are left untouched (a NaN norm is not: that row is written as NaN, as in
+ * the reference).  Replaces detail::coalesced_normalize
  * (linalg/detail/normalize.cuh:36-197) behind raft::linalg::row_normalize
  * (linalg/normalize.cuh:48-110).  Uses the descriptor fields in_dtype (also the
  * output's type: F16, BF16, F32 or F64), n_rows, n_cols, main_op (IDENTITY, SQ, ABS),

@@ -706,7 +706,8 @@ ORC_API int orc_reduce_typed(const rmi_reduce_desc* d,
 }
 
 // Row normalisation in fp64: out[i, :] = in[i, :] / norm_i, rows with norm_i <= eps
-// untouched (cpp/include/raft/linalg/detail/normalize.cuh:36-57).  `out` holds the
+// untouched (cpp/include/raft/linalg/detail/normalize.cuh:36-57); a row whose norm is NaN
+// fails that test and is written (as NaN), like in the reference.  `out` holds the
 // previous contents on entry, as doubles.
 template <class T>
 static int normalize_seq(const rmi_reduce_desc& d, const T* in, double* out, double eps)
@@ -716,7 +717,7 @@ static int normalize_seq(const rmi_reduce_desc& d, const T* in, double* out, dou
     for (int64_t j = 0; j < d.n_cols; ++j)
       acc = red_f(d.reduce_op, acc, main_f(d.main_op, Elem<T>::f64(in[i * d.n_cols + j])));
     const double norm = d.final_op == RMI_FIN_SQRT ? sqrt(acc) : acc;
-    if (!(norm > eps)) continue;
+    if (norm <= eps) continue;  // normalize.cuh:52,120: a NaN norm is not skipped
     for (int64_t j = 0; j < d.n_cols; ++j)
       out[i * d.n_cols + j] = Elem<T>::f64(in[i * d.n_cols + j]) / norm;
   }

@@ -1,7 +1,7 @@
 // Row normalisation fused with its norm: out[i, :] = in[i, :] / norm_i, where
 // norm_i = final_op(reduce_op-fold of main_op(in[i, j])) and rows whose norm is
 // <= eps are left untouched (linalg/detail/normalize.cuh:36-57,112-134 of the
-// reference).  Rows of up to 256 lane-loads stay in registers between the reduction
+// reference; a NaN norm is not <= eps, so such a row is written, as NaN).  Rows of up to 256 lane-loads stay in registers between the reduction
 // and the scaling, so the matrix is read once and written once; longer rows are
 // swept twice by one team (the second sweep finds the row in the caches).
 #pragma once
@@ -112,8 +112,12 @@ __device__ __forceinline__ typename P::nat row_norm(const NormArgs& a, typename 
   return n;
 }
 
-// lane-load `v` of a row, scaled by 1/norm and written to the same place of `orow`
-template <class P, bool VEC16, bool STREAM>
+// lane-load `v` of a row, scaled by 1/norm and written to the same place of `orow`.
+// TAIL_EACH: the overlapping last vector stores only its `tail` new elements, one by one.
+// A kernel that re-reads the row for the scaling needs that when `out` is `in`: the vector's
+// first VEC - tail elements belong to the lane before it, which may sit in another wave and
+// may already have stored them scaled.
+template <class P, bool VEC16, bool STREAM, bool TAIL_EACH = false>
 __device__ __forceinline__ void write_scaled(const NormArgs& a,
                                              char* orow,
                                              const typename Held<P, VEC16>::type& x,
@@ -123,7 +127,27 @@ __device__ __forceinline__ void write_scaled(const NormArgs& a,
   using in_t = typename P::in_t;
   if constexpr (VEC16) {
     // The overlapping last vector (v == nvec) is stored whole where it was read: its first
-    // VEC - tail elements repeat what the lane before it stores, bit for bit.
+    // VEC - tail elements repeat what the lane before it stores, bit for bit (as long as it
+    // was loaded before any lane stored, i.e. the row is held in registers).
+    if constexpr (TAIL_EACH) {
+      if (v >= a.nvec) {
+        in_t* o   = reinterpret_cast<in_t*>(orow) + (a.len - P::VEC);
+        const int first = P::VEC - a.tail;
+        if constexpr (sizeof(in_t) == 2) {
+          const typename P::nat inv = (typename P::nat)1 / norm;
+          static_for<P::VEC>([&](auto j) {
+            if (decltype(j)::value >= first)
+              Put<in_t>::st(o + decltype(j)::value, In<in_t>::template get<decltype(j)::value>(x) * inv);
+          });
+        } else {
+          static_for<P::VEC>([&](auto j) {
+            if (decltype(j)::value >= first)
+              Put<in_t>::st(o + decltype(j)::value, In<in_t>::template get<decltype(j)::value>(x) / norm);
+          });
+        }
+        return;
+      }
+    }
     u32x4 y = x;
     if constexpr (sizeof(in_t) == 2) {
       // 16-bit elements: one division per lane-load, then products in fp32 that are rounded
@@ -195,7 +219,7 @@ __device__ __forceinline__ void normalize_wave_body(const NormArgs& a)
   for (int t = 0; t < TILES; ++t) {
     if (row[t] < a.n_rows) {
       const auto norm = row_norm<P>(a, acc[t]);
-      if (norm > (typename P::nat)a.eps) {  // false for NaN norms too
+      if (!(norm <= (typename P::nat)a.eps)) {  // a NaN norm is not skipped: the row becomes NaN
         char* orow = static_cast<char*>(a.out) + row[t] * a.row_bytes;
 #pragma unroll
         for (int u = 0; u < L; ++u)
@@ -251,7 +275,7 @@ __device__ __forceinline__ void normalize_anyg_body(const NormArgs& a)
     const acc_t total = shfl_acc<P>(acc[t], first);
     if (live && row[t] < a.n_rows) {
       const auto norm = row_norm<P>(a, total);
-      if (norm > (typename P::nat)a.eps)  // false for NaN norms too
+      if (!(norm <= (typename P::nat)a.eps))  // a NaN norm is not skipped: the row becomes NaN
         write_scaled<P, true, STREAM>(a, static_cast<char*>(a.out) + row[t] * a.row_bytes, x[t], c, norm);
     }
   }
@@ -314,7 +338,7 @@ __global__ __launch_bounds__(1024) void normalize_team_kernel(NormArgs a)
   }
   __syncthreads();
   const nat norm = sm_norm;
-  if (!(norm > (nat)a.eps)) return;
+  if (norm <= (nat)a.eps) return;  // a NaN norm is not skipped: the row becomes NaN
   char* orow = static_cast<char*>(a.out) + row * a.row_bytes;
 #pragma unroll
   for (int u = 0; u < UH; ++u)
@@ -360,7 +384,7 @@ __global__ __launch_bounds__(1024) void normalize_sweep_kernel(NormArgs a)
   }
   __syncthreads();
   const nat norm = sm_norm;
-  if (!(norm > (nat)a.eps)) return;
+  if (norm <= (nat)a.eps) return;  // a NaN norm is not skipped: the row becomes NaN
   char* orow = static_cast<char*>(a.out) + row * a.row_bytes;
   for (i64 v = t; v < nload; v += (i64)kUnroll * T) {
     typename H::type x[kUnroll];
@@ -371,7 +395,7 @@ __global__ __launch_bounds__(1024) void normalize_sweep_kernel(NormArgs a)
     }
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u)
-      if (v + (i64)u * T < nload) write_scaled<P, true, true>(a, orow, x[u], v + (i64)u * T, norm);
+      if (v + (i64)u * T < nload) write_scaled<P, true, true, true>(a, orow, x[u], v + (i64)u * T, norm);
   }
 }
 

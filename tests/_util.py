@@ -135,14 +135,59 @@ def approx_ok(actual, expected, eps):
 # The bar of this build for floating results against the fp64 oracle:
 # |x - o| <= 1e-5*|o|, or <= 1e-5 absolute where |o| < 1.
 FP_TOL = 1e-5
-OUT_TOL = {api.F32: 1e-5, api.F64: 1e-5, api.F16: 2e-3, api.BF16: 1.6e-2}
+OUT_TOL = {api.F32: 1e-5, api.F64: 1e-5}
+# 16-bit outputs have no tolerance: the library rounds its f64 result once, so an output must be
+# the correctly rounded oracle value or the 16-bit number next to it (ulp16_ok below).
+
+
+def _ord16(bits):
+    """uint16 sign-magnitude storage bits -> integers ordered like the values (+-0 -> 0)."""
+    b = np.asarray(bits).astype(np.int32)
+    return np.where(b & 0x8000, -(b & 0x7FFF), b)
+
+
+def _bits16(o):
+    o = np.asarray(o, dtype=np.int32)
+    return np.where(o < 0, (-o) | 0x8000, o).astype(np.uint16)
+
+
+def round_to_16(out_dtype, values):
+    """float64 values -> storage bits of the nearest f16 / bf16 number (ties to even)."""
+    v = np.asarray(values, dtype=np.float64)
+    if out_dtype == api.F16:
+        with np.errstate(over="ignore"):
+            return v.astype(np.float16).view(np.uint16)
+    # bf16: round through f32, then repair the rare double rounding by picking, among the
+    # result and its two neighbours, the one strictly nearest to the f64 value
+    with np.errstate(over="ignore"):
+        b0 = to_bf16(v.astype(np.float32))
+    o0 = _ord16(b0)
+    best, bestd = o0.copy(), np.abs(from_bf16(b0).astype(np.float64) - v)
+    for step in (-1, 1):
+        c = o0 + step
+        d = np.abs(from_bf16(_bits16(c)).astype(np.float64) - v)
+        take = np.isfinite(d) & (d < bestd)
+        best, bestd = np.where(take, c, best), np.where(take, d, bestd)
+    return np.where(np.isfinite(v), _bits16(best), b0).astype(np.uint16)
+
+
+def ulp16_ok(out_dtype, got_bits, expected_f64, ulps=1):
+    """True where a 16-bit output is within `ulps` representable numbers of the correctly
+    rounded expected value (NaN matches NaN, infinities match themselves)."""
+    got_bits = np.asarray(got_bits).view(np.uint16)
+    want = round_to_16(out_dtype, expected_f64)
+    gf = got_bits.view(np.float16).astype(np.float64) if out_dtype == api.F16 else \
+        from_bf16(got_bits).astype(np.float64)
+    nan = np.isnan(np.asarray(expected_f64, dtype=np.float64))
+    return np.where(nan, np.isnan(gf), np.abs(_ord16(got_bits) - _ord16(want)) <= ulps)
 
 
 def fp_close(actual, expected, tol=FP_TOL):
     actual = np.asarray(actual, dtype=np.float64)
     expected = np.asarray(expected, dtype=np.float64)
-    diff = np.abs(actual - expected)
-    bound = tol * np.maximum(np.abs(expected), 1.0)
+    with np.errstate(invalid="ignore"):
+        diff = np.abs(actual - expected)
+        bound = tol * np.maximum(np.abs(expected), 1.0)
     same_special = (actual == expected) | (np.isnan(actual) & np.isnan(expected))
     return same_special | (diff <= bound)
 
@@ -238,6 +283,11 @@ def check_against_oracle(desc, data, *, old_raw=None, aux_raw=None, misalign_ele
             exp = exp.astype(np.int32).astype(np.int64)
         assert np.array_equal(got, exp), (
             f"{label}: integer results differ at {np.flatnonzero(got != exp)[:8]}")
+    elif desc.out_dtype in (api.F16, api.BF16) and tol is None:
+        ok = ulp16_ok(desc.out_dtype, got_raw, exp)
+        assert ok.all(), (f"{label}: {np.count_nonzero(~ok)} of {ok.size} 16-bit outputs are more "
+                          f"than one ulp from the rounded oracle value: first bad "
+                          f"{np.flatnonzero(~ok)[:5]} got {got[~ok][:5]} want {exp[~ok][:5]}")
     else:
         t = tol if tol is not None else OUT_TOL[desc.out_dtype]
         ok = fp_close(got, exp, t)

@@ -63,36 +63,32 @@ def test_wave_reduction_vector(gpu):
     assert [int(r["key"][0]), float(r["value"][0])] == W64["argmin"]
 
 
-# cpp/tests/stats/sum.cu:50-98,139-140 ("Accuracy"): per column, every third row holds
-# v*L, the row above -v*L, the one above that 3v; the column sum must still be rows*v.
-@pytest.mark.parametrize("npdt,dt,value,large,rows,cols,tol", [
-    (np.float32, api.F32, 1e-4, 1e7, 1024, 32, 0.001),
-    (np.float32, api.F32, 1e-4, 1e7, 1024, 256, 0.001),
-    (np.float32, api.F32, 1e-4, 1e7, 17, 5, 0.001),
-    (np.float32, api.F32, 1e-4, 1e7, 7, 23, 0.001),
-    (np.float32, api.F32, 1e-4, 1e7, 3, 97, 0.001),
-    (np.float64, api.F64, 1e-6, 1e12, 1024, 256, 0.0001),
-    (np.float64, api.F64, 1e-6, 1e12, 17, 5, 0.0001),
-    (np.float64, api.F64, 1e-6, 1e12, 3, 97, 0.0001),
-])
-@pytest.mark.parametrize("row_major", [True, False])
-def test_sum_compensation(gpu, npdt, dt, value, large, rows, cols, tol, row_major):
-    m = np.full((rows, cols), value, dtype=np.float64)
-    for r in range(2, rows, 3):
-        m[r, :] = value * large
-        m[r - 1, :] = -value * large
-        m[r - 2, :] = 3.0 * value
-    m = m.astype(npdt)
-    flat = m.reshape(-1) if row_major else m.T.reshape(-1)
+# cpp/tests/stats/sum.cu:50-98,108-140: the reference's grid, plain ("Result") and with the
+# (3v, -vL, +vL) triples ("Accuracy"); the column sums must be rows * value.  The cases of 10^8
+# and 2^27 rows are generated on the device in tests/test_gpu_reference_stats.py.
+from tests.test_oracle import SUM_SMALL, sum_case_matrix  # noqa: E402
+
+
+@pytest.mark.parametrize("kind,case", SUM_SMALL, ids=lambda x: str(x))
+@pytest.mark.parametrize("accuracy", [False, True])
+def test_sum_grid(gpu, kind, case, accuracy):
+    g = GOLD["stats_sum"]
+    tol, rows, cols, row_major, value = case
+    npdt, dt = (np.float32, api.F32) if kind == "float" else (np.float64, api.F64)
+    m = sum_case_matrix(npdt, rows, cols, value, g["large_factor"][kind] if accuracy else None)
+    flat = np.ascontiguousarray(m.reshape(-1) if row_major else m.T.reshape(-1))
     d = api.make_desc(dt, dt, rows, cols, apply=api.ALONG_COLUMNS,
                       layout=api.ROW_MAJOR if row_major else api.COL_MAJOR)
-    got = u.gpu_reduce(d, np.ascontiguousarray(flat)).astype(np.float64)
-    expected = np.full(cols, rows * value)
-    # the reference allows 100*tolerance here; this build holds the plain tolerance
+    got = u.gpu_reduce(d, flat).astype(np.float64)
+    expected = np.full(cols, float(npdt(rows * float(npdt(value)))))
+    # the reference allows 100 * tolerance for the Accuracy variant; this build holds the
+    # plain tolerance for both
     assert u.approx_ok(got, expected, tol).all(), (got[:4], expected[:4])
 
 
-# cpp/tests/stats/stddev.cu:139-150,187-190: constant data => stddev 0; one row => 0.
+# Constant data => stddev 0, one row => 0, sqrt(vars) == stddev (what
+# cpp/tests/stats/stddev.cu:148-149,187-202 checks; its own 2^27-row cases run at full size in
+# tests/test_gpu_reference_stats.py).
 @pytest.mark.parametrize("rows,cols", [(1, 1), (1, 257), (31, 1), (4096, 64)])
 @pytest.mark.parametrize("sample", [False, True])
 def test_stddev_constant_data(gpu, rows, cols, sample):

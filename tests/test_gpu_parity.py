@@ -204,6 +204,112 @@ def test_min_max(gpu, in_dt, out_dt, red, main):
                                label=f"minmax {api.DTYPE_NAME[in_dt]} red{red} main{main}")
 
 
+# NaN through max_op / min_op and the Linf norm: the reference's device max / min are fmax / fmin
+# (core/math.hpp:375-397,517-533), which ignore NaN; a row of NaN only returns `init`.  NaN is
+# scattered, fills whole rows and whole columns, and sits in the tail elements after the last
+# whole 16-byte vector (the overlapping last lane-load sees those twice).  Every plan kind: rows
+# inside a vector, one load per lane, lanes of a wave (direct and staged through LDS), teams,
+# split rows with the second pass, and the column kernel with its second pass.  Checked against
+# the oracle (exactly: max / min select one of the inputs) and against numpy's nanmax / nanmin.
+NAN_SHAPES = [
+    # rows, cols, apply, plan hint, expected plan kind
+    (5000, 2, api.ALONG_ROWS, api.PLAN_AUTO, api.PLAN_ROW_LANES),
+    (3000, 21, api.ALONG_ROWS, api.PLAN_AUTO, api.PLAN_ROW_WAVE),     # one load per lane, any G, tail
+    (3000, 30, api.ALONG_ROWS, api.PLAN_AUTO, api.PLAN_ROW_WAVE),     # one load per lane, G = 8, tail
+    (1000, 259, api.ALONG_ROWS, api.PLAN_AUTO, api.PLAN_ROW_WAVE),    # lanes of a wave, tail
+    (1000, 200, api.ALONG_ROWS, api.PLAN_AUTO, api.PLAN_ROW_WAVE),    # staged through LDS
+    (300, 4099, api.ALONG_ROWS, api.PLAN_AUTO, api.PLAN_ROW_BLOCK),   # teams, tail
+    (37, 8197, api.ALONG_ROWS, api.PLAN_ROW_BLOCK, api.PLAN_ROW_BLOCK),
+    (3, 300003, api.ALONG_ROWS, api.PLAN_AUTO, api.PLAN_ROW_SPLIT),   # split rows + second pass
+    (5, 70001, api.ALONG_ROWS, api.PLAN_ROW_SPLIT, api.PLAN_ROW_SPLIT),
+    (20000, 67, api.ALONG_COLUMNS, api.PLAN_AUTO, api.PLAN_COL_TILE),   # dense lanes, tail, 2 passes
+    (30000, 64, api.ALONG_COLUMNS, api.PLAN_AUTO, api.PLAN_COL_TILE),
+    (40000, 3, api.ALONG_COLUMNS, api.PLAN_AUTO, api.PLAN_COL_TILE),    # rows read in groups
+    (700, 1001, api.ALONG_COLUMNS, api.PLAN_AUTO, api.PLAN_COL_TILE),
+]
+
+
+@pytest.mark.parametrize("in_dt,out_dt", [(api.F32, api.F32), (api.F64, api.F64), (api.F16, api.F32),
+                                          (api.BF16, api.F32)])
+@pytest.mark.parametrize("rows,cols,apply,hint,kind", NAN_SHAPES)
+def test_max_min_ignore_nan(gpu, in_dt, out_dt, rows, cols, apply, hint, kind):
+    import warnings
+    rng = np.random.default_rng(rows * 31 + cols)
+    m = rng.standard_normal((rows, cols))
+    m[rng.random((rows, cols)) < 0.1] = np.nan
+    m[rows // 3, :] = np.nan                       # a whole row
+    m[:, cols // 2] = np.nan                       # a whole column
+    m[min(rows - 1, 2), cols - 1] = np.nan         # the last element of a row: a tail element
+    m[:, -1][rng.random(rows) < 0.5] = np.nan
+    if in_dt == api.F32:
+        data = m.astype(np.float32)
+    elif in_dt == api.F64:
+        data = m
+    elif in_dt == api.F16:
+        data = m.astype(np.float16)
+    else:
+        data = u.to_bf16(m.astype(np.float32).reshape(-1)).reshape(rows, cols)
+    vals = u.from_bf16(data).astype(np.float64) if in_dt == api.BF16 else data.astype(np.float64)
+    assert np.isnan(vals).sum() == np.isnan(m).sum()
+    ax = 1 if apply == api.ALONG_ROWS else 0
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore", RuntimeWarning)
+        cases = [(api.MAIN_IDENTITY, api.RED_MAX, -np.inf, np.nanmax(vals, axis=ax)),
+                 (api.MAIN_IDENTITY, api.RED_MIN, np.inf, np.nanmin(vals, axis=ax)),
+                 (api.MAIN_ABS, api.RED_MAX, 0.0, np.nanmax(np.abs(vals), axis=ax))]  # Linf norm
+    for main, red, init, want in cases:
+        want = np.where(np.isnan(want), init, want)
+        d = api.make_desc(in_dt, out_dt, rows, cols, apply=apply, main_op=main, reduce_op=red,
+                          init_f=init, plan_hint=hint)
+        # two f64 fill a 16-byte vector: such rows take one lane each of the wave plan
+        want_kind = api.PLAN_ROW_WAVE if kind == api.PLAN_ROW_LANES and in_dt == api.F64 else kind
+        assert api.plan_query(d).kind == want_kind
+        for shift in (0, 1):
+            raw = u.check_against_oracle(d, data.reshape(-1), tol=0.0, misalign_elems=shift,
+                                         label=f"nan {rows}x{cols} main{main} red{red} +{shift}")
+            assert np.array_equal(raw.astype(np.float64), want), (main, red, shift)
+
+
+# The same through the inplace merge and a 16-bit output: red(out_old, acc) must ignore a NaN
+# on either side the way fmax / fmin do.
+def test_max_nan_inplace_and_init(gpu):
+    rows, cols = 64, 100
+    m = np.full((rows, cols), np.nan, dtype=np.float32)
+    m[1::2, 5] = 3.0
+    d = api.make_desc(api.F32, api.F32, rows, cols, reduce_op=api.RED_MAX, init_f=-np.inf,
+                      inplace=True)
+    old = np.where(np.arange(rows) % 4 < 2, np.float32(np.nan), np.float32(7.0)).astype(np.float32)
+    raw = u.check_against_oracle(d, m.reshape(-1), old_raw=old, tol=0.0, label="nan inplace")
+    want = np.array([np.fmax(np.fmax(-np.inf, 3.0 if r % 2 else np.nan), old[r]) for r in range(rows)])
+    assert np.array_equal(raw.astype(np.float64), want)
+
+
+# Rounding of f32 / f64 results to 16-bit outputs, bit for bit: one-element rows make the
+# output the conversion of the input itself.  torch's bfloat16 and numpy's float16 conversions
+# are the independent statements of round-to-nearest-even; a truncating conversion fails on
+# half of the values, a round-half-up one on the ties.
+@pytest.mark.parametrize("out_dt", [api.BF16, api.F16])
+def test_output_rounding_is_nearest_even(gpu, out_dt):
+    import torch
+    rng = np.random.default_rng(99)
+    n = 1 << 20
+    if out_dt == api.BF16:
+        bits = rng.integers(0, 2**32, n, dtype=np.uint64).astype(np.uint32)
+        bits[: n // 4] = (bits[: n // 4] & 0xFFFF0000) | 0x8000        # exact ties
+        x = bits.view(np.float32)
+        x = x[np.isfinite(x)]
+        want = torch.from_numpy(x).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    else:
+        x = (rng.standard_normal(n) * np.exp(rng.uniform(-12, 11, n))).astype(np.float32)
+        h = x[: n // 4].astype(np.float16).astype(np.float32)           # exact ties: midpoints
+        x[: n // 4] = (h + np.nextafter(h.astype(np.float16), np.float16(np.inf)).astype(np.float32)) / 2
+        x = x[np.isfinite(x) & (np.abs(x) < 60000)]
+        want = x.astype(np.float16).view(np.uint16)
+    d = api.make_desc(api.F32, out_dt, x.size, 1)
+    got = u.gpu_reduce(d, x).view(np.uint16)
+    assert np.array_equal(got, want), np.flatnonzero(got != want)[:8]
+
+
 # L1 / L2 / Linf norms (linalg/detail/norm.cuh:23-61), row and column, with and without sqrt;
 # cpp/tests/linalg/norm.cu:238-306 (incl. half -> float).
 @pytest.mark.parametrize("in_dt,out_dt", [(api.F32, api.F32), (api.F64, api.F64),

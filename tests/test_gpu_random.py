@@ -104,10 +104,14 @@ def test_random_normalize(gpu, seed):
         data = f.astype({api.F32: np.float32, api.F64: np.float64, api.F16: np.float16}[dt])
     d = api.make_desc(dt, dt, rows, cols, main_op=main, reduce_op=red, final_op=fin)
     prev = np.zeros(rows * cols, dtype=data.dtype)
-    got = tn._as_f64(dt, tn._gpu(d, data, prev, 1e-8))
+    raw = tn._gpu(d, data, prev, 1e-8)
+    got = tn._as_f64(dt, raw)
     exp = tn._oracle(d, data, tn._as_f64(dt, prev), 1e-8)
-    tol = {api.F32: 1e-5, api.F64: 1e-8}.get(dt, u.OUT_TOL[dt])
-    assert u.approx_ok(got, exp, tol).all(), (seed, dt, rows, cols, norm, u.worst_rel(got, exp))
+    if dt in (api.F16, api.BF16):
+        ok = u.ulp16_ok(dt, raw, exp)
+    else:
+        ok = u.approx_ok(got, exp, {api.F32: 1e-5, api.F64: 1e-8}[dt])
+    assert ok.all(), (seed, dt, rows, cols, norm, u.worst_rel(got, exp))
 
 
 @pytest.mark.parametrize("seed", range(int(os.environ.get("RMI_RANDOM_CASES", "400")) // 4))

@@ -86,45 +86,133 @@ def test_arg_op_truth_table(oracle):
             assert _arg2(red, pair[x], pair[y]) == f(pair[want]), (red, x, y)
 
 
-# cpp/tests/stats/sum.cu:50-98: triples (3v, -vL, +vL) must still sum to rows*v.
-@pytest.mark.parametrize("case", GOLD["sum_accuracy"]["cases"],
-                         ids=lambda c: f"{c['dtype']}-{c['rows']}x{c['cols']}")
-def test_sum_compensation_fixture(oracle, case):
-    npdt, dt = (np.float32, api.F32) if case["dtype"] == "f32" else (np.float64, api.F64)
-    v, L, rows, cols = case["value"], case["large"], case["rows"], case["cols"]
-    m = np.full((rows, cols), v, dtype=np.float64)
-    for r in range(2, rows, 3):
-        m[r], m[r - 1], m[r - 2] = v * L, -v * L, 3 * v
-    m = m.astype(npdt)
-    d = api.make_desc(dt, dt, rows, cols, apply=api.ALONG_COLUMNS)
+# cpp/tests/stats/sum.cu:50-98,108-140: the reference's grid of constant matrices (Result) and
+# of (3v, -vL, +vL) triples (Accuracy); the column sums must be rows * value.  Cases above a
+# million elements run on the GPU only (tests/test_gpu_reference_stats.py).
+def sum_case_matrix(npdt, rows, cols, value, large=None):
+    """The reference's input for one SumInputs case, as a [rows, cols] array of npdt."""
+    v = float(npdt(value))            # params.value is a T
+    col = np.full(rows, v, dtype=np.float64)
+    if large is not None:
+        r = np.arange(rows)
+        col[r % 3 == 2] = v * large
+        col[(r % 3 == 1) & (r + 1 < rows)] = -v * large
+        col[(r % 3 == 0) & (r + 2 < rows)] = 3.0 * v
+    return np.repeat(col.astype(npdt)[:, None], cols, axis=1)
+
+
+SUM_SMALL = [(k, c) for k in ("float", "double") for c in GOLD["stats_sum"][k] if c[1] * c[2] <= 10**6]
+
+
+@pytest.mark.parametrize("kind,case", SUM_SMALL, ids=lambda x: str(x))
+@pytest.mark.parametrize("accuracy", [False, True])
+def test_sum_grid(oracle, kind, case, accuracy):
+    g = GOLD["stats_sum"]
+    tol, rows, cols, row_major, value = case
+    npdt, dt = (np.float32, api.F32) if kind == "float" else (np.float64, api.F64)
+    m = sum_case_matrix(npdt, rows, cols, value, g["large_factor"][kind] if accuracy else None)
+    flat = np.ascontiguousarray(m.reshape(-1) if row_major else m.T.reshape(-1))
+    d = api.make_desc(dt, dt, rows, cols, apply=api.ALONG_COLUMNS,
+                      layout=api.ROW_MAJOR if row_major else api.COL_MAJOR)
+    expected = np.full(cols, float(npdt(rows * float(npdt(value)))))
+    eps = tol * (g["accuracy_tolerance_factor"] if accuracy else 1)
     # the typed implementation carries the reference's compensation term
     out = np.zeros(cols, dtype=npdt)
-    u.oracle_typed(d, m.reshape(-1), out)
-    tol = 0.1 if npdt == np.float32 else 0.01
-    assert u.approx_ok(out, np.full(cols, rows * float(npdt(v))), tol).all()
-    # the fp64 oracle on fp32 data is exact to far below that
+    u.oracle_typed(d, flat, out)
+    assert u.approx_ok(out, expected, eps).all(), (out[:3], expected[:3])
+    # the sequential fp64 oracle: exact on fp32 data to far below the tolerance
     if npdt == np.float32:
-        seq = u.oracle_reduce(d, m.reshape(-1))
-        assert u.approx_ok(seq, np.full(cols, rows * float(np.float32(v))), 1e-6).all()
+        assert u.approx_ok(u.oracle_reduce(d, flat), expected, 1e-6).all()
 
 
-# cpp/tests/stats/stddev.cu:139-150,187-190,198-202
-def test_stddev_fixtures(oracle):
-    g = GOLD["stddev_constant"]
-    rows, cols = g["rows"], g["cols"]
-    data = np.full(rows * cols, g["value"], dtype=np.float32)
-    mu = np.full(cols, g["value"])
-    for sample in (False, True):
+# cpp/tests/stats/stddev.cu:119-202: stddev of normal(mean, stddev) data within `tolerance` of
+# the distribution's stddev, 0 for a single row, sqrt(vars) == stddev; the reference's RNG is not
+# reproduced, numpy's normal stands in.  The 2^27-row constant cases run on the GPU only; their
+# small-scale counterpart (constant data -> 0) is the last block.
+@pytest.mark.parametrize("kind", ["float", "double"])
+def test_stddev_grid(oracle, kind):
+    npdt, dt = (np.float32, api.F32) if kind == "float" else (np.float64, api.F64)
+    rng = np.random.default_rng(1234)
+    for tol, mean, sd, rows, cols, sample, row_major in GOLD["stats_stddev"][kind]:
+        if rows * cols > 10**6:
+            rows = 4096  # same constant data, a size the CPU finishes at once
+        m = (rng.normal(mean, sd, (rows, cols)) if sd > 0 else np.full((rows, cols), mean)).astype(npdt)
+        flat = np.ascontiguousarray(m.reshape(-1) if row_major else m.T.reshape(-1))
+        lay = api.ROW_MAJOR if row_major else api.COL_MAJOR
+        mu = m.astype(np.float64).mean(axis=0)
         r = 1.0 / (rows - 1 if sample else rows)
         rm = r * rows if sample else 1.0
-        ds = api.make_desc(api.F32, api.F32, rows, cols, apply=api.ALONG_COLUMNS,
+        ds = api.make_desc(dt, dt, rows, cols, layout=lay, apply=api.ALONG_COLUMNS,
                            main_op=api.MAIN_SQ, final_op=api.FIN_STDDEV_FROM_SUMSQ,
                            final_scalar=r, final_scalar2=rm)
-        sd = u.oracle_reduce(ds, data, aux=mu)
-        assert np.all(np.abs(sd) < 1e-6)
+        got = u.oracle_reduce(ds, flat, aux=mu)
+        want = 0.0 if rows == 1 else sd
+        assert u.approx_ok(got, np.full(cols, want), tol).all(), (rows, cols, got[:3])
+        if rows > 1:
+            assert np.allclose(got, m.astype(np.float64).std(axis=0, ddof=1 if sample else 0),
+                               rtol=1e-9, atol=1e-7)
         ds.final_op = api.FIN_VAR_FROM_SUMSQ
-        var = u.oracle_reduce(ds, data, aux=mu)
-        assert np.allclose(np.sqrt(var), sd)
+        var = u.oracle_reduce(ds, flat, aux=mu)
+        assert u.approx_ok(np.sqrt(var), got, tol).all()
+
+
+# cpp/tests/stats/mean.cu:118-215: column means of normal(mean, stddev) data within `tolerance`
+# of the mean, including half -> float and (rounded normals) int8 -> half.
+@pytest.mark.parametrize("kind", ["float", "double", "half_to_float", "int8_to_half"])
+def test_mean_grid(oracle, kind):
+    in_np, in_dt, out_np, out_dt = {
+        "float": (np.float32, api.F32, np.float32, api.F32),
+        "double": (np.float64, api.F64, np.float64, api.F64),
+        "half_to_float": (np.float16, api.F16, np.float32, api.F32),
+        "int8_to_half": (np.int8, api.I8, np.float16, api.F16)}[kind]
+    rng = np.random.default_rng(1234)
+    for tol, mean, rows, cols, row_major, sd in GOLD["stats_mean"][kind]:
+        if rows * cols > 10**7:
+            continue  # GPU only
+        x = rng.normal(mean, sd, (rows, cols))
+        m = np.clip(np.rint(x), -128, 127).astype(np.int8) if in_np == np.int8 else x.astype(in_np)
+        flat = np.ascontiguousarray(m.reshape(-1) if row_major else m.T.reshape(-1))
+        ratio = float(out_np(1) / out_np(rows))   # stats/detail/mean.cuh:22
+        d = api.make_desc(in_dt, out_dt, rows, cols, apply=api.ALONG_COLUMNS,
+                          layout=api.ROW_MAJOR if row_major else api.COL_MAJOR,
+                          final_op=api.FIN_MUL_CONST, final_scalar=ratio)
+        got = u.oracle_reduce(d, flat)
+        if in_np == np.int8:
+            assert np.all(np.abs(got - mean) <= tol)            # ASSERT_NEAR
+        else:
+            assert u.approx_ok(got, np.full(cols, float(in_np(mean))), tol).all()
+        assert np.allclose(got, m.astype(np.float64).sum(axis=0) * ratio, rtol=1e-12)
+        out = np.zeros(cols, dtype=out_np)
+        u.oracle_typed(d, flat, out)
+        assert np.allclose(out.astype(np.float64), got, rtol=2e-3 if out_np == np.float16 else 1e-5)
+
+
+# core/math.hpp:375-397,517-533: the device max / min ignore NaN (fmax / fmin); a row of NaN
+# only returns `init`.  numpy's nanmax / nanmin are the independent statement of that rule.
+@pytest.mark.parametrize("layout,apply", itertools.product([api.ROW_MAJOR, api.COL_MAJOR],
+                                                           [api.ALONG_ROWS, api.ALONG_COLUMNS]))
+def test_max_min_ignore_nan(oracle, layout, apply):
+    rng = np.random.default_rng(17)
+    rows, cols = 23, 31
+    m = rng.standard_normal((rows, cols)).astype(np.float32)
+    m[rng.random((rows, cols)) < 0.2] = np.nan
+    m[4, :] = np.nan
+    m[:, 7] = np.nan
+    flat = np.ascontiguousarray(m.reshape(-1) if layout == api.ROW_MAJOR else m.T.reshape(-1))
+    ax = 1 if apply == api.ALONG_ROWS else 0
+    import warnings
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore", RuntimeWarning)
+        cases = [(api.MAIN_IDENTITY, api.RED_MAX, -np.inf, np.nanmax(m, axis=ax)),
+                 (api.MAIN_IDENTITY, api.RED_MIN, np.inf, np.nanmin(m, axis=ax)),
+                 (api.MAIN_ABS, api.RED_MAX, 0.0, np.nanmax(np.abs(m), axis=ax))]   # Linf norm
+    for main, red, init, want in cases:
+        want = np.where(np.isnan(want), init, want).astype(np.float64)
+        d = api.make_desc(api.F32, api.F32, rows, cols, layout=layout, apply=apply, main_op=main,
+                          reduce_op=red, init_f=init)
+        assert np.array_equal(u.oracle_reduce(d, flat), want), (main, red)
+        out = np.zeros(len(want), dtype=np.float32)
+        assert np.array_equal(u.oracle_typed(d, flat, out).astype(np.float64), want), (main, red)
 
 
 # cpp/tests/linalg/map_then_reduce.cu:140-169
@@ -245,11 +333,20 @@ def test_storage_conversions(oracle):
     oracle.orc_f16_to_f32(allh.ctypes.data, backall.ctypes.data, 65536)
     ref = allh.view(np.float16).astype(np.float32)
     assert np.array_equal(backall.view(np.uint32), ref.view(np.uint32))
-    b = u.to_bf16(x)
-    bits = x.view(np.uint32).astype(np.uint64)
-    want = ((bits + 0x7fff + ((bits >> 16) & 1)) >> 16).astype(np.uint16)
+    # bf16 against torch's conversion (an independent implementation): random bit patterns of
+    # every exponent, and exact ties (the low 16 bits are 0x8000), which must go to even
+    import torch
+    bits = rng.integers(0, 2**32, 4_000_000, dtype=np.uint64).astype(np.uint32)
+    ties = (rng.integers(0, 2**16, 100_000, dtype=np.uint64).astype(np.uint32) << 16) | 0x8000
+    xb = np.concatenate([bits, ties, x.view(np.uint32)]).view(np.float32)
+    xb = xb[~np.isnan(xb)]
+    b = u.to_bf16(xb)
+    want = torch.from_numpy(xb).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
     assert np.array_equal(b, want)
-    assert np.array_equal(u.from_bf16(b).view(np.uint32), b.astype(np.uint32) << 16)
+    assert np.array_equal(u.from_bf16(b).view(np.uint32),
+                          torch.from_numpy(b.view(np.int16)).view(torch.bfloat16).float().numpy().view(np.uint32))
+    nan = u.to_bf16(np.array([np.nan], dtype=np.float32))
+    assert np.isnan(u.from_bf16(nan)[0])
 
 
 # the OpenMP implementation agrees with the sequential oracle on the benchmark's
@@ -300,6 +397,22 @@ def test_row_normalize_against_numpy(oracle):
         want = np.where(norms[:, None] > 1e-8, m / np.where(norms > 0, norms, 1.0)[:, None], -1.0)
         assert np.allclose(out, want, rtol=1e-14, atol=0)
         assert (out[5] == -1.0).all()
+    # A NaN norm is not <= eps (linalg/detail/normalize.cuh:52,120): the row is written, as NaN.
+    # Sums turn NaN with one NaN element; the NaN-ignoring max does not, so that row is divided
+    # by the largest of its other elements.
+    mn = m.copy()
+    mn[2, 11] = np.nan
+    for main, red, fin, norms in cases:
+        d = api.make_desc(api.F64, api.F64, rows, cols, main_op=main, reduce_op=red, final_op=fin)
+        out = np.full(rows * cols, -1.0)
+        assert oracle.orc_row_normalize(C.byref(d), mn.ctypes.data, out.ctypes.data, 1e-8) == 0
+        out = out.reshape(rows, cols)
+        if red == api.RED_ADD:
+            assert np.isnan(out[2]).all()
+        else:
+            want2 = mn[2] / np.nanmax(np.abs(mn[2]))
+            assert np.isnan(out[2, 11]) and np.allclose(np.delete(out[2], 11), np.delete(want2, 11), rtol=1e-14)
+        assert np.allclose(out[3], m[3] / norms[3], rtol=1e-14)
 
 
 # ---- one-pass mean and variance -------------------------------------------------------
