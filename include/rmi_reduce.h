@@ -23,7 +23,7 @@
 extern "C" {
 #endif
 
-#define RMI_ABI_VERSION 1
+#define RMI_ABI_VERSION 2
 
 #if defined(__GNUC__) || defined(__clang__)
 #define RMI_API __attribute__((visibility("default")))
@@ -41,7 +41,9 @@ typedef enum rmi_status {
   RMI_ERR_WORKSPACE      = 5, /* workspace missing, too small or misaligned       */
   RMI_ERR_ALIGNMENT      = 6, /* in/out pointer not aligned to its element size   */
   RMI_ERR_LAUNCH         = 7, /* HIP reported an error at launch                  */
-  RMI_ERR_NO_DEVICE      = 8  /* no usable gfx950 device / code object            */
+  RMI_ERR_NO_DEVICE      = 8, /* no usable gfx950 device / code object            */
+  RMI_ERR_SCRATCH_LIMIT  = 9  /* rmi_reduce_noalloc: the plan needs more scratch
+                                 than RMI_NOALLOC_SCRATCH_BYTES                   */
 } rmi_status;
 
 /* ---- element types ---------------------------------------------------- */
@@ -214,6 +216,26 @@ RMI_API int rmi_reduce(const rmi_reduce_desc* desc,
                void* workspace,
                size_t workspace_bytes,
                void* stream);
+
+/* rmi_reduce for callers that cannot allocate device memory and have no workspace to
+ * pass: code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc.  It has no counterpart in the reference (whose Thick plan allocates an
+ * rmm::device_uvector inside the call, linalg/detail/coalesced_reduction-inl.cuh:560).
+ * Same descriptor, same kernels, same results bit for bit as rmi_reduce; the partials of
+ * two-pass plans go to a buffer of RMI_NOALLOC_SCRATCH_BYTES bytes that the library keeps
+ * in every GPU it runs on for the life of the process (a static device array; its address
+ * is looked up once per device, at the first call made with that device current: make
+ * that first call outside stream capture).  The call itself allocates and frees nothing.
+ * A descriptor whose plan needs more scratch (rmi_reduce_workspace_bytes(desc) >
+ * RMI_NOALLOC_SCRATCH_BYTES) is refused with RMI_ERR_SCRATCH_LIMIT and nothing is
+ * launched.  All calls on one GPU share that GPU's buffer: calls that may run at the same
+ * time (different streams, or branches of one graph) race on it; order them on one stream.
+ * Nothing in the buffer has to start at zero: every partial is written before it is read. */
+#define RMI_NOALLOC_SCRATCH_BYTES ((size_t)4 << 20)
+RMI_API int rmi_reduce_noalloc(const rmi_reduce_desc* desc,
+                               const void* in,
+                               void* out,
+                               void* stream);
 
 /* Whole-array map + reduce to one scalar: replaces detail::mapThenReduceImpl
  * (linalg/detail/map_then_reduce.cuh:72-95) behind mapThenSumReduce /

@@ -13,7 +13,9 @@ LIB_PATH = Path(__file__).resolve().parent / "lib" / "libraft_amd.so"
 
 # rmi_status
 OK, ERR_NULL, ERR_BAD_ENUM, ERR_BAD_SHAPE, ERR_UNSUPPORTED, ERR_WORKSPACE, ERR_ALIGNMENT, \
-    ERR_LAUNCH, ERR_NO_DEVICE = range(9)
+    ERR_LAUNCH, ERR_NO_DEVICE, ERR_SCRATCH_LIMIT = range(10)
+ABI_VERSION = 2
+NOALLOC_SCRATCH_BYTES = 4 << 20
 
 # rmi_dtype
 I8, U8, I32, I64, F16, BF16, F32, F64, KVP_I32_F32, KVP_I32_F64, KVP_I64_F32, KVP_I64_F64 = range(12)
@@ -74,6 +76,7 @@ SYMBOLS = {
     "rmi_reduce_workspace_bytes": (C.c_size_t, [C.POINTER(ReduceDesc)]),
     "rmi_reduce": (C.c_int, [C.POINTER(ReduceDesc), C.c_void_p, C.c_void_p, C.c_void_p,
                              C.c_size_t, C.c_void_p]),
+    "rmi_reduce_noalloc": (C.c_int, [C.POINTER(ReduceDesc), C.c_void_p, C.c_void_p, C.c_void_p]),
     "rmi_map_reduce_workspace_bytes": (C.c_size_t, [C.POINTER(ReduceDesc), C.c_int64]),
     "rmi_row_normalize": (C.c_int, [C.POINTER(ReduceDesc), C.c_void_p, C.c_void_p, C.c_double,
                                     C.c_void_p]),

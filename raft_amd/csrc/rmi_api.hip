@@ -4,8 +4,37 @@
 
 #include "rmi_launch.hpp"
 
+// Scratch of rmi_reduce_noalloc: partials of two-pass plans, for callers that can neither
+// allocate nor pass a workspace.  One copy per GPU, at its own address, for the life of the
+// process.  In host code this name is only a handle for hipGetSymbolAddress, never a device
+// address: kernels get the looked-up pointer as an argument.
+static __device__ __align__(256) unsigned char scratch[RMI_NOALLOC_SCRATCH_BYTES];
+
 namespace rmi {
 namespace {
+
+// Device address of `scratch` on the current device, looked up once per device.
+constexpr int kMaxDevices = 64;
+std::atomic<void*> scratch_ptr[kMaxDevices];
+
+int scratch_of_current_device(void** out)
+{
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    (void)hipGetLastError();
+    return RMI_ERR_NO_DEVICE;
+  }
+  void* p = scratch_ptr[dev].load(std::memory_order_acquire);
+  if (p == nullptr) {
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || p == nullptr) {
+      (void)hipGetLastError();
+      return RMI_ERR_NO_DEVICE;
+    }
+    scratch_ptr[dev].store(p, std::memory_order_release);
+  }
+  *out = p;
+  return RMI_OK;
+}
 
 // CU count of the current device, queried once per process.  Without a
 // visible device the MI355X figure is assumed so that planning works on a
@@ -57,17 +86,16 @@ int plan_for(const rmi_reduce_desc* desc, PlanX& pl, PolicyKey& key, const void*
   return make_plan(*desc, key, acc_bytes, cu_count(), pl, reinterpret_cast<uintptr_t>(in) % 128);
 }
 
-int reduce_impl(const rmi_reduce_desc& d,
-                const void* in,
-                void* out,
-                void* ws,
-                size_t ws_bytes,
-                void* stream)
+// Launches the planned reduction: pointer checks, epilogue set-up, kernel launch.
+int reduce_planned(const rmi_reduce_desc& d,
+                   const PlanX& pl,
+                   const PolicyKey& key,
+                   const void* in,
+                   void* out,
+                   void* ws,
+                   size_t ws_bytes,
+                   void* stream)
 {
-  PlanX pl;
-  PolicyKey key;
-  int rc = plan_for(&d, pl, key, in);
-  if (rc != RMI_OK) return rc;
   if (pl.n_out == 0) return RMI_OK;
   if (out == nullptr) return RMI_ERR_NULL;
   if (pl.len > 0 && in == nullptr) return RMI_ERR_NULL;
@@ -104,6 +132,20 @@ int reduce_impl(const rmi_reduce_desc& d,
   pr.epi.plain         = (!d.inplace && simple_final && natural_out) ? 1 : 0;
   pr.epi.out_aligned16 = aligned(out, 16) ? 1 : 0;
   return lookup(key)(pl, pr, static_cast<hipStream_t>(stream));
+}
+
+int reduce_impl(const rmi_reduce_desc& d,
+                const void* in,
+                void* out,
+                void* ws,
+                size_t ws_bytes,
+                void* stream)
+{
+  PlanX pl;
+  PolicyKey key;
+  const int rc = plan_for(&d, pl, key, in);
+  if (rc != RMI_OK) return rc;
+  return reduce_planned(d, pl, key, in, out, ws, ws_bytes, stream);
 }
 
 // map_reduce is a one-row reduction over the contiguous dimension.
@@ -166,6 +208,9 @@ const char* rmi_status_string(int status)
     case RMI_ERR_ALIGNMENT: return "pointer is not aligned to its element type";
     case RMI_ERR_LAUNCH: return "HIP reported an error at kernel launch";
     case RMI_ERR_NO_DEVICE: return "no usable gfx950 device";
+    case RMI_ERR_SCRATCH_LIMIT:
+      return "the plan needs more scratch than the library's static buffer holds "
+             "(RMI_NOALLOC_SCRATCH_BYTES); use rmi_reduce with a workspace";
     default: return "unknown status";
   }
 }
@@ -203,6 +248,22 @@ int rmi_reduce(const rmi_reduce_desc* desc,
 {
   if (desc == nullptr) return RMI_ERR_NULL;
   return rmi::reduce_impl(*desc, in, out, workspace, workspace_bytes, stream);
+}
+
+int rmi_reduce_noalloc(const rmi_reduce_desc* desc, const void* in, void* out, void* stream)
+{
+  if (desc == nullptr) return RMI_ERR_NULL;
+  rmi::PlanX pl;
+  rmi::PolicyKey key;
+  int rc = rmi::plan_for(desc, pl, key, in);
+  if (rc != RMI_OK) return rc;
+  if (pl.ws_bytes > RMI_NOALLOC_SCRATCH_BYTES) return RMI_ERR_SCRATCH_LIMIT;
+  // looked up at every device's first call, whether or not this plan needs scratch, so
+  // that "the first call" is the only one that does more than launch
+  void* ws = nullptr;
+  rc       = rmi::scratch_of_current_device(&ws);
+  if (rc != RMI_OK) return rc;
+  return rmi::reduce_planned(*desc, pl, key, in, out, ws, RMI_NOALLOC_SCRATCH_BYTES, stream);
 }
 
 size_t rmi_map_reduce_workspace_bytes(const rmi_reduce_desc* desc, int64_t len)

@@ -20,7 +20,7 @@ def test_library_exports_every_declared_symbol():
     lib = api.load()
     for name in declared:
         assert getattr(lib, name) is not None
-    assert lib.rmi_abi_version() == 1
+    assert lib.rmi_abi_version() == api.ABI_VERSION
 
 
 def test_struct_layouts_match_the_header(tmp_path):
@@ -53,8 +53,8 @@ def test_struct_layouts_match_the_header(tmp_path):
 
 def test_status_strings():
     lib = api.load()
-    seen = {lib.rmi_status_string(i).decode() for i in range(9)}
-    assert len(seen) == 9 and "ok" in seen
+    seen = {lib.rmi_status_string(i).decode() for i in range(10)}
+    assert len(seen) == 10 and "ok" in seen
     assert lib.rmi_status_string(1234).decode() == "unknown status"
 
 
