@@ -139,7 +139,7 @@ def main():
                       seed=5, rows=4096, cols=16384, in_dt=api.I8, out_dt=api.I64, kw={}),
         "cfg5b": dict(desc="row sum int8->int64 16777216x8", make=lambda s: mk_int8(16777216, 8, s),
                       seed=6, rows=16777216, cols=8, in_dt=api.I8, out_dt=api.I64, kw={}),
-        "cfg5c": dict(desc="row sum bf16->fp32 8x4194304 (split rows, two passes)",
+        "cfg5c": dict(desc="row sum bf16->fp32 8x4194304 (split rows, last workgroup of a row folds)",
                       make=lambda s: mk_bf16(8, 4194304, s), seed=7, rows=8, cols=4194304,
                       in_dt=api.BF16, out_dt=api.F32, kw={}),
     }
@@ -178,7 +178,9 @@ def main():
         descs = []
         aux = []
         for i in range(nbuf):
-            d = api.make_desc(w["in_dt"], w["out_dt"], w["rows"], w["cols"], **kw)
+            # the workspace below is zero-filled once and then only used by the library
+            d = api.make_desc(w["in_dt"], w["out_dt"], w["rows"], w["cols"],
+                              flags=api.FLAG_WORKSPACE_ZEROED, **kw)
             if w.get("needs_mean"):
                 m = bufs[i].view(w["rows"], w["cols"]).mean(dim=0, dtype=torch.float64).to(torch.float32)
                 aux.append(m)
@@ -186,7 +188,7 @@ def main():
             descs.append(d)
         plan = api.plan_query(descs[0])
         ws_bytes = lib.rmi_reduce_workspace_bytes(C.byref(descs[0]))
-        ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=devc)
+        ws = torch.zeros(max(ws_bytes, 16), dtype=torch.uint8, device=devc)
         wsp = ws.data_ptr()
         in_ptrs = [b.data_ptr() for b in bufs]
         out_ptrs = [o.data_ptr() for o in outs]

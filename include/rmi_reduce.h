@@ -148,8 +148,20 @@ typedef struct rmi_reduce_desc {
   const void* final_aux; /* device vector (out_dtype, one per output) read by
                             VAR/STDDEV (the mean); NULL otherwise            */
   int32_t plan_hint;   /* rmi_plan_kind to force, or 0 = choose by shape      */
-  int32_t reserved;    /* must be 0                                           */
+  int32_t flags;       /* RMI_FLAG_* bits; unknown bits are refused           */
 } rmi_reduce_desc;
+
+/* The caller promises that the first RMI_WORKSPACE_TICKET_BYTES bytes of the workspace passed
+ * with this descriptor were zero when the workspace was first handed to this library and
+ * have only been written by this library since.  Rows split over several workgroups are
+ * then reduced in ONE launch: every workgroup takes a ticket for its row (counters in that
+ * area, one per 16 workgroups of a row plus one per row, each on a 128-byte line of its
+ * own), the last one to arrive folds the row's partials in index order (results stay
+ * bitwise repeatable and equal to the two-launch plan's) and every counter wraps back to
+ * zero, so the area is zero again when the call has run.  Without the flag the workspace
+ * needs no initialisation and such rows take a second, folding launch. */
+#define RMI_FLAG_WORKSPACE_ZEROED 1
+#define RMI_WORKSPACE_TICKET_BYTES 65536
 
 /* ---- launch plans ------------------------------------------------------ */
 typedef enum rmi_plan_kind {
@@ -207,9 +219,10 @@ RMI_API size_t rmi_reduce_workspace_bytes(const rmi_reduce_desc* desc);
  * and detail::stridedReduction (linalg/detail/strided_reduction.cuh:129-196).
  * `in`: n_rows*n_cols elements, contiguous in `layout`.  `out`: one element per
  * output.  `workspace`: at least rmi_reduce_workspace_bytes(desc) bytes, 16-byte
- * aligned, may be NULL when that is 0; its contents need no initialisation and
- * are undefined afterwards.  Calls that share a workspace must be ordered on
- * one stream. */
+ * aligned, may be NULL when that is 0; its contents need no initialisation (unless
+ * desc->flags says RMI_FLAG_WORKSPACE_ZEROED) and, past the first
+ * RMI_WORKSPACE_TICKET_BYTES bytes, are undefined afterwards.  Calls that share a
+ * workspace must be ordered on one stream. */
 RMI_API int rmi_reduce(const rmi_reduce_desc* desc,
                const void* in,
                void* out,
@@ -230,7 +243,9 @@ RMI_API int rmi_reduce(const rmi_reduce_desc* desc,
  * RMI_NOALLOC_SCRATCH_BYTES) is refused with RMI_ERR_SCRATCH_LIMIT and nothing is
  * launched.  All calls on one GPU share that GPU's buffer: calls that may run at the same
  * time (different streams, or branches of one graph) race on it; order them on one stream.
- * Nothing in the buffer has to start at zero: every partial is written before it is read. */
+ * The buffer's ticket words (see RMI_FLAG_WORKSPACE_ZEROED, which this entry point always
+ * applies) are zero when the library is loaded and every launch leaves them zero; nothing
+ * else in it has to start at zero: every partial is written before it is read. */
 #define RMI_NOALLOC_SCRATCH_BYTES ((size_t)4 << 20)
 RMI_API int rmi_reduce_noalloc(const rmi_reduce_desc* desc,
                                const void* in,

@@ -16,6 +16,8 @@ OK, ERR_NULL, ERR_BAD_ENUM, ERR_BAD_SHAPE, ERR_UNSUPPORTED, ERR_WORKSPACE, ERR_A
     ERR_LAUNCH, ERR_NO_DEVICE, ERR_SCRATCH_LIMIT = range(10)
 ABI_VERSION = 2
 NOALLOC_SCRATCH_BYTES = 4 << 20
+FLAG_WORKSPACE_ZEROED = 1
+WORKSPACE_TICKET_BYTES = 65536
 
 # rmi_dtype
 I8, U8, I32, I64, F16, BF16, F32, F64, KVP_I32_F32, KVP_I32_F64, KVP_I64_F32, KVP_I64_F64 = range(12)
@@ -54,7 +56,7 @@ class ReduceDesc(C.Structure):
         ("init", Scalar),
         ("final_scalar", C.c_double), ("final_scalar2", C.c_double),
         ("final_aux", C.c_void_p),
-        ("plan_hint", C.c_int32), ("reserved", C.c_int32),
+        ("plan_hint", C.c_int32), ("flags", C.c_int32),
     ]
 
 
@@ -114,7 +116,7 @@ def status_string(code: int) -> str:
 def make_desc(in_dtype, out_dtype, n_rows, n_cols, *, layout=ROW_MAJOR, apply=ALONG_ROWS,
               main_op=MAIN_IDENTITY, reduce_op=RED_ADD, final_op=FIN_IDENTITY, inplace=False,
               init_f=0.0, init_i=0, final_scalar=0.0, final_scalar2=0.0, final_aux=None,
-              plan_hint=PLAN_AUTO) -> ReduceDesc:
+              plan_hint=PLAN_AUTO, flags=0) -> ReduceDesc:
     d = ReduceDesc()
     d.in_dtype, d.out_dtype = in_dtype, out_dtype
     d.layout, d.apply = layout, apply
@@ -125,7 +127,7 @@ def make_desc(in_dtype, out_dtype, n_rows, n_cols, *, layout=ROW_MAJOR, apply=AL
     d.final_scalar, d.final_scalar2 = float(final_scalar), float(final_scalar2)
     d.final_aux = final_aux
     d.plan_hint = plan_hint
-    d.reserved = 0
+    d.flags = flags
     return d
 
 

@@ -9,6 +9,12 @@
 //   Argmin            cpp/bench/prims/matrix/argmin.cu:55-60
 // One line per case: name, shape, mean time per call, algorithmic GB/s.
 //
+// copy_roof (no counterpart in the reference) measures what this GPU sustains when a kernel
+// writes as many bytes as it reads: a plain streaming copy swept over loads in flight per
+// lane, workgroups per CU (one-shot grid or persistent), and non-temporal loads / stores, at
+// 134 MB + 134 MB and 512 MB + 512 MB, over rotating buffers.  It is the roof that the
+// shapes with 1:1 traffic (row_normalize, row sums of 8-byte rows into int64) are held to.
+//
 // usage: prims_bench [--filter substring] [--min-iters N] [--max-bytes B] [--no-flush]
 #include <raft/core/device_mdarray.hpp>
 #include <raft/core/device_mdspan.hpp>
@@ -323,6 +329,120 @@ void bench_mat_vec_op(Harness& h)
   }
 }
 
+// ---- copy roof ------------------------------------------------------------------------
+typedef unsigned u32x4_t __attribute__((ext_vector_type(4)));
+
+template <int U, bool NT_LD, bool NT_ST, bool PERSIST>
+__global__ __launch_bounds__(256) void stream_copy(const u32x4_t* __restrict__ in,
+                                                   u32x4_t* __restrict__ out, size_t nvec)
+{
+  // nvec is a multiple of 256 * U: no tails, the copy's own best case
+  const size_t step = (size_t)gridDim.x * 256 * U;
+  for (size_t base = (size_t)blockIdx.x * 256 * U; base < nvec; base += step) {
+    u32x4_t x[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const u32x4_t* p = in + base + (size_t)u * 256 + threadIdx.x;
+      x[u]             = NT_LD ? __builtin_nontemporal_load(p) : *p;
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      u32x4_t* q = out + base + (size_t)u * 256 + threadIdx.x;
+      if (NT_ST)
+        __builtin_nontemporal_store(x[u], q);
+      else
+        *q = x[u];
+    }
+    if (!PERSIST) break;
+  }
+}
+
+template <int U, bool NT_LD, bool NT_ST>
+void copy_roof_case(hipStream_t s, int n_cu, size_t bytes, std::vector<void*>& src,
+                    std::vector<void*>& dst, hipEvent_t e0, hipEvent_t e1, double& best,
+                    std::string& best_name)
+{
+  const size_t nvec = bytes / 16;
+  for (int per_cu : {0, 2, 4, 8, 16}) {  // 0: one workgroup per 256 * U vectors
+    const size_t grid = per_cu == 0 ? nvec / (256 * U) : (size_t)n_cu * per_cu;
+    auto launch = [&](int i) {
+      const u32x4_t* a = static_cast<const u32x4_t*>(src[i % src.size()]);
+      u32x4_t* b       = static_cast<u32x4_t*>(dst[i % dst.size()]);
+      if (per_cu == 0)
+        stream_copy<U, NT_LD, NT_ST, false><<<dim3((unsigned)grid), 256, 0, s>>>(a, b, nvec);
+      else
+        stream_copy<U, NT_LD, NT_ST, true><<<dim3((unsigned)grid), 256, 0, s>>>(a, b, nvec);
+    };
+    const int reps = 40;
+    for (int i = 0; i < 5; ++i)
+      launch(i);
+    RAFT_HIP_TRY(hipEventRecord(e0, s));
+    for (int i = 0; i < reps; ++i)
+      launch(i);
+    RAFT_HIP_TRY(hipEventRecord(e1, s));
+    RAFT_HIP_TRY(hipEventSynchronize(e1));
+    float ms = 0.f;
+    RAFT_HIP_TRY(hipEventElapsedTime(&ms, e0, e1));
+    const double us   = ms * 1e3 / reps;
+    const double gbps = 2.0 * bytes / (us * 1e-6) / 1e9;
+    char name[160];
+    std::snprintf(name, sizeof name, "loads=%d nt_load=%d nt_store=%d %s", U, (int)NT_LD, (int)NT_ST,
+                  per_cu == 0 ? "one-shot" : (std::to_string(per_cu) + " wg/cu").c_str());
+    std::printf("%-34s %-22s %10.2f us %9.1f GB/s  %s\n", "copy_roof",
+                (std::to_string(bytes >> 20) + "MiB+" + std::to_string(bytes >> 20) + "MiB").c_str(), us,
+                gbps, name);
+    if (gbps > best) best = gbps, best_name = name;
+  }
+}
+
+void bench_copy_roof(Harness& h)
+{
+  if (!h.wanted("copy_roof")) return;
+  int n_cu = 256;
+  RAFT_HIP_TRY(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, 0));
+  hipEvent_t e0, e1;
+  RAFT_HIP_TRY(hipEventCreate(&e0));
+  RAFT_HIP_TRY(hipEventCreate(&e1));
+  for (size_t bytes : {(size_t)128 << 20, (size_t)512 << 20}) {
+    // enough source / destination pairs that a buffer is long out of the 256 MB memory-side
+    // cache when its turn comes again
+    const int nbuf = bytes >= ((size_t)512 << 20) ? 3 : 6;
+    std::vector<void*> src(nbuf), dst(nbuf);
+    for (int i = 0; i < nbuf; ++i) {
+      RAFT_HIP_TRY(hipMalloc(&src[i], bytes));
+      RAFT_HIP_TRY(hipMalloc(&dst[i], bytes));
+      fill_words<<<2048, 256, 0, h.stream()>>>(static_cast<unsigned*>(src[i]), bytes / 4, 17u + i);
+    }
+    RAFT_HIP_TRY(hipStreamSynchronize(h.stream()));
+    double best = 0.0;
+    std::string best_name;
+#define RAFT_COPY_ROOF(U)                                                                         \
+  copy_roof_case<U, false, false>(h.stream(), n_cu, bytes, src, dst, e0, e1, best, best_name);    \
+  copy_roof_case<U, true, false>(h.stream(), n_cu, bytes, src, dst, e0, e1, best, best_name);     \
+  copy_roof_case<U, false, true>(h.stream(), n_cu, bytes, src, dst, e0, e1, best, best_name);     \
+  copy_roof_case<U, true, true>(h.stream(), n_cu, bytes, src, dst, e0, e1, best, best_name)
+    RAFT_COPY_ROOF(1);
+    RAFT_COPY_ROOF(2);
+    RAFT_COPY_ROOF(4);
+    RAFT_COPY_ROOF(8);
+#undef RAFT_COPY_ROOF
+    std::printf("%-34s %-22s best %9.1f GB/s  %s\n", "copy_roof/best",
+                (std::to_string(bytes >> 20) + "MiB+" + std::to_string(bytes >> 20) + "MiB").c_str(), best,
+                best_name.c_str());
+    // correctness of the last copy, so the sweep cannot time a kernel that moved nothing
+    std::vector<unsigned> a(1024), b(1024);
+    RAFT_HIP_TRY(hipMemcpy(a.data(), static_cast<char*>(src[0]) + bytes - 4096, 4096, hipMemcpyDeviceToHost));
+    RAFT_HIP_TRY(hipMemcpy(b.data(), static_cast<char*>(dst[0]) + bytes - 4096, 4096, hipMemcpyDeviceToHost));
+    if (a != b) std::printf("copy_roof: COPY MISMATCH\n");
+    for (int i = 0; i < nbuf; ++i) {
+      (void)hipFree(src[i]);
+      (void)hipFree(dst[i]);
+    }
+  }
+  (void)hipEventDestroy(e0);
+  (void)hipEventDestroy(e1);
+}
+
 }  // namespace
 
 int main(int argc, char** argv)
@@ -362,5 +482,6 @@ int main(int argc, char** argv)
   bench_mat_vec_op<float, true>(h);
   bench_mat_vec_op<double, false>(h);
   bench_mat_vec_op<double, true>(h);
+  bench_copy_roof(h);
   return 0;
 }

@@ -83,7 +83,8 @@ int plan_for(const rmi_reduce_desc* desc, PlanX& pl, PolicyKey& key, const void*
   int rc        = classify(*desc, key, acc_bytes);
   if (rc != RMI_OK) return rc;
   if (lookup(key) == nullptr) return RMI_ERR_UNSUPPORTED;
-  return make_plan(*desc, key, acc_bytes, cu_count(), pl, reinterpret_cast<uintptr_t>(in) % 128);
+  rc = make_plan(*desc, key, acc_bytes, cu_count(), pl, reinterpret_cast<uintptr_t>(in) % 128);
+  return rc;
 }
 
 // Launches the planned reduction: pointer checks, epilogue set-up, kernel launch.
@@ -253,9 +254,12 @@ int rmi_reduce(const rmi_reduce_desc* desc,
 int rmi_reduce_noalloc(const rmi_reduce_desc* desc, const void* in, void* out, void* stream)
 {
   if (desc == nullptr) return RMI_ERR_NULL;
+  // the buffer's ticket words are zero from load time on and every launch leaves them zero
+  rmi_reduce_desc d = *desc;
+  d.flags |= RMI_FLAG_WORKSPACE_ZEROED;
   rmi::PlanX pl;
   rmi::PolicyKey key;
-  int rc = rmi::plan_for(desc, pl, key, in);
+  int rc = rmi::plan_for(&d, pl, key, in);
   if (rc != RMI_OK) return rc;
   if (pl.ws_bytes > RMI_NOALLOC_SCRATCH_BYTES) return RMI_ERR_SCRATCH_LIMIT;
   // looked up at every device's first call, whether or not this plan needs scratch, so
@@ -263,7 +267,7 @@ int rmi_reduce_noalloc(const rmi_reduce_desc* desc, const void* in, void* out, v
   void* ws = nullptr;
   rc       = rmi::scratch_of_current_device(&ws);
   if (rc != RMI_OK) return rc;
-  return rmi::reduce_planned(*desc, pl, key, in, out, ws, RMI_NOALLOC_SCRATCH_BYTES, stream);
+  return rmi::reduce_planned(d, pl, key, in, out, ws, RMI_NOALLOC_SCRATCH_BYTES, stream);
 }
 
 size_t rmi_map_reduce_workspace_bytes(const rmi_reduce_desc* desc, int64_t len)

@@ -428,47 +428,64 @@ struct PolI {
   {
     a = red<i64>(a, main_i64<MAIN>((i64)x));
   }
-  static __device__ __forceinline__ int32_t vec_i32(const u32x4& v)
+  // main_op of the four bytes of one word, folded in 32 bits (kNarrow inputs only)
+  static __device__ __forceinline__ int32_t word_i32(u32 w)
   {
     if constexpr (RED == RMI_RED_ADD && std::is_same_v<InT, int8_t> &&
                   (MAIN == RMI_MAIN_IDENTITY || MAIN == RMI_MAIN_SQ)) {
       // v_dot4_i32_i8: four signed byte products per instruction.
-      int32_t s = 0;
-#pragma unroll
-      for (int w = 0; w < 4; ++w) {
-        const int x = (int)v[w];
-        s = __builtin_amdgcn_sdot4(x, MAIN == RMI_MAIN_SQ ? x : 0x01010101, s, false);
-      }
-      return s;
+      const int x = (int)w;
+      return __builtin_amdgcn_sdot4(x, MAIN == RMI_MAIN_SQ ? x : 0x01010101, 0, false);
     } else if constexpr (RED == RMI_RED_ADD && std::is_same_v<InT, uint8_t> &&
                          (MAIN == RMI_MAIN_IDENTITY || MAIN == RMI_MAIN_ABS ||
                           MAIN == RMI_MAIN_SQ)) {
-      int32_t s = 0;
-#pragma unroll
-      for (int w = 0; w < 4; ++w) {
-        const u32 x = v[w];
-        s = (int32_t)__builtin_amdgcn_udot4(x, MAIN == RMI_MAIN_SQ ? x : 0x01010101u, (u32)s, false);
-      }
-      return s;
+      return (int32_t)__builtin_amdgcn_udot4(w, MAIN == RMI_MAIN_SQ ? w : 0x01010101u, 0u, false);
     } else if constexpr (RED == RMI_RED_ADD && std::is_same_v<InT, int8_t> &&
                          MAIN == RMI_MAIN_ABS) {
       // |x| summed with v_sad_u8 after biasing signed bytes to unsigned.
-      u32 s = 0;
-#pragma unroll
-      for (int w = 0; w < 4; ++w)
-        s = __builtin_amdgcn_sad_u8(v[w] ^ 0x80808080u, 0x80808080u, s);
-      return (int32_t)s;
+      return (int32_t)__builtin_amdgcn_sad_u8(w ^ 0x80808080u, 0x80808080u, 0u);
     } else {
-      int32_t t[VEC];
-      static_for<VEC>([&](auto j) { t[j] = main_i32<MAIN>(In<InT>::template get<j>(v)); });
-#pragma unroll
-      for (int w = VEC / 2; w >= 1; w /= 2) {
-#pragma unroll
-        for (int j = 0; j < w; ++j)
-          t[j] = red<int32_t>(t[j], t[j + w]);
-      }
-      return t[0];
+      int32_t t[4];
+      static_for<4>([&](auto j) {
+        if constexpr (std::is_same_v<InT, int8_t>)
+          t[j] = main_i32<MAIN>(__builtin_amdgcn_sbfe((int)w, 8 * j, 8));
+        else
+          t[j] = main_i32<MAIN>((int32_t)__builtin_amdgcn_ubfe(w, 8 * j, 8));
+      });
+      return red<int32_t>(red<int32_t>(t[0], t[1]), red<int32_t>(t[2], t[3]));
     }
+  }
+  static __device__ __forceinline__ int32_t vec_i32(const u32x4& v)
+  {
+    if constexpr (RED == RMI_RED_ADD) {
+      // dot products chain their accumulator: one instruction per word
+      if constexpr (std::is_same_v<InT, int8_t> && (MAIN == RMI_MAIN_IDENTITY || MAIN == RMI_MAIN_SQ)) {
+        int32_t s = 0;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          const int x = (int)v[w];
+          s = __builtin_amdgcn_sdot4(x, MAIN == RMI_MAIN_SQ ? x : 0x01010101, s, false);
+        }
+        return s;
+      } else if constexpr (std::is_same_v<InT, uint8_t> &&
+                           (MAIN == RMI_MAIN_IDENTITY || MAIN == RMI_MAIN_ABS || MAIN == RMI_MAIN_SQ)) {
+        int32_t s = 0;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          const u32 x = v[w];
+          s = (int32_t)__builtin_amdgcn_udot4(x, MAIN == RMI_MAIN_SQ ? x : 0x01010101u, (u32)s, false);
+        }
+        return s;
+      } else if constexpr (std::is_same_v<InT, int8_t> && MAIN == RMI_MAIN_ABS) {
+        u32 s = 0;
+#pragma unroll
+        for (int w = 0; w < 4; ++w)
+          s = __builtin_amdgcn_sad_u8(v[w] ^ 0x80808080u, 0x80808080u, s);
+        return (int32_t)s;
+      }
+    }
+    return red<int32_t>(red<int32_t>(word_i32(v[0]), word_i32(v[1])),
+                        red<int32_t>(word_i32(v[2]), word_i32(v[3])));
   }
   static __device__ __forceinline__ void push_vec(acc_t& a, const u32x4& v, i64)
   {

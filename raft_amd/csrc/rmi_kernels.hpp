@@ -26,6 +26,8 @@ constexpr int kColUnroll  = 4;    // rows per lane and tile in the column kernel
 constexpr int kStageBytes  = 4096 + 128 + 16;  // LDS staging area of one wave (row_wave_kernel)
 constexpr int kStageLoads  = 5;  // lane-loads that cover 4096 + 112 bytes
 constexpr int kTeamUnroll = 4;    // lane-loads per batch in the team-per-row kernel
+constexpr int kFan        = 16;   // split rows: workgroups per first-level ticket counter
+constexpr int kLineWords  = 32;   // a ticket counter has a 128-byte line to itself
 
 struct RowArgs {
   const void* in;
@@ -43,6 +45,10 @@ struct RowArgs {
   int R;           // row_short_kernel, any G: 64 / G rows per wave step
   u32 invG;        // row_short_kernel, any G: 65536 / G + 1, so that (x * invG) >> 16 == x / G
   u32 invR;        // likewise for R                              for every x < 64
+  u32* ticket;     // row_block_kernel, B > 1: zeroed ticket counters, each alone on a 128-byte
+                   // line; the workgroup that takes a row's last ticket folds its partials
+                   // (nullptr: a second launch does)
+  int LB;          // ... with LB lanes (a power of two <= 64), as fold_kernel would
   Epilogue epi;
 };
 
@@ -181,10 +187,16 @@ __device__ __forceinline__ typename P::acc_t bperm_acc(const typename P::acc_t& 
   return r;
 }
 
+// policies that fold the four 8-bit elements of a word with one instruction (P::kNarrow)
+template <class P, class = void>
+struct lanes_by_words : std::false_type {};
+template <class P>
+struct lanes_by_words<P, std::void_t<decltype(P::kNarrow)>> : std::bool_constant<P::kNarrow> {};
+
 // ---------------------------------------------------------------------------
-// K rows per 16-byte vector (row length VEC/K elements).  Lane-local.
+// K rows per 16-byte vector (row length VEC/K elements).  Lane-local; U lane-loads per lane.
 // ---------------------------------------------------------------------------
-template <class P, int K>
+template <class P, int K, int U = kUnroll>
 __global__ __launch_bounds__(kBlock) void row_lanes_kernel(RowArgs a)
 {
   using in_t      = typename P::in_t;
@@ -193,28 +205,39 @@ __global__ __launch_bounds__(kBlock) void row_lanes_kernel(RowArgs a)
   const i64 nfull = a.n_out / K; // vectors made only of whole, in-range rows
   const char* inb = static_cast<const char*>(a.in);
 
-  u32x4 x[kUnroll];
+  u32x4 x[U];
   if (nfull > 0) {
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
+    for (int u = 0; u < U; ++u) {
       // consecutive lanes take consecutive vectors within each unroll slot; the loads are
       // unconditional (a vector past the end re-reads the last one): loads under a lane
       // mask make the compiler wait for each of them in turn
-      const i64 v = ((i64)blockIdx.x * kUnroll + u) * kBlock + threadIdx.x;
+      const i64 v = ((i64)blockIdx.x * U + u) * kBlock + threadIdx.x;
       x[u]        = load16(inb + (v < nfull ? v : nfull - 1) * 16);
     }
   }
 #pragma unroll
-  for (int u = 0; u < kUnroll; ++u) {
-    const i64 v = ((i64)blockIdx.x * kUnroll + u) * kBlock + threadIdx.x;
+  for (int u = 0; u < U; ++u) {
+    const i64 v = ((i64)blockIdx.x * U + u) * kBlock + threadIdx.x;
     if (v < nfull) {
       acc_t acc[K];
-      static_for<K>([&](auto r) {
-        acc[r] = P::neutral();
-        static_for<D>([&](auto j) {
-          P::push(acc[r], In<in_t>::template get<r * D + j>(x[u]), (i64)j);
+      if constexpr (lanes_by_words<P>::value && D % 4 == 0) {
+        // rows of whole words of 8-bit elements: a dot-product instruction per word
+        static_for<K>([&](auto r) {
+          int32_t t = P::word_i32(x[u][r * (D / 4)]);
+          static_for<D / 4 - 1>([&](auto w) {
+            t = P::template red<int32_t>(t, P::word_i32(x[u][r * (D / 4) + w + 1]));
+          });
+          acc[r] = (acc_t)t;
         });
-      });
+      } else {
+        static_for<K>([&](auto r) {
+          acc[r] = P::neutral();
+          static_for<D>([&](auto j) {
+            P::push(acc[r], In<in_t>::template get<r * D + j>(x[u]), (i64)j);
+          });
+        });
+      }
       finish_run<P, K>(a.epi, v * K, acc);
     }
   }
@@ -466,11 +489,50 @@ __global__ __launch_bounds__(kBlock) void row_wave_kernel(RowArgs a)
   if (c == 0 && row < a.n_out) finish<P>(a.epi, row, acc);
 }
 
+// Partials that another workgroup of the SAME launch reads (single-launch split rows) are
+// written and read past the caches, word by word as device-scope relaxed atomics
+// (global_store / global_load with sc1): the eight L2 caches of the chip are not coherent
+// with each other inside a launch, and making them so with device-scope fences costs a
+// write-back and an invalidation of a whole L2 per workgroup (2048 workgroups: 100 us).
+template <class T>
+__device__ __forceinline__ void store_coherent(T* p, const T& v)
+{
+  static_assert(sizeof(T) % 8 == 0, "accumulators are moved in 8-byte words");
+  constexpr int NW = sizeof(T) / 8;
+  u64 w[NW];
+  __builtin_memcpy(w, &v, sizeof(T));
+#pragma unroll
+  for (int i = 0; i < NW; ++i)
+    __hip_atomic_store(reinterpret_cast<u64*>(p) + i, w[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+template <class T>
+__device__ __forceinline__ T load_coherent(const T* p)
+{
+  static_assert(sizeof(T) % 8 == 0, "accumulators are moved in 8-byte words");
+  constexpr int NW = sizeof(T) / 8;
+  u64 w[NW];
+#pragma unroll
+  for (int i = 0; i < NW; ++i)
+    w[i] = __hip_atomic_load(reinterpret_cast<const u64*>(p) + i, __ATOMIC_RELAXED,
+                             __HIP_MEMORY_SCOPE_AGENT);
+  T v;
+  __builtin_memcpy(&v, w, sizeof(T));
+  return v;
+}
+
+template <class P, bool COHERENT = false>
+__device__ __forceinline__ typename P::acc_t fold_lane(const typename P::acc_t* p, int B, int LB,
+                                                       int lb);
+
 // ---------------------------------------------------------------------------
 // Teams of T = 64 << logT threads (1..16 waves); each team sweeps one chunk of
 // one row in batches of kTeamUnroll loads per lane.  A workgroup holds
 // blockDim.x / T teams.  B chunks per row: B == 1 writes outputs, B > 1 writes
-// partials for the second pass.
+// partials.  Those are folded by a second launch, or, when the caller brought zeroed
+// ticket words (one per row), by the workgroup that finishes a row last: it learns that
+// from the ticket it takes, reads the B partials in index order like the second launch
+// would, and its ticket wraps the word back to zero.  The order of the fold does not
+// depend on which workgroup does it, so results are bitwise repeatable.
 // ---------------------------------------------------------------------------
 template <class P, bool VEC16>
 __global__ __launch_bounds__(1024) void row_block_kernel(RowArgs a)
@@ -569,8 +631,48 @@ __global__ __launch_bounds__(1024) void row_block_kernel(RowArgs a)
   if (t == 0 && live) {
     if (a.B == 1) {
       finish<P>(a.epi, row, acc);
+    } else if (a.ticket != nullptr) {
+      store_coherent(static_cast<acc_t*>(a.partial) + row * a.B + b, acc);
     } else {
       static_cast<acc_t*>(a.partial)[row * a.B + b] = acc;
+    }
+  }
+  if (a.B > 1 && a.ticket != nullptr) {  // one team per workgroup here (T == blockDim.x)
+    __shared__ int last_of_row;
+    if (threadIdx.x == 0) {
+      int last = 0;
+      if (live) {
+        // Counters wrap to zero with their last ticket (atomicInc), so the area is clean for
+        // the next call.  Up to kFan chunks: one counter per row.  More: chunks count in
+        // groups of kFan, the last of a group counts for the row.  Line 0 of a row's lines
+        // is the row's counter, lines 1.. its groups'.
+        constexpr int kLine = kLineWords;
+        // the partial's stores (past the caches) have completed before the ticket is taken:
+        // a release at workgroup scope waits for them without writing any cache back
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        if (a.B <= kFan) {
+          last = atomicInc(a.ticket + row * kLine, (u32)a.B - 1) == (u32)a.B - 1;
+        } else {
+          const int groups = (a.B + kFan - 1) / kFan;
+          const int g      = b / kFan;
+          const int gsize  = g == groups - 1 ? a.B - g * kFan : kFan;
+          u32* lines       = a.ticket + row * (groups + 1) * kLine;
+          if (atomicInc(lines + (1 + g) * kLine, (u32)gsize - 1) == (u32)gsize - 1)
+            last = atomicInc(lines, (u32)groups - 1) == (u32)groups - 1;
+        }
+      }
+      last_of_row = last;
+    }
+    __syncthreads();
+    if (last_of_row && threadIdx.x < kWave) {
+      // every other workgroup's ticket, and with it its partial, is at the memory side by now
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+      const int lane = threadIdx.x;
+      acc_t total    = P::neutral();
+      if (lane < a.LB)
+        total = fold_lane<P, true>(static_cast<const acc_t*>(a.partial) + row * a.B, a.B, a.LB, lane);
+      group_allreduce<P>(total, a.LB);
+      if (lane == 0) finish<P>(a.epi, row, total);
     }
   }
 }
@@ -763,6 +865,38 @@ __global__ __launch_bounds__(kBlock) void col_kernel(ColArgs a)
 }
 
 // ---------------------------------------------------------------------------
+// Lane `lb` of the LB lanes that fold the B partials of one output: partials lb, lb + LB, ...
+// in that order.  The caller combines the lanes with group_allreduce<P>(acc, LB).
+// ---------------------------------------------------------------------------
+template <class P, bool COHERENT>
+__device__ __forceinline__ typename P::acc_t fold_lane(const typename P::acc_t* p, int B, int LB,
+                                                       int lb)
+{
+  using acc_t = typename P::acc_t;
+  auto get    = [&](int i) {
+    if constexpr (COHERENT) {
+      return load_coherent(p + i);
+    } else {
+      return p[i];
+    }
+  };
+  acc_t acc = P::neutral();
+  int b     = lb;
+  for (; b + (kUnroll - 1) * LB < B; b += kUnroll * LB) {
+    acc_t x[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u)
+      x[u] = get(b + u * LB);
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u)
+      P::merge(acc, x[u]);
+  }
+  for (; b < B; b += LB)
+    P::merge(acc, get(b));
+  return acc;
+}
+
+// ---------------------------------------------------------------------------
 // Second pass: LB lanes fold the B partials of one output in a fixed order,
 // then the epilogue.  B == 0 writes final_op(init) (empty reductions).
 // ---------------------------------------------------------------------------
@@ -774,21 +908,7 @@ __global__ __launch_bounds__(kBlock) void fold_kernel(FoldArgs a)
   const i64 o    = gtid >> a.logLB;
   const int lb   = (int)(gtid & (a.LB - 1));
   acc_t acc      = P::neutral();
-  if (o < a.n_out) {
-    const acc_t* p = static_cast<const acc_t*>(a.partial) + o * a.B;
-    int b          = lb;
-    for (; b + (kUnroll - 1) * a.LB < a.B; b += kUnroll * a.LB) {
-      acc_t x[kUnroll];
-#pragma unroll
-      for (int u = 0; u < kUnroll; ++u)
-        x[u] = p[b + u * a.LB];
-#pragma unroll
-      for (int u = 0; u < kUnroll; ++u)
-        P::merge(acc, x[u]);
-    }
-    for (; b < a.B; b += a.LB)
-      P::merge(acc, p[b]);
-  }
+  if (o < a.n_out) acc = fold_lane<P>(static_cast<const acc_t*>(a.partial) + o * a.B, a.B, a.LB, lb);
   group_allreduce<P>(acc, a.LB);
   if (lb == 0 && o < a.n_out) finish<P>(a.epi, o, acc);
 }

@@ -19,14 +19,18 @@ struct Problem {
 
 using run_fn = int (*)(const PlanX&, const Problem&, hipStream_t);
 
+// partials start after the workspace's ticket words
+inline void* partials_of(void* ws) { return ws == nullptr ? nullptr : static_cast<char*>(ws) + kTicketBytes; }
+inline int fold_lanes(int B) { return B >= 64 ? 64 : pow2ceil(B < 1 ? 1 : B); }
+
 template <class P>
 int launch_fold(const PlanX& pl, const Problem& pr, int B, hipStream_t st)
 {
   FoldArgs f{};
-  f.partial = pr.ws;
+  f.partial = partials_of(pr.ws);
   f.n_out   = pl.n_out;
   f.B       = B;
-  f.LB      = B >= 64 ? 64 : pow2ceil(B < 1 ? 1 : B);
+  f.LB      = fold_lanes(B);
   f.logLB   = ilog2(f.LB);
   f.epi     = pr.epi;
   const int64_t threads = pl.n_out * f.LB;
@@ -40,8 +44,11 @@ template <class P, int K>
 int launch_lanes(const PlanX& pl, const RowArgs& a, hipStream_t st)
 {
   if constexpr (K <= P::VEC) {
-    hipLaunchKernelGGL(
-      (row_lanes_kernel<P, K>), dim3((unsigned)pl.grid_blocks), dim3(kBlock), 0, st, a);
+    const dim3 grid((unsigned)pl.grid_blocks);
+    if (pl.lanes_loads == 1)
+      hipLaunchKernelGGL((row_lanes_kernel<P, K, 1>), grid, dim3(kBlock), 0, st, a);
+    else
+      hipLaunchKernelGGL((row_lanes_kernel<P, K, kUnroll>), grid, dim3(kBlock), 0, st, a);
     return RMI_OK;
   } else {
     return RMI_ERR_UNSUPPORTED;
@@ -52,7 +59,8 @@ template <class P>
 int run(const PlanX& pl, const Problem& pr, hipStream_t st)
 {
   static_assert(kBlock == kPlanBlock && kUnroll == kPlanUnroll && kColUnroll == kPlanUnroll &&
-                  kTeamUnroll == kPlanTeamUnroll && kStageBytes == kStageBytesPerWave,
+                  kTeamUnroll == kPlanTeamUnroll && kStageBytes == kStageBytesPerWave &&
+                  kFan == kTicketFan && kLineWords * 4 == kTicketLineBytes,
                 "plan selector and kernels must agree on block size and unroll");
   int rc = RMI_OK;
   switch (pl.kind) {
@@ -65,7 +73,9 @@ int run(const PlanX& pl, const Problem& pr, hipStream_t st)
     case RMI_PLAN_ROW_SPLIT: {
       RowArgs a{};
       a.in      = pr.in;
-      a.partial = pr.ws;
+      a.partial = partials_of(pr.ws);
+      a.ticket  = pl.fused_fold ? static_cast<u32*>(pr.ws) : nullptr;
+      a.LB      = fold_lanes(pl.B);
       a.n_out   = pl.n_out;
       a.len     = pl.len;
       a.row_bytes = pl.row_bytes;
@@ -112,14 +122,14 @@ int run(const PlanX& pl, const Problem& pr, hipStream_t st)
           hipLaunchKernelGGL((row_block_kernel<P, true>), grid, block, lds, st, a);
         else
           hipLaunchKernelGGL((row_block_kernel<P, false>), grid, block, 0, st, a);
-        if (pl.kind == RMI_PLAN_ROW_SPLIT) rc = launch_fold<P>(pl, pr, pl.B, st);
+        if (pl.kind == RMI_PLAN_ROW_SPLIT && !pl.fused_fold) rc = launch_fold<P>(pl, pr, pl.B, st);
       }
       break;
     }
     case RMI_PLAN_COL_TILE: {
       ColArgs a{};
       a.in             = pr.in;
-      a.partial        = pr.ws;
+      a.partial        = partials_of(pr.ws);
       a.n_out          = pl.n_out;
       a.len            = pl.len;
       a.row_bytes      = pl.row_bytes;
@@ -166,6 +176,7 @@ struct NormPlan {
   int G        = 1;
   int logG     = 0;
   int L        = 4;  // wave kernel: lane-loads per lane and row
+  int tiles    = 1;  // wave kernel: rows per lane group and step
   int hold     = 4;  // team kernel: lane-loads held per thread
   int threads  = kBlock;
   int64_t grid = 0;
@@ -188,8 +199,19 @@ inline NormPlan make_norm_plan(int64_t n_rows, int64_t len, int elem_bytes)
     p.L    = nload <= 8 ? 1 : (nload <= 16 ? 2 : 4);
     p.G    = pow2ceil(ceildiv(nload, p.L));
     p.L    = (int)ceildiv(nload, (int64_t)p.G);  // no load instruction without a lane-load
-    p.logG = ilog2(p.G);
-    p.grid = ceildiv(n_rows, (int64_t)(kWave / p.G) * (kUnroll / p.L) * (kBlock / kWave));
+    p.logG  = ilog2(p.G);
+    p.tiles = kUnroll / p.L;
+    // Rows of 16, 32, 64 or 128 lane-loads: two loads per lane and ONE row per lane group and
+    // step (half the default's bytes in flight per lane, twice the workgroups) measured 2-3 %
+    // faster than four loads per lane or two rows per group on fp32, fp64 and bf16 rows
+    // (1M x 128 floats 167 -> 162 us; a streaming copy is fastest at one load per lane too).
+    if (p.vec16 && nload >= 16 && nload <= 128 && (nload & (nload - 1)) == 0) {
+      p.L     = 2;
+      p.G     = (int)(nload / 2);
+      p.logG  = ilog2(p.G);
+      p.tiles = 1;
+    }
+    p.grid = ceildiv(n_rows, (int64_t)(kWave / p.G) * p.tiles * (kBlock / kWave));
     // Lane-load counts that are not a power of two: one lane per lane-load and 64 / G whole
     // rows per wave step, so that every load and store instruction covers one contiguous
     // span (1M x 33 / 50 / 100 floats: 59 / 60 / 56 % -> 70 / 72 / 71 % of 8 TB/s in + out).
@@ -234,6 +256,7 @@ int run_normalize(const NormPlan& pl, const NormArgs& args, hipStream_t st)
   a.G        = pl.G;
   a.logG     = pl.logG;
   a.L        = pl.L;
+  a.tiles    = pl.tiles;
   a.invG     = 65536u / (unsigned)(pl.G > 0 ? pl.G : 1) + 1;
   if (pl.grid > 0x7fffffffLL) return RMI_ERR_BAD_SHAPE;
   const dim3 grid((unsigned)pl.grid);

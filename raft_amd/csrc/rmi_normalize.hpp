@@ -20,6 +20,7 @@ struct NormArgs {
   int tail;    // elements after the last whole vector
   int G;       // lanes per row (wave kernel)
   int logG;
+  int tiles;   // wave kernel: rows per lane group and step (L * tiles lane-loads in flight)
   int L;       // wave kernel: lane-loads per lane and row (1 to 4); 0: one per lane with
                // G = the row's lane-load count itself (not a power of two)
   u32 invG;    // L == 0: 65536 / G + 1, so that (lane * invG) >> 16 == lane / G
@@ -100,6 +101,32 @@ __device__ __forceinline__ void store16(void* p, const u32x4& v)
   }
 }
 
+// x / d for many x and one d, as the reference's element-wise division computes it, at three
+// instructions per element instead of the ten or more of a division: with r = RN(1 / d), the
+// quotient estimate q = RN(x * r) is corrected once with the exact residual, q' = RN(q + RN(x -
+// q * d) * r), which is the correctly rounded x / d (Markstein) as long as r and the residual
+// stay in the normal range.  A divisor outside [2^-100, 2^100] (fp32; 2^-900, 2^900 fp64), an
+// infinite or a NaN one takes the division itself.
+template <class T>
+struct Quot {
+  T d, r;
+  bool fast;
+  __device__ __forceinline__ explicit Quot(T divisor) : d(divisor), r((T)1 / divisor)
+  {
+    constexpr T lo = sizeof(T) == 4 ? (T)7.888609052210118e-31 : (T)1.183e-271;   // 2^-100, ~2^-900
+    constexpr T hi = sizeof(T) == 4 ? (T)1.2676506002282294e30 : (T)8.452e270;    // 2^100, ~2^900
+    fast = fabs(divisor) >= lo && fabs(divisor) <= hi;
+  }
+  __device__ __forceinline__ T operator()(T x) const
+  {
+    if (!fast) return x / d;
+    const T q  = x * r;
+    const T q2 = fma(fma(-q, d, x), r, q);
+    // an infinite x has no residual (inf - inf): its product with r already is the quotient
+    return q2 == q2 ? q2 : q;
+  }
+};
+
 // norm of a row from its folded accumulator, in the element's own arithmetic
 template <class P>
 __device__ __forceinline__ typename P::nat row_norm(const NormArgs& a, typename P::acc_t acc)
@@ -140,9 +167,10 @@ __device__ __forceinline__ void write_scaled(const NormArgs& a,
               Put<in_t>::st(o + decltype(j)::value, In<in_t>::template get<decltype(j)::value>(x) * inv);
           });
         } else {
+          const Quot<typename P::nat> quot(norm);
           static_for<P::VEC>([&](auto j) {
             if (decltype(j)::value >= first)
-              Put<in_t>::st(o + decltype(j)::value, In<in_t>::template get<decltype(j)::value>(x) / norm);
+              Put<in_t>::st(o + decltype(j)::value, quot(In<in_t>::template get<decltype(j)::value>(x)));
           });
         }
         return;
@@ -158,8 +186,9 @@ __device__ __forceinline__ void write_scaled(const NormArgs& a,
         Put<in_t>::template at<decltype(j)::value>(y, In<in_t>::template get<decltype(j)::value>(x) * inv);
       });
     } else {
+      const Quot<typename P::nat> quot(norm);
       static_for<P::VEC>([&](auto j) {
-        Put<in_t>::template at<decltype(j)::value>(y, In<in_t>::template get<decltype(j)::value>(x) / norm);
+        Put<in_t>::template at<decltype(j)::value>(y, quot(In<in_t>::template get<decltype(j)::value>(x)));
       });
     }
     store16<STREAM>(v < a.nvec ? orow + v * 16 : orow + (a.len - P::VEC) * (i64)sizeof(in_t), y);
@@ -171,12 +200,11 @@ __device__ __forceinline__ void write_scaled(const NormArgs& a,
 // G lanes of one wave per row, L lane-loads per lane and row, kUnroll / L rows per
 // lane group and step: kUnroll loads in flight per lane whatever the row length, and
 // the rows stay in registers from the reduction to the scaling.
-template <class P, bool VEC16, int L, bool STREAM>
+template <class P, bool VEC16, int L, int TILES, bool STREAM>
 __device__ __forceinline__ void normalize_wave_body(const NormArgs& a)
 {
   using acc_t         = typename P::acc_t;
   using H             = Held<P, VEC16>;
-  constexpr int TILES = kUnroll / L;
   const int lane      = threadIdx.x & (kWave - 1);
   const i64 wid       = (i64)blockIdx.x * (kBlock / kWave) + (threadIdx.x >> 6);
   const int G         = a.G;
@@ -185,7 +213,7 @@ __device__ __forceinline__ void normalize_wave_body(const NormArgs& a)
   const int g         = lane >> a.logG;
   const i64 nload     = a.nvec + (a.tail > 0 ? 1 : 0);
 
-  typename H::type x[kUnroll];
+  typename H::type x[L * TILES];
   i64 row[TILES];
 #pragma unroll
   for (int t = 0; t < TILES; ++t) {
@@ -291,13 +319,14 @@ __global__ __launch_bounds__(kBlock) void normalize_wave_kernel(NormArgs a)
     }
   }
   if (a.L == 1) {
-    normalize_wave_body<P, VEC16, 1, STREAM>(a);
+    normalize_wave_body<P, VEC16, 1, 4, STREAM>(a);
   } else if (a.L == 2) {
-    normalize_wave_body<P, VEC16, 2, STREAM>(a);
+    if (a.tiles == 1) normalize_wave_body<P, VEC16, 2, 1, STREAM>(a);
+    else normalize_wave_body<P, VEC16, 2, 2, STREAM>(a);
   } else if (a.L == 3) {
-    normalize_wave_body<P, VEC16, 3, STREAM>(a);
+    normalize_wave_body<P, VEC16, 3, 1, STREAM>(a);
   } else {
-    normalize_wave_body<P, VEC16, 4, STREAM>(a);
+    normalize_wave_body<P, VEC16, 4, 1, STREAM>(a);
   }
 }
 

@@ -91,10 +91,20 @@ template <>
 struct main_tag<identity_op> {
   static constexpr int value = RMI_MAIN_IDENTITY;
 };
+// cast_op<T> is the identity to the library (which widens every element into an f64 or
+// int64 accumulator anyway) only where the cast keeps the value: to a floating type, or
+// between integers without narrowing.  A cast that truncates (cast_op<int> on float data)
+// has no tag; see cast_keeps_value below.
 template <typename T>
 struct main_tag<cast_op<T>> {
   static constexpr int value = RMI_MAIN_IDENTITY;
 };
+template <typename F, typename In>
+struct cast_keeps_value : std::true_type {};
+template <typename T, typename In>
+struct cast_keeps_value<cast_op<T>, In>
+  : std::bool_constant<std::is_floating_point_v<T> || std::is_same_v<T, __half> ||
+                       (std::is_integral_v<T> && std::is_integral_v<In> && sizeof(T) >= sizeof(In))> {};
 template <>
 struct main_tag<sq_op> {
   static constexpr int value = RMI_MAIN_SQ;
@@ -180,6 +190,43 @@ RAFT_RMI_FINAL_CONST(add_op, RMI_FIN_ADD_CONST);
 RAFT_RMI_FINAL_CONST(sub_op, RMI_FIN_SUB_CONST);
 #undef RAFT_RMI_FINAL_CONST
 
+// ---- does the library have a kernel for this combination? ----------------------------
+// The rules of the library's own descriptor check, on the tags: a combination it would
+// refuse at run time (a count of non-zeros into an int from float data, max of integers
+// into a float, ...) is instantiated in the caller's translation unit instead, like any
+// other functor the vocabulary lacks.
+constexpr bool dtype_is_float(int dt)
+{
+  return dt == RMI_F16 || dt == RMI_BF16 || dt == RMI_F32 || dt == RMI_F64;
+}
+constexpr bool dtype_is_int(int dt)
+{
+  return dt == RMI_I8 || dt == RMI_U8 || dt == RMI_I32 || dt == RMI_I64;
+}
+constexpr bool dtype_is_kvp(int dt) { return dt >= RMI_KVP_I32_F32 && dt <= RMI_KVP_I64_F64; }
+
+constexpr bool library_serves(int in_dt, int out_dt, int main_op, int red_op, int final_op)
+{
+  if (in_dt < 0 || out_dt < 0 || main_op < 0 || red_op < 0 || final_op < 0) return false;
+  if (dtype_is_kvp(in_dt)) return false;
+  const bool arg = red_op == RMI_RED_ARGMAX || red_op == RMI_RED_ARGMIN;
+  if (arg) {
+    if (main_op != RMI_MAIN_KVP || !dtype_is_float(in_dt)) return false;
+    // (matrix::argmax names the pair type and overrides the stored type with the key's)
+    if (final_op == RMI_FIN_KEY) return out_dt == RMI_I32 || out_dt == RMI_I64 || dtype_is_kvp(out_dt);
+    if (final_op != RMI_FIN_IDENTITY || !dtype_is_kvp(out_dt)) return false;
+    const bool out_val64 = out_dt == RMI_KVP_I32_F64 || out_dt == RMI_KVP_I64_F64;
+    return out_val64 == (in_dt == RMI_F64);
+  }
+  if (main_op == RMI_MAIN_KVP || final_op == RMI_FIN_KEY || dtype_is_kvp(out_dt)) return false;
+  if (main_op == RMI_MAIN_NZ && red_op != RMI_RED_ADD) return false;
+  if (dtype_is_float(out_dt)) return !(dtype_is_int(in_dt) && red_op != RMI_RED_ADD);
+  // integer output: integer arithmetic end to end
+  return dtype_is_int(in_dt) && (out_dt == RMI_I32 || out_dt == RMI_I64) &&
+         final_op != RMI_FIN_SQRT && final_op != RMI_FIN_VAR_FROM_SUMSQ &&
+         final_op != RMI_FIN_STDDEV_FROM_SUMSQ;
+}
+
 // ---- status -> exception ----------------------------------------------------------
 inline void check(int status, const char* what)
 {
@@ -194,8 +241,9 @@ inline void check(int status, const char* what)
 }
 
 // ---- workspace ----------------------------------------------------------------------
-// With a handle the workspace belongs to the handle and is reused; with a bare
-// stream it is a stream-ordered allocation released after the launches (what the
+// With a handle the workspace belongs to the handle and is reused (its ticket words are
+// zero, see raft::resources::workspace, so split rows are reduced in one launch); with a
+// bare stream it is a stream-ordered allocation released after the launches (what the
 // reference does with rmm::device_uvector, coalesced_reduction-inl.cuh:560).
 class workspace_lease {
  public:
@@ -204,7 +252,8 @@ class workspace_lease {
     if (bytes == 0) return;
     bytes_ = bytes;
     if (res != nullptr) {
-      ptr_ = res->workspace(bytes);
+      ptr_    = res->workspace(bytes);
+      zeroed_ = true;
     } else {
       ptr_   = scratch_alloc(bytes, stream);
       owned_ = true;
@@ -218,11 +267,13 @@ class workspace_lease {
   }
   void* data() const { return ptr_; }
   size_t size() const { return bytes_; }
+  int flags() const { return zeroed_ ? RMI_FLAG_WORKSPACE_ZEROED : 0; }
 
  private:
   void* ptr_     = nullptr;
   size_t bytes_  = 0;
   bool owned_    = false;
+  bool zeroed_   = false;
   hipStream_t stream_;
 };
 
@@ -287,11 +338,11 @@ void reduce(const resources* res,
 {
   // Functor and element types the library implements go through the C ABI; anything
   // else is instantiated in this translation unit when it is compiled by hipcc.
-  constexpr bool lowered = main_tag<MainLambda>::value >= 0 &&
-                           reduce_tag<ReduceLambda>::value >= 0 &&
-                           final_tag<FinalLambda>::value >= 0 &&
-                           dtype_of<std::remove_cv_t<InType>>::value >= 0 &&
-                           dtype_of<std::remove_cv_t<OutType>>::value >= 0;
+  constexpr bool lowered =
+    cast_keeps_value<MainLambda, std::remove_cv_t<InType>>::value &&
+    library_serves(dtype_of<std::remove_cv_t<InType>>::value,
+                   dtype_of<std::remove_cv_t<OutType>>::value, main_tag<MainLambda>::value,
+                   reduce_tag<ReduceLambda>::value, final_tag<FinalLambda>::value);
   if constexpr (!lowered) {
 #if defined(__HIPCC__)
     (void)res;
@@ -314,6 +365,12 @@ void reduce(const resources* res,
                     dtype_of<std::remove_cv_t<OutType>>::value >= 0,
                   "element type not supported by the reduction library; compile this translation "
                   "unit with hipcc to reduce arbitrary trivially copyable types");
+    static_assert(always_false<MainLambda>,
+                  "the reduction library has no kernel for this combination of element types and "
+                  "functors (floating data into an integer output, max / min of integers into a "
+                  "floating output, a cast_op that narrows or truncates, nz_op with a reduce_op "
+                  "other than add_op, an arg-reduction whose output is not the matching "
+                  "KeyValuePair or its key); compile this translation unit with hipcc");
 #endif
   } else {
   rmi_reduce_desc d{};
@@ -333,9 +390,10 @@ void reduce(const resources* res,
   d.final_scalar2 = scalar2;
   d.final_aux     = final_aux;
   d.plan_hint     = RMI_PLAN_AUTO;
-  d.reserved      = 0;
+  d.flags         = 0;
   const size_t ws_bytes = rmi_reduce_workspace_bytes(&d);
   workspace_lease ws(res, stream, ws_bytes);
+  d.flags = ws.flags();
   check(rmi_reduce(&d, data, dots, ws.data(), ws.size(), stream), "rmi_reduce");
   (void)main_op;
   (void)reduce_op;

@@ -54,10 +54,17 @@ void check(const rmi_reduce_desc& d, int n_cu, uintptr_t in_misalign)
   }
   REQUIRE(p.grid_blocks >= 1 && p.grid_blocks <= 0x7fffffffLL);
   REQUIRE(p.lds_reserve >= 0 && p.lds_reserve <= 64 * 1024);
-  REQUIRE((p.ws_bytes > 0) == (p.passes == 2));
+  // partials behind the workspace's ticket words; a second launch folds them unless the
+  // caller vouches for zeroed tickets and the plan splits rows (at most one ticket per row)
+  REQUIRE((p.ws_bytes > 0) == (p.passes == 2 || p.fused_fold));
   REQUIRE(p.B >= 1 && p.B <= 4096);
-  if (p.passes == 2)
-    REQUIRE(p.ws_bytes == (size_t)p.n_out * p.B * (p.group > 0 ? p.group : 1) * acc_bytes);
+  if (p.ws_bytes > 0)
+    REQUIRE(p.ws_bytes == rmi::kTicketBytes +
+                            (size_t)p.n_out * p.B * (p.group > 0 ? p.group : 1) * acc_bytes);
+  REQUIRE(p.fused_fold == ((d.flags & RMI_FLAG_WORKSPACE_ZEROED) != 0 &&
+                           p.kind == RMI_PLAN_ROW_SPLIT &&
+                           p.n_out * rmi::ticket_lines_per_row(p.B) <= rmi::kTicketLines));
+  if (p.fused_fold) REQUIRE(p.passes == 1 && p.threads == rmi::kPlanBlock);
   const int es = dtype_size(d.in_dtype);
   if (p.kind != RMI_PLAN_ROW_LANES) {
     REQUIRE(p.row_bytes == contiguous * es);
@@ -151,6 +158,7 @@ int main()
     d.layout    = (int)(g() % 2);
     d.apply     = (int)(g() % 2);
     d.plan_hint = (int)(g() % 7);
+    d.flags     = (int)(g() % 2) * RMI_FLAG_WORKSPACE_ZEROED;
     const int kind = (int)(g() % 4);
     if (kind == 0) {  // sums
       d.out_dtype = d.in_dtype >= RMI_F16 ? RMI_F32 : (g() % 2 ? RMI_I64 : RMI_F32);

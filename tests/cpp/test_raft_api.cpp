@@ -666,6 +666,45 @@ void handle_workspace_reuse()
   RAFT_HIP_TRY(hipStreamDestroy(s));
 }
 
+// Handles are copyable (the reference passes raft::resources by value in places) and copies
+// share the workspace; a copy on another stream must not overwrite partials that work queued
+// on the first stream still reads: results of interleaved calls on two streams stay right.
+void handle_copies_and_stream_changes()
+{
+  hipStream_t s1, s2;
+  RAFT_HIP_TRY(hipStreamCreate(&s1));
+  RAFT_HIP_TRY(hipStreamCreate(&s2));
+  {
+    raft::resources a(s1);
+    raft::resources b = a;  // shares a's workspace
+    b.set_stream(s2);
+    const int rows = 4, cols = 1 << 20;
+    auto h1 = uniform<float>((size_t)rows * cols, -1.0, 1.0, 5);
+    auto h2 = uniform<float>((size_t)rows * cols, -1.0, 1.0, 6);
+    auto d1 = raft::make_device_matrix<float, int, raft::row_major>(a, rows, cols);
+    auto d2 = raft::make_device_matrix<float, int, raft::row_major>(b, rows, cols);
+    auto o1 = raft::make_device_vector<float, int>(a, rows);
+    auto o2 = raft::make_device_vector<float, int>(b, rows);
+    raft::update_device(d1.data_handle(), h1.data(), h1.size(), s1);
+    raft::update_device(d2.data_handle(), h2.data(), h2.size(), s2);
+    auto add = [](double x, double y) { return x + y; };
+    auto idm = [](double x, int) { return x; };
+    auto idf = [](double x) { return x; };
+    auto w1  = host_reduce(h1, rows, cols, true, true, 0.0, nullptr, idm, add, idf);
+    auto w2  = host_reduce(h2, rows, cols, true, true, 0.0, nullptr, idm, add, idf);
+    for (int rep = 0; rep < 4; ++rep) {
+      raft::linalg::reduce<raft::Apply::ALONG_ROWS>(a, raft::make_const_mdspan(d1.view()), o1.view(), 0.0f);
+      raft::linalg::reduce<raft::Apply::ALONG_ROWS>(b, raft::make_const_mdspan(d2.view()), o2.view(), 0.0f);
+    }
+    CHECK(all_close(to_host(o1.data_handle(), (size_t)rows, s1), w1, 1e-5));
+    CHECK(all_close(to_host(o2.data_handle(), (size_t)rows, s2), w2, 1e-5));
+    auto by_value = [](raft::resources r, hipStream_t want) { return r.get_stream() == want; };
+    CHECK(by_value(a, s1) && by_value(b, s2));
+  }
+  RAFT_HIP_TRY(hipStreamDestroy(s1));
+  RAFT_HIP_TRY(hipStreamDestroy(s2));
+}
+
 // cpp/tests/linalg/normalize.cu:40-135: row_normalize against rowNorm followed by a
 // per-row division, rows {11,101,12345} x cols {2,3,7,12,33,125,254} x {L1,L2,Linf}
 template <typename T, typename Idx>
@@ -734,6 +773,7 @@ TEST_CASE(ArgFixturesF) { arg_fixtures<float>(); }
 TEST_CASE(ArgFixturesD) { arg_fixtures<double>(); }
 TEST_CASE(MapReduce) { map_reduce_cases(); }
 TEST_CASE(HandleWorkspaceReuse) { handle_workspace_reuse(); }
+TEST_CASE(HandleCopiesAndStreamChanges) { handle_copies_and_stream_changes(); }
 
 int main()
 {

@@ -513,6 +513,133 @@ void weighted_mean_cases(double tol)
 TEST_CASE(WeightedMeanF) { weighted_mean_cases<float>(1e-6); }
 TEST_CASE(WeightedMeanD) { weighted_mean_cases<double>(1e-14); }
 
+// Combinations whose functors all have tags but which the library has no kernel for are
+// instantiated here like any other functor: a count of non-zeros of float data into an int
+// (nz_op + add_op), the maximum of integers into a float, and cast_op<int> on float data,
+// whose truncation must not be lost (sum of the truncated values, not the truncated sum).
+TEST_CASE(TagValidCombinationsWithoutALibraryKernel)
+{
+  raft::resources handle;
+  auto stream = raft::resource::get_cuda_stream(handle);
+  const int rows = 300, cols = 517;
+  auto h = uniform<float>((size_t)rows * cols, -3.0, 3.0, 77);
+  for (size_t i = 0; i < h.size(); i += 7)
+    h[i] = 0.0f;
+  auto in = raft::make_device_matrix<float, int, raft::row_major>(handle, rows, cols);
+  raft::update_device(in.data_handle(), h.data(), h.size(), stream);
+  auto in_c = raft::make_const_mdspan(in.view());
+  {
+    auto out = raft::make_device_vector<int, int>(handle, rows);
+    raft::linalg::reduce<raft::Apply::ALONG_ROWS>(handle, in_c, out.view(), 0, false, raft::nz_op{},
+                                                  raft::add_op{});
+    auto got = to_host(out.data_handle(), (size_t)rows, stream);
+    bool ok  = true;
+    for (int r = 0; r < rows; ++r) {
+      int want = 0;
+      for (int c = 0; c < cols; ++c)
+        want += h[(size_t)r * cols + c] != 0.0f;
+      ok &= got[r] == want;
+    }
+    CHECK(ok);
+  }
+  {
+    auto out = raft::make_device_vector<int, int>(handle, cols);
+    raft::linalg::reduce<raft::Apply::ALONG_COLUMNS>(handle, in_c, out.view(), 0, false,
+                                                     raft::cast_op<int>{}, raft::add_op{});
+    auto got = to_host(out.data_handle(), (size_t)cols, stream);
+    bool ok  = true;
+    for (int c = 0; c < cols; ++c) {
+      int want = 0;
+      for (int r = 0; r < rows; ++r)
+        want += (int)h[(size_t)r * cols + c];
+      ok &= got[c] == want;
+    }
+    CHECK(ok);
+  }
+  {
+    std::vector<int> hi((size_t)rows * cols);
+    for (size_t i = 0; i < hi.size(); ++i)
+      hi[i] = (int)(h[i] * 1000.0f);
+    auto ini = raft::make_device_matrix<int, int, raft::row_major>(handle, rows, cols);
+    raft::update_device(ini.data_handle(), hi.data(), hi.size(), stream);
+    auto out = raft::make_device_vector<float, int>(handle, rows);
+    raft::linalg::reduce<raft::Apply::ALONG_ROWS>(handle, raft::make_const_mdspan(ini.view()), out.view(),
+                                                  -1e30f, false, raft::cast_op<float>{}, raft::max_op{});
+    auto got = to_host(out.data_handle(), (size_t)rows, stream);
+    bool ok  = true;
+    for (int r = 0; r < rows; ++r) {
+      int want = hi[(size_t)r * cols];
+      for (int c = 1; c < cols; ++c)
+        want = std::max(want, hi[(size_t)r * cols + c]);
+      ok &= got[r] == (float)want;
+    }
+    CHECK(ok);
+  }
+}
+
+// The weight sum stays on the device (the reference brings it to the host and synchronises,
+// stats/detail/weighted_mean.cuh:38-42), so the whole call can be captured into a HIP graph:
+// captured once, replayed over new data and weights, each replay against the host.
+TEST_CASE(WeightedMeanUnderGraphCapture)
+{
+  hipStream_t s;
+  RAFT_HIP_TRY(hipStreamCreate(&s));
+  {
+    raft::resources handle(s);
+    const int rows = 1024, cols = 256;
+    auto dd = raft::make_device_vector<float, int>(handle, rows * cols);
+    auto dw = raft::make_device_vector<float, int>(handle, cols);
+    auto mu = raft::make_device_vector<float, int>(handle, rows);
+    auto in = raft::make_device_matrix_view<const float, int, raft::row_major>(dd.data_handle(), rows, cols);
+    auto wv = raft::make_device_vector_view<const float, int>(dw.data_handle(), cols);
+    auto upload = [&](unsigned long long seed) {
+      auto hd = uniform<float>((size_t)rows * cols, -1.0, 1.0, seed);
+      auto hw = uniform<float>((size_t)cols, 0.1, 1.0, seed + 1);
+      RAFT_HIP_TRY(hipMemcpy(dd.data_handle(), hd.data(), hd.size() * sizeof(float), hipMemcpyHostToDevice));
+      RAFT_HIP_TRY(hipMemcpy(dw.data_handle(), hw.data(), hw.size() * sizeof(float), hipMemcpyHostToDevice));
+      std::vector<double> want(rows);
+      double ws = 0;
+      for (float w : hw)
+        ws += w;
+      for (int r = 0; r < rows; ++r) {
+        double acc = 0;
+        for (int c = 0; c < cols; ++c)
+          acc += (double)hd[(size_t)r * cols + c] * hw[c];
+        want[r] = acc / ws;
+      }
+      return want;
+    };
+    auto check_mu = [&](const std::vector<double>& want) {
+      auto got = to_host(mu.data_handle(), (size_t)rows, s);
+      bool ok  = true;
+      for (int r = 0; r < rows; ++r)
+        ok &= std::fabs((double)got[r] - want[r]) <= 1e-5 * (1.0 + std::fabs(want[r]));
+      CHECK(ok);
+    };
+    // eager once: the handle allocates its scalar slot here, outside the capture
+    auto want = upload(11);
+    raft::stats::row_weighted_mean(handle, in, wv, mu.view());
+    check_mu(want);
+
+    hipGraph_t graph;
+    hipGraphExec_t exec;
+    RAFT_HIP_TRY(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal));
+    raft::stats::row_weighted_mean(handle, in, wv, mu.view());
+    RAFT_HIP_TRY(hipStreamEndCapture(s, &graph));
+    RAFT_HIP_TRY(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0));
+    for (int rep = 0; rep < 3; ++rep) {
+      want = upload(100 + 7 * rep);
+      RAFT_HIP_TRY(hipMemsetAsync(mu.data_handle(), 0, rows * sizeof(float), s));
+      RAFT_HIP_TRY(hipStreamSynchronize(s));
+      RAFT_HIP_TRY(hipGraphLaunch(exec, s));
+      check_mu(want);
+    }
+    RAFT_HIP_TRY(hipGraphExecDestroy(exec));
+    RAFT_HIP_TRY(hipGraphDestroy(graph));
+  }
+  RAFT_HIP_TRY(hipStreamDestroy(s));
+}
+
 // map over two arrays, then sum: the call shape of linalg/detail/mean_squared_error.cuh:18-24
 // (sq_diff(a, b) summed over two arrays) and stats/detail/kl_divergence.cuh:62
 TEST_CASE(MapReduceTwoArrays)

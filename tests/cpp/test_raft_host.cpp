@@ -148,7 +148,7 @@ TEST_CASE(plan_selector)
   p = plan(RMI_I8, RMI_I64, 4096, 16384);
   CHECK(p.kind == RMI_PLAN_ROW_BLOCK && p.passes == 1);
   p = plan(RMI_BF16, RMI_F32, 8, 4194304);
-  CHECK(p.kind == RMI_PLAN_ROW_SPLIT && p.passes == 2 && p.workspace_bytes > 0);
+  CHECK(p.kind == RMI_PLAN_ROW_SPLIT && p.passes == 2 && p.workspace_bytes > RMI_WORKSPACE_TICKET_BYTES);
   p = plan(RMI_F32, RMI_F32, 10000000, 64, RMI_ALONG_COLUMNS);
   CHECK(p.kind == RMI_PLAN_COL_TILE && p.n_outputs == 64 && p.reduce_len == 10000000);
   p = plan(RMI_F32, RMI_KVP_I32_F32, 65536, 32000, RMI_ALONG_ROWS, RMI_RED_ARGMAX, RMI_MAIN_KVP);

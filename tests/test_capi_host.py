@@ -94,7 +94,7 @@ def test_plan_hints_and_fallbacks():
     d = api.make_desc(api.F32, api.F32, 4, 1 << 20, plan_hint=api.PLAN_ROW_SPLIT)
     p = api.plan_query(d)
     assert p.kind == api.PLAN_ROW_SPLIT and p.blocks_per_out >= 2
-    assert p.workspace_bytes == 4 * p.blocks_per_out * 8
+    assert p.workspace_bytes == api.WORKSPACE_TICKET_BYTES + 4 * p.blocks_per_out * 8
     # rows of 7 floats (28 B) are one 16-byte vector plus three tail elements;
     # rows of 3 floats (12 B) are read element by element
     p = api.plan_query(api.make_desc(api.F32, api.F32, 1000, 7))
@@ -104,7 +104,11 @@ def test_plan_hints_and_fallbacks():
     # f64 sums carry a 16-byte (sum, compensation) accumulator through the partials
     d = api.make_desc(api.F64, api.F64, 4, 1 << 20, plan_hint=api.PLAN_ROW_SPLIT)
     p = api.plan_query(d)
-    assert p.workspace_bytes == 4 * p.blocks_per_out * 16
+    assert p.workspace_bytes == api.WORKSPACE_TICKET_BYTES + 4 * p.blocks_per_out * 16
+    # with zeroed ticket words in the workspace the last workgroup of a row folds: one launch
+    d.flags = api.FLAG_WORKSPACE_ZEROED
+    p1 = api.plan_query(d)
+    assert (p1.kind, p1.passes, p1.workspace_bytes) == (api.PLAN_ROW_SPLIT, 1, p.workspace_bytes)
     # column-major along rows is a strided fold
     p = api.plan_query(api.make_desc(api.F32, api.F32, 64, 100000, layout=api.COL_MAJOR))
     assert p.kind == api.PLAN_COL_TILE and p.n_outputs == 64
@@ -122,7 +126,7 @@ def test_plan_hints_and_fallbacks():
      api.ERR_UNSUPPORTED),                                      # value type mismatch
     (dict(final_op=api.FIN_STDDEV_FROM_SUMSQ), api.ERR_NULL),   # needs final_aux
     (dict(in_dtype=api.KVP_I32_F32), api.ERR_UNSUPPORTED),
-    (dict(reserved=1), api.ERR_BAD_ENUM),
+    (dict(flags=2), api.ERR_BAD_ENUM),
 ])
 def test_descriptor_validation(kw, status):
     d = api.make_desc(api.F32, api.F32, 100, 100)

@@ -181,6 +181,29 @@ def test_nan_rows_are_written(gpu, cols, norm):
     assert not np.isnan(got[[0, 1, 3, 4, 6, 7, 8]]).any() and not (got == -3.0).any()
 
 
+# fp32 and fp64 rows are divided element by element in the reference (in / norm, a correctly
+# rounded IEEE division).  The kernels compute the same quotient from one reciprocal and a
+# residual correction; with the Linf norm the divisor is one of the row's own elements, so
+# numpy's division in the same type gives the expected bits.  Rows scaled to 1e+-35 have a
+# divisor outside the range where the shortcut is exact and take the division itself.
+@pytest.mark.parametrize("dt,npdt", [(api.F32, np.float32), (api.F64, np.float64)])
+@pytest.mark.parametrize("cols", [8, 100, 128, 1024, 5000, 70001])
+def test_quotients_are_correctly_rounded(gpu, dt, npdt, cols):
+    rows = 40
+    rng = np.random.default_rng(cols)
+    m = rng.standard_normal((rows, cols)) * np.exp(rng.uniform(-3, 3, (rows, cols)))
+    m *= np.exp(rng.uniform(-20, 20, (rows, 1)))
+    m[5] *= 1e35 / np.abs(m[5]).max()
+    m[6] *= 1e-35 / np.abs(m[6]).max()
+    m = m.astype(npdt)
+    main, red, fin = NORMS["linf"]
+    d = api.make_desc(dt, dt, rows, cols, main_op=main, reduce_op=red, final_op=fin)
+    got = _gpu(d, m.reshape(-1), np.zeros(rows * cols, dtype=npdt), 0.0).reshape(rows, cols)
+    want = m / np.abs(m).max(axis=1, keepdims=True)
+    assert want.dtype == npdt
+    assert np.array_equal(got, want), np.argwhere(got != want)[:5]
+
+
 def test_full_size_embedding_shape(gpu):
     """1,000,000 x 128 fp32 (the shape of benchmark config 2): unit L2 rows, and the
     oracle on a slice."""

@@ -459,6 +459,88 @@ def test_bitwise_repeatable(gpu):
             assert np.array_equal(a, u.gpu_reduce(d, data))
 
 
+# Rows split over several workgroups, reduced in ONE launch: with RMI_FLAG_WORKSPACE_ZEROED the
+# workgroup that finishes a row last folds its partials (in index order, so the result equals
+# the two-launch plan's bit for bit) and its ticket wraps the row's ticket word back to zero.
+# One zeroed workspace serves every call of the test, split and column plans mixed, shapes
+# growing and shrinking; the ticket words must read zero after every call.
+@pytest.mark.parametrize("in_dt,out_dt,kw", [
+    (api.F32, api.F32, {}),
+    (api.F32, api.F32, dict(main_op=api.MAIN_SQ, final_op=api.FIN_SQRT)),
+    (api.BF16, api.F32, {}),
+    (api.F64, api.F64, {}),
+    (api.F16, api.F16, dict(main_op=api.MAIN_ABS, reduce_op=api.RED_MAX)),
+    (api.I8, api.I64, dict(main_op=api.MAIN_SQ)),
+    (api.I32, api.I32, dict(reduce_op=api.RED_MIN, init_i=2**31 - 1)),
+    (api.F32, api.KVP_I32_F32, dict(main_op=api.MAIN_KVP, reduce_op=api.RED_ARGMAX, init_f=-np.inf)),
+    (api.F64, api.KVP_I64_F64, dict(main_op=api.MAIN_KVP, reduce_op=api.RED_ARGMIN, init_f=np.inf)),
+    (api.F32, api.F32, dict(inplace=True)),
+])
+def test_split_rows_single_launch(gpu, in_dt, out_dt, kw):
+    import ctypes as C
+    import torch
+    lib = api.load()
+    sptr = torch.cuda.current_stream().cuda_stream
+    ws = torch.zeros(1 << 20, dtype=torch.uint8, device="cuda")   # zeroed once, then only reused
+    scratch = torch.empty(1 << 20, dtype=torch.uint8, device="cuda")
+    rng = np.random.default_rng(in_dt * 7 + out_dt)
+    odt = u.out_numpy_dtype(out_dt)
+    shapes = [(8, 300_001, api.PLAN_AUTO), (1, 2_000_000, api.PLAN_AUTO), (3, 70_001, api.PLAN_ROW_SPLIT),
+              (40, 80_000, api.PLAN_ROW_SPLIT), (2, 1_000_003, api.PLAN_AUTO), (512, 70_000, api.PLAN_ROW_SPLIT),
+              (5, 100_003, api.PLAN_ROW_SPLIT)]
+    for rows, cols, hint in shapes:
+        data = _rand(rng, in_dt, rows * cols)
+        x = torch.from_numpy(data.view(np.uint8).reshape(-1)).cuda()
+        old = u.encode_out(out_dt, rng.integers(-3, 4, rows).astype(np.float64)) if kw.get("inplace") else None
+        outs = []
+        for flags in (api.FLAG_WORKSPACE_ZEROED, 0):
+            d = api.make_desc(in_dt, out_dt, rows, cols, plan_hint=hint, flags=flags, **kw)
+            pl = api.plan_query(d)
+            assert pl.kind == api.PLAN_ROW_SPLIT and pl.passes == (1 if flags else 2), (rows, cols)
+            assert pl.workspace_bytes <= ws.numel()
+            for rep in range(2 if flags else 1):
+                o = torch.zeros(rows * odt.itemsize, dtype=torch.uint8, device="cuda")
+                if old is not None:
+                    o.copy_(torch.from_numpy(old.view(np.uint8).reshape(-1)))
+                w = ws if flags else scratch.random_(0, 255)
+                rc = lib.rmi_reduce(C.byref(d), x.data_ptr(), o.data_ptr(), w.data_ptr(), w.numel(), sptr)
+                assert rc == api.OK, api.status_string(rc)
+                torch.cuda.synchronize()
+                outs.append(o.cpu().numpy().view(odt).copy())
+            if flags:
+                assert int(ws[: api.WORKSPACE_TICKET_BYTES].max().item()) == 0, "tickets must wrap to zero"
+        assert all(np.array_equal(outs[0].view(np.uint8), o.view(np.uint8)) for o in outs[1:]), (rows, cols)
+        # and the oracle, at the usual bar
+        d = api.make_desc(in_dt, out_dt, rows, cols, **kw)
+        got = u.decode_out(out_dt, outs[0])
+        exp = u.oracle_reduce(d, data, old=u.decode_out(out_dt, old) if old is not None else None)
+        if u.is_arg(d):
+            assert np.array_equal(got[0], exp[0]) and np.array_equal(got[1], exp[1])
+        elif out_dt in (api.I32, api.I64):
+            assert np.array_equal(got, exp)
+        elif out_dt in (api.F16, api.BF16):
+            assert u.ulp16_ok(out_dt, outs[0], exp).all()
+        else:
+            assert u.fp_close(got, exp).all(), u.worst_rel(got, exp)
+        # a column reduction through the same workspace in between leaves the tickets alone
+        dc = api.make_desc(api.F32, api.F32, 5000, 64, apply=api.ALONG_COLUMNS,
+                           flags=api.FLAG_WORKSPACE_ZEROED)
+        xc = torch.ones(5000 * 64, device="cuda")
+        oc = torch.zeros(64, device="cuda")
+        assert lib.rmi_reduce(C.byref(dc), xc.data_ptr(), oc.data_ptr(), ws.data_ptr(), ws.numel(), sptr) == api.OK
+        torch.cuda.synchronize()
+        assert bool((oc == 5000).all()) and int(ws[: api.WORKSPACE_TICKET_BYTES].max().item()) == 0
+
+
+# More rows than ticket words: the plan falls back to the folding launch.
+def test_split_rows_beyond_the_ticket_words(gpu):
+    d = api.make_desc(api.F32, api.F32, 513, 9000, plan_hint=api.PLAN_ROW_SPLIT,
+                      flags=api.FLAG_WORKSPACE_ZEROED)
+    assert api.plan_query(d).passes == 2
+    rng = np.random.default_rng(1)
+    u.check_against_oracle(d, _rand(rng, api.F32, 513 * 9000), label="split, two launches")
+
+
 # Column reductions over rows that are not a power-of-two number of lane-loads: a workgroup
 # takes as many whole rows as fit its 256 threads and combines them through LDS.  Rows shorter
 # than a 16-byte vector are read in groups of 2..16 consecutive rows that make whole vectors

@@ -129,3 +129,18 @@ def test_noalloc_under_graph_capture(gpu):
         assert rc == api.OK
         torch.cuda.synchronize()
         assert torch.equal(out, ref), rep
+
+
+def test_noalloc_splits_rows_in_one_launch(gpu):
+    """The static buffer's ticket words are zero from load time on, so rows split over several
+    workgroups take the single-launch plan here; bit for bit the two-launch result."""
+    import torch
+    lib = api.load()
+    d = api.make_desc(api.BF16, api.F32, 8, 4194304, flags=api.FLAG_WORKSPACE_ZEROED)
+    assert api.plan_query(d).passes == 1
+    d.flags = 0
+    assert api.plan_query(d).passes == 2
+    x = torch.randn(8 * 4194304, device="cuda").to(torch.bfloat16)
+    for rep in range(3):
+        a, b, nws = _both(d, x, 4, 8)
+        assert nws > 0 and np.array_equal(a, b), rep
