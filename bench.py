@@ -8,13 +8,20 @@ headline workload is the L2 row norm of a row-major fp32 1,000,000 x 128 matrix
 (N(0,1), sqrt fused); the other benchmark shapes are timed the same way and
 reported under "configs".  Inputs are generated on the device from fixed seeds and
 are resident in HBM before timing starts; consecutive steps read different
-buffers whose total size exceeds the 256 MB Infinity Cache, so every step streams
-from HBM.  Timing uses HIP events recorded on the stream the kernels run on.
+buffers whose total size is at least twice the 256 MB Infinity Cache, so every step
+streams from HBM.  Timing uses HIP events recorded on the stream the kernels run on.
+Per config, beside the back-to-back average: the same launches replayed from a HIP
+graph, the same buffer every step (cache-resident where it fits), and single calls
+timed one by one after a 768 MB scratch sweep has evicted the caches (median and
+minimum of the repetitions; the method of the reference's benchmark fixture,
+cpp/bench/prims/common/benchmark.hpp:138-155).
 
 Prints one JSON line.  `roofline.achieved` = algorithmic bytes (input read once +
-output written once) / average launch duration.  `cpu_baseline` times the OpenMP
-host implementation of the same semantics (oracle/, kind "port") on this
-machine's cores.
+output written once) / average launch duration.  `roofline.traffic` is NOT measured in
+this run: it is read from profiles/traffic.json, which raft_amd/bench/profile_summary.py
+writes from rocprofv3 counter runs of this same program (the file names the commit it
+was measured at).  `cpu_baseline` times the OpenMP host implementation of the same
+semantics (oracle/, kind "port") on this machine's cores.
 """
 from __future__ import annotations
 
@@ -130,11 +137,24 @@ def main():
                                     final_op=api.FIN_STDDEV_FROM_SUMSQ,
                                     final_scalar=float(f32(1.0) / f32(10000000)), final_scalar2=1.0),
                             needs_mean=True),
+        "cfg3_stddev_sample": dict(desc="column stddev (sample) fp32 10000000x64 N(3,2)",
+                                   make=lambda s: mk_normal(10000000, 64, s, 3.0, 2.0),
+                                   seed=3, rows=10000000, cols=64, in_dt=api.F32, out_dt=api.F32,
+                                   kw=dict(apply=api.ALONG_COLUMNS, main_op=api.MAIN_SQ,
+                                           final_op=api.FIN_STDDEV_FROM_SUMSQ,
+                                           final_scalar=float(f32(1.0) / f32(9999999)),
+                                           final_scalar2=float(f32(f32(1.0) / f32(9999999)) * f32(10000000))),
+                                   needs_mean=True),
         "cfg4": dict(desc="row argmax (KVP int32,fp32) fp32 65536x32000 N(0,1), ties in 1% of rows",
                      make=lambda s: mk_logits_with_ties(65536, 32000, s), seed=4, rows=65536, cols=32000,
                      in_dt=api.F32, out_dt=api.KVP_I32_F32,
                      kw=dict(main_op=api.MAIN_KVP, reduce_op=api.RED_ARGMAX, init_i=0,
                              init_f=float("-inf"))),
+        "cfg4_keys": dict(desc="matrix::argmax (int32 index only) fp32 65536x32000 N(0,1), ties in 1% of rows",
+                          make=lambda s: mk_logits_with_ties(65536, 32000, s), seed=4, rows=65536, cols=32000,
+                          in_dt=api.F32, out_dt=api.I32,
+                          kw=dict(main_op=api.MAIN_KVP, reduce_op=api.RED_ARGMAX, final_op=api.FIN_KEY,
+                                  init_i=0, init_f=float("-inf"))),
         "cfg5a": dict(desc="row sum int8->int64 4096x16384", make=lambda s: mk_int8(4096, 16384, s),
                       seed=5, rows=4096, cols=16384, in_dt=api.I8, out_dt=api.I64, kw={}),
         "cfg5b": dict(desc="row sum int8->int64 16777216x8", make=lambda s: mk_int8(16777216, 8, s),
@@ -163,13 +183,17 @@ def main():
         return (w["rows"] * w["cols"] * api.DTYPE_SIZE[w["in_dt"]]
                 + n_out(w) * api.DTYPE_SIZE[w["out_dt"]])
 
-    TORCH_OUT = {api.F32: torch.float32, api.I64: torch.int64}
+    TORCH_OUT = {api.F32: torch.float32, api.I64: torch.int64, api.I32: torch.int32}
 
-    def run_config(name, steps, warmup, check=True):
+    # > 512 MB written between single timed calls: evicts the 256 MB memory-side cache
+    flush_buf = torch.empty(768 << 20, dtype=torch.uint8, device=devc)
+
+    def run_config(name, steps, warmup, check=True, extras=True):
         w = WORK[name]
         in_bytes = w["rows"] * w["cols"] * api.DTYPE_SIZE[w["in_dt"]]
-        # enough distinct inputs to defeat the 256 MB Infinity Cache, at most ~17 GB
-        nbuf = max(2, min(16, -(-(1 << 30) // in_bytes)))
+        # enough distinct inputs that a buffer is long out of the 256 MB Infinity Cache when
+        # its turn comes again: at least 512 MB in rotation (cfg1: 53 buffers of 10 MB)
+        nbuf = max(2, min(64, -(-(512 << 20) // in_bytes)))
         bufs = [w["make"](w["seed"] + 7919 * i) for i in range(nbuf)]
         no = n_out(w)
         out_bytes = no * api.DTYPE_SIZE[w["out_dt"]]
@@ -221,7 +245,9 @@ def main():
                    alg_bytes=alg_bytes(w), GBps=alg_bytes(w) / (ms * 1e-3) / 1e9,
                    rows_per_s=w["rows"] / (ms * 1e-3))
         res["pct_of_peak"] = 100.0 * res["GBps"] / PEAK_HBM_GBPS
-        res["hbm_traffic_bytes_rocprof"] = MEASURED_TRAFFIC.get(name)
+        res["hbm_traffic_bytes_profile"] = PROFILE_TRAFFIC.get(name)
+        if not extras:  # profiler runs: the timed launches only
+            return res, bufs, outs
 
         # the same launches replayed from a HIP graph: removes host launch gaps, which
         # dominate the shapes whose kernel is only a few microseconds long
@@ -268,6 +294,21 @@ def main():
             res["same_buffer_ms_per_step"] = cms
             res["same_buffer_GBps"] = alg_bytes(w) / (cms * 1e-3) / 1e9
 
+        # single calls, caches evicted before each: median and minimum of the repetitions
+        # (a pair of events around one call carries a few microseconds of its own)
+        reps = 20
+        times = []
+        for i in range(reps):
+            flush_buf.fill_(i & 0xFF)
+            e0.record(stream)
+            step(i)
+            e1.record(stream)
+            torch.cuda.synchronize()
+            times.append(e0.elapsed_time(e1))
+        times.sort()
+        res["flushed_single_call_us"] = {"median": times[reps // 2] * 1e3, "min": times[0] * 1e3,
+                                         "reps": reps}
+
         if check:
             res["check"] = check_config(name, w, bufs[0], outs[0], aux[0] if aux else None)
         return res, bufs, outs
@@ -280,6 +321,25 @@ def main():
         rows, cols = w["rows"], w["cols"]
         info = {}
         kw = dict(w["kw"])
+        if w["out_dt"] == api.I32 and kw.get("final_op") == api.FIN_KEY:
+            keys = out_raw.view(torch.int32).to(torch.int64)
+            x = buf.view(rows, cols)
+            ok = True
+            ar = torch.arange(cols, device=devc, dtype=torch.int64)
+            for r0 in range(0, rows, 4096):
+                blk = x[r0:r0 + 4096]
+                eq = blk == blk.amax(dim=1)[:, None]
+                first = torch.where(eq, ar[None, :], torch.full((), cols, device=devc, dtype=torch.int64)).amin(dim=1)
+                ok &= bool(torch.equal(first, keys[r0:r0 + 4096]))
+            info["full_size_first_max_property"] = ok
+            ns = 256
+            sample = x[:ns].contiguous().cpu().numpy().reshape(-1)
+            d = api.make_desc(w["in_dt"], w["out_dt"], ns, cols, **kw)
+            ek, _ = u.oracle_reduce(d, sample)
+            info["oracle_sample_rows"] = ns
+            info["oracle_exact"] = bool(np.array_equal(keys[:ns].cpu().numpy(), ek))
+            info["pass"] = ok and info["oracle_exact"]
+            return info
         if w["out_dt"] == api.KVP_I32_F32:
             kv = out_raw.view(torch.int32).view(rows, 2)
             keys = kv[:, 0].to(torch.int64)
@@ -331,19 +391,21 @@ def main():
             # strided: fp64 reference over the whole matrix on the device (independent
             # implementation), plus the CPU oracle on the first 200k rows as its own problem
             x = buf.view(rows, cols)
+            sample_sd = name.endswith("_sample")
             if name == "cfg3_mean":
                 ref = x.mean(dim=0, dtype=torch.float64).cpu().numpy()
             else:
-                ref = x.to(torch.float64).std(dim=0, unbiased=False).cpu().numpy() \
-                    if rows * cols <= (1 << 28) else \
-                    torch.sqrt(torch.clamp((sum((c.to(torch.float64) ** 2).sum(dim=0) for c in x.split(1 << 21)) / rows)
-                               - x.mean(dim=0, dtype=torch.float64) ** 2, min=0)).cpu().numpy()
+                m64 = x.mean(dim=0, dtype=torch.float64)
+                ss = sum(((c.to(torch.float64) - m64) ** 2).sum(dim=0) for c in x.split(1 << 21))
+                ref = torch.sqrt(ss / (rows - 1 if sample_sd else rows)).cpu().numpy()
             got = out_raw.view(torch.float32).cpu().numpy()
             info["worst_rel_err_vs_fp64_full"] = u.worst_rel(got, ref)
             ns = 200000
             sub = x[:ns].contiguous()
             d = api.make_desc(w["in_dt"], w["out_dt"], ns, cols, **{**kw, "final_scalar": 1.0 / ns})
-            d.final_scalar = float(np.float32(1.0) / np.float32(ns))
+            d.final_scalar = float(np.float32(1.0) / np.float32(ns - 1 if sample_sd else ns))
+            if sample_sd:
+                d.final_scalar2 = float(np.float32(d.final_scalar) * np.float32(ns))
             o = torch.zeros(cols, dtype=torch.float32, device=devc)
             auxs = None
             if w.get("needs_mean"):
@@ -373,7 +435,9 @@ def main():
         host = (t.view(torch.int16).cpu().numpy().view(np.uint16) if w["in_dt"] == api.BF16
                 else t.cpu().numpy()).reshape(-1)
         if "final_scalar" in kw and name.startswith("cfg3"):
-            kw["final_scalar"] = float(np.float32(1.0) / np.float32(ns))
+            kw["final_scalar"] = float(np.float32(1.0) / np.float32(ns - 1 if name.endswith("_sample") else ns))
+            if name.endswith("_sample"):
+                kw["final_scalar2"] = float(np.float32(kw["final_scalar"]) * np.float32(ns))
         d = api.make_desc(w["in_dt"], w["out_dt"], ns, cols, **kw)
         no = ns if kw.get("apply", api.ALONG_ROWS) == api.ALONG_ROWS else cols
         out = np.zeros(no, dtype=u.out_numpy_dtype(w["out_dt"]))
@@ -399,7 +463,7 @@ def main():
     # ------------------------------------------------------------------
     if args.only_kernel:
         for nm in args.only_kernel.split(","):
-            run_config(nm, args.steps, args.warmup, check=False)
+            run_config(nm, args.steps, args.warmup, check=False, extras=False)
             torch.cuda.empty_cache()
         if args.calib_copy:
             a = torch.empty(512 << 20, dtype=torch.uint8, device=devc).random_(0, 255)
@@ -522,7 +586,8 @@ def main():
         "pct_of_hbm_peak": head["pct_of_peak"],
         "roofline": {"bound": "hbm", "achieved": head["GBps"], "peak": PEAK_HBM_GBPS,
                      "unit": "GB/s", "frac": head["GBps"] / PEAK_HBM_GBPS,
-                     "traffic": MEASURED_TRAFFIC.get(HEADLINE)},
+                     "traffic": PROFILE_TRAFFIC.get(HEADLINE),
+                     "traffic_source": PROFILE_SOURCE},
         "cpu_baseline": cpu.get(HEADLINE),
         "launch_floor_us": launch_floor_us(),
         "extras": ({"row_normalize": extra_row_normalize(), "meanvar": extra_meanvar()}
@@ -534,12 +599,22 @@ def main():
     print(json.dumps(line))
 
 
-# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs (see
-# profiles/), scaled by the same counters' reading for a copy kernel of known size.
-MEASURED_TRAFFIC: dict[str, float | None] = {
-    "cfg1": 10.36e6, "cfg2": 516.04e6, "cfg3_mean": 2561.39e6, "cfg3_stddev": 2561.38e6,
-    "cfg4": 8394.23e6, "cfg5a": 67.26e6, "cfg5b": 268.53e6, "cfg5c": 67.33e6,
-}
+def _load_profile_traffic():
+    """HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this program,
+    scaled by the same counters' reading for a copy of known size: written by
+    raft_amd/bench/profile_summary.py into profiles/traffic.json together with the commit the
+    library was at.  Not measured in this run; None where the file has no entry."""
+    path = ROOT / "profiles" / "traffic.json"
+    try:
+        with open(path) as f:
+            doc = json.load(f)
+    except (OSError, ValueError):
+        return {}, "profiles/traffic.json missing"
+    traffic = {k: v.get("hbm_bytes") for k, v in doc.get("configs", {}).items()}
+    return traffic, f"profiles/traffic.json (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE; commit {doc.get('commit', 'unknown')})"
+
+
+PROFILE_TRAFFIC, PROFILE_SOURCE = _load_profile_traffic()
 
 
 if __name__ == "__main__":

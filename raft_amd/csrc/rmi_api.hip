@@ -1,6 +1,7 @@
 // C ABI of the reduction library (declared in include/rmi_reduce.h):
 // validation, plan selection, policy lookup, launch.
 #include <atomic>
+#include <cstring>
 
 #include "rmi_launch.hpp"
 
@@ -74,29 +75,92 @@ run_fn lookup(const PolicyKey& k)
 
 bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 
-// `in` is the input pointer when the plan is made for a launch (its position within a
-// 128-byte line decides whether rows are staged through LDS), nullptr for queries.
-int plan_for(const rmi_reduce_desc* desc, PlanX& pl, PolicyKey& key, const void* in = nullptr)
+// A planned reduction: the launch plan, the accumulator policy's key and its launcher.
+struct Planned {
+  PlanX pl;
+  PolicyKey key;
+  run_fn fn = nullptr;
+};
+
+// What a plan depends on: every descriptor field but the values that only the epilogue
+// reads (init, the final scalars, the address behind final_aux), and the input's position
+// within a 128-byte line (it decides whether rows are staged through LDS).
+struct PlanKey {
+  int32_t in_dtype, out_dtype, layout, apply;
+  int64_t n_rows, n_cols;
+  int32_t main_op, reduce_op, final_op, inplace, plan_hint, flags;
+  int32_t has_aux, misalign;
+  bool operator==(const PlanKey& o) const { return memcmp(this, &o, sizeof(PlanKey)) == 0; }
+};
+static_assert(sizeof(PlanKey) == 16 + 16 + 24 + 8, "no padding: keys are compared bytewise");
+
+PlanKey plan_key(const rmi_reduce_desc& d, uintptr_t misalign)
+{
+  PlanKey k;
+  k.in_dtype = d.in_dtype, k.out_dtype = d.out_dtype, k.layout = d.layout, k.apply = d.apply;
+  k.n_rows = d.n_rows, k.n_cols = d.n_cols;
+  k.main_op = d.main_op, k.reduce_op = d.reduce_op, k.final_op = d.final_op;
+  k.inplace = d.inplace ? 1 : 0, k.plan_hint = d.plan_hint, k.flags = d.flags;
+  k.has_aux  = d.final_aux != nullptr;
+  k.misalign = (int32_t)misalign;
+  return k;
+}
+
+int plan_uncached(const rmi_reduce_desc& d, uintptr_t misalign, Planned& p)
+{
+  int acc_bytes = 8;
+  int rc        = classify(d, p.key, acc_bytes);
+  if (rc != RMI_OK) return rc;
+  p.fn = lookup(p.key);
+  if (p.fn == nullptr) return RMI_ERR_UNSUPPORTED;
+  return make_plan(d, p.key, acc_bytes, cu_count(), p.pl, misalign);
+}
+
+// `in` is the input pointer when the plan is made for a launch, nullptr for queries.  A
+// caller that repeats a call (a serving loop, a solver's iteration) repeats its descriptor:
+// the last few plans of every host thread are kept, so such a call goes from its arguments
+// to the launch without validating and planning again.  Only successful plans are kept.
+int plan_for(const rmi_reduce_desc* desc, const Planned*& out, const void* in = nullptr)
 {
   if (desc == nullptr) return RMI_ERR_NULL;
-  int acc_bytes = 8;
-  int rc        = classify(*desc, key, acc_bytes);
+  constexpr int kSlots = 8;
+  struct Slot {
+    PlanKey k;
+    Planned p;
+    bool used = false;
+  };
+  thread_local Slot slots[kSlots];
+  thread_local int next = 0;
+  const uintptr_t misalign = reinterpret_cast<uintptr_t>(in) % 128;
+  const PlanKey k          = plan_key(*desc, misalign);
+  for (int i = 0; i < kSlots; ++i) {
+    if (slots[i].used && slots[i].k == k) {
+      out = &slots[i].p;
+      return RMI_OK;
+    }
+  }
+  Slot& s = slots[next];
+  s.used  = false;
+  const int rc = plan_uncached(*desc, misalign, s.p);
   if (rc != RMI_OK) return rc;
-  if (lookup(key) == nullptr) return RMI_ERR_UNSUPPORTED;
-  rc = make_plan(*desc, key, acc_bytes, cu_count(), pl, reinterpret_cast<uintptr_t>(in) % 128);
-  return rc;
+  s.k    = k;
+  s.used = true;
+  next   = (next + 1) % kSlots;
+  out    = &s.p;
+  return RMI_OK;
 }
 
 // Launches the planned reduction: pointer checks, epilogue set-up, kernel launch.
 int reduce_planned(const rmi_reduce_desc& d,
-                   const PlanX& pl,
-                   const PolicyKey& key,
+                   const Planned& planned,
                    const void* in,
                    void* out,
                    void* ws,
                    size_t ws_bytes,
                    void* stream)
 {
+  const PlanX& pl      = planned.pl;
+  const PolicyKey& key = planned.key;
   if (pl.n_out == 0) return RMI_OK;
   if (out == nullptr) return RMI_ERR_NULL;
   if (pl.len > 0 && in == nullptr) return RMI_ERR_NULL;
@@ -132,7 +196,7 @@ int reduce_planned(const rmi_reduce_desc& d,
     (key.family != kFamInt && (d.final_op == RMI_FIN_SQRT || d.final_op == RMI_FIN_MUL_CONST));
   pr.epi.plain         = (!d.inplace && simple_final && natural_out) ? 1 : 0;
   pr.epi.out_aligned16 = aligned(out, 16) ? 1 : 0;
-  return lookup(key)(pl, pr, static_cast<hipStream_t>(stream));
+  return planned.fn(pl, pr, static_cast<hipStream_t>(stream));
 }
 
 int reduce_impl(const rmi_reduce_desc& d,
@@ -142,11 +206,10 @@ int reduce_impl(const rmi_reduce_desc& d,
                 size_t ws_bytes,
                 void* stream)
 {
-  PlanX pl;
-  PolicyKey key;
-  const int rc = plan_for(&d, pl, key, in);
+  const Planned* p = nullptr;
+  const int rc     = plan_for(&d, p, in);
   if (rc != RMI_OK) return rc;
-  return reduce_planned(d, pl, key, in, out, ws, ws_bytes, stream);
+  return reduce_planned(d, *p, in, out, ws, ws_bytes, stream);
 }
 
 // map_reduce is a one-row reduction over the contiguous dimension.
@@ -221,11 +284,10 @@ size_t rmi_dtype_size(int dtype) { return (size_t)rmi::dtype_size(dtype); }
 int rmi_plan_query(const rmi_reduce_desc* desc, rmi_plan* plan)
 {
   if (plan == nullptr) return RMI_ERR_NULL;
-  rmi::PlanX pl;
-  rmi::PolicyKey key;
-  const int rc = rmi::plan_for(desc, pl, key);
+  const rmi::Planned* p = nullptr;
+  const int rc          = rmi::plan_for(desc, p);
   if (rc != RMI_OK) return rc;
-  rmi::export_plan(pl, *plan);
+  rmi::export_plan(p->pl, *plan);
   return RMI_OK;
 }
 
@@ -233,11 +295,11 @@ int rmi_plan_query(const rmi_reduce_desc* desc, rmi_plan* plan)
 // groups need a 16-byte aligned start): a query answers for the larger of the two.
 size_t rmi_reduce_workspace_bytes(const rmi_reduce_desc* desc)
 {
-  rmi::PlanX pl, pu;
-  rmi::PolicyKey key;
-  if (rmi::plan_for(desc, pl, key) != RMI_OK) return 0;
-  if (rmi::plan_for(desc, pu, key, reinterpret_cast<const void*>(uintptr_t{1})) != RMI_OK) return 0;
-  return pl.ws_bytes > pu.ws_bytes ? pl.ws_bytes : pu.ws_bytes;
+  if (desc == nullptr) return 0;
+  rmi::Planned pa, pu;
+  if (rmi::plan_uncached(*desc, 0, pa) != RMI_OK) return 0;
+  if (rmi::plan_uncached(*desc, 1, pu) != RMI_OK) return 0;
+  return pa.pl.ws_bytes > pu.pl.ws_bytes ? pa.pl.ws_bytes : pu.pl.ws_bytes;
 }
 
 int rmi_reduce(const rmi_reduce_desc* desc,
@@ -257,17 +319,16 @@ int rmi_reduce_noalloc(const rmi_reduce_desc* desc, const void* in, void* out, v
   // the buffer's ticket words are zero from load time on and every launch leaves them zero
   rmi_reduce_desc d = *desc;
   d.flags |= RMI_FLAG_WORKSPACE_ZEROED;
-  rmi::PlanX pl;
-  rmi::PolicyKey key;
-  int rc = rmi::plan_for(&d, pl, key, in);
+  const rmi::Planned* p = nullptr;
+  int rc                = rmi::plan_for(&d, p, in);
   if (rc != RMI_OK) return rc;
-  if (pl.ws_bytes > RMI_NOALLOC_SCRATCH_BYTES) return RMI_ERR_SCRATCH_LIMIT;
+  if (p->pl.ws_bytes > RMI_NOALLOC_SCRATCH_BYTES) return RMI_ERR_SCRATCH_LIMIT;
   // looked up at every device's first call, whether or not this plan needs scratch, so
   // that "the first call" is the only one that does more than launch
   void* ws = nullptr;
   rc       = rmi::scratch_of_current_device(&ws);
   if (rc != RMI_OK) return rc;
-  return rmi::reduce_planned(d, pl, key, in, out, ws, RMI_NOALLOC_SCRATCH_BYTES, stream);
+  return rmi::reduce_planned(d, *p, in, out, ws, RMI_NOALLOC_SCRATCH_BYTES, stream);
 }
 
 size_t rmi_map_reduce_workspace_bytes(const rmi_reduce_desc* desc, int64_t len)

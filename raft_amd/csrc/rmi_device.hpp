@@ -629,6 +629,21 @@ struct PolMeanVar {
     // per-column selects: a branch here measured slower on ragged widths
     static_for<VEC>([&](auto j) { push(a[j], In<InT>::template get<j>(v), 0); });
   }
+  // The column kernel's main loop, where a lane folds one vector after the other into the
+  // same VEC columns: the shift is taken from the first vector before the loop, a step is
+  // three operations per element, and the count is added once after the loop.
+  static __device__ __forceinline__ void cols_set_shift(acc_t (&a)[VEC], const u32x4& v)
+  {
+    static_for<VEC>([&](auto j) { a[j].k = (double)In<InT>::template get<j>(v); });
+  }
+  static __device__ __forceinline__ void cols_steps(acc_t (&a)[VEC], const u32x4& v)
+  {
+    static_for<VEC>([&](auto j) { step(a[j], (double)In<InT>::template get<j>(v)); });
+  }
+  static __device__ __forceinline__ void cols_count(acc_t (&a)[VEC], double n)
+  {
+    static_for<VEC>([&](auto j) { a[j].w += n; });
+  }
   static __device__ __forceinline__ void merge(acc_t& a, const acc_t& b)
   {
     const double cw = a.w + b.w;
