@@ -647,9 +647,14 @@ __global__ __launch_bounds__(1024) void row_block_kernel(RowArgs a)
         // groups of kFan, the last of a group counts for the row.  Line 0 of a row's lines
         // is the row's counter, lines 1.. its groups'.
         constexpr int kLine = kLineWords;
-        // the partial's stores (past the caches) have completed before the ticket is taken:
-        // a release at workgroup scope waits for them without writing any cache back
+        // The partial's stores (past the caches, same thread) must have completed before the
+        // ticket is taken.  A device-scope release would do that and write a whole L2 back
+        // besides; a workgroup-scope one orders the compiler but emits no wait (the waves of
+        // a workgroup share their CU's cache).  So: wait for this wave's outstanding memory
+        // operations (s_waitcnt vmcnt(0), gfx9 encoding: expcnt and lgkmcnt left at their
+        // maxima), after which a write-through store has been acknowledged by the memory side.
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __builtin_amdgcn_s_waitcnt(0x0F70);
         if (a.B <= kFan) {
           last = atomicInc(a.ticket + row * kLine, (u32)a.B - 1) == (u32)a.B - 1;
         } else {

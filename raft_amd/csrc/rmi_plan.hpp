@@ -35,11 +35,10 @@ constexpr int64_t kBytesInFlightPerCu = 80 * 1024;  // target of the wave-per-ro
 constexpr int kStageBytesPerWave = 4096 + 128 + 16;
 // The first bytes of every workspace are the ticket counters of the single-launch split
 // plan; partials start after them, whatever the plan, so that a workspace shared by calls of
-// different shapes keeps the counters intact.  A counter sits alone on a 128-byte line:
-// device-wide atomics are carried out at the memory side, one after the other per line
-// (2048 workgroups taking tickets from eight adjacent words took 100 us).  For the same
-// reason a row's workgroups first count in groups of kTicketFan, and the last of each group
-// counts once more for the row: the longest queue on one line is kTicketFan atomics.
+// different shapes keeps the counters intact.  A counter sits alone on a 128-byte line, and
+// a row's workgroups first count in groups of kTicketFan, the last of each group counting
+// once more for the row: atomics on one word are carried out one after the other (256
+// workgroups per counter: 15.5 us on 8 rows of 4M bf16, groups of 16: 13.6 us).
 inline int64_t ceildiv_i(int64_t a, int64_t b) { return (a + b - 1) / b; }
 constexpr size_t kTicketBytes    = RMI_WORKSPACE_TICKET_BYTES;
 constexpr int kTicketLineBytes   = 128;
@@ -386,7 +385,20 @@ inline int make_plan(const rmi_reduce_desc& d,
 
   if (kind == RMI_PLAN_ROW_WAVE) {
     p.kind = RMI_PLAN_ROW_WAVE;
-    if (nload <= 8) {
+    // An input that starts off a 16-byte boundary makes every 128-byte piece of the default
+    // layout (8 or 16 lanes per row, several loads per lane) straddle two lines, and each
+    // line is then asked for by two load instructions.  With one load per lane and the
+    // rows of a wave side by side, a load instruction reads ONE contiguous span and a line
+    // is asked for once (plus one per instruction).  Measured on fp32 sums at +4 and +8
+    // bytes: 1M x 128 80 -> 74 us (81 -> 87 %), 1M x 100 74 -> 67 us, 1M x 64 43 -> 38 us,
+    // 2M x 48 82 -> 64 us.  Not for rows beyond 32 lane-loads (1M x 256: 141 -> 160 us), rows
+    // that leave more than a quarter of the lanes idle or end in tail elements (1M x 66:
+    // 50 -> 62 us), arg-reductions (85 -> 92 us) or 1- and 2-byte elements (no change).
+    const bool side_by_side = (in_misalign % 16) != 0 && es == 4 && key.family != kFamKvp &&
+                              p.vec16 && p.tail == 0 && nload <= 32 &&
+                              nload * 4 >= (int64_t)pow2ceil(nload) * 3 &&
+                              (hint == RMI_PLAN_AUTO || hint == RMI_PLAN_ROW_WAVE);
+    if (nload <= 8 || side_by_side) {
       p.short_rows = true;
       p.G          = pow2ceil(nload);  // lane c == nvec loads the overlapping last vector
     } else {

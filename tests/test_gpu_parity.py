@@ -411,6 +411,28 @@ def test_unaligned_input(gpu, in_dt, out_dt, rows, cols, apply):
     u.check_against_oracle(d, data, misalign_elems=1, label="unaligned")
 
 
+# fp32 / int32 rows of whole vectors whose input starts off a 16-byte boundary are laid side by
+# side in the wave, one load per lane (up to 32 lanes per row), so that a load instruction reads
+# one contiguous span; the same shapes on a boundary, and their neighbours (tails, longer rows,
+# arg-reductions, which keep the default layout), sit beside them.
+@pytest.mark.parametrize("in_dt,out_dt,kw", [
+    (api.F32, api.F32, dict(main_op=api.MAIN_SQ, final_op=api.FIN_SQRT)),
+    (api.F32, api.F64, {}),
+    (api.I32, api.I64, dict(main_op=api.MAIN_ABS)),
+    (api.F32, api.F32, dict(reduce_op=api.RED_MAX, init_f=-np.inf)),
+    (api.F32, api.KVP_I32_F32, dict(main_op=api.MAIN_KVP, reduce_op=api.RED_ARGMIN, init_f=np.inf)),
+])
+@pytest.mark.parametrize("cols", [36, 48, 64, 96, 100, 104, 124, 128, 132, 66])
+@pytest.mark.parametrize("rows,shift", [(1, 1), (7, 2), (63, 3), (1000, 1), (5003, 2), (5003, 0), (4096, 5)])
+def test_rows_off_a_vector_boundary(gpu, in_dt, out_dt, kw, cols, rows, shift):
+    rng = np.random.default_rng(rows * 13 + cols + shift)
+    data = _rand(rng, in_dt, rows * cols)
+    d = api.make_desc(in_dt, out_dt, rows, cols, **kw)
+    assert api.plan_query(d).kind == api.PLAN_ROW_WAVE
+    u.check_against_oracle(d, data, misalign_elems=shift,
+                           label=f"off boundary {rows}x{cols} dt{in_dt} +{shift}")
+
+
 # Empty extents: no rows -> nothing written; no columns -> final_op(init) per output
 # (and red(old, init) when inplace).
 def test_empty_inputs(gpu):
