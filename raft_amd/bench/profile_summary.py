@@ -11,10 +11,14 @@ Run the three profiler passes on the GPU box from the repository root (TMPDIR=/t
   rocprofv3 --pmc WRITE_SIZE -d OUT/write -o write --output-format csv -- \\
       python3 bench.py --only-kernel $ALL --steps 6 --warmup 2 --calib-copy
 
+  rocprofv3 --kernel-trace --stats -d OUT/ex -o ex --output-format csv -- \
+      python3 bench.py --configs all --steps 40 --warmup 5 --no-cpu          (optional)
+
 then, where git is available:  python raft_amd/bench/profile_summary.py OUT
 
 It writes profiles/reduce_all_configs_rocprofv3.txt (per-kernel durations, raw counters, the
-copy-kernel scaling, GB/s per config) and profiles/traffic.json (HBM bytes per launch and
+copy-kernel scaling, GB/s per config), profiles/row_normalize_meanvar_rocprofv3.txt when OUT/ex
+exists (kernel durations of the two extra workloads of bench.py) and profiles/traffic.json (HBM bytes per launch and
 kernel durations per config, with the commit they were measured at), which bench.py reads
 for the `roofline.traffic` field of its report.
 """
@@ -162,6 +166,52 @@ def main():
     (ROOT / "profiles" / "reduce_all_configs_rocprofv3.txt").write_text("\n".join(lines) + "\n")
     (ROOT / "profiles" / "traffic.json").write_text(json.dumps(doc, indent=1) + "\n")
     print("\n".join(lines[:40]))
+    if (out / "ex").exists():
+        extras(out, commit)
+
+
+def extras(out: Path, commit: str):
+    """Kernel durations of bench.py's extra workloads (row_normalize, meanvar) from OUT/ex."""
+    rows = list(csv.DictReader(open(_find_csv(out / "ex", "kernel_stats.csv"))))
+    kt = {r["Name"]: r for r in rows}
+    lines = []
+    w = lines.append
+    w("rocprofv3 summary: row_normalize and meanvar on the benchmark shapes, one MI355X (gfx950)")
+    w("=" * 88)
+    w("")
+    w(f"Library at commit {commit}.  Command (run from the repository root on the GPU box, TMPDIR=/tmp):")
+    w("")
+    w("  rocprofv3 --kernel-trace --stats -d OUT/ex -o ex --output-format csv -- \\")
+    w("      python3 bench.py --configs all --steps 40 --warmup 5 --no-cpu")
+    w("")
+    w("GB/s = algorithmic bytes / (kernel + fold average duration); %peak against 8000 GB/s.")
+    w("")
+    w(f"{'workload':50s} {'kernel':58s} {'calls':>5s} {'avg us':>8s} {'alg MB':>8s} {'GB/s':>6s} {'%peak':>6s}")
+    work = [("row_normalize L2 fp32 1000000x128 (read + write)", "normalize_wave_kernel<rmi::PolF<float, 1, 0>", None,
+             1024000000),
+            ("meanvar fp32 10000000x64 row-major (one read)", "col_kernel<rmi::PolMeanVar<float>",
+             "fold_kernel<rmi::PolMeanVar<float>", 2560000512)]
+    for label, k1, k2, alg in work:
+        s1 = pick(kt, k1)
+        if s1 is None:
+            continue
+        s2 = pick(kt, k2)
+        t1 = float(s1["AverageNs"]) / 1e3
+        t2 = float(s2["AverageNs"]) / 1e3 if s2 else 0.0
+        gbps = alg / (t1 + t2) / 1e3
+        name1 = [n for n in kt if k1 in n][0].replace("rmi::", "").replace("void ", "")[:58]
+        w(f"{label:50s} {name1:58s} {s1['Calls']:>5s} {t1:8.2f} {alg / 1e6:8.2f} {gbps:6.0f} {100 * gbps / PEAK_GBPS:6.1f}")
+        if s2:
+            name2 = [n for n in kt if k2 in n][0].replace("rmi::", "").replace("void ", "")[:58]
+            w(f"{'':50s} {'+ ' + name2:58s} {s2['Calls']:>5s} {t2:8.2f}")
+    w("")
+    w("The same run's durations of the reduction kernels (ns; the caches are swept between the")
+    w("single timed calls, so launch counts include those):")
+    for n, r in kt.items():
+        if "rmi::" in n and "normalize" not in n and "MeanVar" not in n:
+            w(f"  {n[:100]:100s} {r['Calls']:>6s} {float(r['AverageNs']):12.1f}")
+    (ROOT / "profiles" / "row_normalize_meanvar_rocprofv3.txt").write_text("\n".join(lines) + "\n")
+    print("\n".join(lines[:16]))
 
 
 if __name__ == "__main__":
