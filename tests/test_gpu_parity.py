@@ -53,15 +53,21 @@ def test_reduce_grid(gpu, in_dt, out_dt, rows, cols):
                                label=f"{rows}x{cols} l{layout} a{apply} inplace")
 
 
-# cpp/tests/linalg/reduce.cu:321-341 ("thick"): {3,9} x {17771,33333,100000}.
+# cpp/tests/linalg/reduce.cu:321-341 ("thick"): {3,9} x {17771,33333,100000}, float -> float,
+# double -> double and float -> double, inplace = false then true (the reference runs row-major
+# along rows; the other three layout / axis combinations ride along for float).
+@pytest.mark.parametrize("in_dt,out_dt", [(api.F32, api.F32), (api.F64, api.F64), (api.F32, api.F64)])
 @pytest.mark.parametrize("rows,cols", itertools.product([3, 9], [17771, 33333, 100000]))
-def test_reduce_thick(gpu, rows, cols):
+def test_reduce_thick(gpu, in_dt, out_dt, rows, cols):
     rng = np.random.default_rng(1234)
-    data = _rand(rng, api.F32, rows * cols)
-    for layout, apply in LAYOUT_AXIS:
-        d = api.make_desc(api.F32, api.F32, rows, cols, layout=layout, apply=apply,
+    data = _rand(rng, in_dt, rows * cols)
+    for layout, apply in LAYOUT_AXIS if in_dt == out_dt == api.F32 else [(api.ROW_MAJOR, api.ALONG_ROWS)]:
+        d = api.make_desc(in_dt, out_dt, rows, cols, layout=layout, apply=apply,
                           main_op=api.MAIN_SQ, final_op=api.FIN_SQRT)
-        u.check_against_oracle(d, data, label=f"thick {rows}x{cols} l{layout} a{apply}")
+        first = u.check_against_oracle(d, data, label=f"thick {rows}x{cols} l{layout} a{apply}")
+        d.inplace = 1
+        u.check_against_oracle(d, data, old_raw=first,
+                               label=f"thick {rows}x{cols} l{layout} a{apply} inplace")
 
 
 # Many long rows: the automatic plan gives each row a team of 64, 128 or 256 threads
@@ -344,6 +350,11 @@ def test_kvp_arg_reduce(gpu, in_dt, out_dt, red):
         first = u.check_against_oracle(d, data, label=f"kvp {rows}x{cols}")
         d.inplace = 1
         u.check_against_oracle(d, data, old_raw=first, label=f"kvp {rows}x{cols} inplace")
+        # the reference's own init, {0, 0} (reduce.cu:360-385): a row whose values all lose
+        # against 0 returns it
+        d0 = api.make_desc(in_dt, out_dt, rows, cols, main_op=api.MAIN_KVP, reduce_op=red,
+                           init_i=0, init_f=0.0)
+        u.check_against_oracle(d0, data, label=f"kvp {rows}x{cols} init {{0, 0}}")
 
 
 @pytest.mark.parametrize("plan", [api.PLAN_AUTO, api.PLAN_ROW_WAVE, api.PLAN_ROW_BLOCK,
