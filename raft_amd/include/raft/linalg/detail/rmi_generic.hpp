@@ -15,8 +15,12 @@
 // The kernels are wave64 / gfx950 code: 16-byte lane loads for arithmetic element
 // types, ds_bpermute butterflies on 32-bit words for accumulators of any trivially
 // copyable type, LDS across waves.  They are simpler than the library's tuned
-// kernels (no compensated sums: accumulation happens in OutType with the caller's
-// reduce_op, exactly as written).
+// kernels.  Accumulation happens in OutType with the caller's reduce_op, exactly as
+// written, with one exception the reference makes too
+// (coalesced_reduction-inl.cuh:255,421,568, strided_reduction.cuh:146): when reduce_op is
+// raft::add_op and OutType is float or double, lanes, workgroups and partial results carry
+// a wider sum (fp64 for float; a Kahan-Babuska-Neumaier pair for double) that is rounded
+// to OutType once, before final_op.
 #pragma once
 
 #if !defined(__HIPCC__)
@@ -63,6 +67,55 @@ __device__ __forceinline__ T group_reduce(T acc, int G, Red& red)
     acc = red(acc, shfl_xor_any(acc, m));
   return acc;
 }
+
+// ---- wider accumulators for sums --------------------------------------------------------
+// sum + running compensation (Kahan-Babuska-Neumaier); value = s + c
+struct kbn_sum {
+  double s, c;
+  kbn_sum() = default;
+  __host__ __device__ kbn_sum(double v) : s(v), c(0.0) {}
+  __host__ __device__ explicit operator double() const { return s + c; }
+};
+struct wide_add {
+  __host__ __device__ double operator()(double a, double b) const { return a + b; }
+  __host__ __device__ kbn_sum operator()(const kbn_sum& a, const kbn_sum& b) const
+  {
+    kbn_sum r;
+    r.s = a.s + b.s;
+    // the low-order bits that the addition dropped, taken from the smaller operand
+    const double lost = (a.s < 0 ? -a.s : a.s) >= (b.s < 0 ? -b.s : b.s) ? (a.s - r.s) + b.s
+                                                                          : (b.s - r.s) + a.s;
+    r.c = (a.c + b.c) + lost;
+    return r;
+  }
+};
+template <typename Out>
+struct wide_sum {
+  using type = Out;
+};
+template <>
+struct wide_sum<float> {
+  using type = double;
+};
+template <>
+struct wide_sum<double> {
+  using type = kbn_sum;
+};
+template <typename Out, typename Red>
+constexpr bool sums_wide()
+{
+  return std::is_same_v<Red, raft::add_op> && (std::is_same_v<Out, float> || std::is_same_v<Out, double>);
+}
+// final_op behind the rounding of a wide sum to the caller's OutType
+template <typename Out, typename Fin>
+struct narrow_then {
+  Fin fin;
+  template <typename Acc>
+  __host__ __device__ auto operator()(const Acc& a) const
+  {
+    return fin(static_cast<Out>(static_cast<double>(a)));
+  }
+};
 
 // One 16-byte lane load (global_load_dwordx4) at any element-aligned address.  The input
 // is streamed once, so the load is marked non-temporal, except where the cache lines of a
@@ -158,8 +211,9 @@ __device__ __forceinline__ Out sweep_row(const In* row, Idx D, int first, int st
 }
 
 // G lanes of a wave per row (rows are contiguous, D elements each)
-template <typename In, typename Out, typename Idx, typename Main, typename Red, typename Fin>
-__global__ __launch_bounds__(kBlock) void rows_group_kernel(Out* dots, const In* data, Idx D,
+template <typename In, typename Out, typename Idx, typename Main, typename Red, typename Fin,
+          typename Dst>
+__global__ __launch_bounds__(kBlock) void rows_group_kernel(Dst* dots, const In* data, Idx D,
                                                             Idx N, Out init, bool inplace,
                                                             Main main_op, Red red, Fin fin,
                                                             int G, int logG, bool nt)
@@ -174,7 +228,8 @@ __global__ __launch_bounds__(kBlock) void rows_group_kernel(Out* dots, const In*
              : sweep_row<In, Out, Idx, false>(data + row * D, D, c, G, acc, main_op, red);
   }
   acc = group_reduce(acc, G, red);
-  if (c == 0 && row < (std::int64_t)N) dots[row] = fin(inplace ? red(dots[row], acc) : acc);
+  if (c == 0 && row < (std::int64_t)N)
+    dots[row] = fin(inplace ? red(static_cast<Out>(dots[row]), acc) : acc);
 }
 
 // Rows of G 16-byte lane loads, G not a power of two (3..32, the row's last load may be the
@@ -196,8 +251,9 @@ __device__ __forceinline__ T shfl_any(const T& v, int src)
   return r;
 }
 
-template <typename In, typename Out, typename Idx, typename Main, typename Red, typename Fin>
-__global__ __launch_bounds__(kBlock) void rows_anyg_kernel(Out* dots, const In* data, Idx D, Idx N,
+template <typename In, typename Out, typename Idx, typename Main, typename Red, typename Fin,
+          typename Dst>
+__global__ __launch_bounds__(kBlock) void rows_anyg_kernel(Dst* dots, const In* data, Idx D, Idx N,
                                                            Out init, bool inplace, Main main_op,
                                                            Red red, Fin fin, int G, unsigned invG)
 {
@@ -245,13 +301,14 @@ __global__ __launch_bounds__(kBlock) void rows_anyg_kernel(Out* dots, const In* 
 #pragma unroll
   for (int u = 0; u < U; ++u)
     if (live && c == 0 && row[u] < (std::int64_t)N)
-      dots[row[u]] = fin(inplace ? red(dots[row[u]], acc[u]) : acc[u]);
+      dots[row[u]] = fin(inplace ? red(static_cast<Out>(dots[row[u]]), acc[u]) : acc[u]);
 }
 
 // one 256-thread workgroup per chunk of a row; B chunks per row.  B == 1 writes the
 // outputs, B > 1 writes partials[row * B + b].
-template <typename In, typename Out, typename Idx, typename Main, typename Red, typename Fin>
-__global__ __launch_bounds__(kBlock) void rows_block_kernel(Out* dots, Out* partial,
+template <typename In, typename Out, typename Idx, typename Main, typename Red, typename Fin,
+          typename Dst>
+__global__ __launch_bounds__(kBlock) void rows_block_kernel(Dst* dots, Out* partial,
                                                             const In* data, Idx D, Idx N, Out init,
                                                             bool inplace, Main main_op, Red red,
                                                             Fin fin, int B, std::int64_t chunk)
@@ -272,7 +329,7 @@ __global__ __launch_bounds__(kBlock) void rows_block_kernel(Out* dots, Out* part
     for (int w = 1; w < kBlock / kWave; ++w)
       acc = red(acc, sm[w]);
     if (B == 1) {
-      dots[row] = fin(inplace ? red(dots[row], acc) : acc);
+      dots[row] = fin(inplace ? red(static_cast<Out>(dots[row]), acc) : acc);
     } else {
       partial[row * B + b] = acc;
     }
@@ -289,8 +346,9 @@ __global__ __launch_bounds__(kBlock) void rows_block_kernel(Out* dots, Out* part
 // contiguous span and the last 256 - TX * TY threads idle.  blockIdx.y strides over the steps
 // with four independent loads in flight per thread; the rows of a step are combined
 // through LDS.
-template <int V, typename In, typename Out, typename Idx, typename Main, typename Red, typename Fin>
-__global__ __launch_bounds__(kBlock) void cols_kernel(Out* dots, Out* partial, const In* data,
+template <int V, typename In, typename Out, typename Idx, typename Main, typename Red, typename Fin,
+          typename Dst>
+__global__ __launch_bounds__(kBlock) void cols_kernel(Dst* dots, Out* partial, const In* data,
                                                       Idx D, Idx N, Out init, bool inplace,
                                                       Main main_op, Red red, Fin fin, int TX,
                                                       int TY, int treeTY, int B)
@@ -356,7 +414,7 @@ __global__ __launch_bounds__(kBlock) void cols_kernel(Out* dots, Out* partial, c
       if (j >= first) {
         const std::int64_t col = col0 + j;
         if (B == 1) {
-          dots[col] = fin(inplace ? red(dots[col], sm[t * V + j]) : sm[t * V + j]);
+          dots[col] = fin(inplace ? red(static_cast<Out>(dots[col]), sm[t * V + j]) : sm[t * V + j]);
         } else {
           partial[col * B + blockIdx.y] = sm[t * V + j];
         }
@@ -367,8 +425,8 @@ __global__ __launch_bounds__(kBlock) void cols_kernel(Out* dots, Out* partial, c
 
 // second pass over partials[n_out][B]: LB lanes of a wave per output (LB a power of
 // two <= 64), each folding every LB-th partial, then a butterfly: a fixed order
-template <typename Out, typename Red, typename Fin>
-__global__ __launch_bounds__(kBlock) void fold_kernel(Out* dots, const Out* partial,
+template <typename Out, typename Red, typename Fin, typename Dst>
+__global__ __launch_bounds__(kBlock) void fold_kernel(Dst* dots, const Out* partial,
                                                       std::int64_t n_out, int B, Out init,
                                                       bool inplace, Red red, Fin fin, int LB,
                                                       int logLB)
@@ -393,7 +451,7 @@ __global__ __launch_bounds__(kBlock) void fold_kernel(Out* dots, const Out* part
       acc = red(acc, p[b]);
   }
   acc = group_reduce(acc, LB, red);
-  if (lb == 0 && o < n_out) dots[o] = fin(inplace ? red(dots[o], acc) : acc);
+  if (lb == 0 && o < n_out) dots[o] = fin(inplace ? red(static_cast<Out>(dots[o]), acc) : acc);
 }
 
 inline int pow2ceil(std::int64_t x)
@@ -419,19 +477,20 @@ inline void check_launch(const char* what)
                           hipGetErrorString(e));
 }
 
-template <typename Out, typename Red, typename Fin>
-void launch_fold(Out* dots, const Out* partial, std::int64_t n_out, int B, Out init, bool inplace,
+template <typename Out, typename Red, typename Fin, typename Dst>
+void launch_fold(Dst* dots, const Out* partial, std::int64_t n_out, int B, Out init, bool inplace,
                  Red red, Fin fin, hipStream_t stream)
 {
   const int LB             = B >= 64 ? 64 : pow2ceil(B);
   const std::int64_t grid  = (n_out * LB + kBlock - 1) / kBlock;
-  hipLaunchKernelGGL((fold_kernel<Out, Red, Fin>), dim3((unsigned)grid), dim3(kBlock), 0, stream,
+  hipLaunchKernelGGL((fold_kernel<Out, Red, Fin, Dst>), dim3((unsigned)grid), dim3(kBlock), 0, stream,
                      dots, partial, n_out, B, init, inplace, red, fin, LB, ilog2(LB));
 }
 
 // dots[N] from N contiguous rows of D elements
-template <typename In, typename Out, typename Idx, typename Main, typename Red, typename Fin>
-void coalesced(Out* dots, const In* data, Idx D, Idx N, Out init, hipStream_t stream, bool inplace,
+template <typename In, typename Out, typename Idx, typename Main, typename Red, typename Fin,
+          typename Dst>
+void coalesced(Dst* dots, const In* data, Idx D, Idx N, Out init, hipStream_t stream, bool inplace,
                Main main_op, Red red, Fin fin)
 {
   if (N <= 0) return;
@@ -445,7 +504,7 @@ void coalesced(Out* dots, const In* data, Idx D, Idx N, Out init, hipStream_t st
       const int G              = (int)nloads;
       const int rows_per_block = (kWave / G) * 4 * (kBlock / kWave);
       const std::int64_t grid  = ((std::int64_t)N + rows_per_block - 1) / rows_per_block;
-      hipLaunchKernelGGL((rows_anyg_kernel<In, Out, Idx, Main, Red, Fin>), dim3((unsigned)grid),
+      hipLaunchKernelGGL((rows_anyg_kernel<In, Out, Idx, Main, Red, Fin, Dst>), dim3((unsigned)grid),
                          dim3(kBlock), 0, stream, dots, data, D, N, init, inplace, main_op, red, fin,
                          G, 65536u / (unsigned)G + 1);
       check_launch("rows_anyg_kernel");
@@ -461,7 +520,7 @@ void coalesced(Out* dots, const In* data, Idx D, Idx N, Out init, hipStream_t st
     const bool nt = ((std::int64_t)D * (std::int64_t)sizeof(In)) % 128 == 0 &&
                     reinterpret_cast<std::uintptr_t>(data) % 128 == 0;
     const std::int64_t grid  = ((std::int64_t)N + rows_per_block - 1) / rows_per_block;
-    hipLaunchKernelGGL((rows_group_kernel<In, Out, Idx, Main, Red, Fin>), dim3((unsigned)grid),
+    hipLaunchKernelGGL((rows_group_kernel<In, Out, Idx, Main, Red, Fin, Dst>), dim3((unsigned)grid),
                        dim3(kBlock), 0, stream, dots, data, D, N, init, inplace, main_op, red, fin,
                        G, ilog2(G), nt);
     check_launch("rows_group_kernel");
@@ -480,7 +539,7 @@ void coalesced(Out* dots, const In* data, Idx D, Idx N, Out init, hipStream_t st
   B                  = ((std::int64_t)D + chunk - 1) / chunk;
   Out* partial             = nullptr;
   if (B > 1) partial = static_cast<Out*>(scratch_alloc(sizeof(Out) * (std::size_t)N * B, stream));
-  hipLaunchKernelGGL((rows_block_kernel<In, Out, Idx, Main, Red, Fin>),
+  hipLaunchKernelGGL((rows_block_kernel<In, Out, Idx, Main, Red, Fin, Dst>),
                      dim3((unsigned)((std::int64_t)N * B)), dim3(kBlock), 0, stream, dots, partial,
                      data, D, N, init, inplace, main_op, red, fin, (int)B, chunk);
   check_launch("rows_block_kernel");
@@ -491,8 +550,9 @@ void coalesced(Out* dots, const In* data, Idx D, Idx N, Out init, hipStream_t st
   }
 }
 
-template <int V, typename In, typename Out, typename Idx, typename Main, typename Red, typename Fin>
-void launch_cols(Out* dots, const In* data, Idx D, Idx N, Out init, hipStream_t stream, bool inplace,
+template <int V, typename In, typename Out, typename Idx, typename Main, typename Red, typename Fin,
+          typename Dst>
+void launch_cols(Dst* dots, const In* data, Idx D, Idx N, Out init, hipStream_t stream, bool inplace,
                  Main main_op, Red red, Fin fin)
 {
   const std::int64_t lanes = ((std::int64_t)D + V - 1) / V;
@@ -510,7 +570,7 @@ void launch_cols(Out* dots, const In* data, Idx D, Idx N, Out init, hipStream_t 
   if (B > 4096) B = 4096;
   Out* partial = nullptr;
   if (B > 1) partial = static_cast<Out*>(scratch_alloc(sizeof(Out) * (std::size_t)D * B, stream));
-  hipLaunchKernelGGL((cols_kernel<V, In, Out, Idx, Main, Red, Fin>),
+  hipLaunchKernelGGL((cols_kernel<V, In, Out, Idx, Main, Red, Fin, Dst>),
                      dim3((unsigned)gridx, (unsigned)B), dim3(kBlock), 0, stream, dots, partial,
                      data, D, N, init, inplace, main_op, red, fin, TX, TY, pow2ceil(TY), (int)B);
   check_launch("cols_kernel");
@@ -522,8 +582,9 @@ void launch_cols(Out* dots, const In* data, Idx D, Idx N, Out init, hipStream_t 
 }
 
 // dots[D] from N rows of D contiguous elements (one output per column)
-template <typename In, typename Out, typename Idx, typename Main, typename Red, typename Fin>
-void strided(Out* dots, const In* data, Idx D, Idx N, Out init, hipStream_t stream, bool inplace,
+template <typename In, typename Out, typename Idx, typename Main, typename Red, typename Fin,
+          typename Dst>
+void strided(Dst* dots, const In* data, Idx D, Idx N, Out init, hipStream_t stream, bool inplace,
              Main main_op, Red red, Fin fin)
 {
   if (D <= 0) return;
@@ -540,19 +601,33 @@ void strided(Out* dots, const In* data, Idx D, Idx N, Out init, hipStream_t stre
 }
 
 // layout x axis dispatch of linalg/detail/reduce.cuh:36-48
+template <typename In, typename Acc, typename Out, typename Main, typename Red, typename Fin>
+void reduce_as(hipStream_t stream, Out* dots, const In* data, std::int64_t n_rows,
+               std::int64_t n_cols, bool row_major, bool along_rows, Acc init, bool inplace,
+               Main main_op, Red red, Fin fin)
+{
+  using Idx = std::int64_t;
+  const Idx D = row_major ? n_cols : n_rows, N = row_major ? n_rows : n_cols;
+  if (row_major == along_rows) {
+    // fold the contiguous dimension
+    coalesced<In, Acc, Idx>(dots, data, D, N, init, stream, inplace, main_op, red, fin);
+  } else {
+    strided<In, Acc, Idx>(dots, data, D, N, init, stream, inplace, main_op, red, fin);
+  }
+}
+
 template <typename In, typename Out, typename Main, typename Red, typename Fin>
 void reduce(hipStream_t stream, Out* dots, const In* data, std::int64_t n_rows,
             std::int64_t n_cols, bool row_major, bool along_rows, Out init, bool inplace,
             Main main_op, Red red, Fin fin)
 {
-  using Idx = std::int64_t;
-  if (row_major == along_rows) {
-    // fold the contiguous dimension
-    const Idx D = row_major ? n_cols : n_rows, N = row_major ? n_rows : n_cols;
-    coalesced<In, Out, Idx>(dots, data, D, N, init, stream, inplace, main_op, red, fin);
+  if constexpr (sums_wide<Out, Red>()) {
+    using Acc = typename wide_sum<Out>::type;
+    reduce_as<In, Acc>(stream, dots, data, n_rows, n_cols, row_major, along_rows,
+                       Acc((double)init), inplace, main_op, wide_add{}, narrow_then<Out, Fin>{fin});
   } else {
-    const Idx D = row_major ? n_cols : n_rows, N = row_major ? n_rows : n_cols;
-    strided<In, Out, Idx>(dots, data, D, N, init, stream, inplace, main_op, red, fin);
+    reduce_as<In, Out>(stream, dots, data, n_rows, n_cols, row_major, along_rows, init, inplace,
+                       main_op, red, fin);
   }
 }
 
@@ -617,9 +692,9 @@ __global__ __launch_bounds__(kBlock) void map_reduce_multi_kernel(Out* partial, 
   }
 }
 
-template <typename Out, typename Map, typename Red, typename... InTs>
-void map_reduce_multi(hipStream_t stream, Out* out, std::int64_t len, Out neutral, Map map, Red red,
-                      const InTs*... ins)
+template <typename Out, typename Dst, typename Map, typename Red, typename Fin, typename... InTs>
+void map_reduce_multi_as(hipStream_t stream, Dst* out, std::int64_t len, Out neutral, Map map,
+                         Red red, Fin fin, const InTs*... ins)
 {
   using raft::linalg::detail::map_min;
   using raft::linalg::detail::map_ratio_of;
@@ -638,10 +713,22 @@ void map_reduce_multi(hipStream_t stream, Out* out, std::int64_t len, Out neutra
   hipLaunchKernelGGL((map_reduce_multi_kernel<R, Out, Map, Red, InTs...>), dim3((unsigned)B),
                      dim3(kBlock), 0, stream, partial, len, per, neutral, map, red, ins...);
   check_launch("map_reduce_multi_kernel");
-  launch_fold(out, partial, (std::int64_t)1, (int)B, neutral, false, red, raft::identity_op(),
-              stream);
+  launch_fold(out, partial, (std::int64_t)1, (int)B, neutral, false, red, fin, stream);
   check_launch("fold_kernel");
   scratch_free(partial, stream);
+}
+
+template <typename Out, typename Map, typename Red, typename... InTs>
+void map_reduce_multi(hipStream_t stream, Out* out, std::int64_t len, Out neutral, Map map, Red red,
+                      const InTs*... ins)
+{
+  if constexpr (sums_wide<Out, Red>()) {
+    using Acc = typename wide_sum<Out>::type;
+    map_reduce_multi_as<Acc>(stream, out, len, Acc((double)neutral), map, wide_add{},
+                             narrow_then<Out, raft::identity_op>{raft::identity_op()}, ins...);
+  } else {
+    map_reduce_multi_as<Out>(stream, out, len, neutral, map, red, raft::identity_op(), ins...);
+  }
 }
 
 }  // namespace raft::detail::rmi::generic

@@ -685,6 +685,83 @@ TEST_CASE(MapReduceTwoArrays)
   }
 }
 
+// Sums of a caller's own main_op carry a wider accumulator, as the reference's kernels carry a
+// Kahan-Babuska-Neumaier compensation whenever reduce_op is raft::add_op
+// (linalg/detail/coalesced_reduction-inl.cuh:255,421,568).  The data is that of the reference's
+// accuracy test (cpp/tests/stats/sum.cu:54-76): along the reduced axis 3v, -v * L, +v * L repeat
+// with L = 1e7 (float) / 1e12 (double), so a plain accumulation in the element type loses the
+// small terms' low bits at every step and the exact sum is (len / 3) * T(3v).
+template <typename T>
+void compensated_lambda_sums(double large, double tol)
+{
+  raft::resources handle;
+  auto stream = raft::resource::get_cuda_stream(handle);
+  const T v   = (T)0.1;
+  struct shape {
+    int n_out, len;
+  };
+  // lane-group rows (power-of-two and other lane counts), split rows, few and many columns
+  for (bool contiguous : {true, false})
+    for (shape sh : {shape{501, 96}, shape{300, 3072}, shape{3, 3 << 19}, shape{40, 3 << 15}}) {
+      std::vector<T> h((size_t)sh.n_out * sh.len);
+      for (int k = 0; k < sh.n_out; ++k)
+        for (int i = 0; i < sh.len; ++i) {
+          const T x = i % 3 == 0 ? (T)(3.0 * (double)v)
+                                 : (T)((i % 3 == 1 ? -1.0 : 1.0) * (double)v * large);
+          h[contiguous ? (size_t)k * sh.len + i : (size_t)i * sh.n_out + k] = x;
+        }
+      auto d   = raft::make_device_vector<T, int>(handle, (int)h.size());
+      auto out = raft::make_device_vector<T, int>(handle, sh.n_out);
+      raft::update_device(d.data_handle(), h.data(), h.size(), stream);
+      auto main_op = [] __device__(T a, int) { return a; };  // a lambda: no library kernel
+      auto fin_op  = [] __device__(T x) { return x; };
+      for (bool inplace : {false, true}) {
+        std::vector<T> before((size_t)sh.n_out, (T)1000);
+        raft::update_device(out.data_handle(), before.data(), before.size(), stream);
+        if (contiguous) {
+          auto view = raft::make_device_matrix_view<const T, int, raft::row_major>(
+            d.data_handle(), sh.n_out, sh.len);
+          raft::linalg::reduce<raft::Apply::ALONG_ROWS>(handle, view, out.view(), (T)0, inplace,
+                                                        main_op, raft::add_op(), fin_op);
+        } else {
+          auto view = raft::make_device_matrix_view<const T, int, raft::row_major>(
+            d.data_handle(), sh.len, sh.n_out);
+          raft::linalg::reduce<raft::Apply::ALONG_COLUMNS>(handle, view, out.view(), (T)0, inplace,
+                                                           main_op, raft::add_op(), fin_op);
+        }
+        const double want =
+          (double)(sh.len / 3) * (double)(T)(3.0 * (double)v) + (inplace ? 1000.0 : 0.0);
+        auto got = to_host(out.data_handle(), (size_t)sh.n_out, stream);
+        bool ok  = true;
+        for (int k = 0; k < sh.n_out; ++k)
+          ok &= close(got[k], want, tol);
+        if (!ok)
+          std::printf("    contiguous=%d n_out=%d len=%d inplace=%d got %.17g want %.17g\n",
+                      (int)contiguous, sh.n_out, sh.len, (int)inplace, (double)got[0], want);
+        CHECK(ok);
+      }
+    }
+  // map over two arrays, then sum: the same pattern split over the two operands
+  const int len = 3 << 20;
+  std::vector<T> ha(len), hb(len);
+  for (int i = 0; i < len; ++i) {
+    ha[i] = i % 3 == 0 ? (T)(3.0 * (double)v) : (T)((i % 3 == 1 ? -1.0 : 1.0) * (double)v * large);
+    hb[i] = (T)0;
+  }
+  auto da  = raft::make_device_vector<T, int>(handle, len);
+  auto db  = raft::make_device_vector<T, int>(handle, len);
+  auto out = raft::make_device_scalar<T>(handle);
+  raft::update_device(da.data_handle(), ha.data(), ha.size(), stream);
+  raft::update_device(db.data_handle(), hb.data(), hb.size(), stream);
+  raft::linalg::mapReduce<T>(
+    out.data_handle(), (size_t)len, (T)0, [] __device__(T a, T b) { return a + b; },
+    raft::add_op(), stream, (const T*)da.data_handle(), (const T*)db.data_handle());
+  CHECK(close(to_host(out.data_handle(), 1, stream)[0],
+              (double)(len / 3) * (double)(T)(3.0 * (double)v), tol));
+}
+TEST_CASE(CompensatedLambdaSumsF) { compensated_lambda_sums<float>(1e7, 2e-7); }
+TEST_CASE(CompensatedLambdaSumsD) { compensated_lambda_sums<double>(1e12, 1e-13); }
+
 int main()
 {
   int n = 0;
