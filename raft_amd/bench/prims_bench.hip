@@ -14,6 +14,8 @@
 // lane, workgroups per CU (one-shot grid or persistent), and non-temporal loads / stores, at
 // 134 MB + 134 MB and 512 MB + 512 MB, over rotating buffers.  It is the roof that the
 // shapes with 1:1 traffic (row_normalize, row sums of 8-byte rows into int64) are held to.
+// read_roof is the same for kernels that only read (16-byte loads XORed into a register), at the
+// input sizes of the benchmark shapes from 10 MiB to 2.4 GiB.
 //
 // usage: prims_bench [--filter substring] [--min-iters N] [--max-bytes B] [--no-flush]
 #include <raft/core/device_mdarray.hpp>
@@ -443,6 +445,114 @@ void bench_copy_roof(Harness& h)
   (void)hipEventDestroy(e1);
 }
 
+// ---- read roof ------------------------------------------------------------------------
+// What the GPU sustains when a kernel only reads: every lane XORs its 16-byte loads into a
+// register and one word per workgroup is written at the end (so that nothing can be dropped).
+template <int U, bool NT_LD, bool PERSIST>
+__global__ __launch_bounds__(256) void stream_read(const u32x4_t* __restrict__ in,
+                                                   unsigned* __restrict__ out, size_t nvec)
+{
+  __shared__ unsigned sm[4];
+  u32x4_t acc       = {0u, 0u, 0u, 0u};
+  const size_t step = (size_t)gridDim.x * 256 * U;
+  for (size_t base = (size_t)blockIdx.x * 256 * U; base < nvec; base += step) {
+    u32x4_t x[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const u32x4_t* p = in + base + (size_t)u * 256 + threadIdx.x;
+      x[u]             = NT_LD ? __builtin_nontemporal_load(p) : *p;
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      acc ^= x[u];
+    if (!PERSIST) break;
+  }
+  unsigned w = acc[0] ^ acc[1] ^ acc[2] ^ acc[3];
+  for (int m = 32; m >= 1; m >>= 1)
+    w ^= (unsigned)__shfl_xor((int)w, m, 64);
+  if ((threadIdx.x & 63) == 0) sm[threadIdx.x >> 6] = w;
+  __syncthreads();
+  if (threadIdx.x == 0) out[blockIdx.x] = sm[0] ^ sm[1] ^ sm[2] ^ sm[3];
+}
+
+template <int U, bool NT_LD>
+void read_roof_case(hipStream_t s, int n_cu, size_t bytes, std::vector<void*>& src, unsigned* out,
+                    hipEvent_t e0, hipEvent_t e1, double& best, std::string& best_name)
+{
+  const size_t nvec = bytes / 16;
+  for (int per_cu : {0, 2, 4, 8, 16}) {  // 0: one workgroup per 256 * U vectors
+    const size_t grid = per_cu == 0 ? nvec / (256 * U) : (size_t)n_cu * per_cu;
+    auto launch = [&](int i) {
+      const u32x4_t* a = static_cast<const u32x4_t*>(src[i % src.size()]);
+      if (per_cu == 0)
+        stream_read<U, NT_LD, false><<<dim3((unsigned)grid), 256, 0, s>>>(a, out, nvec);
+      else
+        stream_read<U, NT_LD, true><<<dim3((unsigned)grid), 256, 0, s>>>(a, out, nvec);
+    };
+    const int reps = 40;
+    for (int i = 0; i < 5; ++i)
+      launch(i);
+    RAFT_HIP_TRY(hipEventRecord(e0, s));
+    for (int i = 0; i < reps; ++i)
+      launch(i);
+    RAFT_HIP_TRY(hipEventRecord(e1, s));
+    RAFT_HIP_TRY(hipEventSynchronize(e1));
+    float ms = 0.f;
+    RAFT_HIP_TRY(hipEventElapsedTime(&ms, e0, e1));
+    const double us   = ms * 1e3 / reps;
+    const double gbps = (double)bytes / (us * 1e-6) / 1e9;
+    char name[160];
+    std::snprintf(name, sizeof name, "loads=%d nt_load=%d %s", U, (int)NT_LD,
+                  per_cu == 0 ? "one-shot" : (std::to_string(per_cu) + " wg/cu").c_str());
+    std::printf("%-34s %-22s %10.2f us %9.1f GB/s  %s\n", "read_roof",
+                (std::to_string(bytes >> 20) + "MiB").c_str(), us, gbps, name);
+    if (gbps > best) best = gbps, best_name = name;
+  }
+}
+
+// Sizes: those of the benchmark shapes (10, 32, 64, 128, 512 and 2440 MiB); the buffers rotate over
+// at least 512 MiB so that none is read from the memory-side cache.
+void bench_read_roof(Harness& h)
+{
+  if (!h.wanted("read_roof")) return;
+  int n_cu = 256;
+  RAFT_HIP_TRY(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, 0));
+  hipEvent_t e0, e1;
+  RAFT_HIP_TRY(hipEventCreate(&e0));
+  RAFT_HIP_TRY(hipEventCreate(&e1));
+  unsigned* out = nullptr;
+  RAFT_HIP_TRY(hipMalloc(&out, ((size_t)2560 << 20) / (16 * 256) * sizeof(unsigned)));
+  for (size_t mib : {(size_t)10, (size_t)32, (size_t)64, (size_t)128, (size_t)512, (size_t)2440}) {
+    const size_t bytes = mib << 20;
+    int nbuf           = (int)((((size_t)640 << 20) + bytes - 1) / bytes);
+    if (nbuf < 2) nbuf = 2;
+    if (nbuf > 64) nbuf = 64;
+    std::vector<void*> src(nbuf);
+    for (int i = 0; i < nbuf; ++i) {
+      RAFT_HIP_TRY(hipMalloc(&src[i], bytes));
+      fill_words<<<2048, 256, 0, h.stream()>>>(static_cast<unsigned*>(src[i]), bytes / 4, 29u + i);
+    }
+    RAFT_HIP_TRY(hipStreamSynchronize(h.stream()));
+    double best = 0.0;
+    std::string best_name;
+#define RAFT_READ_ROOF(U)                                                              \
+  read_roof_case<U, false>(h.stream(), n_cu, bytes, src, out, e0, e1, best, best_name); \
+  read_roof_case<U, true>(h.stream(), n_cu, bytes, src, out, e0, e1, best, best_name)
+    RAFT_READ_ROOF(1);
+    RAFT_READ_ROOF(2);
+    RAFT_READ_ROOF(4);
+    RAFT_READ_ROOF(8);
+#undef RAFT_READ_ROOF
+    std::printf("%-34s %-22s best %9.1f GB/s  %s\n", "read_roof/best",
+                (std::to_string(bytes >> 20) + "MiB").c_str(), best, best_name.c_str());
+    for (int i = 0; i < nbuf; ++i)
+      (void)hipFree(src[i]);
+  }
+  (void)hipFree(out);
+  (void)hipEventDestroy(e0);
+  (void)hipEventDestroy(e1);
+}
+
 }  // namespace
 
 int main(int argc, char** argv)
@@ -483,5 +593,6 @@ int main(int argc, char** argv)
   bench_mat_vec_op<double, false>(h);
   bench_mat_vec_op<double, true>(h);
   bench_copy_roof(h);
+  bench_read_roof(h);
   return 0;
 }
