@@ -15,7 +15,8 @@
 // 134 MB + 134 MB and 512 MB + 512 MB, over rotating buffers.  It is the roof that the
 // shapes with 1:1 traffic (row_normalize, row sums of 8-byte rows into int64) are held to.
 // read_roof is the same for kernels that only read (16-byte loads XORed into a register), at the
-// input sizes of the benchmark shapes from 10 MiB to 2.4 GiB.
+// input sizes of the benchmark shapes from 10 MiB to 2.4 GiB.  call_path times back-to-back calls of
+// the smallest benchmark shape from a native loop (C ABI, header API, HIP graph replay).
 //
 // usage: prims_bench [--filter substring] [--min-iters N] [--max-bytes B] [--no-flush]
 #include <raft/core/device_mdarray.hpp>
@@ -29,7 +30,10 @@
 #include <raft/matrix/argmin.cuh>
 #include <raft/util/cudart_utils.hpp>
 
+#include <rmi_reduce.h>
+
 #include <algorithm>
+#include <chrono>
 #include <cstdint>
 #include <cstdio>
 #include <cstdlib>
@@ -553,6 +557,85 @@ void bench_read_roof(Harness& h)
   (void)hipEventDestroy(e1);
 }
 
+// ---- call path ------------------------------------------------------------------------
+// Back-to-back calls of the smallest benchmark shape (row sums of 10000 x 256 floats, 10 MB:
+// 1.3 us at 8 TB/s) over 64 rotating inputs, issued from C++ so that the caller's own cost per
+// call is that of a native loop: through the C ABI, through the header API, and as the replay of
+// one HIP graph holding the same launches.  Prints the time per call by events and the host's
+// time to issue a call.
+void bench_call_path(Harness& h)
+{
+  if (!h.wanted("call_path")) return;
+  const int rows = 10000, cols = 256, nbuf = 64, reps = 2048;
+  std::vector<DeviceBuf<float>*> in;
+  for (int i = 0; i < nbuf; ++i) {
+    in.push_back(new DeviceBuf<float>((size_t)rows * cols));
+    in.back()->uniform(-1.0, 1.0, h.stream());
+  }
+  DeviceBuf<float> out((size_t)rows);
+  hipStream_t s = h.stream();
+  hipEvent_t e0, e1;
+  RAFT_HIP_TRY(hipEventCreate(&e0));
+  RAFT_HIP_TRY(hipEventCreate(&e1));
+  rmi_reduce_desc d{};
+  d.in_dtype = RMI_F32, d.out_dtype = RMI_F32, d.layout = RMI_ROW_MAJOR, d.apply = RMI_ALONG_ROWS;
+  d.n_rows = rows, d.n_cols = cols;
+  d.main_op = RMI_MAIN_IDENTITY, d.reduce_op = RMI_RED_ADD, d.final_op = RMI_FIN_IDENTITY;
+  auto via_abi = [&](int i) {
+    if (rmi_reduce(&d, in[i % nbuf]->p, out.p, nullptr, 0, s) != RMI_OK) std::abort();
+  };
+  auto via_header = [&](int i) {
+    raft::linalg::reduce<true, true>(out.p, (const float*)in[i % nbuf]->p, cols, rows, 0.0f, s);
+  };
+  auto timed = [&](const char* what, auto&& call) {
+    for (int i = 0; i < 64; ++i)
+      call(i);
+    RAFT_HIP_TRY(hipStreamSynchronize(s));
+    const auto t0 = std::chrono::steady_clock::now();
+    RAFT_HIP_TRY(hipEventRecord(e0, s));
+    for (int i = 0; i < reps; ++i)
+      call(i);
+    RAFT_HIP_TRY(hipEventRecord(e1, s));
+    const auto t1 = std::chrono::steady_clock::now();
+    RAFT_HIP_TRY(hipEventSynchronize(e1));
+    float ms = 0.f;
+    RAFT_HIP_TRY(hipEventElapsedTime(&ms, e0, e1));
+    const double us = ms * 1e3 / reps;
+    std::printf("%-34s %-22s %10.2f us %9.1f GB/s  host issues a call in %.2f us\n",
+                (std::string("call_path/") + what).c_str(), shape2(rows, cols).c_str(), us,
+                (double)rows * (cols + 1) * 4 / (us * 1e-6) / 1e9,
+                std::chrono::duration<double, std::micro>(t1 - t0).count() / reps);
+  };
+  timed("c_abi", via_abi);
+  timed("header", via_header);
+  // the same launches as one graph: 256 calls captured, replayed reps / 256 times
+  hipGraph_t graph;
+  hipGraphExec_t exec;
+  RAFT_HIP_TRY(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal));
+  for (int i = 0; i < 256; ++i)
+    via_abi(i);
+  RAFT_HIP_TRY(hipStreamEndCapture(s, &graph));
+  RAFT_HIP_TRY(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0));
+  RAFT_HIP_TRY(hipGraphLaunch(exec, s));
+  RAFT_HIP_TRY(hipStreamSynchronize(s));
+  RAFT_HIP_TRY(hipEventRecord(e0, s));
+  for (int i = 0; i < reps / 256; ++i)
+    RAFT_HIP_TRY(hipGraphLaunch(exec, s));
+  RAFT_HIP_TRY(hipEventRecord(e1, s));
+  RAFT_HIP_TRY(hipEventSynchronize(e1));
+  float ms = 0.f;
+  RAFT_HIP_TRY(hipEventElapsedTime(&ms, e0, e1));
+  std::printf("%-34s %-22s %10.2f us %9.1f GB/s\n", "call_path/hip_graph",
+              shape2(rows, cols).c_str(), ms * 1e3 / reps,
+              (double)rows * (cols + 1) * 4 / (ms * 1e-3 / reps) / 1e9);
+  RAFT_HIP_TRY(hipGraphExecDestroy(exec));
+  RAFT_HIP_TRY(hipGraphDestroy(graph));
+  for (auto* b : in)
+    delete b;
+  (void)hipEventDestroy(e0);
+  (void)hipEventDestroy(e1);
+}
+
 }  // namespace
 
 int main(int argc, char** argv)
@@ -594,5 +677,6 @@ int main(int argc, char** argv)
   bench_mat_vec_op<double, true>(h);
   bench_copy_roof(h);
   bench_read_roof(h);
+  bench_call_path(h);
   return 0;
 }
