@@ -171,7 +171,8 @@ typedef enum rmi_plan_kind {
   RMI_PLAN_ROW_BLOCK  = 3, /* a team of 128..1024 threads per row, LDS combine       */
   RMI_PLAN_ROW_SPLIT  = 4, /* several blocks per row + second pass over partials    */
   RMI_PLAN_COL_TILE   = 5, /* column reduction: column-contiguous lanes, row ranges
-                              per block, LDS combine, second pass over partials    */
+                              per block, LDS combine, second pass over partials
+                              (rows of 2 KB..20 KB: whole adjacent rows per block)  */
   RMI_PLAN_EMPTY      = 6  /* nothing to read: outputs get final_op(init) only      */
 } rmi_plan_kind;
 

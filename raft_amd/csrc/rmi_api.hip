@@ -106,8 +106,10 @@ PlanKey plan_key(const rmi_reduce_desc& d, uintptr_t misalign)
   return k;
 }
 
-int plan_uncached(const rmi_reduce_desc& d, uintptr_t misalign, Planned& p)
+int plan_uncached(const rmi_reduce_desc& d, uintptr_t misalign, Planned& p,
+                  bool own_descriptor = false)
 {
+  if (!own_descriptor && (d.flags & kFlagSmallWorkspace) != 0) return RMI_ERR_BAD_ENUM;
   int acc_bytes = 8;
   int rc        = classify(d, p.key, acc_bytes);
   if (rc != RMI_OK) return rc;
@@ -120,9 +122,11 @@ int plan_uncached(const rmi_reduce_desc& d, uintptr_t misalign, Planned& p)
 // caller that repeats a call (a serving loop, a solver's iteration) repeats its descriptor:
 // the last few plans of every host thread are kept, so such a call goes from its arguments
 // to the launch without validating and planning again.  Only successful plans are kept.
-int plan_for(const rmi_reduce_desc* desc, const Planned*& out, const void* in = nullptr)
+int plan_for(const rmi_reduce_desc* desc, const Planned*& out, const void* in = nullptr,
+             bool own_descriptor = false)
 {
   if (desc == nullptr) return RMI_ERR_NULL;
+  if (!own_descriptor && (desc->flags & kFlagSmallWorkspace) != 0) return RMI_ERR_BAD_ENUM;
   constexpr int kSlots = 8;
   struct Slot {
     PlanKey k;
@@ -141,7 +145,7 @@ int plan_for(const rmi_reduce_desc* desc, const Planned*& out, const void* in = 
   }
   Slot& s = slots[next];
   s.used  = false;
-  const int rc = plan_uncached(*desc, misalign, s.p);
+  const int rc = plan_uncached(*desc, misalign, s.p, own_descriptor);
   if (rc != RMI_OK) return rc;
   s.k    = k;
   s.used = true;
@@ -318,9 +322,10 @@ int rmi_reduce_noalloc(const rmi_reduce_desc* desc, const void* in, void* out, v
   if (desc == nullptr) return RMI_ERR_NULL;
   // the buffer's ticket words are zero from load time on and every launch leaves them zero
   rmi_reduce_desc d = *desc;
-  d.flags |= RMI_FLAG_WORKSPACE_ZEROED;
+  if ((d.flags & rmi::kFlagSmallWorkspace) != 0) return RMI_ERR_BAD_ENUM;
+  d.flags |= RMI_FLAG_WORKSPACE_ZEROED | rmi::kFlagSmallWorkspace;
   const rmi::Planned* p = nullptr;
-  int rc                = rmi::plan_for(&d, p, in);
+  int rc                = rmi::plan_for(&d, p, in, true);
   if (rc != RMI_OK) return rc;
   if (p->pl.ws_bytes > RMI_NOALLOC_SCRATCH_BYTES) return RMI_ERR_SCRATCH_LIMIT;
   // looked up at every device's first call, whether or not this plan needs scratch, so

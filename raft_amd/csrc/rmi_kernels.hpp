@@ -13,7 +13,9 @@
 //   row_block_kernel  teams of 64..1024 threads per row chunk, B chunks per row;
 //                     B == 1 writes outputs, B > 1 writes partials
 //   col_kernel        reduction along the strided dimension
+//   col_wide_kernel   ... of rows of more than 128 lane-loads: whole rows per workgroup step
 //   fold_kernel       second pass: partials[n_out][B] -> outputs
+//   fold_rows_kernel  second pass of col_wide_kernel: partials[B][n_out] -> outputs
 #pragma once
 
 #include "rmi_device.hpp"
@@ -883,6 +885,155 @@ __global__ __launch_bounds__(kBlock) void col_kernel(ColArgs a)
       }
     }
   }
+}
+
+// ---------------------------------------------------------------------------
+// Column reduction of wide rows: more than 128 lane-loads, and few enough for a workgroup to
+// hold a whole row.  The workgroup streams whole adjacent rows, i.e. one contiguous span of
+// the matrix, where col_kernel reads pieces of at most 2 KB at the row's stride (32768 x 4097
+// floats: 96 us there, 81 us this way; x 2049: 99 / 80 us).
+// A thread has K load slots with a set of accumulators each, as many as 256 bytes of
+// accumulators allow.  The 256 * K slots of the workgroup are dealt to the lane-loads of
+// a.TY adjacent rows (a bundle) in order: slot k of thread t is lane-load (k * 256 + t) %
+// nload of row (k * 256 + t) / nload of the bundle, so a slot always meets the same columns
+// and at most nload - 1 slots idle.  R bundles are in flight, and bundles are dealt
+// round-robin to the B workgroups.  Every load of a step is issued before the first is
+// used, none under a condition (a load behind a branch makes the compiler wait for all
+// earlier ones): idle slots load the row's first vector and their accumulators are dropped.
+// At the end the bundle's rows are combined through LDS in row order, and the partials are
+// stored [B][n_out], whole lines per workgroup; the epilogue is left to the second pass.
+// ---------------------------------------------------------------------------
+template <class P>
+constexpr int col_wide_sets()
+{
+  constexpr int k = 256 / (P::VEC * (int)sizeof(typename P::acc_t));
+  return k < 1 ? 1 : (k > 5 ? 5 : k);
+}
+constexpr int col_wide_bundles(int K) { return (10 + K - 1) / K; }
+
+template <class P>
+__global__ __launch_bounds__(kBlock) void col_wide_kernel(ColArgs a)
+{
+  using acc_t     = typename P::acc_t;
+  using in_t      = typename P::in_t;
+  constexpr int S = P::VEC;
+  constexpr int K = col_wide_sets<P>();
+  constexpr int R = col_wide_bundles(K);
+  extern __shared__ __align__(16) unsigned char col_wide_lds[];
+  acc_t* sm       = reinterpret_cast<acc_t*>(col_wide_lds);  // [rows of a bundle][nload * S]
+  const int t     = threadIdx.x;
+  const int nload = a.TX;  // lane-loads of a row: nvec + (tail > 0)
+  const int rb    = a.TY;  // rows of a bundle: 256 * K / nload
+  // byte offset of lane-load l within a row: whole vector l, or the vector that ends at the
+  // row's end (its first S - tail columns belong to the lane-load before it)
+  auto offset_of = [&](int l) { return l < a.nvec ? (i64)l * 16 : (a.n_out - S) * (i64)sizeof(in_t); };
+  i64 off[K];   // ... of slot k, counted from the bundle's first row
+  int sub[K];   // row of the bundle that slot k reads
+  int lane[K];  // its lane-load of that row
+  bool live[K];
+#pragma unroll
+  for (int k = 0; k < K; ++k) {
+    const unsigned f = (unsigned)(k * kBlock + t);
+    const unsigned q = f / (unsigned)nload;
+    sub[k]           = (int)q;
+    lane[k]          = (int)(f - q * (unsigned)nload);
+    live[k]          = (int)q < rb;
+    off[k]           = live[k] ? (i64)q * a.row_bytes + offset_of(lane[k]) : 0;
+  }
+  acc_t acc[K][S];
+#pragma unroll
+  for (int k = 0; k < K; ++k)
+#pragma unroll
+    for (int j = 0; j < S; ++j)
+      acc[k][j] = P::neutral();
+
+  const char* inb  = static_cast<const char*>(a.in);
+  const i64 step   = (i64)R * rb;  // rows per step
+  const i64 stride = (i64)a.B * step;
+  i64 r            = (i64)blockIdx.y * step;
+  for (; r + step <= a.len; r += stride) {
+    u32x4 x[R][K];
+#pragma unroll
+    for (int q = 0; q < R; ++q)
+#pragma unroll
+      for (int k = 0; k < K; ++k)
+        x[q][k] = load16(inb + (r + (i64)q * rb) * a.row_bytes + off[k]);
+    // all of the step's loads first: left to itself the scheduler trades loads in flight for
+    // registers and issues four or five of the ten before the first use
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int q = 0; q < R; ++q)
+#pragma unroll
+      for (int k = 0; k < K; ++k)
+        P::push_cols(acc[k], x[q][k], r + (i64)q * rb + sub[k]);
+  }
+  // the rows after the last whole step go to the workgroup whose turn it is, bundle by bundle
+  for (; r < a.len; r += rb) {
+#pragma unroll
+    for (int k = 0; k < K; ++k)
+      if (live[k] && r + sub[k] < a.len)
+        P::push_cols(acc[k], load16(inb + r * a.row_bytes + off[k]), r + sub[k]);
+  }
+
+  const int width = nload * S;
+#pragma unroll
+  for (int k = 0; k < K; ++k) {
+    if (live[k]) {
+#pragma unroll
+      for (int j = 0; j < S; ++j)
+        sm[sub[k] * width + lane[k] * S + j] = acc[k][j];
+    }
+  }
+  __syncthreads();
+  acc_t* out = static_cast<acc_t*>(a.partial) + (i64)blockIdx.y * a.n_out;
+  for (int idx = t; idx < width; idx += kBlock) {
+    const int l = idx / S, j = idx - l * S;
+    // the last, partial lane-load holds the row's last S columns; its first S - tail are
+    // already covered by the lane-load before it
+    if (l == a.nvec && j < S - a.tail) continue;
+    acc_t v = sm[idx];
+    for (int q = 1; q < rb; ++q)
+      P::merge(v, sm[q * width + idx]);
+    out[l < a.nvec ? (i64)idx : a.n_out - S + j] = v;
+  }
+}
+
+// Second pass of col_wide_kernel over partials[B][n_out]: a workgroup folds 16 adjacent
+// outputs (its loads cover whole lines of 8-byte accumulators); thread (c, s) folds partials
+// s, s + 16, ... of output c in that order, then the 16 s are combined in a fixed tree.
+template <class P>
+__global__ __launch_bounds__(kBlock) void fold_rows_kernel(FoldArgs a)
+{
+  using acc_t = typename P::acc_t;
+  __shared__ acc_t sm[kBlock];
+  const int t = threadIdx.x;
+  const int c = t & 15;
+  const int s = t >> 4;
+  const i64 o = (i64)blockIdx.x * 16 + c;
+  acc_t acc   = P::neutral();
+  if (o < a.n_out) {
+    const acc_t* p = static_cast<const acc_t*>(a.partial) + o;
+    int b          = s;
+    constexpr int U = 8;  // 256 partials per output: two rounds of loads per thread
+    for (; b + (U - 1) * 16 < a.B; b += U * 16) {
+      acc_t x[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        x[u] = p[(i64)(b + u * 16) * a.n_out];
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        P::merge(acc, x[u]);
+    }
+    for (; b < a.B; b += 16)
+      P::merge(acc, p[(i64)b * a.n_out]);
+  }
+  sm[t] = acc;
+  __syncthreads();
+  for (int h = 8; h >= 1; h >>= 1) {
+    if (s < h) P::merge(sm[t], sm[t + h * 16]);
+    __syncthreads();
+  }
+  if (s == 0 && o < a.n_out) finish<P>(a.epi, o, sm[t]);
 }
 
 // ---------------------------------------------------------------------------

@@ -62,6 +62,10 @@ int run(const PlanX& pl, const Problem& pr, hipStream_t st)
                   kTeamUnroll == kPlanTeamUnroll && kStageBytes == kStageBytesPerWave &&
                   kFan == kTicketFan && kLineWords * 4 == kTicketLineBytes,
                 "plan selector and kernels must agree on block size and unroll");
+  static_assert(col_wide_bundles(1) == col_wide_bundles_of(1) && col_wide_bundles(2) == col_wide_bundles_of(2) &&
+                  col_wide_bundles(3) == col_wide_bundles_of(3) && col_wide_bundles(4) == col_wide_bundles_of(4) &&
+                  col_wide_bundles(5) == col_wide_bundles_of(5) && kColWideMaxSets == 5,
+                "plan selector and wide-row column kernel must agree on rows per step");
   int rc = RMI_OK;
   switch (pl.kind) {
     case RMI_PLAN_EMPTY:
@@ -153,6 +157,24 @@ int run(const PlanX& pl, const Problem& pr, hipStream_t st)
         a.rem       = (pl.len - pl.group_len * pl.group) * pl.n_out;
       }
       const dim3 grid((unsigned)pl.gridx, (unsigned)pl.B);
+      if (pl.wide > 0) {
+        if constexpr (P::CLS != kClsFloat) {
+          return RMI_ERR_UNSUPPORTED;  // planned for plain and compensated floating sums only
+        } else {
+          if (col_wide_sets<P>() != pl.wide) return RMI_ERR_UNSUPPORTED;
+          const size_t lds_bytes =
+            (size_t)pl.TY * pl.TX * P::VEC * sizeof(typename P::acc_t);  // at most 64 KB
+          hipLaunchKernelGGL((col_wide_kernel<P>), grid, dim3(kBlock), lds_bytes, st, a);
+          FoldArgs f{};
+          f.partial = partials_of(pr.ws);
+          f.n_out   = pl.n_out;
+          f.B       = pl.B;
+          f.epi     = pr.epi;
+          hipLaunchKernelGGL((fold_rows_kernel<P>), dim3((unsigned)ceildiv(pl.n_out, 16)),
+                             dim3(kBlock), 0, st, f);
+        }
+        break;
+      }
       if (pl.vec16)
         hipLaunchKernelGGL((col_kernel<P, true>), grid, dim3(kBlock), 0, st, a);
       else

@@ -27,6 +27,9 @@ constexpr int kWavesPerCu = 32;  // 8 resident waves on each of the 4 SIMDs
 // lose 2 and 8 points to queueing in the memory system.
 constexpr int kColBlocksPerCu = 2;
 constexpr int kColMaxLanes = 128;     // COL_TILE: most lanes of a workgroup along one row
+constexpr int kColWideMaxSets = 5;    // COL_TILE, wide rows: most load slots per thread
+// row bundles in flight in the wide-row column kernel whose threads have K load slots
+constexpr int col_wide_bundles_of(int K) { return (10 + K - 1) / K; }
 constexpr int64_t kGroupMinLen = 256;  // COL_TILE: fewest row groups worth reading rows in groups
 constexpr int kLdsPerCu       = 160 * 1024;  // LDS bytes of one gfx950 CU
 constexpr int64_t kBytesInFlightPerCu = 80 * 1024;  // target of the wave-per-row plan
@@ -46,6 +49,12 @@ constexpr int64_t kTicketLines   = kTicketBytes / kTicketLineBytes;
 constexpr int kTicketFan         = 16;
 // lines a split row needs: one per group of kTicketFan chunks, and the row's own
 inline int64_t ticket_lines_per_row(int B) { return B <= kTicketFan ? 1 : ceildiv_i(B, kTicketFan) + 1; }
+
+// Descriptor flag of the library's own (rmi_reduce_noalloc sets it on its copy of the
+// descriptor, callers' descriptors that carry it are refused): the partials have to fit the
+// static buffer of RMI_NOALLOC_SCRATCH_BYTES, so a plan whose partials outgrow it is passed
+// over when another one serves the shape with fewer.
+constexpr int32_t kFlagSmallWorkspace = 1 << 30;
 
 struct PlanX {
   int kind        = RMI_PLAN_EMPTY;
@@ -78,6 +87,9 @@ struct PlanX {
   int group       = 0;  // COL_TILE: > 0 when `group` consecutive rows are read as one row
   int64_t group_len  = 0;  // COL_TILE, grouped: whole groups (rows of the widened matrix)
   int64_t group_nvec = 0;  // COL_TILE, grouped: 16-byte vectors per group
+  int wide        = 0;  // COL_TILE: > 0 when a workgroup streams whole rows (TX lane-loads each,
+                        // TY rows side by side in the `wide` load slots of its threads;
+                        // partials laid out [B][n_out])
   int64_t grid_blocks    = 0;
   int passes             = 1;
   bool fused_fold        = false;  // ROW_SPLIT: the last workgroup of a row folds its partials
@@ -155,7 +167,7 @@ inline int classify(const rmi_reduce_desc& d, PolicyKey& key, int& acc_bytes)
   if (d.reduce_op < RMI_RED_ADD || d.reduce_op > RMI_RED_ARGMIN) return RMI_ERR_BAD_ENUM;
   if (d.final_op < RMI_FIN_IDENTITY || d.final_op > RMI_FIN_KEY) return RMI_ERR_BAD_ENUM;
   if (d.plan_hint < RMI_PLAN_AUTO || d.plan_hint > RMI_PLAN_EMPTY) return RMI_ERR_BAD_ENUM;
-  if ((d.flags & ~RMI_FLAG_WORKSPACE_ZEROED) != 0) return RMI_ERR_BAD_ENUM;
+  if ((d.flags & ~(RMI_FLAG_WORKSPACE_ZEROED | kFlagSmallWorkspace)) != 0) return RMI_ERR_BAD_ENUM;
   if (d.n_rows < 0 || d.n_cols < 0) return RMI_ERR_BAD_SHAPE;
   if (is_kvp_dtype(d.in_dtype)) return RMI_ERR_UNSUPPORTED;
 
@@ -304,6 +316,42 @@ inline int make_plan(const rmi_reduce_desc& d,
       p.gridx = ceildiv(lanes, p.TX);
       p.dense = (p.TX & (p.TX - 1)) != 0 || p.TX > 64;
       p.logTX = p.dense ? 0 : ilog2(p.TX);
+    }
+    // Rows of more than kColMaxLanes lane-loads that a workgroup can hold whole: it streams
+    // adjacent rows, one contiguous span of the matrix.  A thread has K load slots, as many as
+    // 256 bytes of accumulators allow (5 for 4- and 8-byte elements, 4 for 2-byte ones); the
+    // workgroup's 256 * K slots take the lane-loads of 256 * K / lanes adjacent rows (a
+    // bundle: more than half of the slots get a lane-load), ten or so lane-loads per thread
+    // are in flight, one workgroup per CU.  Taken when every workgroup gets sixteen steps or
+    // more (4096 x 4097 floats lose 16 % with eight).  Longer rows, and accumulators whose step
+    // is arithmetic-bound at four waves per CU (arg-reductions 33-38 % slower, byte sums
+    // 25 %), keep the layout above.  Measured at 512 MB, % of 8 TB/s, the layout above / this
+    // one: fp32 D = 513: 76 / 81, 768: 74 / 82, 1025: 70 / 80, 1536: 73 / 82, 2049: 66 / 80,
+    // 3000: 65 / 78, 4096: 72 / 81, 4097: 67 / 78 (640 and 1024: 84 / 81 and 82 / 81);
+    // fp64 D = 300: 76 / 82, 513: 70 / 83, 1025: 67 / 82, 2049: 69 / 80; bf16 D = 1030: 72 / 80.
+    if (p.group == 0 && p.vec16 && lanes > kColMaxLanes &&
+        (key.family == kFamFloat || key.family == kFamKbn)) {
+      int K = 256 / (p.step * acc_bytes);
+      K     = K < 1 ? 1 : (K > kColWideMaxSets ? kColWideMaxSets : K);
+      const int64_t slots = (int64_t)kPlanBlock * K;
+      if (lanes <= slots) {
+        const int64_t bundle = slots / lanes;
+        const int64_t step   = bundle * col_wide_bundles_of(K);
+        const int64_t B      = n_cu;
+        const size_t ws      = kTicketBytes + (size_t)p.n_out * B * acc_bytes;
+        const bool too_large = (d.flags & kFlagSmallWorkspace) != 0 && ws > RMI_NOALLOC_SCRATCH_BYTES;
+        if (rows >= B * step * 16 && !too_large) {
+          p.wide        = K;
+          p.TX          = (int)lanes;
+          p.TY          = (int)bundle;
+          p.gridx       = 1;
+          p.B           = (int)B;
+          p.grid_blocks = p.B;
+          p.passes      = 2;  // the epilogue is the second pass's
+          p.ws_bytes    = ws;
+          return RMI_OK;
+        }
+      }
     }
     // row tiles of TY*unroll rows are dealt round-robin to B blocks: kColBlocksPerCu
     // blocks per CU, but at least two tiles per block

@@ -13,6 +13,7 @@ int failures = 0;
 long planned[8] = {0, 0, 0, 0, 0, 0, 0, 0};
 long staged_plans = 0;
 long grouped_plans = 0;
+long wide_plans = 0;
 #define REQUIRE(cond)                                                              \
   do {                                                                             \
     if (!(cond)) {                                                                 \
@@ -116,6 +117,22 @@ void check(const rmi_reduce_desc& d, int n_cu, uintptr_t in_misalign)
       break;
     case RMI_PLAN_COL_TILE:
       REQUIRE(p.strided);
+      if (p.wide > 0) {
+        ++wide_plans;
+        // whole rows per workgroup: the slots of its threads hold TY adjacent rows of TX
+        // lane-loads, more than half of them in use, in at most 64 KB of LDS at the end
+        const int64_t slots = (int64_t)kPlanBlock * p.wide;
+        REQUIRE(p.wide >= 1 && p.wide <= rmi::kColWideMaxSets && p.wide * p.step * p.acc_bytes <= 256);
+        REQUIRE(key.family == rmi::kFamFloat || key.family == rmi::kFamKbn);
+        REQUIRE(p.group == 0 && p.vec16 && p.TX == nload && p.TX > rmi::kColMaxLanes && p.TX <= slots);
+        REQUIRE(p.TY >= 1 && (int64_t)p.TY * p.TX <= slots && (int64_t)(p.TY + 1) * p.TX > slots);
+        REQUIRE((int64_t)p.TY * p.TX * 2 > slots);
+        REQUIRE((int64_t)p.TY * p.TX * p.step * p.acc_bytes <= 65536);
+        REQUIRE(p.gridx == 1 && p.B == n_cu && p.grid_blocks == p.B && p.passes == 2);
+        REQUIRE(p.len >= (int64_t)p.B * p.TY * rmi::col_wide_bundles_of(p.wide) * 16);
+        REQUIRE(p.ws_bytes == rmi::kTicketBytes + (size_t)p.n_out * p.B * p.acc_bytes);
+        break;
+      }
       REQUIRE(p.TX >= 1 && p.TX <= 128 && p.TY == kPlanBlock / p.TX && p.TY >= 2);
       REQUIRE(p.dense == ((p.TX & (p.TX - 1)) != 0 || p.TX > 64));
       if (!p.dense) REQUIRE((1 << p.logTX) == p.TX);
@@ -201,9 +218,9 @@ int main()
       ++failures;
     }
   }
-  std::printf("plans checked: lanes %ld wave %ld block %ld split %ld col %ld empty %ld\n",
+  std::printf("plans checked: lanes %ld wave %ld block %ld split %ld col %ld (whole rows %ld) empty %ld\n",
               planned[RMI_PLAN_ROW_LANES], planned[RMI_PLAN_ROW_WAVE], planned[RMI_PLAN_ROW_BLOCK],
-              planned[RMI_PLAN_ROW_SPLIT], planned[RMI_PLAN_COL_TILE], planned[RMI_PLAN_EMPTY]);
+              planned[RMI_PLAN_ROW_SPLIT], planned[RMI_PLAN_COL_TILE], wide_plans, planned[RMI_PLAN_EMPTY]);
   for (int k = RMI_PLAN_ROW_LANES; k <= RMI_PLAN_EMPTY; ++k)
     if (planned[k] < 1000) {
       std::printf("  plan kind %d was hardly exercised\n", k);
@@ -211,6 +228,10 @@ int main()
     }
   if (grouped_plans < 1000) {
     std::printf("  grouped column plans were hardly exercised (%ld)\n", grouped_plans);
+    ++failures;
+  }
+  if (wide_plans < 1000) {
+    std::printf("  whole-row column plans were hardly exercised (%ld)\n", wide_plans);
     ++failures;
   }
   if (staged_plans < 1000) {

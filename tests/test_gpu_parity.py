@@ -610,6 +610,61 @@ def test_grouped_columns(gpu, in_dt, out_dt, kw, rows, cols, shift):
                            label=f"grouped {rows}x{cols} dt{in_dt} +{shift}")
 
 
+# Column reductions over rows of more than 128 lane-loads that one workgroup can hold whole
+# (floating sums, max and min): workgroups stream bundles of adjacent rows, one per CU, the
+# rows of a bundle are combined through LDS and the partials [workgroup][column] are folded
+# by a second launch.  Widths around the lane-load and slot boundaries, with and without
+# tail elements; row counts from the fewest that take this plan, with rows left over after
+# the last whole step; starts off a 16-byte boundary; both layouts; inplace.
+def _whole_row_rows(lanes, slots_per_thread, bundles):
+    """Fewest rows for which the planner streams whole rows: sixteen steps per workgroup."""
+    n_cu = 256
+    return n_cu * (256 * slots_per_thread // lanes) * bundles * 16
+
+
+@pytest.mark.parametrize("in_dt,out_dt,kw,slots,bundles,cols_list", [
+    (api.F32, api.F32, {}, 5, 2, (513, 516, 517, 700, 1024, 1025, 1300, 2049, 2560, 4097, 5119, 5120)),
+    (api.F32, api.F32, dict(main_op=api.MAIN_SQ, final_op=api.FIN_SQRT), 5, 2, (1027, 4099)),
+    (api.F32, api.F32, dict(reduce_op=api.RED_MAX, init_f=-np.inf), 5, 2, (519, 3001)),
+    (api.F32, api.F16, dict(main_op=api.MAIN_ABS, final_op=api.FIN_MUL_CONST, final_scalar=1e-3), 5, 2, (2051,)),
+    (api.F64, api.F64, {}, 5, 2, (257, 300, 513, 1025, 2049, 2560)),
+    (api.F64, api.F64, dict(reduce_op=api.RED_MIN, init_f=np.inf), 5, 2, (301, 1281)),
+    (api.BF16, api.F32, {}, 4, 3, (1025, 1030, 2056, 5500, 8191, 8192)),
+    (api.F16, api.F32, dict(main_op=api.MAIN_ABS), 4, 3, (1100, 2741)),
+])
+@pytest.mark.parametrize("extra,shift,col_major,inplace", [(0, 0, False, False), (37, 1, False, True),
+                                                           (5, 0, True, False)])
+def test_whole_row_columns(gpu, in_dt, out_dt, kw, slots, bundles, cols_list, extra, shift,
+                           col_major, inplace):
+    es = api.load().rmi_dtype_size(in_dt)
+    for cols in cols_list:
+        lanes = -(-cols * es // 16)
+        rows = _whole_row_rows(lanes, slots, bundles) + extra
+        rng = np.random.default_rng(cols * 3 + extra + shift)
+        data = _rand(rng, in_dt, rows * cols)
+        if kw.get("reduce_op") in (api.RED_MAX, api.RED_MIN):
+            data[rng.integers(0, data.size, 5000)] = np.nan
+            data.reshape(rows, cols)[:, 7] = np.nan  # a column of nothing but NaN keeps init
+        if col_major:
+            d = api.make_desc(in_dt, out_dt, cols, rows, layout=api.COL_MAJOR, apply=api.ALONG_ROWS,
+                              inplace=inplace, **kw)
+        else:
+            d = api.make_desc(in_dt, out_dt, rows, cols, apply=api.ALONG_COLUMNS, inplace=inplace, **kw)
+        pl = api.plan_query(d)
+        assert pl.kind == api.PLAN_COL_TILE and pl.passes == 2
+        assert pl.grid_blocks == 256 and pl.blocks_per_out == 256, (cols, pl.grid_blocks)
+        old = None
+        if inplace:
+            old = u.encode_out(out_dt, rng.uniform(1, 2, cols))
+        u.check_against_oracle(d, data, misalign_elems=shift, old_raw=old,
+                               label=f"whole rows {rows}x{cols} dt{in_dt} +{shift}")
+        # one row fewer than the plan needs: the layout for short matrices, the same values
+        if extra == 0 and cols == cols_list[0]:
+            d2 = api.make_desc(in_dt, out_dt, rows - 1, cols, apply=api.ALONG_COLUMNS, **kw)
+            assert api.plan_query(d2).grid_blocks != 256
+            u.check_against_oracle(d2, data[:(rows - 1) * cols], label="one row fewer")
+
+
 # Rows of 5 lane-loads, or of 6, 9..16, 18..21 and 28..32 with tail elements (up to 12 only for
 # 16-byte accumulators): one lane per lane-load, 64 / G whole
 # rows per wave step (G is not a power of two, the wave's last lanes idle).  Row counts around

@@ -93,6 +93,31 @@ def test_noalloc_refuses_plans_beyond_its_buffer(gpu):
     assert bool((out == 7.0).all()), "nothing may be launched"
 
 
+def test_noalloc_passes_over_plans_with_large_partials(gpu):
+    """Column sums of wide rows: rmi_reduce streams whole rows with one set of partials per
+    CU, more than the static buffer holds at this width; the entry point that allocates nothing
+    takes the layout with fewer partials instead of refusing the call."""
+    import torch
+    lib = api.load()
+    rows, cols = 16384, 4097
+    d = api.make_desc(api.F32, api.F32, rows, cols, apply=api.ALONG_COLUMNS)
+    assert lib.rmi_reduce_workspace_bytes(C.byref(d)) > api.NOALLOC_SCRATCH_BYTES
+    x = torch.randn(rows * cols, device="cuda")
+    a, b, _ = _both(d, x, 4, cols)
+    a, b = a.view(np.float32), b.view(np.float32)
+    # both accumulate in fp64 and round once; the partial sums are grouped differently
+    assert np.allclose(a, b, rtol=3e-7, atol=0), np.abs(a - b).max()
+    want = x.view(rows, cols).sum(dim=0, dtype=torch.float64).cpu().numpy()
+    assert np.allclose(b, want, rtol=1e-6, atol=1e-6)
+    # the library's own flag bit is refused from callers
+    d.flags = 1 << 30
+    assert lib.rmi_reduce_workspace_bytes(C.byref(d)) == 0
+    out = torch.zeros(cols, device="cuda")
+    sptr = torch.cuda.current_stream().cuda_stream
+    assert lib.rmi_reduce_noalloc(C.byref(d), x.data_ptr(), out.data_ptr(), sptr) == api.ERR_BAD_ENUM
+    assert lib.rmi_reduce(C.byref(d), x.data_ptr(), out.data_ptr(), None, 0, sptr) == api.ERR_BAD_ENUM
+
+
 def test_noalloc_under_graph_capture(gpu):
     """The caller this entry point is for: a captured stream, replayed over new inputs."""
     import torch
