@@ -555,6 +555,40 @@ def main():
                     pct_of_peak=100.0 * nb / (ms * 1e-3) / 1e9 / PEAK_HBM_GBPS,
                     check={"torch_fp64": ok})
 
+    def extra_wide_columns():
+        # column sums over rows of 16 KB that are not whole vectors: every workgroup streams
+        # whole adjacent rows (partials per workgroup, folded by the second launch)
+        rows, cols = 32768, 4097
+        xs = [mk_normal(rows, cols, 11 + 7919 * i) for i in range(3)]
+        out = torch.empty(cols, dtype=torch.float32, device="cuda")
+        d = api.make_desc(api.F32, api.F32, rows, cols, apply=api.ALONG_COLUMNS)
+        ref = C.byref(d)
+        nws = lib.rmi_reduce_workspace_bytes(ref)
+        ws = torch.empty(max(nws, 16), dtype=torch.uint8, device="cuda")
+
+        def call(i):
+            return lib.rmi_reduce(ref, xs[i % 3].data_ptr(), out.data_ptr(), ws.data_ptr(), nws, sptr)
+        for i in range(5):
+            rc = call(i)
+            assert rc == 0, api.status_string(rc)
+        torch.cuda.synchronize()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        n = max(10, args.steps // 4)
+        e0.record(stream)
+        for i in range(n):
+            call(i)
+        e1.record(stream)
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / n
+        nb = rows * cols * 4 + cols * 4
+        want = xs[(n - 1) % 3].view(rows, cols).sum(dim=0, dtype=torch.float64)
+        ok = bool(torch.allclose(out.double(), want, rtol=1e-5, atol=1e-5))
+        return dict(workload="column sum fp32 32768x4097 (whole rows per workgroup)", ms_per_step=ms,
+                    alg_bytes=nb, GBps=nb / (ms * 1e-3) / 1e9,
+                    pct_of_peak=100.0 * nb / (ms * 1e-3) / 1e9 / PEAK_HBM_GBPS,
+                    check={"torch_fp64": ok})
+
     results = {}
     cpu = {}
     for name in names:
@@ -590,7 +624,8 @@ def main():
                      "traffic_source": PROFILE_SOURCE},
         "cpu_baseline": cpu.get(HEADLINE),
         "launch_floor_us": launch_floor_us(),
-        "extras": ({"row_normalize": extra_row_normalize(), "meanvar": extra_meanvar()}
+        "extras": ({"row_normalize": extra_row_normalize(), "meanvar": extra_meanvar(),
+                    "wide_columns": extra_wide_columns()}
                    if args.configs == "all" else {}),
         "configs": results,
         "cpu_baselines": cpu,

@@ -171,12 +171,13 @@ def main():
 
 
 def extras(out: Path, commit: str):
-    """Kernel durations of bench.py's extra workloads (row_normalize, meanvar) from OUT/ex."""
+    """Kernel durations of bench.py's extra workloads (row_normalize, meanvar, wide-row column sums)
+    from OUT/ex."""
     rows = list(csv.DictReader(open(_find_csv(out / "ex", "kernel_stats.csv"))))
     kt = {r["Name"]: r for r in rows}
     lines = []
     w = lines.append
-    w("rocprofv3 summary: row_normalize and meanvar on the benchmark shapes, one MI355X (gfx950)")
+    w("rocprofv3 summary: row_normalize, meanvar and wide-row column sums, one MI355X (gfx950)")
     w("=" * 88)
     w("")
     w(f"Library at commit {commit}.  Command (run from the repository root on the GPU box, TMPDIR=/tmp):")
@@ -190,7 +191,9 @@ def extras(out: Path, commit: str):
     work = [("row_normalize L2 fp32 1000000x128 (read + write)", "normalize_wave_kernel<rmi::PolF<float, 1, 0>", None,
              1024000000),
             ("meanvar fp32 10000000x64 row-major (one read)", "col_kernel<rmi::PolMeanVar<float>",
-             "fold_kernel<rmi::PolMeanVar<float>", 2560000512)]
+             "fold_kernel<rmi::PolMeanVar<float>", 2560000512),
+            ("column sum fp32 32768x4097 (whole rows)", "col_wide_kernel<rmi::PolF<float, 0, 0>",
+             "fold_rows_kernel<rmi::PolF<float, 0, 0>", 32768 * 4097 * 4 + 4097 * 4)]
     for label, k1, k2, alg in work:
         s1 = pick(kt, k1)
         if s1 is None:
@@ -208,7 +211,8 @@ def extras(out: Path, commit: str):
     w("The same run's durations of the reduction kernels (ns; the caches are swept between the")
     w("single timed calls, so launch counts include those):")
     for n, r in kt.items():
-        if "rmi::" in n and "normalize" not in n and "MeanVar" not in n:
+        if "rmi::" in n and "normalize" not in n and "MeanVar" not in n and "col_wide" not in n \
+                and "fold_rows" not in n:
             w(f"  {n[:100]:100s} {r['Calls']:>6s} {float(r['AverageNs']):12.1f}")
     (ROOT / "profiles" / "row_normalize_meanvar_rocprofv3.txt").write_text("\n".join(lines) + "\n")
     print("\n".join(lines[:16]))
