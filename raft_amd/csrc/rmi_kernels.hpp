@@ -10,6 +10,8 @@
 //                     or the row's own lane-load count up to 32), 4 row-tiles in
 //                     flight per wave
 //   row_wave_kernel   G<=64 lanes of one wave per row, at most 4 loads per lane
+//   row_dense_kernel  whole adjacent rows per workgroup, one lane-load per load slot, rows
+//                     combined through LDS (rows whose lane-loads fill no power of two)
 //   row_block_kernel  teams of 64..1024 threads per row chunk, B chunks per row;
 //                     B == 1 writes outputs, B > 1 writes partials
 //   col_kernel        reduction along the strided dimension
@@ -884,6 +886,84 @@ __global__ __launch_bounds__(kBlock) void col_kernel(ColArgs a)
         }
       }
     }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Rows whose lane-load count fits neither a power-of-two lane group nor whole rows per
+// wave (17 lane-loads: 17 of 32 lanes, or 51 of 64).  The 256 * K load slots of a workgroup
+// are dealt densely over the lane-loads of a.R adjacent rows (a bundle): slot k of thread t
+// is lane-load (k * 256 + t) % G of row (k * 256 + t) / G, so the workgroup reads one
+// contiguous span and at most G - 1 slots idle.  Every slot reduces its own vector, the
+// values meet in LDS, and one thread per row folds the row's G values in lane order and
+// writes the output.  kDenseBundles bundles are in flight (8 loads per thread, all issued
+// before the first use); four workgroups per CU take turns between their LDS phases.
+// Loads of rows past the matrix are clamped to its last vector and their values dropped.
+// ---------------------------------------------------------------------------
+constexpr int kDenseSlots   = 2;
+constexpr int kDenseBundles = 4;
+
+template <class P>
+__global__ __launch_bounds__(kBlock) void row_dense_kernel(RowArgs a)
+{
+  using acc_t     = typename P::acc_t;
+  using in_t      = typename P::in_t;
+  using H         = Held<P, true>;
+  constexpr int K = kDenseSlots, R = kDenseBundles;
+  extern __shared__ __align__(16) unsigned char row_dense_lds[];
+  acc_t* sm       = reinterpret_cast<acc_t*>(row_dense_lds);  // [R][rows of a bundle * G]
+  const int t     = threadIdx.x;
+  const int G     = a.G;  // lane-loads of a row
+  const int rb    = a.R;  // rows of a bundle: 256 * K / G
+  const int width = rb * G;
+  i64 off[K];
+  int lane[K];
+  bool live[K];
+#pragma unroll
+  for (int k = 0; k < K; ++k) {
+    const unsigned f = (unsigned)(k * kBlock + t);
+    const unsigned q = f / (unsigned)G;
+    lane[k]          = (int)(f - q * (unsigned)G);
+    live[k]          = (int)q < rb;
+    off[k] = !live[k] ? 0
+                      : (i64)q * a.row_bytes +
+                          (lane[k] < a.nvec ? (i64)lane[k] * 16 : (a.len - P::VEC) * (i64)sizeof(in_t));
+  }
+  const char* inb = static_cast<const char*>(a.in);
+  const i64 last  = a.n_out * a.row_bytes - 16;  // the matrix's last whole vector
+  const i64 step  = (i64)R * rb;
+  for (i64 r = (i64)blockIdx.x * step; r < a.n_out; r += (i64)gridDim.x * step) {
+    u32x4 x[R][K];
+#pragma unroll
+    for (int q = 0; q < R; ++q)
+#pragma unroll
+      for (int k = 0; k < K; ++k) {
+        const i64 o = (r + (i64)q * rb) * a.row_bytes + off[k];
+        x[q][k]     = load16(inb + (o < last ? o : last));
+      }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int q = 0; q < R; ++q)
+#pragma unroll
+      for (int k = 0; k < K; ++k) {
+        acc_t v = P::neutral();
+        H::push_any(v, x[q][k], lane[k], a.nvec, a.len, a.tail);
+        if (live[k]) sm[q * width + k * kBlock + t] = v;
+      }
+    __syncthreads();
+    for (int i = t; i < R * rb; i += kBlock) {
+      const int q   = i / rb;
+      const int rr  = i - q * rb;
+      const i64 row = r + (i64)q * rb + rr;
+      if (row < a.n_out) {
+        const acc_t* p = sm + q * width + rr * G;
+        acc_t acc      = p[0];
+        for (int l = 1; l < G; ++l)
+          P::merge(acc, p[l]);
+        finish<P>(a.epi, row, acc);
+      }
+    }
+    __syncthreads();
   }
 }
 

@@ -64,7 +64,8 @@ int run(const PlanX& pl, const Problem& pr, hipStream_t st)
                 "plan selector and kernels must agree on block size and unroll");
   static_assert(col_wide_bundles(1) == col_wide_bundles_of(1) && col_wide_bundles(2) == col_wide_bundles_of(2) &&
                   col_wide_bundles(3) == col_wide_bundles_of(3) && col_wide_bundles(4) == col_wide_bundles_of(4) &&
-                  col_wide_bundles(5) == col_wide_bundles_of(5) && kColWideMaxSets == 5,
+                  col_wide_bundles(5) == col_wide_bundles_of(5) && kColWideMaxSets == 5 &&
+                  kDenseSlots == kPlanDenseSlots && kDenseBundles == kPlanDenseBundles,
                 "plan selector and wide-row column kernel must agree on rows per step");
   int rc = RMI_OK;
   switch (pl.kind) {
@@ -102,7 +103,12 @@ int run(const PlanX& pl, const Problem& pr, hipStream_t st)
           default: rc = RMI_ERR_UNSUPPORTED;
         }
       } else if (pl.kind == RMI_PLAN_ROW_WAVE && !pl.team_kernel) {
-        if (pl.short_rows) {
+        if (pl.dense_rows) {
+          a.R = (kBlock * kDenseSlots) / pl.G;
+          const size_t lds_bytes =
+            (size_t)kDenseBundles * a.R * pl.G * sizeof(typename P::acc_t);  // at most 32 KB
+          hipLaunchKernelGGL((row_dense_kernel<P>), grid, dim3(kBlock), lds_bytes, st, a);
+        } else if (pl.short_rows) {
           if (pl.any_g) {
             a.R    = 64 / pl.G;
             a.invG = 65536u / (unsigned)pl.G + 1;

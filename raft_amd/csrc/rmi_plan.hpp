@@ -27,6 +27,8 @@ constexpr int kWavesPerCu = 32;  // 8 resident waves on each of the 4 SIMDs
 // lose 2 and 8 points to queueing in the memory system.
 constexpr int kColBlocksPerCu = 2;
 constexpr int kColMaxLanes = 128;     // COL_TILE: most lanes of a workgroup along one row
+constexpr int kPlanDenseSlots   = 2;  // ROW_WAVE, dense rows: load slots per thread
+constexpr int kPlanDenseBundles = 4;  // ... and bundles of rows in flight
 constexpr int kColWideMaxSets = 5;    // COL_TILE, wide rows: most load slots per thread
 // row bundles in flight in the wide-row column kernel whose threads have K load slots
 constexpr int col_wide_bundles_of(int K) { return (10 + K - 1) / K; }
@@ -62,6 +64,8 @@ struct PlanX {
   bool vec16      = false;  // 16-byte lane loads
   bool short_rows = false;  // ROW_WAVE served by the one-load-per-lane kernel
   bool any_g      = false;  // short_rows with G = the row's lane-load count (not a power of two)
+  bool dense_rows = false;  // ROW_WAVE: G = the row's lane-load count, a workgroup's load slots
+                            // dealt over whole adjacent rows, rows combined through LDS
   bool team_kernel = false; // served by the team-per-row kernel
   bool stage_ok    = false; // ROW_WAVE: rows could be staged through LDS
   bool staged      = false; // ROW_WAVE: rows are staged through LDS (line-aligned span reads)
@@ -481,9 +485,37 @@ inline int make_plan(const rmi_reduce_desc& d,
       p.any_g      = true;
       p.G          = (int)nload;
     }
-    p.logG               = p.any_g ? 0 : ilog2(p.G);
-    const int64_t rows_w = (int64_t)(64 / p.G) * (p.short_rows ? kPlanUnroll : 1);
+    // Some lane-load counts suit neither layout: 17 fill 17 of 32 lanes, or 51 of 64 as three
+    // whole rows per wave.  There a workgroup's load slots are dealt densely over whole adjacent
+    // rows, one lane-load each, and the rows are combined through LDS (row_dense_kernel).  It
+    // costs a pass through LDS and two barriers per step, so the rule is what was measured on
+    // 512 MB matrices (% of 8 TB/s, before -> dense): rows ending in tail elements with 17 or 18
+    // lane-loads (fp32 D = 65 / 66 / 67 / 69: 65 / 64 / 67 / 72 -> 76 / 76 / 75 / 77, bf16 D = 130:
+    // 65 -> 75, int8 D = 270: 58 -> 63, arg-max D = 66: 61 -> 73), with 33 (fp32 D = 129: 76 -> 79,
+    // bf16 D = 260: 73 -> 78, f64 D = 65: 68 -> 73; not arg-reductions: 69 -> 63), 16-bit rows of 9
+    // to 16 (bf16 D = 66 / 100: 64 / 63 -> 70 / 72) and compensated f64 sums of 5 to 18 or 34 (D =
+    // 9 / 17 / 25 / 33 / 35 / 67: 53 / 52 / 59 / 60 / 62 / 70 -> 60 / 67 / 68 / 71 / 72 / 74).  Everywhere
+    // else it measured 1 to 30 % slower than the layouts above (fp32 D = 100: 88 -> 78 %).
+    const bool dense_ok =
+      p.vec16 && p.tail > 0 && hint == RMI_PLAN_AUTO &&
+      (nload == 17 || nload == 18 || (nload == 33 && key.family != kFamKvp) ||
+       (key.family == kFamFloat && es == 2 && nload >= 9 && nload <= 16) ||
+       (key.family == kFamKbn && ((nload >= 5 && nload <= 18) || nload == 34)));
+    if (dense_ok) {
+      p.dense_rows = true;
+      p.short_rows = false;
+      p.any_g      = false;
+      p.G          = (int)nload;
+    }
+    p.logG               = (p.any_g || p.dense_rows) ? 0 : ilog2(p.G);
+    const int64_t rows_w = p.dense_rows ? 1 : (int64_t)(64 / p.G) * (p.short_rows ? kPlanUnroll : 1);
     p.grid_blocks        = ceildiv(p.n_out, rows_w * (kPlanBlock / 64));
+    if (p.dense_rows) {
+      const int64_t step = (int64_t)kPlanDenseBundles * ((kPlanBlock * kPlanDenseSlots) / p.G);
+      p.grid_blocks      = ceildiv(p.n_out, step);
+      if (p.grid_blocks > (int64_t)4 * n_cu) p.grid_blocks = (int64_t)4 * n_cu;
+      return RMI_OK;
+    }
     if (!p.short_rows && p.vec16) {
       // Bytes in flight per CU are what the memory system is sensitive to: about
       // 80 KB sustains the most (5 workgroups when 256 lanes hold 4 loads of 16 B); the

@@ -14,6 +14,7 @@ long planned[8] = {0, 0, 0, 0, 0, 0, 0, 0};
 long staged_plans = 0;
 long grouped_plans = 0;
 long wide_plans = 0;
+long dense_plans = 0;
 #define REQUIRE(cond)                                                              \
   do {                                                                             \
     if (!(cond)) {                                                                 \
@@ -82,6 +83,17 @@ void check(const rmi_reduce_desc& d, int n_cu, uintptr_t in_misalign)
       REQUIRE(!p.strided);
       if (p.team_kernel) {
         REQUIRE(p.threads == 64 && p.B == 1 && p.chunk == p.nvec);
+      } else if (p.dense_rows) {
+        ++dense_plans;
+        // one lane-load per load slot, whole adjacent rows per workgroup, rows met in LDS
+        const int64_t slots = (int64_t)kPlanBlock * rmi::kPlanDenseSlots;
+        REQUIRE(p.vec16 && p.tail > 0 && !p.short_rows && !p.any_g && !p.staged && p.G == nload);
+        REQUIRE(p.G >= 5 && p.G <= 34 && slots / p.G >= 1);
+        REQUIRE((int64_t)rmi::kPlanDenseBundles * (slots / p.G) * p.G * p.acc_bytes <= 32768);
+        REQUIRE(p.grid_blocks >= 1 && p.grid_blocks <= (int64_t)4 * n_cu);
+        REQUIRE(p.grid_blocks * rmi::kPlanDenseBundles * (slots / p.G) >= p.n_out ||
+                p.grid_blocks == (int64_t)4 * n_cu);
+        REQUIRE(p.passes == 1 && p.ws_bytes == 0 && p.lds_reserve == 0);
       } else {
         if (p.any_g) {
           // one lane per lane-load, whole rows per wave, one run of at most 64 outputs
@@ -191,7 +203,7 @@ int main()
     }
     // log-uniform extents with the edge values mixed in
     auto extent = [&]() -> int64_t {
-      if (g() % 8 == 0) return pick({0, 1, 2, 3, 7, 15, 16, 17, 63, 64, 65, 255, 256, 257, 1023, 1024, 1025, 4095, 4096, 4097});
+      if (g() % 8 == 0) return pick({0, 1, 2, 3, 7, 9, 15, 16, 17, 25, 33, 35, 63, 64, 65, 66, 67, 69, 100, 129, 130, 255, 256, 257, 260, 270, 1023, 1024, 1025, 4095, 4096, 4097});
       const int bits = (int)(g() % 34);
       return (int64_t)(g() & ((1ull << bits) - 1)) + (g() % 2);
     };
@@ -218,9 +230,10 @@ int main()
       ++failures;
     }
   }
-  std::printf("plans checked: lanes %ld wave %ld block %ld split %ld col %ld (whole rows %ld) empty %ld\n",
+  std::printf("plans checked: lanes %ld wave %ld block %ld split %ld col %ld (whole rows %ld) empty %ld, dense rows %ld\n",
               planned[RMI_PLAN_ROW_LANES], planned[RMI_PLAN_ROW_WAVE], planned[RMI_PLAN_ROW_BLOCK],
-              planned[RMI_PLAN_ROW_SPLIT], planned[RMI_PLAN_COL_TILE], wide_plans, planned[RMI_PLAN_EMPTY]);
+              planned[RMI_PLAN_ROW_SPLIT], planned[RMI_PLAN_COL_TILE], wide_plans, planned[RMI_PLAN_EMPTY],
+              dense_plans);
   for (int k = RMI_PLAN_ROW_LANES; k <= RMI_PLAN_EMPTY; ++k)
     if (planned[k] < 1000) {
       std::printf("  plan kind %d was hardly exercised\n", k);
@@ -232,6 +245,10 @@ int main()
   }
   if (wide_plans < 1000) {
     std::printf("  whole-row column plans were hardly exercised (%ld)\n", wide_plans);
+    ++failures;
+  }
+  if (dense_plans < 1000) {
+    std::printf("  dense row plans were hardly exercised (%ld)\n", dense_plans);
     ++failures;
   }
   if (staged_plans < 1000) {

@@ -172,7 +172,9 @@ def test_lane_groups_follow_the_row_length():
     lanes = lambda cols, dt=api.F32, out=api.F32: api.plan_query(
         api.make_desc(dt, out, 1000000, cols)).lanes_per_row
     assert lanes(20) == 5 and lanes(17) == 5            # 5 lane-loads, without and with a tail
-    assert lanes(33) == 9 and lanes(45) == 12 and lanes(62) == 16 and lanes(66) == 8
+    assert lanes(33) == 9 and lanes(45) == 12 and lanes(62) == 16
+    # 17, 18 and 33 lane-loads with a tail: the row's own count (slots dealt over whole rows)
+    assert lanes(66) == 17 and lanes(70) == 18 and lanes(129) == 33 and lanes(68) == 8
     assert lanes(83) == 21 and lanes(125) == 32 and lanes(90) == 8   # 23 lane-loads: 46 lanes, no
     assert lanes(21) == 6                               # 5 whole vectors + one element
     assert lanes(24) == 8 and lanes(28) == 8            # 6 and 7 whole lane-loads stay on 8 lanes
@@ -180,7 +182,10 @@ def test_lane_groups_follow_the_row_length():
     assert lanes(128) == 8 and lanes(256) == 16
     assert lanes(100, api.BF16) == 13                   # 12 whole + 4 elements
     # 16-byte accumulators (f64 sums) keep it up to 12 lane-loads
-    assert lanes(17, api.F64, api.F64) == 9 and lanes(25, api.F64, api.F64) == 8
+    assert lanes(17, api.F64, api.F64) == 9 and lanes(63, api.F64, api.F64) == 8
+    # ... and take their own count again from 5 to 18 lane-loads with a tail, whole rows dealt
+    # over the workgroup's load slots
+    assert lanes(25, api.F64, api.F64) == 13 and lanes(35, api.F64, api.F64) == 18
     # arg-reductions follow the same rule
     d = api.make_desc(api.F32, api.KVP_I32_F32, 1000, 33, main_op=api.MAIN_KVP,
                       reduce_op=api.RED_ARGMAX)

@@ -610,6 +610,55 @@ def test_grouped_columns(gpu, in_dt, out_dt, kw, rows, cols, shift):
                            label=f"grouped {rows}x{cols} dt{in_dt} +{shift}")
 
 
+# Rows whose lane-load count suits neither a power-of-two lane group nor whole rows per wave
+# (17, 18 or 33 lane-loads ending in tail elements; 16-bit rows of 9..16; compensated f64 sums
+# of 5..18 or 34): a workgroup's load slots are dealt densely over whole adjacent rows and the
+# rows are combined through LDS.  Row counts below one bundle, around one step, and beyond one
+# round of the grid; starts off a 16-byte boundary; inplace.
+@pytest.mark.parametrize("in_dt,out_dt,kw,cols_list", [
+    (api.F32, api.F32, {}, (65, 66, 67, 69, 70, 71, 129, 130, 131)),
+    (api.F32, api.F32, dict(main_op=api.MAIN_SQ, final_op=api.FIN_SQRT), (66, 129)),
+    (api.F32, api.F32, dict(reduce_op=api.RED_MAX, init_f=-np.inf), (67, 131)),
+    (api.F32, api.F16, dict(main_op=api.MAIN_ABS), (65,)),
+    (api.BF16, api.F32, {}, (66, 76, 100, 127, 130, 132, 140, 260)),
+    (api.F16, api.F32, dict(reduce_op=api.RED_MIN, init_f=np.inf), (73, 133, 259)),
+    (api.F64, api.F64, {}, (9, 11, 17, 25, 33, 35, 65, 67)),
+    (api.I8, api.I64, {}, (257, 270, 285, 520)),
+    (api.U8, api.I32, {}, (260,)),
+    (api.I32, api.I64, {}, (66, 129)),
+    (api.F32, api.KVP_I32_F32, dict(main_op=api.MAIN_KVP, reduce_op=api.RED_ARGMAX, init_f=-np.inf),
+     (65, 66, 70)),
+    (api.F64, api.KVP_I64_F64, dict(main_op=api.MAIN_KVP, reduce_op=api.RED_ARGMIN, init_f=np.inf),
+     (33, 35)),
+])
+@pytest.mark.parametrize("rows,shift,inplace", [(1, 0, False), (7, 1, False), (29, 0, True), (121, 3, False),
+                                                (1000, 0, False), (40003, 1, True), (150001, 0, False)])
+def test_dense_rows(gpu, in_dt, out_dt, kw, cols_list, rows, shift, inplace):
+    for cols in cols_list:
+        rng = np.random.default_rng(rows * 13 + cols + shift)
+        data = _rand(rng, in_dt, rows * cols)
+        if kw.get("reduce_op") in (api.RED_MAX, api.RED_MIN):
+            data[rng.integers(0, data.size, max(1, data.size // 50))] = np.nan
+        if kw.get("main_op") == api.MAIN_KVP:  # ties: the lowest index has to win
+            m = data.reshape(rows, cols)
+            v = 9.0 if kw["reduce_op"] == api.RED_ARGMAX else -9.0
+            m[:, cols - 1] = v
+            m[:, cols // 2] = v
+        d = api.make_desc(in_dt, out_dt, rows, cols, inplace=inplace, **kw)
+        pl = api.plan_query(d)
+        assert pl.kind == api.PLAN_ROW_WAVE and pl.passes == 1
+        es = api.load().rmi_dtype_size(in_dt)
+        assert pl.lanes_per_row == -(-cols * es // 16), (cols, pl.lanes_per_row)
+        assert pl.grid_blocks <= 4 * 256
+        old = None
+        if inplace and kw.get("main_op") != api.MAIN_KVP:
+            old = u.encode_out(out_dt, rng.integers(1, 5, rows))
+        elif inplace:
+            continue
+        u.check_against_oracle(d, data, misalign_elems=shift, old_raw=old,
+                               label=f"dense rows {rows}x{cols} dt{in_dt} +{shift}")
+
+
 # Column reductions over rows of more than 128 lane-loads that one workgroup can hold whole
 # (floating sums, max and min): workgroups stream bundles of adjacent rows, one per CU, the
 # rows of a bundle are combined through LDS and the partials [workgroup][column] are folded
