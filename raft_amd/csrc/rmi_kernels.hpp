@@ -968,15 +968,16 @@ __global__ __launch_bounds__(kBlock) void row_dense_kernel(RowArgs a)
 }
 
 // ---------------------------------------------------------------------------
-// Column reduction of wide rows: more than 128 lane-loads, and few enough for a workgroup to
-// hold a whole row.  The workgroup streams whole adjacent rows, i.e. one contiguous span of
-// the matrix, where col_kernel reads pieces of at most 2 KB at the row's stride (32768 x 4097
-// floats: 96 us there, 81 us this way; x 2049: 99 / 80 us).
+// Column reduction of wide rows (more than 128 lane-loads).  The workgroup streams whole
+// adjacent rows, i.e. one contiguous span of the matrix, where col_kernel reads pieces of at
+// most 2 KB at the row's stride (32768 x 4097 floats: 96 us there, 81 us this way; x 2049:
+// 99 / 80 us); rows too long for its load slots are cut into gridDim.x equal pieces of a.TX
+// lane-loads, up to 20 KB each, and blockIdx.x names the piece.
 // A thread has K load slots with a set of accumulators each, as many as 256 bytes of
 // accumulators allow.  The 256 * K slots of the workgroup are dealt to the lane-loads of
 // a.TY adjacent rows (a bundle) in order: slot k of thread t is lane-load (k * 256 + t) %
-// nload of row (k * 256 + t) / nload of the bundle, so a slot always meets the same columns
-// and at most nload - 1 slots idle.  R bundles are in flight, and bundles are dealt
+// TX of row (k * 256 + t) / TX of the bundle, so a slot always meets the same columns
+// and at most TX - 1 slots idle.  R bundles are in flight, and bundles are dealt
 // round-robin to the B workgroups.  Every load of a step is issued before the first is
 // used, none under a condition (a load behind a branch makes the compiler wait for all
 // earlier ones): idle slots load the row's first vector and their accumulators are dropped.
@@ -1002,11 +1003,15 @@ __global__ __launch_bounds__(kBlock) void col_wide_kernel(ColArgs a)
   extern __shared__ __align__(16) unsigned char col_wide_lds[];
   acc_t* sm       = reinterpret_cast<acc_t*>(col_wide_lds);  // [rows of a bundle][nload * S]
   const int t     = threadIdx.x;
-  const int nload = a.TX;  // lane-loads of a row: nvec + (tail > 0)
-  const int rb    = a.TY;  // rows of a bundle: 256 * K / nload
+  const int piece = a.TX;  // lane-loads of this workgroup's piece of a row (the whole row
+                           // when it fits the slots), the last piece may hold fewer
+  const int rb    = a.TY;  // rows of a bundle: 256 * K / piece
+  const i64 total = a.nvec + (a.tail > 0 ? 1 : 0);
+  const i64 l0    = (i64)blockIdx.x * piece;
+  const int nload = (int)(total - l0 < piece ? total - l0 : piece);
   // byte offset of lane-load l within a row: whole vector l, or the vector that ends at the
   // row's end (its first S - tail columns belong to the lane-load before it)
-  auto offset_of = [&](int l) { return l < a.nvec ? (i64)l * 16 : (a.n_out - S) * (i64)sizeof(in_t); };
+  auto offset_of = [&](i64 l) { return l < a.nvec ? l * 16 : (a.n_out - S) * (i64)sizeof(in_t); };
   i64 off[K];   // ... of slot k, counted from the bundle's first row
   int sub[K];   // row of the bundle that slot k reads
   int lane[K];  // its lane-load of that row
@@ -1014,11 +1019,11 @@ __global__ __launch_bounds__(kBlock) void col_wide_kernel(ColArgs a)
 #pragma unroll
   for (int k = 0; k < K; ++k) {
     const unsigned f = (unsigned)(k * kBlock + t);
-    const unsigned q = f / (unsigned)nload;
+    const unsigned q = f / (unsigned)piece;
     sub[k]           = (int)q;
-    lane[k]          = (int)(f - q * (unsigned)nload);
-    live[k]          = (int)q < rb;
-    off[k]           = live[k] ? (i64)q * a.row_bytes + offset_of(lane[k]) : 0;
+    lane[k]          = (int)(f - q * (unsigned)piece);
+    live[k]          = (int)q < rb && lane[k] < nload;
+    off[k]           = live[k] ? (i64)q * a.row_bytes + offset_of(l0 + lane[k]) : offset_of(l0);
   }
   acc_t acc[K][S];
 #pragma unroll
@@ -1067,14 +1072,15 @@ __global__ __launch_bounds__(kBlock) void col_wide_kernel(ColArgs a)
   __syncthreads();
   acc_t* out = static_cast<acc_t*>(a.partial) + (i64)blockIdx.y * a.n_out;
   for (int idx = t; idx < width; idx += kBlock) {
-    const int l = idx / S, j = idx - l * S;
+    const int ll = idx / S, j = idx - ll * S;
+    const i64 l  = l0 + ll;
     // the last, partial lane-load holds the row's last S columns; its first S - tail are
     // already covered by the lane-load before it
     if (l == a.nvec && j < S - a.tail) continue;
     acc_t v = sm[idx];
     for (int q = 1; q < rb; ++q)
       P::merge(v, sm[q * width + idx]);
-    out[l < a.nvec ? (i64)idx : a.n_out - S + j] = v;
+    out[l < a.nvec ? l * S + j : a.n_out - S + j] = v;
   }
 }
 

@@ -91,9 +91,9 @@ struct PlanX {
   int group       = 0;  // COL_TILE: > 0 when `group` consecutive rows are read as one row
   int64_t group_len  = 0;  // COL_TILE, grouped: whole groups (rows of the widened matrix)
   int64_t group_nvec = 0;  // COL_TILE, grouped: 16-byte vectors per group
-  int wide        = 0;  // COL_TILE: > 0 when a workgroup streams whole rows (TX lane-loads each,
-                        // TY rows side by side in the `wide` load slots of its threads;
-                        // partials laid out [B][n_out])
+  int wide        = 0;  // COL_TILE: > 0 when a workgroup streams whole rows, or one of gridx equal
+                        // pieces of them (TX lane-loads each, TY rows side by side in the `wide`
+                        // load slots of its threads; partials laid out [B][n_out])
   int64_t grid_blocks    = 0;
   int passes             = 1;
   bool fused_fold        = false;  // ROW_SPLIT: the last workgroup of a row folds its partials
@@ -321,36 +321,44 @@ inline int make_plan(const rmi_reduce_desc& d,
       p.dense = (p.TX & (p.TX - 1)) != 0 || p.TX > 64;
       p.logTX = p.dense ? 0 : ilog2(p.TX);
     }
-    // Rows of more than kColMaxLanes lane-loads that a workgroup can hold whole: it streams
-    // adjacent rows, one contiguous span of the matrix.  A thread has K load slots, as many as
-    // 256 bytes of accumulators allow (5 for 4- and 8-byte elements, 4 for 2-byte ones); the
-    // workgroup's 256 * K slots take the lane-loads of 256 * K / lanes adjacent rows (a
-    // bundle: more than half of the slots get a lane-load), ten or so lane-loads per thread
-    // are in flight, one workgroup per CU.  Taken when every workgroup gets sixteen steps or
-    // more (4096 x 4097 floats lose 16 % with eight).  Longer rows, and accumulators whose step
-    // is arithmetic-bound at four waves per CU (arg-reductions 33-38 % slower, byte sums
-    // 25 %), keep the layout above.  Measured at 512 MB, % of 8 TB/s, the layout above / this
-    // one: fp32 D = 513: 76 / 81, 768: 74 / 82, 1025: 70 / 80, 1536: 73 / 82, 2049: 66 / 80,
-    // 3000: 65 / 78, 4096: 72 / 81, 4097: 67 / 78 (640 and 1024: 84 / 81 and 82 / 81);
-    // fp64 D = 300: 76 / 82, 513: 70 / 83, 1025: 67 / 82, 2049: 69 / 80; bf16 D = 1030: 72 / 80.
+    // Rows of more than kColMaxLanes lane-loads: a workgroup streams whole adjacent rows (or,
+    // of rows that outgrow it, one of the fewest equal pieces), i.e. long contiguous spans.
+    // A thread has K load slots, as many as 256 bytes of accumulators allow (5 for 4- and
+    // 8-byte elements, 4 for 2-byte ones); the workgroup's 256 * K slots take the lane-loads of
+    // 256 * K / piece adjacent rows (a bundle: more than half of the slots get a lane-load),
+    // ten or so lane-loads per thread are in flight, one workgroup per CU in all (a 257th
+    // workgroup would share a CU and finish last: 3 pieces x 86 workgroups ran 15 % slower than
+    // the layout above, 3 x 85 run 20 % faster).  Taken when every workgroup gets sixteen steps
+    // or more (4096 x 4097 floats lose 16 % with eight).  Accumulators whose step is
+    // arithmetic-bound at four waves per CU (arg-reductions 33-38 % slower, byte sums 25 %)
+    // keep the layout above, and so do rows of several pieces that are whole multiples of 64
+    // whole lane-loads, its best case (fp32 D = 32768 / 65536: 80 / 83 % there, 76 / 75 % this
+    // way).
+    // Measured at 512 MB, % of 8 TB/s, the layout above / this one: fp32 D = 513: 76 / 81,
+    // 768: 74 / 82, 1025: 70 / 80, 1536: 73 / 82, 2049: 66 / 80, 3000: 65 / 78, 4096: 72 / 81,
+    // 4097: 67 / 78, 8191: 71 / 77, 11000: 66 / 81, 14000: 67 / 78, 22000: 66 / 79, 50000: 70 / 77,
+    // 200000: 66 / 72 (640 and 1024: 84 / 81 and 82 / 81); fp64 D = 300: 76 / 82, 1025: 67 / 82,
+    // 4097: 61 / 80, 8191: 70 / 79; bf16 D = 1030: 72 / 80, 10000: 62 / 72, 16400: 59 / 75.
     if (p.group == 0 && p.vec16 && lanes > kColMaxLanes &&
         (key.family == kFamFloat || key.family == kFamKbn)) {
       int K = 256 / (p.step * acc_bytes);
       K     = K < 1 ? 1 : (K > kColWideMaxSets ? kColWideMaxSets : K);
       const int64_t slots = (int64_t)kPlanBlock * K;
-      if (lanes <= slots) {
-        const int64_t bundle = slots / lanes;
+      const int64_t cuts  = ceildiv(lanes, slots);
+      if (cuts <= n_cu && (cuts == 1 || lanes % 64 != 0 || p.tail > 0)) {
+        const int64_t piece  = ceildiv(lanes, cuts);
+        const int64_t bundle = slots / piece;
         const int64_t step   = bundle * col_wide_bundles_of(K);
-        const int64_t B      = n_cu;
+        const int64_t B      = (int64_t)n_cu / cuts;
         const size_t ws      = kTicketBytes + (size_t)p.n_out * B * acc_bytes;
         const bool too_large = (d.flags & kFlagSmallWorkspace) != 0 && ws > RMI_NOALLOC_SCRATCH_BYTES;
         if (rows >= B * step * 16 && !too_large) {
           p.wide        = K;
-          p.TX          = (int)lanes;
+          p.TX          = (int)piece;
           p.TY          = (int)bundle;
-          p.gridx       = 1;
+          p.gridx       = ceildiv(lanes, piece);
           p.B           = (int)B;
-          p.grid_blocks = p.B;
+          p.grid_blocks = p.gridx * p.B;
           p.passes      = 2;  // the epilogue is the second pass's
           p.ws_bytes    = ws;
           return RMI_OK;

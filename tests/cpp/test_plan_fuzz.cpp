@@ -131,16 +131,21 @@ void check(const rmi_reduce_desc& d, int n_cu, uintptr_t in_misalign)
       REQUIRE(p.strided);
       if (p.wide > 0) {
         ++wide_plans;
-        // whole rows per workgroup: the slots of its threads hold TY adjacent rows of TX
-        // lane-loads, more than half of them in use, in at most 64 KB of LDS at the end
+        // whole rows (or the fewest equal pieces of them) per workgroup: the slots of its
+        // threads hold TY adjacent rows of TX lane-loads, more than half of them in use, in at
+        // most 64 KB of LDS at the end; no more workgroups than CUs
         const int64_t slots = (int64_t)kPlanBlock * p.wide;
         REQUIRE(p.wide >= 1 && p.wide <= rmi::kColWideMaxSets && p.wide * p.step * p.acc_bytes <= 256);
         REQUIRE(key.family == rmi::kFamFloat || key.family == rmi::kFamKbn);
-        REQUIRE(p.group == 0 && p.vec16 && p.TX == nload && p.TX > rmi::kColMaxLanes && p.TX <= slots);
+        REQUIRE(p.group == 0 && p.vec16 && nload > rmi::kColMaxLanes && p.TX <= slots);
+        REQUIRE(p.gridx >= 1 && p.gridx <= n_cu && p.gridx * p.TX >= nload && (p.gridx - 1) * p.TX < nload);
+        REQUIRE(p.gridx == (nload + slots - 1) / slots);
+        if (p.gridx > 1) REQUIRE(nload % 64 != 0 || p.tail > 0);
         REQUIRE(p.TY >= 1 && (int64_t)p.TY * p.TX <= slots && (int64_t)(p.TY + 1) * p.TX > slots);
         REQUIRE((int64_t)p.TY * p.TX * 2 > slots);
         REQUIRE((int64_t)p.TY * p.TX * p.step * p.acc_bytes <= 65536);
-        REQUIRE(p.gridx == 1 && p.B == n_cu && p.grid_blocks == p.B && p.passes == 2);
+        REQUIRE(p.B == n_cu / p.gridx && p.B >= 1 && p.grid_blocks == p.B * p.gridx && p.grid_blocks <= n_cu);
+        REQUIRE(p.passes == 2);
         REQUIRE(p.len >= (int64_t)p.B * p.TY * rmi::col_wide_bundles_of(p.wide) * 16);
         REQUIRE(p.ws_bytes == rmi::kTicketBytes + (size_t)p.n_out * p.B * p.acc_bytes);
         break;

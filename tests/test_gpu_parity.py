@@ -702,16 +702,50 @@ def test_whole_row_columns(gpu, in_dt, out_dt, kw, slots, bundles, cols_list, ex
         pl = api.plan_query(d)
         assert pl.kind == api.PLAN_COL_TILE and pl.passes == 2
         assert pl.grid_blocks == 256 and pl.blocks_per_out == 256, (cols, pl.grid_blocks)
-        old = None
-        if inplace:
-            old = u.encode_out(out_dt, rng.uniform(1, 2, cols))
-        u.check_against_oracle(d, data, misalign_elems=shift, old_raw=old,
-                               label=f"whole rows {rows}x{cols} dt{in_dt} +{shift}")
+        _check_whole_rows(d, data, rng, cols, out_dt, shift, inplace)
         # one row fewer than the plan needs: the layout for short matrices, the same values
         if extra == 0 and cols == cols_list[0]:
             d2 = api.make_desc(in_dt, out_dt, rows - 1, cols, apply=api.ALONG_COLUMNS, **kw)
             assert api.plan_query(d2).grid_blocks != 256
             u.check_against_oracle(d2, data[:(rows - 1) * cols], label="one row fewer")
+
+
+def _check_whole_rows(d, data, rng, cols, out_dt, shift, inplace):
+    old = u.encode_out(out_dt, rng.uniform(1, 2, cols)) if inplace else None
+    u.check_against_oracle(d, data, misalign_elems=shift, old_raw=old,
+                           label=f"whole rows x{cols} dt{d.in_dtype} +{shift}")
+
+
+# ... and rows that outgrow a workgroup's 1280 (16-bit elements: 1024) load slots, cut into the
+# fewest equal pieces, 256 // pieces workgroups each: two to forty pieces, the last one shorter,
+# with and without tail elements.  Rows that are whole multiples of 64 lane-loads keep the
+# other layout.
+@pytest.mark.parametrize("in_dt,out_dt,kw,slots,bundles,shapes", [
+    (api.F32, api.F32, {}, 5, 2, ((5121, 2), (8191, 2), (11001, 3), (20003, 4), (50001, 10), (204700, 40))),
+    (api.F32, api.F32, dict(reduce_op=api.RED_MIN, init_f=np.inf), 5, 2, ((6000, 2), (30000, 6))),
+    (api.F64, api.F64, {}, 5, 2, ((2561, 2), (4097, 2), (12001, 5))),
+    (api.BF16, api.F32, dict(main_op=api.MAIN_SQ, final_op=api.FIN_SQRT), 4, 3, ((10000, 2), (16400, 3))),
+])
+@pytest.mark.parametrize("extra,shift,inplace", [(0, 0, False), (3, 1, True)])
+def test_whole_row_columns_in_pieces(gpu, in_dt, out_dt, kw, slots, bundles, shapes, extra, shift, inplace):
+    es = api.load().rmi_dtype_size(in_dt)
+    for cols, pieces in shapes:
+        lanes = -(-cols * es // 16)
+        piece = -(-lanes // pieces)
+        b = 256 // pieces
+        rows = b * (256 * slots // piece) * bundles * 16 + extra
+        rng = np.random.default_rng(cols + extra)
+        data = _rand(rng, in_dt, rows * cols)
+        if kw.get("reduce_op") == api.RED_MIN:
+            data[rng.integers(0, data.size, 5000)] = np.nan
+        d = api.make_desc(in_dt, out_dt, rows, cols, apply=api.ALONG_COLUMNS, inplace=inplace, **kw)
+        pl = api.plan_query(d)
+        assert pl.kind == api.PLAN_COL_TILE and pl.passes == 2
+        assert pl.blocks_per_out == b and pl.grid_blocks == b * pieces, (cols, pl.grid_blocks)
+        _check_whole_rows(d, data, rng, cols, out_dt, shift, inplace)
+    # whole multiples of 64 lane-loads in several pieces: not this plan
+    d = api.make_desc(api.F32, api.F32, 4096, 32768, apply=api.ALONG_COLUMNS)
+    assert api.plan_query(d).grid_blocks > 256
 
 
 # Rows of 5 lane-loads, or of 6, 9..16, 18..21 and 28..32 with tail elements (up to 12 only for
