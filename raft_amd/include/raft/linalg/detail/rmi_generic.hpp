@@ -563,7 +563,8 @@ void launch_cols(Dst* dots, const In* data, Idx D, Idx N, Out init, hipStream_t 
   // 16-byte lane loads: two workgroups per CU of a 256-CU device read one compact, advancing
   // window of the matrix (measured 74 % of 8 TB/s on 10M x 64 floats where 1024 workgroups
   // give 63 %); element loads want eight times as many in flight.  At least four steps each.
-  std::int64_t B           = ((V > 1 ? 512 : 4096) + gridx - 1) / gridx;
+  // (rounded down: a 513th workgroup lands on a CU that then finishes last)
+  std::int64_t B           = (V > 1 ? 512 : 4096) / gridx;
   const std::int64_t max_b = ((std::int64_t)N + 4 * TY - 1) / (4 * TY);
   if (B > max_b) B = max_b;
   if (B < 1) B = 1;
