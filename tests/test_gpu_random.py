@@ -125,3 +125,51 @@ def test_random_meanvar(gpu, seed):
     layout = int(rng.choice([api.ROW_MAJOR, api.COL_MAJOR]))
     stored = tm._make(rng, dt, layout, rows, cols, float(rng.uniform(-50, 50)), float(rng.uniform(0.1, 5)))
     tm._check(dt, layout, rows, cols, bool(rng.random() < 0.5), stored)
+
+
+# Column reductions of wide rows take their own layout only from a few hundred megabytes on
+# (every workgroup has to get sixteen steps), which the draw above never reaches: random widths
+# from 513 columns up to some hundred thousand, in one piece or several, with just enough rows
+# for that layout plus a random remainder.
+@pytest.mark.parametrize("seed", range(int(os.environ.get("RMI_RANDOM_CASES", "400")) // 10))
+def test_random_wide_columns(gpu, seed):
+    rng = np.random.default_rng(30_000 + seed)
+    in_dt, out_dt = [(api.F32, api.F32), (api.F64, api.F64), (api.BF16, api.F32), (api.F16, api.F32),
+                     (api.F32, api.F64)][rng.integers(5)]
+    es = api.DTYPE_SIZE[in_dt]
+    slots, bundles = (1024, 3) if es == 2 else (1280, 2)
+    lanes = int(np.exp(rng.uniform(np.log(129), np.log(8 * slots))))
+    cols = lanes * (16 // es) - int(rng.integers(0, 16 // es))
+    lanes = -(-cols * es // 16)
+    pieces = -(-lanes // slots)
+    if pieces > 1 and lanes % 64 == 0 and cols * es % 16 == 0:
+        cols -= 1                                   # rows of whole multiples of 64 lane-loads: other layout
+        lanes = -(-cols * es // 16)
+        pieces = -(-lanes // slots)
+    piece = -(-lanes // pieces)
+    b = 256 // pieces
+    rows = b * (slots // piece) * bundles * 16 + int(rng.integers(0, 40))
+    kw = {}
+    op = rng.choice(["sum", "sq", "abs", "max", "min"])
+    if op == "sq":
+        kw.update(main_op=api.MAIN_SQ, final_op=api.FIN_SQRT)
+    elif op == "abs":
+        kw.update(main_op=api.MAIN_ABS)
+    elif op in ("max", "min"):
+        kw.update(reduce_op=api.RED_MAX if op == "max" else api.RED_MIN,
+                  init_f=-np.inf if op == "max" else np.inf)
+    inplace = bool(rng.random() < 0.3)
+    col_major = bool(rng.random() < 0.3)
+    data = _rand(rng, in_dt, rows * cols)
+    if col_major:
+        d = api.make_desc(in_dt, out_dt, cols, rows, layout=api.COL_MAJOR, apply=api.ALONG_ROWS,
+                          inplace=inplace, **kw)
+    else:
+        d = api.make_desc(in_dt, out_dt, rows, cols, apply=api.ALONG_COLUMNS, inplace=inplace, **kw)
+    pl = api.plan_query(d)
+    assert pl.kind == api.PLAN_COL_TILE and pl.passes == 2
+    assert pl.blocks_per_out == b and pl.grid_blocks == b * pieces, (seed, rows, cols, pl.grid_blocks)
+    old = u.encode_out(out_dt, rng.integers(-3, 4, cols).astype(np.float64)) if inplace else None
+    shift = int(rng.choice([0, 0, 1, 3]))
+    u.check_against_oracle(d, data, old_raw=old, misalign_elems=shift,
+                           label=f"seed {seed}: wide columns {rows}x{cols} dt{in_dt}->{out_dt} {op} +{shift}")
