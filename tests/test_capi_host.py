@@ -214,3 +214,30 @@ def test_column_plans_of_rows_that_are_not_whole_vectors():
     p = api.plan_query(d)
     assert p.kind == api.PLAN_COL_TILE and p.vec_bytes == 16 and p.blocks_per_out <= 4096
     assert p.grid_blocks == p.blocks_per_out            # 33 lane-loads: one workgroup column
+
+
+def test_column_plans_of_wide_rows():
+    """Floating sums, max and min down rows of more than 128 lane-loads: whole adjacent rows
+    per workgroup (one workgroup per CU of the 256 a build host is planned for, one set of
+    partials each, a second pass), rows beyond 1280 lane-loads in the fewest equal pieces;
+    arg-reductions, byte sums, short matrices and whole multiples of 64 lane-loads in several
+    pieces keep the other layout; the library's own descriptor flag is refused."""
+    lib = api.load()
+    q = lambda rows, cols, in_dt=api.F32, out_dt=api.F32, **kw: api.plan_query(
+        api.make_desc(in_dt, out_dt, rows, cols, apply=api.ALONG_COLUMNS, **kw))
+    p = q(32768, 4097)
+    assert (p.kind, p.passes, p.grid_blocks, p.blocks_per_out) == (api.PLAN_COL_TILE, 2, 256, 256)
+    assert p.workspace_bytes == api.WORKSPACE_TICKET_BYTES + 4097 * 256 * 8
+    p = q(16384, 11000)                                  # 2750 lane-loads: three pieces of 917
+    assert (p.grid_blocks, p.blocks_per_out) == (3 * 85, 85)
+    p = q(16384, 4097, api.F64, api.F64)                 # compensated sums: 16-byte partials
+    assert p.grid_blocks == 2 * 128 and p.workspace_bytes == api.WORKSPACE_TICKET_BYTES + 4097 * 128 * 16
+    assert q(8191, 4097).grid_blocks != 256              # fewer than sixteen steps per workgroup
+    assert q(4096, 32768).grid_blocks > 256              # 8192 whole lane-loads: pieces of 64 lanes
+    kvp = dict(main_op=api.MAIN_KVP, reduce_op=api.RED_ARGMAX)
+    assert q(32768, 4097, api.F32, api.KVP_I32_F32, **kvp).grid_blocks > 256
+    assert q(131072, 4100, api.I8, api.I64).grid_blocks > 256
+    d = api.make_desc(api.F32, api.F32, 32768, 4097, apply=api.ALONG_COLUMNS, flags=1 << 30)
+    plan = api.Plan()
+    assert lib.rmi_plan_query(C.byref(d), C.byref(plan)) == api.ERR_BAD_ENUM
+    assert lib.rmi_reduce_workspace_bytes(C.byref(d)) == 0
