@@ -42,11 +42,12 @@ struct RowArgs {
   i64 nvec;        // whole lane-loads per row: len / VEC (VEC16) or len (element-wise)
   i64 chunk;       // lane-loads per team chunk (row_block_kernel)
   int tail;        // VEC16: elements after the last whole vector (len % VEC)
-  int G;           // lanes per row (row_short / row_wave)
+  int G;           // lanes per row (row_short / row_wave); row_dense_kernel: lane-loads of a row
   int logG;
   int B;           // chunks per row (row_block_kernel)
   int logT;        // row_block_kernel: a team is 64 << logT threads
-  int R;           // row_short_kernel, any G: 64 / G rows per wave step
+  int R;           // row_short_kernel, any G: 64 / G rows per wave step;
+                   // row_dense_kernel: rows of a bundle, 256 * kDenseSlots / G
   u32 invG;        // row_short_kernel, any G: 65536 / G + 1, so that (x * invG) >> 16 == x / G
   u32 invR;        // likewise for R                              for every x < 64
   u32* ticket;     // row_block_kernel, B > 1: zeroed ticket counters, each alone on a 128-byte
@@ -64,8 +65,9 @@ struct ColArgs {
   i64 row_bytes;   // D * sizeof(element)
   i64 nvec;        // whole lane-loads per row: D / VEC (VEC16) or D (element-wise)
   int tail;        // VEC16: columns after the last whole vector (D % VEC)
-  int TX;          // lanes along the contiguous dimension (<= 128)
-  int TY;          // rows per step: kBlock / TX, rounded down
+  int TX;          // lanes along the contiguous dimension (<= 128); col_wide_kernel: lane-loads
+                   // of a workgroup's piece of a row
+  int TY;          // rows per step: kBlock / TX, rounded down; col_wide_kernel: rows of a bundle
   int logTX;       // log2(TX) when TX is a power of two
   int dense;       // TX is not a power of two or exceeds a wave: thread t is lane t % TX of
                    // row t / TX, the last kBlock - TX * TY threads idle, and the rows of a
