@@ -582,6 +582,193 @@ void launch_cols(Dst* dots, const In* data, Idx D, Idx N, Out init, hipStream_t 
   }
 }
 
+// ---- columns of wide rows ------------------------------------------------------------------
+// Rows of more than 128 lane-loads: a workgroup streams whole adjacent rows (of rows that
+// outgrow its load slots, one of the fewest equal pieces), i.e. long contiguous spans, where
+// cols_kernel reads pieces of at most 2 KB at the row's stride.  A thread has K load slots
+// with V accumulators each, as many as 256 bytes hold (at most 5); the workgroup's 256 * K
+// slots are dealt densely over the lane-loads of `rb` adjacent rows (a bundle): slot k of
+// thread t is lane-load (256 k + t) % piece of row (256 k + t) / piece, so a slot always meets
+// the same columns.  R bundles are in flight, every load issued before the first use and none
+// under a condition (idle slots load the piece's first vector and are dropped).  At the end the
+// rows of a bundle are combined through LDS in row order and the partials are stored
+// [workgroup][column], whole lines at a time; fold_rows_kernel is the second pass.
+template <typename Out, int V>
+constexpr int cols_wide_slots()
+{
+  constexpr int k = 256 / (V * (int)sizeof(Out));
+  return k < 1 ? 1 : (k > 5 ? 5 : k);
+}
+constexpr int cols_wide_bundles(int K) { return (10 + K - 1) / K; }
+
+template <int V, typename In, typename Out, typename Idx, typename Main, typename Red>
+__global__ __launch_bounds__(kBlock) void cols_wide_kernel(Out* partial, const In* data, Idx D,
+                                                           Idx N, Out init, Main main_op, Red red,
+                                                           int piece, int rb, int B)
+{
+  static_assert(std::is_trivially_copyable_v<Out>, "accumulators must be trivially copyable");
+  constexpr int K = cols_wide_slots<Out, V>();
+  constexpr int R = cols_wide_bundles(K);
+  extern __shared__ __align__(16) unsigned char cols_wide_lds[];
+  Out* sm                  = reinterpret_cast<Out*>(cols_wide_lds);  // [rb][lane-loads of the piece * V]
+  const int t              = threadIdx.x;
+  const std::int64_t nvec  = (std::int64_t)D / V;
+  const int tail           = (int)((std::int64_t)D - nvec * V);
+  const std::int64_t total = nvec + (tail > 0 ? 1 : 0);
+  const std::int64_t l0    = (std::int64_t)blockIdx.x * piece;
+  const int nload          = (int)(total - l0 < piece ? total - l0 : piece);
+  // element offset of lane-load l within a row: whole vector l, or the vector that ends at the
+  // row's end (its first V - tail columns belong to the lane-load before it)
+  auto first_col = [&](std::int64_t l) { return l < nvec ? l * V : (std::int64_t)D - V; };
+  std::int64_t off[K];
+  int sub[K], lane[K];
+  bool live[K];
+#pragma unroll
+  for (int k = 0; k < K; ++k) {
+    const unsigned f = (unsigned)(k * kBlock + t);
+    const unsigned q = f / (unsigned)piece;
+    sub[k]           = (int)q;
+    lane[k]          = (int)(f - q * (unsigned)piece);
+    live[k]          = (int)q < rb && lane[k] < nload;
+    off[k] = live[k] ? (std::int64_t)q * (std::int64_t)D + first_col(l0 + lane[k]) : first_col(l0);
+  }
+  Out acc[K][V];
+#pragma unroll
+  for (int k = 0; k < K; ++k)
+#pragma unroll
+    for (int j = 0; j < V; ++j)
+      acc[k][j] = init;
+
+  const std::int64_t step   = (std::int64_t)R * rb;
+  const std::int64_t stride = (std::int64_t)B * step;
+  std::int64_t r            = (std::int64_t)blockIdx.y * step;
+  for (; r + step <= (std::int64_t)N; r += stride) {
+    pack16 x[R][K];
+#pragma unroll
+    for (int q = 0; q < R; ++q)
+#pragma unroll
+      for (int k = 0; k < K; ++k)
+        x[q][k] = load_pack16<true>(data + (r + (std::int64_t)q * rb) * (std::int64_t)D + off[k]);
+    __builtin_amdgcn_sched_barrier(0);  // all of the step's loads before the first use
+#pragma unroll
+    for (int q = 0; q < R; ++q)
+#pragma unroll
+      for (int k = 0; k < K; ++k) {
+        In e[V];
+        __builtin_memcpy(e, x[q][k].w, 16);
+        const Idx row = static_cast<Idx>(r + (std::int64_t)q * rb + sub[k]);
+#pragma unroll
+        for (int j = 0; j < V; ++j)
+          acc[k][j] = red(acc[k][j], static_cast<Out>(main_op(e[j], row)));
+      }
+  }
+  // the rows after the last whole step go to the workgroup whose turn it is, bundle by bundle
+  for (; r < (std::int64_t)N; r += rb) {
+#pragma unroll
+    for (int k = 0; k < K; ++k)
+      if (live[k] && r + sub[k] < (std::int64_t)N) {
+        const pack16 x = load_pack16<true>(data + r * (std::int64_t)D + off[k]);
+        In e[V];
+        __builtin_memcpy(e, x.w, 16);
+#pragma unroll
+        for (int j = 0; j < V; ++j)
+          acc[k][j] = red(acc[k][j], static_cast<Out>(main_op(e[j], static_cast<Idx>(r + sub[k]))));
+      }
+  }
+
+  const int width = nload * V;
+#pragma unroll
+  for (int k = 0; k < K; ++k) {
+    if (live[k]) {
+#pragma unroll
+      for (int j = 0; j < V; ++j)
+        sm[sub[k] * width + lane[k] * V + j] = acc[k][j];
+    }
+  }
+  __syncthreads();
+  Out* out = partial + (std::int64_t)blockIdx.y * (std::int64_t)D;
+  for (int idx = t; idx < width; idx += kBlock) {
+    const int ll = idx / V, j = idx - ll * V;
+    const std::int64_t l = l0 + ll;
+    if (l == nvec && j < V - tail) continue;  // columns of the lane-load before the last, partial one
+    Out v = sm[idx];
+    for (int q = 1; q < rb; ++q)
+      v = red(v, sm[q * width + idx]);
+    out[l < nvec ? l * V + j : (std::int64_t)D - V + j] = v;
+  }
+}
+
+// second pass over partials[B][n_out]: a workgroup folds 16 adjacent outputs; thread (c, s)
+// folds partials s, s + 16, ... of output c in that order, then the 16 s in a fixed tree
+template <typename Out, typename Red, typename Fin, typename Dst>
+__global__ __launch_bounds__(kBlock) void fold_rows_kernel(Dst* dots, const Out* partial,
+                                                           std::int64_t n_out, int B, Out init,
+                                                           bool inplace, Red red, Fin fin)
+{
+  __shared__ Out sm[kBlock];
+  const int t          = threadIdx.x;
+  const int c          = t & 15;
+  const int s          = t >> 4;
+  const std::int64_t o = (std::int64_t)blockIdx.x * 16 + c;
+  Out acc              = init;
+  if (o < n_out) {
+    const Out* p = partial + o;
+    int b        = s;
+    for (; b + 7 * 16 < B; b += 8 * 16) {
+      Out x[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        x[u] = p[(std::int64_t)(b + u * 16) * n_out];
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        acc = red(acc, x[u]);
+    }
+    for (; b < B; b += 16)
+      acc = red(acc, p[(std::int64_t)b * n_out]);
+  }
+  sm[t] = acc;
+  __syncthreads();
+  for (int h = 8; h >= 1; h >>= 1) {
+    if (s < h) sm[t] = red(sm[t], sm[t + h * 16]);
+    __syncthreads();
+  }
+  if (s == 0 && o < n_out) dots[o] = fin(inplace ? red(static_cast<Out>(dots[o]), sm[t]) : sm[t]);
+}
+
+// true when the wide-row layout was taken
+template <int V, typename In, typename Out, typename Idx, typename Main, typename Red, typename Fin,
+          typename Dst>
+bool launch_cols_wide(Dst* dots, const In* data, Idx D, Idx N, Out init, hipStream_t stream,
+                      bool inplace, Main main_op, Red red, Fin fin)
+{
+  constexpr int K          = cols_wide_slots<Out, V>();
+  constexpr int kCus       = 256;  // one workgroup per CU of the device this is tuned for
+  const std::int64_t lanes = ((std::int64_t)D + V - 1) / V;
+  const std::int64_t slots = (std::int64_t)kBlock * K;
+  const std::int64_t cuts  = (lanes + slots - 1) / slots;
+  // rows of several pieces that are whole multiples of 64 lane-loads are cols_kernel's best case
+  if (lanes <= 128 || cuts > kCus || (cuts > 1 && lanes % 64 == 0 && (std::int64_t)D % V == 0))
+    return false;
+  const std::int64_t piece = (lanes + cuts - 1) / cuts;
+  const std::int64_t rb    = slots / piece;
+  const std::int64_t step  = rb * cols_wide_bundles(K);
+  const std::int64_t B     = kCus / cuts;
+  if ((std::int64_t)N < B * step * 16) return false;  // every workgroup gets sixteen steps
+  const std::int64_t gridx = (lanes + piece - 1) / piece;
+  Out* partial = static_cast<Out*>(scratch_alloc(sizeof(Out) * (std::size_t)D * B, stream));
+  const std::size_t lds = (std::size_t)rb * piece * V * sizeof(Out);  // at most 64 KB
+  hipLaunchKernelGGL((cols_wide_kernel<V, In, Out, Idx, Main, Red>),
+                     dim3((unsigned)gridx, (unsigned)B), dim3(kBlock), lds, stream, partial, data, D,
+                     N, init, main_op, red, (int)piece, (int)rb, (int)B);
+  check_launch("cols_wide_kernel");
+  hipLaunchKernelGGL((fold_rows_kernel<Out, Red, Fin, Dst>),
+                     dim3((unsigned)(((std::int64_t)D + 15) / 16)), dim3(kBlock), 0, stream, dots,
+                     partial, (std::int64_t)D, (int)B, init, inplace, red, fin);
+  check_launch("fold_rows_kernel");
+  scratch_free(partial, stream);
+  return true;
+}
+
 // dots[D] from N rows of D contiguous elements (one output per column)
 template <typename In, typename Out, typename Idx, typename Main, typename Red, typename Fin,
           typename Dst>
@@ -594,6 +781,8 @@ void strided(Dst* dots, const In* data, Idx D, Idx N, Out init, hipStream_t stre
   constexpr int V = vec_width<In>();
   if constexpr (V > 1 && sizeof(Out) * V * kBlock <= 32 * 1024) {
     if ((std::int64_t)D >= V) {
+      if (launch_cols_wide<V, In, Out, Idx>(dots, data, D, N, init, stream, inplace, main_op, red, fin))
+        return;
       launch_cols<V, In, Out, Idx>(dots, data, D, N, init, stream, inplace, main_op, red, fin);
       return;
     }

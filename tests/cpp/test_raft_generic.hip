@@ -762,6 +762,65 @@ void compensated_lambda_sums(double large, double tol)
 TEST_CASE(CompensatedLambdaSumsF) { compensated_lambda_sums<float>(1e7, 2e-7); }
 TEST_CASE(CompensatedLambdaSumsD) { compensated_lambda_sums<double>(1e12, 1e-13); }
 
+// Column reductions with the caller's functors over rows of more than 128 lane-loads: whole
+// adjacent rows per workgroup (D = 4097: one piece, D = 6001: two), partials per workgroup and a
+// second pass; sums through the wide accumulator, a maximum of a lambda, and an arg-max with the
+// test's own functors (ties: the lowest row wins).  Row counts are the fewest that take this
+// layout plus a remainder; one more case stays just below and takes the other layout.
+TEST_CASE(WideColumnsLambdas)
+{
+  raft::resources handle;
+  auto stream = raft::resource::get_cuda_stream(handle);
+  using KVP   = raft::KeyValuePair<int, float>;
+  struct shape {
+    int rows, cols;
+  };
+  for (shape sh : {shape{8192 + 5, 4097}, shape{4096 + 3, 6001}, shape{16384 + 9, 2049}, shape{8191, 4097}}) {
+    const int rows = sh.rows, cols = sh.cols;
+    auto h = uniform<float>((size_t)rows * cols, -1.0, 1.0, 1000 + cols);
+    for (int j = 0; j < cols; j += 97)  // planted ties for the arg-max
+      h[(size_t)(rows - 1) * cols + j] = h[(size_t)(rows / 3) * cols + j] = 2.0f;
+    auto d = raft::make_device_matrix<float, int, raft::row_major>(handle, rows, cols);
+    raft::update_device(d.data_handle(), h.data(), h.size(), stream);
+    auto sums = raft::make_device_vector<float, int>(handle, cols);
+    auto maxs = raft::make_device_vector<float, int>(handle, cols);
+    auto args = raft::make_device_vector<KVP, int>(handle, cols);
+    const float scale = 0.5f;
+    raft::linalg::strided_reduction(
+      handle, raft::make_const_mdspan(d.view()), sums.view(), 0.0f, false,
+      [scale] __device__(float a, int i) { return a * scale + (i % 3 == 0 ? 0.25f : 0.0f); },
+      raft::add_op(), [] __device__(float x) { return 2.0f * x; });
+    raft::linalg::strided_reduction(handle, raft::make_const_mdspan(d.view()), maxs.view(), -1e30f,
+                                    false, [] __device__(float a, int) { return a * a; },
+                                    raft::max_op());
+    raft::linalg::strided_reduction(handle, raft::make_const_mdspan(d.view()), args.view(),
+                                    KVP{0, -std::numeric_limits<float>::infinity()}, false,
+                                    ValueToKVP<float, int>{}, ArgMaxOp<int, float>{});
+    auto got_s = to_host(sums.data_handle(), (size_t)cols, stream);
+    auto got_m = to_host(maxs.data_handle(), (size_t)cols, stream);
+    auto got_a = to_host(args.data_handle(), (size_t)cols, stream);
+    bool ok_s = true, ok_m = true, ok_a = true;
+    for (int j = 0; j < cols; ++j) {
+      double acc = 0;
+      float mx   = -1e30f;
+      int best   = 0;
+      for (int i = 0; i < rows; ++i) {
+        const float x = h[(size_t)i * cols + j];
+        acc += (double)(x * scale + (i % 3 == 0 ? 0.25f : 0.0f));
+        mx = std::max(mx, x * x);
+        if (x > h[(size_t)best * cols + j]) best = i;
+      }
+      ok_s &= close(got_s[j], 2.0 * acc, 1e-6);
+      ok_m &= got_m[j] == mx;
+      ok_a &= got_a[j].key == best && got_a[j].value == h[(size_t)best * cols + j];
+    }
+    if (!(ok_s && ok_m && ok_a)) std::printf("    %d x %d: sums %d max %d arg %d\n", rows, cols, ok_s, ok_m, ok_a);
+    CHECK(ok_s);
+    CHECK(ok_m);
+    CHECK(ok_a);
+  }
+}
+
 int main()
 {
   int n = 0;
