@@ -589,6 +589,38 @@ def main():
                     pct_of_peak=100.0 * nb / (ms * 1e-3) / 1e9 / PEAK_HBM_GBPS,
                     check={"torch_fp64": ok})
 
+    def extra_dense_rows():
+        # row sums over rows of 17 lane-loads with tail elements (66 floats): a workgroup's load
+        # slots dealt over whole adjacent rows, the rows combined through LDS
+        rows, cols = 2000000, 66
+        xs = [mk_normal(rows, cols, 13 + 7919 * i) for i in range(3)]
+        out = torch.empty(rows, dtype=torch.float32, device="cuda")
+        d = api.make_desc(api.F32, api.F32, rows, cols)
+        ref = C.byref(d)
+
+        def call(i):
+            return lib.rmi_reduce(ref, xs[i % 3].data_ptr(), out.data_ptr(), None, 0, sptr)
+        for i in range(5):
+            rc = call(i)
+            assert rc == 0, api.status_string(rc)
+        torch.cuda.synchronize()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        n = max(10, args.steps // 4)
+        e0.record(stream)
+        for i in range(n):
+            call(i)
+        e1.record(stream)
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / n
+        nb = rows * cols * 4 + rows * 4
+        want = xs[(n - 1) % 3].view(rows, cols).sum(dim=1, dtype=torch.float64)
+        ok = bool(torch.allclose(out.double(), want, rtol=1e-5, atol=1e-5))
+        return dict(workload="row sum fp32 2000000x66 (17 lane-loads with a tail, dense slots)",
+                    ms_per_step=ms, alg_bytes=nb, GBps=nb / (ms * 1e-3) / 1e9,
+                    pct_of_peak=100.0 * nb / (ms * 1e-3) / 1e9 / PEAK_HBM_GBPS,
+                    check={"torch_fp64": ok})
+
     results = {}
     cpu = {}
     for name in names:
@@ -625,7 +657,7 @@ def main():
         "cpu_baseline": cpu.get(HEADLINE),
         "launch_floor_us": launch_floor_us(),
         "extras": ({"row_normalize": extra_row_normalize(), "meanvar": extra_meanvar(),
-                    "wide_columns": extra_wide_columns()}
+                    "wide_columns": extra_wide_columns(), "dense_rows": extra_dense_rows()}
                    if args.configs == "all" else {}),
         "configs": results,
         "cpu_baselines": cpu,

@@ -177,7 +177,7 @@ def extras(out: Path, commit: str):
     kt = {r["Name"]: r for r in rows}
     lines = []
     w = lines.append
-    w("rocprofv3 summary: row_normalize, meanvar and wide-row column sums, one MI355X (gfx950)")
+    w("rocprofv3 summary: row_normalize, meanvar, wide-row column sums and dense-slot row sums, one MI355X (gfx950)")
     w("=" * 88)
     w("")
     w(f"Library at commit {commit}.  Command (run from the repository root on the GPU box, TMPDIR=/tmp):")
@@ -193,7 +193,9 @@ def extras(out: Path, commit: str):
             ("meanvar fp32 10000000x64 row-major (one read)", "col_kernel<rmi::PolMeanVar<float>",
              "fold_kernel<rmi::PolMeanVar<float>", 2560000512),
             ("column sum fp32 32768x4097 (whole rows)", "col_wide_kernel<rmi::PolF<float, 0, 0>",
-             "fold_rows_kernel<rmi::PolF<float, 0, 0>", 32768 * 4097 * 4 + 4097 * 4)]
+             "fold_rows_kernel<rmi::PolF<float, 0, 0>", 32768 * 4097 * 4 + 4097 * 4),
+            ("row sum fp32 2000000x66 (dense slots)", "row_dense_kernel<rmi::PolF<float, 0, 0>", None,
+             2000000 * 67 * 4)]
     for label, k1, k2, alg in work:
         s1 = pick(kt, k1)
         if s1 is None:
@@ -212,7 +214,7 @@ def extras(out: Path, commit: str):
     w("single timed calls, so launch counts include those):")
     for n, r in kt.items():
         if "rmi::" in n and "normalize" not in n and "MeanVar" not in n and "col_wide" not in n \
-                and "fold_rows" not in n:
+                and "fold_rows" not in n and "row_dense" not in n:
             w(f"  {n[:100]:100s} {r['Calls']:>6s} {float(r['AverageNs']):12.1f}")
     (ROOT / "profiles" / "row_normalize_meanvar_rocprofv3.txt").write_text("\n".join(lines) + "\n")
     print("\n".join(lines[:16]))
