@@ -23,7 +23,7 @@
 extern "C" {
 #endif
 
-#define RMI_ABI_VERSION 2
+#define RMI_ABI_VERSION 3
 
 #if defined(__GNUC__) || defined(__clang__)
 #define RMI_API __attribute__((visibility("default")))
@@ -306,6 +306,34 @@ RMI_API int rmi_meanvar(int dtype,
                         void* workspace,
                         size_t workspace_bytes,
                         void* stream);
+
+/* Covariance matrix of the columns of an [n_rows, n_cols] matrix around a given mean
+ * vector: covar[i][j] = sum_n (x[n,i] - mu[i]) * (x[n,j] - mu[j]) / (sample ? n_rows - 1 :
+ * n_rows).  Replaces detail::cov (stats/detail/cov.cuh:38-66: meanCenter in place, then a
+ * cuBLAS GEMM X^T X scaled by alpha) behind raft::stats::cov (stats/cov.cuh:38-50 pointer
+ * form, :77-106 mdspan form).  `dtype` is F32 or F64 (data, mu and covar share it), `layout`
+ * the rmi_layout of `data`; `covar` is [n_cols][n_cols] and symmetric, so its layout does not
+ * matter.  The contraction runs on the matrix cores in `dtype` (fp32 or fp64 products and
+ * sums), partial sums of row slabs are added in f64.  `mu` may be NULL: the data is taken
+ * as centred already.  With RMI_COV_CENTER_DATA in `flags` the call leaves x - mu in `data`,
+ * which is what the reference documents ("this will get mean-centered at the end!") and its
+ * callers rely on; without it `data` is only read and the matrix is moved once instead of
+ * read and written.  n_rows == 0 writes zeros.  The workspace follows the rules of
+ * rmi_reduce (rmi_cov_workspace_bytes bytes, 16-byte aligned, no initialisation needed). */
+#define RMI_COV_CENTER_DATA 1
+RMI_API size_t rmi_cov_workspace_bytes(int dtype, int layout, int64_t n_rows, int64_t n_cols);
+RMI_API int rmi_cov(int dtype,
+                    int layout,
+                    int64_t n_rows,
+                    int64_t n_cols,
+                    int sample,
+                    int flags,
+                    void* data,
+                    const void* mu,
+                    void* covar,
+                    void* workspace,
+                    size_t workspace_bytes,
+                    void* stream);
 
 #ifdef __cplusplus
 } /* extern "C" */

@@ -35,6 +35,7 @@
 //   row normalisation: include/raft/linalg/detail/normalize.cuh:36-57,
 //       include/raft/linalg/normalize.cuh:91-107
 //   one-pass mean and variance: include/raft/stats/detail/meanvar.cuh:16-99
+//   covariance: include/raft/stats/detail/cov.cuh:38-66 (mean-centre, then alpha * X^T X)
 //
 // Pinned by (tests/test_oracle.py): the closed-form fixtures of
 // tests/linalg/reduce.cu:108-177, tests/matrix/argmax.cu:71-75,
@@ -42,7 +43,8 @@
 // tests/core/operators_host.cpp:134-172, tests/stats/sum.cu:50-98,
 // tests/stats/stddev.cu:139-150, tests/linalg/map_then_reduce.cu:140-169, and
 // by numpy closed forms on random inputs (orc_meanvar: numpy's two-pass mean / var
-// and the statistical tolerances of tests/stats/meanvar.cu:27-33).  The summation ORDER of the
+// and the statistical tolerances of tests/stats/meanvar.cu:27-33; orc_cov: the 3 x 2
+// known answer of tests/stats/cov.cu:88-100 and numpy.cov with both ddof in both layouts).  The summation ORDER of the
 // reference's device kernels (CUB block reductions, float atomics) is not
 // recoverable from its sources and is not pinned by its own tests either; both
 // implementations here fix an order of their own.
@@ -776,6 +778,52 @@ ORC_API int orc_meanvar(int dtype, int layout, int64_t n_rows, int64_t n_cols, i
     case RMI_F64: return meanvar_seq(layout, n_rows, n_cols, sample, (const double*)in, mean, var);
     case RMI_F16: return meanvar_seq(layout, n_rows, n_cols, sample, (const f16*)in, mean, var);
     case RMI_BF16: return meanvar_seq(layout, n_rows, n_cols, sample, (const bf16*)in, mean, var);
+    default: return RMI_ERR_UNSUPPORTED;
+  }
+}
+
+// Covariance around a given mean vector, as the reference computes it
+// (cpp/include/raft/stats/detail/cov.cuh:49-60): the data is mean-centred in its own type
+// (meanCenter, stats/detail/mean_center.cuh: data[n][j] - mu[j] rounded to Type), then
+// covar = alpha * X^T X with alpha = Type(1) / Type(sample ? N - 1 : N).  The products and
+// sums of the GEMM are restated in fp64 (the reference's order inside cuBLAS is not
+// recoverable); `centered`, when given, receives the centred data in the input's type, which
+// is what the reference leaves in `data`.  covar is [D][D], symmetric.
+template <class T>
+static int cov_seq(int layout, int64_t N, int64_t D, int sample, const T* in, const T* mu,
+                   double* covar, T* centered)
+{
+  std::vector<T> c((size_t)N * D);  // centred, row-major [N][D]
+  for (int64_t n = 0; n < N; ++n)
+    for (int64_t j = 0; j < D; ++j) {
+      const T x = layout == RMI_ROW_MAJOR ? in[n * D + j] : in[j * N + n];
+      const T d = mu != nullptr ? (T)(x - mu[j]) : x;
+      c[n * D + j] = d;
+      if (centered != nullptr) centered[layout == RMI_ROW_MAJOR ? n * D + j : j * N + n] = d;
+    }
+  const double alpha = N == 0 ? 0.0 : (double)(T(1) / (sample ? T(N - 1) : T(N)));
+#pragma omp parallel for schedule(dynamic, 1)
+  for (int64_t i = 0; i < D; ++i)
+    for (int64_t j = i; j < D; ++j) {
+      double s = 0.0;
+      for (int64_t n = 0; n < N; ++n)
+        s += (double)c[n * D + i] * (double)c[n * D + j];
+      covar[i * D + j] = covar[j * D + i] = s * alpha;
+    }
+  return RMI_OK;
+}
+
+ORC_API int orc_cov(int dtype, int layout, int64_t n_rows, int64_t n_cols, int sample,
+                    const void* in, const void* mu, double* covar, void* centered)
+{
+  if (layout != RMI_ROW_MAJOR && layout != RMI_COL_MAJOR) return RMI_ERR_BAD_ENUM;
+  switch (dtype) {
+    case RMI_F32:
+      return cov_seq(layout, n_rows, n_cols, sample, (const float*)in, (const float*)mu, covar,
+                     (float*)centered);
+    case RMI_F64:
+      return cov_seq(layout, n_rows, n_cols, sample, (const double*)in, (const double*)mu, covar,
+                     (double*)centered);
     default: return RMI_ERR_UNSUPPORTED;
   }
 }

@@ -14,9 +14,10 @@ LIB_PATH = Path(__file__).resolve().parent / "lib" / "libraft_amd.so"
 # rmi_status
 OK, ERR_NULL, ERR_BAD_ENUM, ERR_BAD_SHAPE, ERR_UNSUPPORTED, ERR_WORKSPACE, ERR_ALIGNMENT, \
     ERR_LAUNCH, ERR_NO_DEVICE, ERR_SCRATCH_LIMIT = range(10)
-ABI_VERSION = 2
+ABI_VERSION = 3
 NOALLOC_SCRATCH_BYTES = 4 << 20
 FLAG_WORKSPACE_ZEROED = 1
+COV_CENTER_DATA = 1
 WORKSPACE_TICKET_BYTES = 65536
 
 # rmi_dtype
@@ -87,6 +88,9 @@ SYMBOLS = {
     "rmi_meanvar_workspace_bytes": (C.c_size_t, [C.c_int, C.c_int, C.c_int64, C.c_int64]),
     "rmi_meanvar": (C.c_int, [C.c_int, C.c_int, C.c_int64, C.c_int64, C.c_int, C.c_void_p,
                               C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
+    "rmi_cov_workspace_bytes": (C.c_size_t, [C.c_int, C.c_int, C.c_int64, C.c_int64]),
+    "rmi_cov": (C.c_int, [C.c_int, C.c_int, C.c_int64, C.c_int64, C.c_int, C.c_int, C.c_void_p,
+                          C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
 }
 
 _lib = None

@@ -12,6 +12,28 @@
 static __device__ __align__(256) unsigned char scratch[RMI_NOALLOC_SCRATCH_BYTES];
 
 namespace rmi {
+
+// CU count of the current device, queried once per process.  Without a
+// visible device the MI355X figure is assumed so that planning works on a
+// build host.
+int cu_count()
+{
+  static std::atomic<int> cached{0};
+  int n = cached.load(std::memory_order_relaxed);
+  if (n > 0) return n;
+  int dev = 0;
+  hipDeviceProp_t prop;
+  if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess &&
+      prop.multiProcessorCount > 0) {
+    n = prop.multiProcessorCount;
+  } else {
+    (void)hipGetLastError();
+    n = 256;
+  }
+  cached.store(n, std::memory_order_relaxed);
+  return n;
+}
+
 namespace {
 
 // Device address of `scratch` on the current device, looked up once per device.
@@ -35,27 +57,6 @@ int scratch_of_current_device(void** out)
   }
   *out = p;
   return RMI_OK;
-}
-
-// CU count of the current device, queried once per process.  Without a
-// visible device the MI355X figure is assumed so that planning works on a
-// build host.
-int cu_count()
-{
-  static std::atomic<int> cached{0};
-  int n = cached.load(std::memory_order_relaxed);
-  if (n > 0) return n;
-  int dev = 0;
-  hipDeviceProp_t prop;
-  if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess &&
-      prop.multiProcessorCount > 0) {
-    n = prop.multiProcessorCount;
-  } else {
-    (void)hipGetLastError();
-    n = 256;
-  }
-  cached.store(n, std::memory_order_relaxed);
-  return n;
 }
 
 run_fn lookup(const PolicyKey& k)

@@ -1,0 +1,157 @@
+// rmi_cov / rmi_cov_workspace_bytes (include/rmi_reduce.h): shape checks, the split of the
+// work into column-block pairs and slabs of rows, and the launches.
+#include "rmi_cov.hpp"
+
+namespace rmi {
+int cu_count();  // rmi_api.hip
+
+namespace {
+
+// Workgroups per CU when one pair of column blocks covers the matrix (D <= 64, the
+// shape that is bound by HBM as much as by the matrix cores), and the number of queued
+// workgroups per CU otherwise (diagonal pairs issue 10 matrix instructions per wave-load,
+// the others 16: small units even the CUs out).
+#ifndef RMI_COV_WG_PER_CU
+#define RMI_COV_WG_PER_CU 3
+#endif
+constexpr int kWgPerCuOnePair = RMI_COV_WG_PER_CU;
+constexpr int kWgPerCuPairs   = 8;
+
+struct CovPlan {
+  int nb       = 0;
+  int npairs   = 0;
+  int S        = 1;
+  int total    = 0;
+  int grid     = 0;
+  bool vec     = false;  // row-major: rows are whole quads of columns
+  size_t ws_bytes = 0;
+};
+
+int make_cov_plan(int dtype, int layout, int64_t N, int64_t D, CovPlan& p)
+{
+  if (dtype != RMI_F32 && dtype != RMI_F64)
+    return dtype >= 0 && dtype < RMI_DTYPE_COUNT_ ? RMI_ERR_UNSUPPORTED : RMI_ERR_BAD_ENUM;
+  if (layout != RMI_ROW_MAJOR && layout != RMI_COL_MAJOR) return RMI_ERR_BAD_ENUM;
+  if (N < 0 || D < 0) return RMI_ERR_BAD_SHAPE;
+  const int64_t nb = (D + cov::kBlockCols - 1) / cov::kBlockCols;
+  if (nb > 8192) return RMI_ERR_BAD_SHAPE;  // 512k columns: the result alone would be 1 TB
+  p.nb     = (int)nb;
+  p.npairs = (int)(nb * (nb + 1) / 2);
+  p.vec    = D % 4 == 0;
+  const int es          = dtype == RMI_F32 ? 4 : 8;
+  const int step_rows   = layout == RMI_ROW_MAJOR ? 4 * cov::kRowLoads : (dtype == RMI_F32 ? 32 : 16);
+  const int64_t steps   = N / step_rows > 0 ? N / step_rows : 1;
+  const int n_cu        = cu_count();
+  int64_t S             = p.npairs <= 1 ? (int64_t)kWgPerCuOnePair * n_cu
+                                        : ((int64_t)kWgPerCuPairs * n_cu) / p.npairs;
+  // every wave gets two steps or more
+  const int64_t maxS = (steps + 2 * cov::kWaves - 1) / (2 * cov::kWaves);
+  if (S > maxS) S = maxS;
+  if (S < 1) S = 1;
+  p.S        = (int)S;
+  p.total    = p.S * p.npairs;
+  p.grid     = (p.total + 7) / 8 * 8;
+  p.ws_bytes = (size_t)p.total * cov::kTilesPerPair * cov::kTile * es;
+  return RMI_OK;
+}
+
+bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
+
+template <class T>
+int launch(const CovPlan& pl, int layout, int64_t N, int64_t D, int sample, bool center, T* data,
+           const T* mu, T* covar, void* ws, hipStream_t st)
+{
+  cov::GramArgs g{};
+  g.data    = data;
+  g.mu      = mu;
+  g.partial = ws;
+  g.N       = N;
+  g.D       = D;
+  g.nb      = pl.nb;
+  g.npairs  = pl.npairs;
+  g.S       = pl.S;
+  g.total   = pl.total;
+  g.center  = (center && mu != nullptr) ? 1 : 0;
+  if (g.center && pl.npairs > 1) {
+    // several workgroups read every column block: centre first, then contract what is left
+    const int64_t total = N * D;
+    const int64_t lead  = layout == RMI_ROW_MAJOR ? D : N;
+    int64_t blocks      = (total + cov::kThreads - 1) / cov::kThreads;
+    const int64_t cap   = (int64_t)cu_count() * 16;
+    if (blocks > cap) blocks = cap;
+    hipLaunchKernelGGL((cov::center_kernel<T>), dim3((unsigned)blocks), dim3(cov::kThreads), 0, st,
+                       data, mu, total, lead, layout == RMI_ROW_MAJOR ? 1 : 0);
+    g.mu     = nullptr;
+    g.center = 0;
+  }
+  const dim3 grid((unsigned)pl.grid);
+  if (layout == RMI_ROW_MAJOR) {
+    if (pl.vec)
+      hipLaunchKernelGGL((cov::gram_rows_kernel<T, true>), grid, dim3(cov::kThreads), 0, st, g);
+    else
+      hipLaunchKernelGGL((cov::gram_rows_kernel<T, false>), grid, dim3(cov::kThreads), 0, st, g);
+  } else {
+    hipLaunchKernelGGL((cov::gram_cols_kernel<T>), grid, dim3(cov::kThreads), 0, st, g);
+  }
+  cov::FoldArgs f{};
+  f.partial  = ws;
+  f.out      = covar;
+  f.D        = D;
+  f.nb       = pl.nb;
+  f.npairs   = pl.npairs;
+  f.S        = pl.S;
+  f.permuted = layout == RMI_ROW_MAJOR ? 1 : 0;
+  // the reference's scalar: Type(1) / Type(N - 1 | N), handed to the GEMM in Type
+  f.alpha = N == 0 ? 0.0 : (double)(T(1) / (sample ? T(N - 1) : T(N)));  // no rows: zeros, as a GEMM with k = 0
+  hipLaunchKernelGGL((cov::cov_fold_kernel<T>), dim3((unsigned)(pl.npairs * cov::kTilesPerPair)),
+                     dim3(cov::kTile * cov::kFoldSplit), 0, st, f);
+  return hipGetLastError() == hipSuccess ? RMI_OK : RMI_ERR_LAUNCH;
+}
+
+}  // namespace
+}  // namespace rmi
+
+extern "C" {
+
+size_t rmi_cov_workspace_bytes(int dtype, int layout, int64_t n_rows, int64_t n_cols)
+{
+  rmi::CovPlan pl;
+  if (rmi::make_cov_plan(dtype, layout, n_rows, n_cols, pl) != RMI_OK) return 0;
+  return n_cols > 0 ? pl.ws_bytes : 0;
+}
+
+int rmi_cov(int dtype,
+            int layout,
+            int64_t n_rows,
+            int64_t n_cols,
+            int sample,
+            int flags,
+            void* data,
+            const void* mu,
+            void* covar,
+            void* workspace,
+            size_t workspace_bytes,
+            void* stream)
+{
+  using namespace rmi;
+  if ((flags & ~RMI_COV_CENTER_DATA) != 0) return RMI_ERR_BAD_ENUM;
+  CovPlan pl;
+  const int rc = make_cov_plan(dtype, layout, n_rows, n_cols, pl);
+  if (rc != RMI_OK) return rc;
+  if (n_cols == 0) return RMI_OK;
+  if (covar == nullptr) return RMI_ERR_NULL;
+  if (n_rows > 0 && data == nullptr) return RMI_ERR_NULL;
+  const size_t es = dtype == RMI_F32 ? 4 : 8;
+  if (!aligned(data, es) || !aligned(mu, es) || !aligned(covar, es)) return RMI_ERR_ALIGNMENT;
+  if (workspace == nullptr || workspace_bytes < pl.ws_bytes || !aligned(workspace, 16))
+    return RMI_ERR_WORKSPACE;
+  hipStream_t st    = static_cast<hipStream_t>(stream);
+  const bool center = (flags & RMI_COV_CENTER_DATA) != 0;
+  if (dtype == RMI_F32)
+    return launch<float>(pl, layout, n_rows, n_cols, sample, center, static_cast<float*>(data),
+                         static_cast<const float*>(mu), static_cast<float*>(covar), workspace, st);
+  return launch<double>(pl, layout, n_rows, n_cols, sample, center, static_cast<double*>(data),
+                        static_cast<const double*>(mu), static_cast<double*>(covar), workspace, st);
+}
+
+}  // extern "C"

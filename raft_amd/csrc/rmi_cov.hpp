@@ -1,0 +1,582 @@
+// Covariance of the columns of a dense matrix around a given mean vector:
+//   covar = (X - 1 mu^T)^T (X - 1 mu^T) * alpha,   X: [N][D], covar: [D][D].
+// The one contraction on this path, so the one place that uses the matrix cores.
+//
+// The columns are cut into blocks of 64; a workgroup owns one pair of blocks (bi <= bj: the
+// upper triangle, the fold mirrors it) and one of S interleaved sets of rows (a slab), and
+// accumulates that pair's 64 x 64 piece of X^T X as sixteen 16 x 16 tiles (ten on the
+// diagonal) with v_mfma_f32_16x16x4_f32 / v_mfma_f64_16x16x4_f64.  The operands go from
+// global memory straight into the registers the instruction reads them from:
+//
+//   row-major X   lane l loads four consecutive columns 4 * (l % 16) .. + 3 of row l / 16 of
+//                 a wave-load of four rows; register j then holds, for the lanes 16 k .. 16 k
+//                 + 15, the columns {4 m + j} of row k, which is the A (and B) operand of a
+//                 16 x 16 x 4 step.  The result tile (ja, jb) is therefore the columns
+//                 {4 m + ja} x {4 n + jb}: a permutation the fold undoes.
+//   col-major X   lane l loads R consecutive rows of column 16 a + l % 16, the four lane
+//                 quarters reading four consecutive runs of rows; register j of column group
+//                 a and register j of group b are one 16 x 16 x 4 step of tile (a, b).
+//
+// x - mu happens in registers; with `center` set (one pair only, i.e. D <= 64) the centred
+// values are also written back, which is what the reference leaves in `data`.  Every wave
+// keeps its tiles for its whole share of the rows, the four waves of a workgroup meet in
+// LDS, and the workgroup stores its tiles as a partial [slab][pair][tile][256] that
+// cov_fold_kernel sums over the slabs in f64, in slab order, scales and writes to both
+// halves of the symmetric result.  Nothing is accumulated with atomics: results are
+// bitwise repeatable.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "rmi_reduce.h"
+
+namespace rmi {
+namespace cov {
+
+constexpr int kBlockCols    = 64;   // columns of a column block
+constexpr int kThreads      = 256;  // a workgroup: four waves
+constexpr int kWaves        = 4;
+constexpr int kTile         = 256;  // elements of a 16 x 16 result tile
+constexpr int kTilesPerPair = 16;   // 4 x 4 tiles of a 64 x 64 piece
+constexpr int kRowLoads     = 4;    // row-major: wave-loads (of four rows) per step
+constexpr int kFoldSplit    = 4;    // fold: threads that share the slabs of one element
+
+template <class T>
+struct Mma;
+template <>
+struct Mma<float> {
+  using acc_t = float __attribute__((ext_vector_type(4)));
+  static __device__ __forceinline__ acc_t mma(float a, float b, acc_t c)
+  {
+    return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
+  }
+  // row of the 16 x 16 result that register i of lane l holds (its column is l % 16)
+  static __device__ __forceinline__ int row(int lane, int i) { return 4 * (lane >> 4) + i; }
+  static constexpr int kColRows = 8;  // col-major: rows per lane, column group and step
+};
+template <>
+struct Mma<double> {
+  using acc_t = double __attribute__((ext_vector_type(4)));
+  static __device__ __forceinline__ acc_t mma(double a, double b, acc_t c)
+  {
+    return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ int row(int lane, int i) { return (lane >> 4) + 4 * i; }
+  static constexpr int kColRows = 4;
+};
+
+struct GramArgs {
+  void* data;        // [N][D] row-major or [D][N] col-major; written only with `center`
+  const void* mu;    // D means, or nullptr: the data is centred already
+  void* partial;     // [S][npairs][16][256] accumulators of T
+  int64_t N;
+  int64_t D;
+  int nb;            // column blocks
+  int npairs;        // nb * (nb + 1) / 2
+  int S;             // slabs
+  int total;         // S * npairs workgroups do work; the grid is rounded up to 8
+  int center;        // write x - mu back (npairs == 1 only)
+};
+
+struct FoldArgs {
+  const void* partial;
+  void* out;         // [D][D]
+  int64_t D;
+  int nb;
+  int npairs;
+  int S;
+  int permuted;      // tiles hold the columns {4 m + ja} x {4 n + jb} (row-major kernel)
+  double alpha;      // 1 / (N - 1) or 1 / N, rounded to T as the reference's scalar is
+};
+
+// Four elements at any element-aligned address (gfx950 serves unaligned vector loads).
+template <class T>
+struct Quad {
+  T v[4];
+};
+template <class T>
+__device__ __forceinline__ Quad<T> load_quad(const T* p, bool stream)
+{
+  typedef T full_t __attribute__((ext_vector_type(4)));
+  typedef full_t vec_t __attribute__((aligned(sizeof(T))));
+  const vec_t x = stream ? __builtin_nontemporal_load(reinterpret_cast<const vec_t*>(p))
+                         : *reinterpret_cast<const vec_t*>(p);
+  Quad<T> q;
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+    q.v[j] = x[j];
+  return q;
+}
+template <class T>
+__device__ __forceinline__ void store_quad(T* p, const Quad<T>& q)
+{
+  typedef T full_t __attribute__((ext_vector_type(4)));
+  typedef full_t vec_t __attribute__((aligned(sizeof(T))));
+  vec_t x;
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+    x[j] = q.v[j];
+  *reinterpret_cast<vec_t*>(p) = x;
+}
+
+// Workgroup ids are dealt round-robin over the 8 XCDs, each with an L2 of its own.  The
+// pairs of one slab read the same rows, so they are given ids that land on one XCD: id
+// 8 q + x becomes unit x * (grid / 8) + q, and units are numbered slab-major.
+__device__ __forceinline__ int xcd_local_unit()
+{
+  const int per_xcd = gridDim.x >> 3;
+  return (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+}
+
+__device__ __forceinline__ void pair_blocks(int p, int nb, int& bi, int& bj)
+{
+  bi = 0;
+  while (p >= nb - bi) {
+    p -= nb - bi;
+    ++bi;
+  }
+  bj = bi + p;
+}
+
+// The four waves' tiles meet in LDS, one wave at a time; wave 0 ends up with the sums.
+template <class T, int NT>
+__device__ __forceinline__ void combine_waves(typename Mma<T>::acc_t (&acc)[NT], T* sm, int wave,
+                                              int lane)
+{
+  for (int w = 1; w < kWaves; ++w) {
+    __syncthreads();
+    if (wave == w) {
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          sm[t * kTile + i * 64 + lane] = acc[t][i];
+    }
+    __syncthreads();
+    if (wave == 0) {
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          acc[t][i] += sm[t * kTile + i * 64 + lane];
+    }
+  }
+}
+
+template <class T>
+__device__ __forceinline__ void store_tile(T* partial, const typename Mma<T>::acc_t& acc, int lane)
+{
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    partial[i * 64 + lane] = acc[i];
+}
+
+// ---------------------------------------------------------------------------
+// Row-major X.  VEC: rows are whole quads of columns (D % 4 == 0), one vector load per
+// lane and block; otherwise four element loads with the column clamped.
+// ---------------------------------------------------------------------------
+template <class T, bool VEC, bool DIAG>
+__device__ __forceinline__ void gram_rows_body(const GramArgs& a, int unit, int slab, int bi, int bj,
+                                               T* sm)
+{
+  using M     = Mma<T>;
+  using acc_t = typename M::acc_t;
+  constexpr int NS = DIAG ? 1 : 2;  // blocks read: one on the diagonal
+
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int lr   = lane >> 4;  // row of the wave-load
+  const int cg   = lane & 15;  // quad of columns within the block
+  T* const data  = static_cast<T*>(a.data);
+  const T* mu    = static_cast<const T*>(a.mu);
+  const int64_t D = a.D;
+
+  // columns of this lane in the block(s), whether they exist, and their means
+  int64_t col[NS][4];
+  bool ok[NS][4];
+  T mean[NS][4];
+#pragma unroll
+  for (int s = 0; s < NS; ++s) {
+    const int64_t c0 = (int64_t)(s == 0 ? bi : bj) * kBlockCols + 4 * cg;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      ok[s][j]   = c0 + j < D;
+      col[s][j]  = ok[s][j] ? c0 + j : 0;
+      mean[s][j] = (mu != nullptr && ok[s][j]) ? mu[col[s][j]] : T(0);
+    }
+  }
+  const bool stream = a.npairs == 1;  // read once: keep it out of the caches
+
+  acc_t acc[kTilesPerPair];
+#pragma unroll
+  for (int t = 0; t < kTilesPerPair; ++t)
+    acc[t] = acc_t{0, 0, 0, 0};
+
+  constexpr int kStepRows = 4 * kRowLoads;
+  const int64_t G         = (int64_t)a.S * kWaves;  // waves that share the rows of a pair
+  const int64_t g         = (int64_t)slab * kWaves + wave;
+  const int64_t nfull     = a.N / kStepRows;
+
+  // one step: kRowLoads wave-loads of four rows for block bi (and bj off the diagonal)
+  auto load_step = [&](Quad<T> (&x)[NS][kRowLoads], int64_t step, bool guard) {
+#pragma unroll
+    for (int u = 0; u < kRowLoads; ++u) {
+      int64_t r = step * kStepRows + u * 4 + lr;
+      if (guard && r >= a.N) r = a.N - 1;
+      const T* rp = data + r * D;
+#pragma unroll
+      for (int s = 0; s < NS; ++s) {
+        if constexpr (VEC) {
+          x[s][u] = load_quad<T>(rp + col[s][0], stream);
+        } else {
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            x[s][u].v[j] = rp[col[s][j]];
+        }
+      }
+    }
+  };
+  auto fold_step = [&](const Quad<T> (&x)[NS][kRowLoads], int64_t step, bool guard) {
+#pragma unroll
+    for (int u = 0; u < kRowLoads; ++u) {
+      const int64_t r = step * kStepRows + u * 4 + lr;
+      const bool live = !guard || r < a.N;
+      T xa[4], xb[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        xa[j] = (ok[0][j] && live) ? x[0][u].v[j] - mean[0][j] : T(0);
+      if constexpr (DIAG) {
+        if (a.center && live) {
+          if constexpr (VEC) {
+            if (ok[0][0]) {
+              Quad<T> q;
+#pragma unroll
+              for (int j = 0; j < 4; ++j)
+                q.v[j] = xa[j];
+              store_quad<T>(data + r * D + col[0][0], q);
+            }
+          } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+              if (ok[0][j]) data[r * D + col[0][j]] = xa[j];
+          }
+        }
+#pragma unroll
+        for (int ja = 0; ja < 4; ++ja)
+#pragma unroll
+          for (int jb = ja; jb < 4; ++jb)
+            acc[ja * 4 + jb] = M::mma(xa[ja], xa[jb], acc[ja * 4 + jb]);
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          xb[j] = (ok[NS - 1][j] && live) ? x[NS - 1][u].v[j] - mean[NS - 1][j] : T(0);
+#pragma unroll
+        for (int ja = 0; ja < 4; ++ja)
+#pragma unroll
+          for (int jb = 0; jb < 4; ++jb)
+            acc[ja * 4 + jb] = M::mma(xa[ja], xb[jb], acc[ja * 4 + jb]);
+      }
+    }
+  };
+
+  // Steps are dealt round-robin over the G waves, so the grid reads one compact,
+  // advancing window of the matrix; a wave's next step is in flight while it feeds the
+  // current one to the matrix cores.
+  int64_t step = g;
+  Quad<T> x[NS][kRowLoads];
+  if (step < nfull) load_step(x, step, false);
+  while (step < nfull) {
+    const int64_t next = step + G;
+    Quad<T> y[NS][kRowLoads];
+    if (next < nfull) load_step(y, next, false);
+    fold_step(x, step, false);
+#pragma unroll
+    for (int s = 0; s < NS; ++s)
+#pragma unroll
+      for (int u = 0; u < kRowLoads; ++u)
+        x[s][u] = y[s][u];
+    step = next;
+  }
+  // the rows after the last whole step
+  if (nfull * kStepRows < a.N && g == nfull % G) {
+    load_step(x, nfull, true);
+    fold_step(x, nfull, true);
+  }
+
+  combine_waves<T, kTilesPerPair>(acc, sm, wave, lane);
+  if (wave == 0) {
+    T* out = static_cast<T*>(a.partial) + (int64_t)unit * kTilesPerPair * kTile;
+#pragma unroll
+    for (int ja = 0; ja < 4; ++ja)
+#pragma unroll
+      for (int jb = 0; jb < 4; ++jb)
+        if (!DIAG || jb >= ja) store_tile<T>(out + (ja * 4 + jb) * kTile, acc[ja * 4 + jb], lane);
+  }
+}
+
+template <class T, bool VEC>
+__global__ __launch_bounds__(kThreads) void gram_rows_kernel(GramArgs a)
+{
+  __shared__ T sm[kTilesPerPair * kTile];
+  const int unit = xcd_local_unit();
+  if (unit >= a.total) return;
+  const int slab = unit / a.npairs;
+  int bi, bj;
+  pair_blocks(unit - slab * a.npairs, a.nb, bi, bj);
+  // one wave-uniform branch around two bodies whose loads are unconditional
+  if (bi == bj)
+    gram_rows_body<T, VEC, true>(a, unit, slab, bi, bj, sm);
+  else
+    gram_rows_body<T, VEC, false>(a, unit, slab, bi, bj, sm);
+}
+
+// ---------------------------------------------------------------------------
+// Col-major X: column c is N consecutive values at data + c * N.
+// ---------------------------------------------------------------------------
+template <class T, bool DIAG>
+__device__ __forceinline__ void gram_cols_body(const GramArgs& a, int unit, int slab, int bi, int bj,
+                                               T* sm)
+{
+  using M     = Mma<T>;
+  using acc_t = typename M::acc_t;
+  constexpr int R  = M::kColRows;  // rows per lane, column group and step: two 16-byte loads
+  constexpr int NS = DIAG ? 1 : 2;
+
+  const int lane  = threadIdx.x & 63;
+  const int wave  = threadIdx.x >> 6;
+  const int rq    = lane >> 4;  // quarter of the step's rows
+  const int cl    = lane & 15;  // column within a group of 16
+  T* const data   = static_cast<T*>(a.data);
+  const T* mu     = static_cast<const T*>(a.mu);
+  const int64_t N = a.N;
+
+  // the lane's column in each of the four groups of the block(s)
+  T* colp[NS][4];
+  bool ok[NS][4];
+  T mean[NS][4];
+#pragma unroll
+  for (int s = 0; s < NS; ++s) {
+#pragma unroll
+    for (int gq = 0; gq < 4; ++gq) {
+      const int64_t c = (int64_t)(s == 0 ? bi : bj) * kBlockCols + 16 * gq + cl;
+      ok[s][gq]       = c < a.D;
+      colp[s][gq]     = data + (ok[s][gq] ? c : 0) * N;
+      mean[s][gq]     = (mu != nullptr && ok[s][gq]) ? mu[c] : T(0);
+    }
+  }
+  const bool stream = a.npairs == 1;
+
+  acc_t acc[kTilesPerPair];
+#pragma unroll
+  for (int t = 0; t < kTilesPerPair; ++t)
+    acc[t] = acc_t{0, 0, 0, 0};
+
+  constexpr int kStepRows = 4 * R;
+  const int64_t G         = (int64_t)a.S * kWaves;
+  const int64_t g         = (int64_t)slab * kWaves + wave;
+  const int64_t nfull     = N / kStepRows;
+
+  // x[s][gq][j]: row step * kStepRows + rq * R + j of the lane's column in group gq
+  auto load_step = [&](T (&x)[NS][4][R], int64_t step, bool guard) {
+    const int64_t r0 = step * kStepRows + rq * R;
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+#pragma unroll
+      for (int gq = 0; gq < 4; ++gq) {
+        if (!guard) {
+#pragma unroll
+          for (int q = 0; q < R / 4; ++q) {
+            const Quad<T> v = load_quad<T>(colp[s][gq] + r0 + 4 * q, stream);
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+              x[s][gq][4 * q + j] = v.v[j];
+          }
+        } else {
+#pragma unroll
+          for (int j = 0; j < R; ++j) {
+            const int64_t r = r0 + j < N ? r0 + j : N - 1;
+            x[s][gq][j]     = colp[s][gq][r];
+          }
+        }
+      }
+    }
+  };
+  auto fold_step = [&](T (&x)[NS][4][R], int64_t step, bool guard) {
+    const int64_t r0 = step * kStepRows + rq * R;
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+#pragma unroll
+      for (int gq = 0; gq < 4; ++gq)
+#pragma unroll
+        for (int j = 0; j < R; ++j) {
+          const bool live = ok[s][gq] && (!guard || r0 + j < N);
+          x[s][gq][j]     = live ? x[s][gq][j] - mean[s][gq] : T(0);
+        }
+    }
+    if constexpr (DIAG) {
+      if (a.center) {
+#pragma unroll
+        for (int gq = 0; gq < 4; ++gq) {
+          if (!ok[0][gq]) continue;
+          if (!guard) {
+#pragma unroll
+            for (int q = 0; q < R / 4; ++q) {
+              Quad<T> v;
+#pragma unroll
+              for (int j = 0; j < 4; ++j)
+                v.v[j] = x[0][gq][4 * q + j];
+              store_quad<T>(colp[0][gq] + r0 + 4 * q, v);
+            }
+          } else {
+#pragma unroll
+            for (int j = 0; j < R; ++j)
+              if (r0 + j < N) colp[0][gq][r0 + j] = x[0][gq][j];
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int ga = 0; ga < 4; ++ga)
+#pragma unroll
+      for (int gb = DIAG ? ga : 0; gb < 4; ++gb) {
+#pragma unroll
+        for (int j = 0; j < R; ++j)
+          acc[ga * 4 + gb] = M::mma(x[0][ga][j], x[NS - 1][gb][j], acc[ga * 4 + gb]);
+      }
+  };
+
+  int64_t step = g;
+  T x[NS][4][R];
+  if (step < nfull) load_step(x, step, false);
+  while (step < nfull) {
+    const int64_t next = step + G;
+    T y[NS][4][R];
+    if (next < nfull) load_step(y, next, false);
+    fold_step(x, step, false);
+#pragma unroll
+    for (int s = 0; s < NS; ++s)
+#pragma unroll
+      for (int gq = 0; gq < 4; ++gq)
+#pragma unroll
+        for (int j = 0; j < R; ++j)
+          x[s][gq][j] = y[s][gq][j];
+    step = next;
+  }
+  if (nfull * kStepRows < N && g == nfull % G) {
+    load_step(x, nfull, true);
+    fold_step(x, nfull, true);
+  }
+
+  combine_waves<T, kTilesPerPair>(acc, sm, wave, lane);
+  if (wave == 0) {
+    T* out = static_cast<T*>(a.partial) + (int64_t)unit * kTilesPerPair * kTile;
+#pragma unroll
+    for (int ga = 0; ga < 4; ++ga)
+#pragma unroll
+      for (int gb = 0; gb < 4; ++gb)
+        if (!DIAG || gb >= ga) store_tile<T>(out + (ga * 4 + gb) * kTile, acc[ga * 4 + gb], lane);
+  }
+}
+
+template <class T>
+__global__ __launch_bounds__(kThreads) void gram_cols_kernel(GramArgs a)
+{
+  __shared__ T sm[kTilesPerPair * kTile];
+  const int unit = xcd_local_unit();
+  if (unit >= a.total) return;
+  const int slab = unit / a.npairs;
+  int bi, bj;
+  pair_blocks(unit - slab * a.npairs, a.nb, bi, bj);
+  if (bi == bj)
+    gram_cols_body<T, true>(a, unit, slab, bi, bj, sm);
+  else
+    gram_cols_body<T, false>(a, unit, slab, bi, bj, sm);
+}
+
+// ---------------------------------------------------------------------------
+// Second pass: one workgroup per (pair, tile).  Thread (e, q) sums the slabs q, q + 4, ...
+// of element e in f64, the four meet in LDS in q order, the total is scaled and written
+// to covar[r][c] and covar[c][r].
+// ---------------------------------------------------------------------------
+template <class T>
+__global__ __launch_bounds__(kTile* kFoldSplit) void cov_fold_kernel(FoldArgs a)
+{
+  using M = Mma<T>;
+  __shared__ double sm[kFoldSplit][kTile];
+  const int pair = blockIdx.x / kTilesPerPair;
+  const int tile = blockIdx.x - pair * kTilesPerPair;
+  const int ta   = tile >> 2;
+  const int tb   = tile & 3;
+  int bi, bj;
+  pair_blocks(pair, a.nb, bi, bj);
+  if (bi == bj && tb < ta) return;  // the lower triangle is the mirror of the upper
+
+  const int e = threadIdx.x & (kTile - 1);
+  const int q = threadIdx.x / kTile;
+  const T* p  = static_cast<const T*>(a.partial) + ((int64_t)pair * kTilesPerPair + tile) * kTile + e;
+  const int64_t slab_stride = (int64_t)a.npairs * kTilesPerPair * kTile;
+  double sum = 0.0;
+  int s      = q;
+  for (; s + 3 * kFoldSplit < a.S; s += 4 * kFoldSplit) {
+    const T v0 = p[(int64_t)s * slab_stride];
+    const T v1 = p[(int64_t)(s + kFoldSplit) * slab_stride];
+    const T v2 = p[(int64_t)(s + 2 * kFoldSplit) * slab_stride];
+    const T v3 = p[(int64_t)(s + 3 * kFoldSplit) * slab_stride];
+    sum += (double)v0;
+    sum += (double)v1;
+    sum += (double)v2;
+    sum += (double)v3;
+  }
+  for (; s < a.S; s += kFoldSplit)
+    sum += (double)p[(int64_t)s * slab_stride];
+  sm[q][e] = sum;
+  __syncthreads();
+  if (q != 0) return;
+  for (int k = 1; k < kFoldSplit; ++k)
+    sum += sm[k][e];
+
+  const int lane = e & 63;
+  const int m    = M::row(lane, e >> 6);
+  const int n    = lane & 15;
+  const int64_t r = (int64_t)bi * kBlockCols + (a.permuted ? 4 * m + ta : 16 * ta + m);
+  const int64_t c = (int64_t)bj * kBlockCols + (a.permuted ? 4 * n + tb : 16 * tb + n);
+  if (r >= a.D || c >= a.D) return;
+  const T val = (T)(sum * a.alpha);
+  T* out      = static_cast<T*>(a.out);
+  out[r * a.D + c] = val;
+  // a diagonal tile holds both (r, c) and (c, r); everything else is mirrored
+  if (!(bi == bj && ta == tb)) out[c * a.D + r] = val;
+}
+
+// ---------------------------------------------------------------------------
+// data[n][c] -= mu[c], for matrices of more than one column block whose caller wants the
+// centred data left behind (the kernels above then run with mu == nullptr).
+// `lead` is the extent of the contiguous dimension, `by_lead` says that dimension is the
+// columns (row-major); `total` = N * D.
+// ---------------------------------------------------------------------------
+template <class T>
+__global__ __launch_bounds__(kThreads) void center_kernel(T* data, const T* mu, int64_t total,
+                                                          int64_t lead, int by_lead)
+{
+  // element i sits at position i % lead of line i / lead; both are carried along the
+  // grid-stride loop instead of divided out again
+  const int64_t stride    = (int64_t)gridDim.x * kThreads;
+  const int64_t step_line = stride / lead;
+  const int64_t step_pos  = stride - step_line * lead;
+  int64_t i               = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  int64_t line            = i / lead;
+  int64_t pos             = i - line * lead;
+  for (; i < total; i += stride) {
+    data[i] -= mu[by_lead ? pos : line];
+    line += step_line;
+    pos += step_pos;
+    if (pos >= lead) {
+      pos -= lead;
+      ++line;
+    }
+  }
+}
+
+}  // namespace cov
+}  // namespace rmi

@@ -495,6 +495,17 @@ __global__ __launch_bounds__(kBlock) void row_wave_kernel(RowArgs a)
   if (c == 0 && row < a.n_out) finish<P>(a.epi, row, acc);
 }
 
+// The hand-off between workgroups of one launch below is written for the cache hierarchy and
+// the s_waitcnt encoding of gfx942 / gfx950 and is outside the HIP memory model; refuse to
+// build it for anything else.
+#if defined(__HIP_DEVICE_COMPILE__) && !defined(__gfx950__) && !defined(__gfx942__)
+#error "the single-launch hand-off between workgroups is written for gfx942 / gfx950"
+#endif
+// s_waitcnt immediate, gfx9 encoding: vmcnt = 0 (bits 3:0 and 15:14), expcnt (6:4) and
+// lgkmcnt (11:8) left at their maxima, i.e. "wait until every vector memory operation of
+// this wave has completed or been acknowledged".
+constexpr int kWaitVmcnt0 = 0x0F70;
+
 // Partials that another workgroup of the SAME launch reads (single-launch split rows) are
 // written and read past the caches, word by word as device-scope relaxed atomics
 // (global_store / global_load with sc1): the eight L2 caches of the chip are not coherent
@@ -644,38 +655,38 @@ __global__ __launch_bounds__(1024) void row_block_kernel(RowArgs a)
     }
   }
   if (a.B > 1 && a.ticket != nullptr) {  // one team per workgroup here (T == blockDim.x)
-    __shared__ int last_of_row;
-    if (threadIdx.x == 0) {
-      int last = 0;
-      if (live) {
-        // Counters wrap to zero with their last ticket (atomicInc), so the area is clean for
-        // the next call.  Up to kFan chunks: one counter per row.  More: chunks count in
-        // groups of kFan, the last of a group counts for the row.  Line 0 of a row's lines
-        // is the row's counter, lines 1.. its groups'.
-        constexpr int kLine = kLineWords;
-        // The partial's stores (past the caches, same thread) must have completed before the
-        // ticket is taken.  A device-scope release would do that and write a whole L2 back
-        // besides; a workgroup-scope one orders the compiler but emits no wait (the waves of
-        // a workgroup share their CU's cache).  So: wait for this wave's outstanding memory
-        // operations (s_waitcnt vmcnt(0), gfx9 encoding: expcnt and lgkmcnt left at their
-        // maxima), after which a write-through store has been acknowledged by the memory side.
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-        __builtin_amdgcn_s_waitcnt(0x0F70);
-        if (a.B <= kFan) {
-          last = atomicInc(a.ticket + row * kLine, (u32)a.B - 1) == (u32)a.B - 1;
-        } else {
-          const int groups = (a.B + kFan - 1) / kFan;
-          const int g      = b / kFan;
-          const int gsize  = g == groups - 1 ? a.B - g * kFan : kFan;
-          u32* lines       = a.ticket + row * (groups + 1) * kLine;
-          if (atomicInc(lines + (1 + g) * kLine, (u32)gsize - 1) == (u32)gsize - 1)
-            last = atomicInc(lines, (u32)groups - 1) == (u32)groups - 1;
-        }
+    // Only the first wave goes on: it holds the thread that stored the partial, and its
+    // lanes learn from that thread whether they fold (a value read from its first lane,
+    // no barrier and no trip through LDS).
+    if (threadIdx.x >= kWave) return;
+    int last = 0;
+    if (threadIdx.x == 0 && live) {
+      // Counters wrap to zero with their last ticket (atomicInc), so the area is clean for
+      // the next call.  Up to kFan chunks: one counter per row.  More: chunks count in
+      // groups of kFan, the last of a group counts for the row.  Line 0 of a row's lines
+      // is the row's counter, lines 1.. its groups'.
+      constexpr int kLine = kLineWords;
+      // The partial's stores (past the caches, same thread) must have completed before the
+      // ticket is taken.  A device-scope release would do that and write a whole L2 back
+      // besides; a workgroup-scope one orders the compiler but emits no wait (the waves of
+      // a workgroup share their CU's cache).  So: wait for this wave's outstanding memory
+      // operations, after which a write-through store has been acknowledged by the memory
+      // side.
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+      __builtin_amdgcn_s_waitcnt(kWaitVmcnt0);
+      if (a.B <= kFan) {
+        last = atomicInc(a.ticket + row * kLine, (u32)a.B - 1) == (u32)a.B - 1;
+      } else {
+        const int groups = (a.B + kFan - 1) / kFan;
+        const int g      = b / kFan;
+        const int gsize  = g == groups - 1 ? a.B - g * kFan : kFan;
+        u32* lines       = a.ticket + row * (groups + 1) * kLine;
+        if (atomicInc(lines + (1 + g) * kLine, (u32)gsize - 1) == (u32)gsize - 1)
+          last = atomicInc(lines, (u32)groups - 1) == (u32)groups - 1;
       }
-      last_of_row = last;
     }
-    __syncthreads();
-    if (last_of_row && threadIdx.x < kWave) {
+    last = __builtin_amdgcn_readfirstlane(last);
+    if (last) {
       // every other workgroup's ticket, and with it its partial, is at the memory side by now
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
       const int lane = threadIdx.x;

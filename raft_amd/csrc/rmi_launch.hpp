@@ -434,6 +434,9 @@ run_fn lookup_for(const PolicyKey& k)
 #undef RMI_MAIN3_CASES
 }
 
+// CU count of the current device (256 when none is visible), cached; rmi_api.hip
+int cu_count();
+
 // one definition per input type, each in its own translation unit
 run_fn lookup_i8(const PolicyKey&);
 run_fn lookup_u8(const PolicyKey&);

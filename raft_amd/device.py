@@ -67,3 +67,18 @@ def meanvar(dtype: int, layout: int, n_rows: int, n_cols: int, sample: bool,
                          current_stream_ptr())
     if rc != api.OK:
         raise RmiError(rc, "rmi_meanvar")
+
+
+def cov(dtype: int, layout: int, n_rows: int, n_cols: int, sample: bool, data: torch.Tensor,
+        mu: torch.Tensor | None, covar: torch.Tensor, *, center: bool = False) -> None:
+    """Run rmi_cov on the current torch stream; with `center` the call leaves x - mu in `data`."""
+    lib = api.load()
+    n = lib.rmi_cov_workspace_bytes(dtype, layout, n_rows, n_cols)
+    ws = torch.empty(max(n, 16), dtype=torch.uint8, device=covar.device)
+    rc = lib.rmi_cov(dtype, layout, n_rows, n_cols, 1 if sample else 0,
+                     api.COV_CENTER_DATA if center else 0,
+                     data.data_ptr() if data is not None else None,
+                     mu.data_ptr() if mu is not None else None, covar.data_ptr(), ws.data_ptr(), n,
+                     current_stream_ptr())
+    if rc != api.OK:
+        raise RmiError(rc, "rmi_cov")

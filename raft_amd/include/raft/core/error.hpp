@@ -72,6 +72,12 @@ inline std::string format_failure(char const* prefix, char const* file, int line
       "exception occurred! ", __FILE__, __LINE__, fmt, ##__VA_ARGS__));                    \
   } while (0)
 
+// core/error.hpp:297-300 in the reference: a failed check raises raft::exception
+#define ASSERT(check, fmt, ...)              \
+  do {                                       \
+    if (!(check)) THROW(fmt, ##__VA_ARGS__); \
+  } while (0)
+
 #define RAFT_HIP_TRY(call)                                                                 \
   do {                                                                                     \
     hipError_t const raft_status_ = (call);                                                \

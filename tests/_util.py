@@ -46,6 +46,9 @@ def load_oracle() -> C.CDLL:
         lib.orc_meanvar.restype = C.c_int
         lib.orc_meanvar.argtypes = [C.c_int, C.c_int, C.c_int64, C.c_int64, C.c_int, C.c_void_p,
                                     C.c_void_p, C.c_void_p]
+        lib.orc_cov.restype = C.c_int
+        lib.orc_cov.argtypes = [C.c_int, C.c_int, C.c_int64, C.c_int64, C.c_int, C.c_void_p,
+                                C.c_void_p, C.c_void_p, C.c_void_p]
         for name in ("orc_f32_to_bf16", "orc_bf16_to_f32", "orc_f32_to_f16", "orc_f16_to_f32"):
             getattr(lib, name).restype = None
             getattr(lib, name).argtypes = [C.c_void_p, C.c_void_p, C.c_int64]

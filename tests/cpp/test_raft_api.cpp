@@ -18,6 +18,7 @@
 #include <raft/linalg/strided_reduction.cuh>
 #include <raft/matrix/argmax.cuh>
 #include <raft/matrix/argmin.cuh>
+#include <raft/stats/cov.cuh>
 #include <raft/stats/mean.cuh>
 #include <raft/stats/meanvar.cuh>
 #include <raft/stats/stddev.cuh>
@@ -509,6 +510,126 @@ void meanvar_cases(double tol)
   CHECK(threw);
 }
 
+// cpp/tests/stats/cov.cu:37-105: the mean through stats::mean, cov through the mdspan form (the
+// grid, rows cut to keep the host reference short, plus a width that is no multiple of four), the
+// 3 x 2 column-major known answer through the pointer form, the centred data left behind, and
+// the refusal of stable == false.
+template <typename T>
+void cov_cases(double tol)
+{
+  raft::resources handle;
+  auto stream = raft::resource::get_cuda_stream(handle);
+  struct Case { double mean, var; int rows, cols; bool sample, row_major; };
+  std::vector<Case> cases;
+  for (bool rm : {false, true})
+    for (int cols : {32, 64, 128, 256, 70})
+      for (bool sample : {true, false})
+        cases.push_back({sample ? 1.0 : -1.0, 2.0, 4096, cols, sample, rm});
+  for (const auto& c : cases) {
+    const size_t n = (size_t)c.rows * c.cols;
+    auto data_h    = normal<T>(n, c.mean, c.var, 1234);
+    auto data_d    = raft::make_device_vector<T, int>(handle, (int)n);
+    raft::update_device(data_d.data_handle(), data_h.data(), n, stream);
+    auto mu   = raft::make_device_vector<T, int>(handle, c.cols);
+    auto cv   = raft::make_device_vector<T, int>(handle, c.cols * c.cols);
+    if (c.row_major) {
+      using layout = raft::row_major;
+      raft::stats::mean<true>(mu.data_handle(), data_d.data_handle(), c.cols, c.rows, stream);
+      raft::stats::cov(handle,
+                       raft::make_device_matrix_view<T, std::uint32_t, layout>(data_d.data_handle(), c.rows, c.cols),
+                       raft::make_device_vector_view<const T, std::uint32_t>(mu.data_handle(), c.cols),
+                       raft::make_device_matrix_view<T, std::uint32_t, layout>(cv.data_handle(), c.cols, c.cols),
+                       c.sample, true);
+    } else {
+      using layout = raft::col_major;
+      raft::stats::mean<false>(mu.data_handle(), data_d.data_handle(), c.cols, c.rows, stream);
+      raft::stats::cov(handle,
+                       raft::make_device_matrix_view<T, std::uint32_t, layout>(data_d.data_handle(), c.rows, c.cols),
+                       raft::make_device_vector_view<const T, std::uint32_t>(mu.data_handle(), c.cols),
+                       raft::make_device_matrix_view<T, std::uint32_t, layout>(cv.data_handle(), c.cols, c.cols),
+                       c.sample, true);
+    }
+    auto mu_h  = to_host(mu.data_handle(), (size_t)c.cols, stream);
+    auto cv_h  = to_host(cv.data_handle(), (size_t)c.cols * c.cols, stream);
+    auto cen_h = to_host(data_d.data_handle(), n, stream);
+    // host reference: centre in T around the device's mean, contract in double
+    std::vector<T> cen(n);
+    for (int i = 0; i < c.rows; ++i)
+      for (int j = 0; j < c.cols; ++j) {
+        const size_t k = at(c.row_major, c.rows, c.cols, i, j);
+        cen[k]         = (T)(data_h[k] - mu_h[j]);
+      }
+    CHECK(cen_h == cen);  // "this will get mean-centered at the end!"
+    const double alpha = (double)(T(1) / (c.sample ? T(c.rows - 1) : T(c.rows)));
+    bool ok = true, diag_ok = true;
+    std::vector<double> dg(c.cols);
+    for (int a = 0; a < c.cols; ++a) {
+      double s = 0;
+      for (int i = 0; i < c.rows; ++i) {
+        const double v = (double)cen[at(c.row_major, c.rows, c.cols, i, a)];
+        s += v * v;
+      }
+      dg[a] = s * alpha;
+    }
+    for (int a = 0; a < c.cols; ++a)
+      for (int b = a; b < c.cols; ++b) {
+        double s = 0;
+        for (int i = 0; i < c.rows; ++i)
+          s += (double)cen[at(c.row_major, c.rows, c.cols, i, a)] *
+               (double)cen[at(c.row_major, c.rows, c.cols, i, b)];
+        const double want = s * alpha;
+        const double lim  = tol * std::sqrt(dg[a] * dg[b]);
+        ok &= std::fabs((double)cv_h[(size_t)a * c.cols + b] - want) <= lim;
+        ok &= cv_h[(size_t)a * c.cols + b] == cv_h[(size_t)b * c.cols + a];
+      }
+    CHECK(ok);
+    // diagonalMatch(var * var, ..., CompareApprox(2 * 0.03)) with a sample of 4096 rows
+    for (int a = 0; a < c.cols; ++a) {
+      const double d = (double)cv_h[(size_t)a * c.cols + a], w = c.var * c.var;
+      diag_ok &= std::fabs(d - w) / std::max(std::fabs(d), w) <= 0.12;
+    }
+    CHECK(diag_ok);
+  }
+  {
+    T data_h[6]       = {1.0, 2.0, 5.0, 4.0, 2.0, 1.0};
+    T cov_cm_ref_h[4] = {4.3333, -2.8333, -2.8333, 2.333};
+    auto data_cm = raft::make_device_vector<T, int>(handle, 6);
+    auto mean_cm = raft::make_device_vector<T, int>(handle, 2);
+    auto cov_cm  = raft::make_device_vector<T, int>(handle, 4);
+    raft::update_device(data_cm.data_handle(), data_h, 6, stream);
+    raft::stats::mean<false>(mean_cm.data_handle(), data_cm.data_handle(), 2, 3, stream);
+    raft::stats::cov<false>(handle, cov_cm.data_handle(), data_cm.data_handle(),
+                            mean_cm.data_handle(), 2, 3, true, true, stream);
+    auto got = to_host(cov_cm.data_handle(), 4, stream);
+    bool ok  = true;
+    for (int i = 0; i < 4; ++i) {
+      const double a = (double)got[i], b = (double)cov_cm_ref_h[i];
+      ok &= std::fabs(a - b) / std::max(std::fabs(a), std::fabs(b)) <= 0.06;
+    }
+    CHECK(ok);
+    bool threw = false;
+    try {
+      raft::stats::cov<false>(handle, cov_cm.data_handle(), data_cm.data_handle(),
+                              mean_cm.data_handle(), 2, 3, true, false, stream);
+    } catch (const raft::exception&) {
+      threw = true;
+    }
+    CHECK(threw);
+    // size mismatch between data and covar (stats/cov.cuh:88-89)
+    threw = false;
+    try {
+      raft::stats::cov(handle,
+                       raft::make_device_matrix_view<T, int, raft::row_major>(data_cm.data_handle(), 3, 2),
+                       raft::make_device_vector_view<const T, int>(mean_cm.data_handle(), 2),
+                       raft::make_device_matrix_view<T, int, raft::row_major>(cov_cm.data_handle(), 2, 1),
+                       true, true);
+    } catch (const raft::logic_error&) {
+      threw = true;
+    }
+    CHECK(threw);
+  }
+}
+
 // cpp/tests/stats/mean.cu:177-185: int8 -> half
 void mean_int8_to_half()
 {
@@ -766,6 +887,8 @@ TEST_CASE(MeanStddevF) { mean_stddev<float>(1e-5); }
 TEST_CASE(MeanStddevD) { mean_stddev<double>(1e-9); }
 TEST_CASE(MeanVarF) { meanvar_cases<float>(1e-5); }
 TEST_CASE(MeanVarD) { meanvar_cases<double>(1e-9); }
+TEST_CASE(CovF) { cov_cases<float>(1e-5); }
+TEST_CASE(CovD) { cov_cases<double>(1e-12); }
 TEST_CASE(MeanInt8ToHalf) { mean_int8_to_half(); }
 TEST_CASE(SumAccuracyF) { sum_accuracy<float>(0.0001f, 1e7, 0.001); }
 TEST_CASE(SumAccuracyD) { sum_accuracy<double>(0.000001, 1e12, 0.0001); }

@@ -442,3 +442,54 @@ def test_meanvar_against_numpy(oracle, npdt, dt, layout, sample):
         if rows >= 700 and sd == 2.0:
             assert np.all(np.abs(mean - mu) <= 6 * sd / np.sqrt(rows))
             assert np.all(np.abs(var - sd * sd) <= 6 * sd * sd * np.sqrt(2.0 / (rows - 1)))
+
+
+# ---- covariance ------------------------------------------------------------------------
+# orc_cov restates "mean-centre in the data's type, then alpha * X^T X".  The reference's
+# own known answer (cpp/tests/stats/cov.cu:88-100,163-177) and numpy.cov fix what it must
+# produce: ddof distinguishes N from N - 1, the non-square shapes and both layouts catch a
+# transposed operand or a wrong stride, a mean far from zero catches a dropped centring.
+def _orc_cov(oracle, dt, layout, rows, cols, sample, stored, mu, want_centered=False):
+    covar = np.zeros((cols, cols))
+    cen = np.zeros_like(stored) if want_centered else None
+    rc = oracle.orc_cov(dt, layout, rows, cols, int(sample), stored.ctypes.data,
+                        mu.ctypes.data if mu is not None else None, covar.ctypes.data,
+                        cen.ctypes.data if cen is not None else None)
+    assert rc == 0
+    return covar, cen
+
+
+@pytest.mark.parametrize("npdt,dt", [(np.float32, api.F32), (np.float64, api.F64)])
+def test_cov_known_answer_fixture(oracle, npdt, dt):
+    k = GOLD["stats_cov"]["known_answer"]
+    data = np.array(k["data"], dtype=npdt)  # column-major 3 x 2
+    m = data.reshape(k["cols"], k["rows"]).T
+    mu = m.mean(axis=0).astype(npdt)
+    covar, _ = _orc_cov(oracle, dt, api.COL_MAJOR, k["rows"], k["cols"], k["sample"], data, mu)
+    tol = 2 * GOLD["stats_cov"]["cases"][0][0]
+    exp = np.array(k["covar"]).reshape(2, 2)
+    assert np.all(np.abs(covar - exp) <= tol * np.maximum(1.0, np.abs(exp)))
+    np.testing.assert_allclose(covar, np.cov(m.astype(np.float64), rowvar=False, ddof=1), rtol=1e-6)
+
+
+@pytest.mark.parametrize("npdt,dt,rtol", [(np.float32, api.F32, 2e-6), (np.float64, api.F64, 1e-12)])
+@pytest.mark.parametrize("layout", [api.ROW_MAJOR, api.COL_MAJOR])
+@pytest.mark.parametrize("sample", [False, True])
+def test_cov_against_numpy(oracle, npdt, dt, rtol, layout, sample):
+    rng = np.random.default_rng(99)
+    for rows, cols, mean in [(1000, 7, 3.0), (257, 33, -1.0), (64, 70, 100.0), (2, 3, 0.5)]:
+        m = (rng.normal(mean, 2.0, (rows, cols)) * rng.uniform(0.5, 2.0, cols)).astype(npdt)
+        stored = np.ascontiguousarray(m if layout == api.ROW_MAJOR else m.T).reshape(-1)
+        mu = m.astype(np.float64).mean(axis=0).astype(npdt)
+        covar, cen = _orc_cov(oracle, dt, layout, rows, cols, sample, stored, mu, True)
+        exp = np.cov(m.astype(np.float64), rowvar=False, ddof=1 if sample else 0)
+        scale = np.sqrt(np.outer(np.diag(exp), np.diag(exp)))
+        # the data is centred in its own type around a mean rounded to that type
+        assert np.all(np.abs(covar - exp) <= rtol * scale * max(1.0, abs(mean))), (rows, cols)
+        assert np.array_equal(covar, covar.T)
+        # what the reference leaves in `data`
+        cen_m = cen.reshape(rows, cols) if layout == api.ROW_MAJOR else cen.reshape(cols, rows).T
+        assert np.array_equal(cen_m, (m - mu[None, :]).astype(npdt))
+        # mu == NULL: the data is taken as centred
+        c2, _ = _orc_cov(oracle, dt, layout, rows, cols, sample, cen, None)
+        assert np.array_equal(c2, covar)
