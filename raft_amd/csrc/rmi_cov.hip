@@ -12,7 +12,7 @@ namespace {
 // workgroups per CU otherwise (diagonal pairs issue 10 matrix instructions per wave-load,
 // the others 16: small units even the CUs out).
 #ifndef RMI_COV_WG_PER_CU
-#define RMI_COV_WG_PER_CU 3
+#define RMI_COV_WG_PER_CU 2
 #endif
 constexpr int kWgPerCuOnePair = RMI_COV_WG_PER_CU;
 constexpr int kWgPerCuPairs   = 8;
@@ -39,13 +39,13 @@ int make_cov_plan(int dtype, int layout, int64_t N, int64_t D, CovPlan& p)
   p.npairs = (int)(nb * (nb + 1) / 2);
   p.vec    = D % 4 == 0;
   const int es          = dtype == RMI_F32 ? 4 : 8;
-  const int step_rows   = layout == RMI_ROW_MAJOR ? 4 * cov::kRowLoads : (dtype == RMI_F32 ? 32 : 16);
+  const int step_rows   = layout == RMI_ROW_MAJOR ? cov::kRowUnitRows : cov::kColUnitRows;
   const int64_t steps   = N / step_rows > 0 ? N / step_rows : 1;
   const int n_cu        = cu_count();
   int64_t S             = p.npairs <= 1 ? (int64_t)kWgPerCuOnePair * n_cu
                                         : ((int64_t)kWgPerCuPairs * n_cu) / p.npairs;
-  // every wave gets two steps or more
-  const int64_t maxS = (steps + 2 * cov::kWaves - 1) / (2 * cov::kWaves);
+  // every wave gets eight units or more
+  const int64_t maxS = (steps + 8 * cov::kWaves - 1) / (8 * cov::kWaves);
   if (S > maxS) S = maxS;
   if (S < 1) S = 1;
   p.S        = (int)S;
@@ -71,8 +71,8 @@ int launch(const CovPlan& pl, int layout, int64_t N, int64_t D, int sample, bool
   g.npairs  = pl.npairs;
   g.S       = pl.S;
   g.total   = pl.total;
-  g.center  = (center && mu != nullptr) ? 1 : 0;
-  if (g.center && pl.npairs > 1) {
+  bool write_back = center && mu != nullptr;
+  if (write_back && pl.npairs > 1) {
     // several workgroups read every column block: centre first, then contract what is left
     const int64_t total = N * D;
     const int64_t lead  = layout == RMI_ROW_MAJOR ? D : N;
@@ -81,17 +81,32 @@ int launch(const CovPlan& pl, int layout, int64_t N, int64_t D, int sample, bool
     if (blocks > cap) blocks = cap;
     hipLaunchKernelGGL((cov::center_kernel<T>), dim3((unsigned)blocks), dim3(cov::kThreads), 0, st,
                        data, mu, total, lead, layout == RMI_ROW_MAJOR ? 1 : 0);
-    g.mu     = nullptr;
-    g.center = 0;
+    g.mu       = nullptr;
+    write_back = false;
   }
   const dim3 grid((unsigned)pl.grid);
-  if (layout == RMI_ROW_MAJOR) {
-    if (pl.vec)
-      hipLaunchKernelGGL((cov::gram_rows_kernel<T, true>), grid, dim3(cov::kThreads), 0, st, g);
+  const dim3 block(cov::kThreads);
+  const bool one = pl.npairs == 1;
+  if (write_back) {  // one column block: the same pass leaves x - mu behind
+    if (layout != RMI_ROW_MAJOR)
+      hipLaunchKernelGGL((cov::gram_cols_kernel<T, true, true>), grid, block, 0, st, g);
+    else if (pl.vec)
+      hipLaunchKernelGGL((cov::gram_rows_kernel<T, true, true, true>), grid, block, 0, st, g);
     else
-      hipLaunchKernelGGL((cov::gram_rows_kernel<T, false>), grid, dim3(cov::kThreads), 0, st, g);
+      hipLaunchKernelGGL((cov::gram_rows_kernel<T, false, true, true>), grid, block, 0, st, g);
+  } else if (layout == RMI_ROW_MAJOR) {
+    if (pl.vec && one)
+      hipLaunchKernelGGL((cov::gram_rows_kernel<T, true, true>), grid, block, 0, st, g);
+    else if (pl.vec)
+      hipLaunchKernelGGL((cov::gram_rows_kernel<T, true, false>), grid, block, 0, st, g);
+    else if (one)
+      hipLaunchKernelGGL((cov::gram_rows_kernel<T, false, true>), grid, block, 0, st, g);
+    else
+      hipLaunchKernelGGL((cov::gram_rows_kernel<T, false, false>), grid, block, 0, st, g);
+  } else if (one) {
+    hipLaunchKernelGGL((cov::gram_cols_kernel<T, true>), grid, block, 0, st, g);
   } else {
-    hipLaunchKernelGGL((cov::gram_cols_kernel<T>), grid, dim3(cov::kThreads), 0, st, g);
+    hipLaunchKernelGGL((cov::gram_cols_kernel<T, false>), grid, block, 0, st, g);
   }
   cov::FoldArgs f{};
   f.partial  = ws;

@@ -39,8 +39,25 @@ constexpr int kThreads      = 256;  // a workgroup: four waves
 constexpr int kWaves        = 4;
 constexpr int kTile         = 256;  // elements of a 16 x 16 result tile
 constexpr int kTilesPerPair = 16;   // 4 x 4 tiles of a 64 x 64 piece
-constexpr int kRowLoads     = 4;    // row-major: wave-loads (of four rows) per step
+#ifndef RMI_COV_ROW_UNIT_LOADS
+#define RMI_COV_ROW_UNIT_LOADS 4
+#endif
+#ifndef RMI_COV_ROW_RING
+#define RMI_COV_ROW_RING 3
+#endif
+constexpr int kRowUnitLoads = RMI_COV_ROW_UNIT_LOADS;  // row-major: wave-loads of a unit
+constexpr int kRowRing      = RMI_COV_ROW_RING;        // ... and units in the ring
+constexpr int kRowUnitRows  = 4 * kRowUnitLoads;      // rows of a unit
+constexpr int kColUnitRows  = 16;   // col-major: rows of a unit (four per lane quarter)
 constexpr int kFoldSplit    = 4;    // fold: threads that share the slabs of one element
+
+// units a wave keeps in flight, given the 32-bit registers one unit takes: about 64
+// registers' worth, at least two and at most eight
+constexpr int ring_depth(int unit_regs)
+{
+  const int p = 64 / unit_regs;
+  return p < 2 ? 2 : (p > 8 ? 8 : p);
+}
 
 template <class T>
 struct Mma;
@@ -53,7 +70,6 @@ struct Mma<float> {
   }
   // row of the 16 x 16 result that register i of lane l holds (its column is l % 16)
   static __device__ __forceinline__ int row(int lane, int i) { return 4 * (lane >> 4) + i; }
-  static constexpr int kColRows = 8;  // col-major: rows per lane, column group and step
 };
 template <>
 struct Mma<double> {
@@ -63,7 +79,6 @@ struct Mma<double> {
     return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0);
   }
   static __device__ __forceinline__ int row(int lane, int i) { return (lane >> 4) + 4 * i; }
-  static constexpr int kColRows = 4;
 };
 
 struct GramArgs {
@@ -76,7 +91,6 @@ struct GramArgs {
   int npairs;        // nb * (nb + 1) / 2
   int S;             // slabs
   int total;         // S * npairs workgroups do work; the grid is rounded up to 8
-  int center;        // write x - mu back (npairs == 1 only)
 };
 
 struct FoldArgs {
@@ -95,13 +109,18 @@ template <class T>
 struct Quad {
   T v[4];
 };
-template <class T>
-__device__ __forceinline__ Quad<T> load_quad(const T* p, bool stream)
+// STREAM: the data is read once, keep it out of the caches (non-temporal).  A template
+// parameter: chosen by a run-time flag, the two forms are merged into one plain load.
+template <class T, bool STREAM>
+__device__ __forceinline__ Quad<T> load_quad(const T* p)
 {
   typedef T full_t __attribute__((ext_vector_type(4)));
   typedef full_t vec_t __attribute__((aligned(sizeof(T))));
-  const vec_t x = stream ? __builtin_nontemporal_load(reinterpret_cast<const vec_t*>(p))
-                         : *reinterpret_cast<const vec_t*>(p);
+  vec_t x;
+  if constexpr (STREAM)
+    x = __builtin_nontemporal_load(reinterpret_cast<const vec_t*>(p));
+  else
+    x = *reinterpret_cast<const vec_t*>(p);
   Quad<T> q;
 #pragma unroll
   for (int j = 0; j < 4; ++j)
@@ -176,16 +195,22 @@ __device__ __forceinline__ void store_tile(T* partial, const typename Mma<T>::ac
 // Row-major X.  VEC: rows are whole quads of columns (D % 4 == 0), one vector load per
 // lane and block; otherwise four element loads with the column clamped.
 // ---------------------------------------------------------------------------
-template <class T, bool VEC, bool DIAG>
+template <class T, bool VEC, bool DIAG, bool CENTER, bool STREAM>
 __device__ __forceinline__ void gram_rows_body(const GramArgs& a, int unit, int slab, int bi, int bj,
                                                T* sm)
 {
   using M     = Mma<T>;
   using acc_t = typename M::acc_t;
   constexpr int NS = DIAG ? 1 : 2;  // blocks read: one on the diagonal
+  constexpr int UL = kRowUnitLoads;
+  constexpr int UR = 4 * UL;        // rows of a unit
+  constexpr int P  = kRowRing;
 
   const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
+  // (read from the first lane so that the compiler knows it, and every row and unit index
+  // derived from it, to be the same for the whole wave: scalar registers and scalar
+  // arithmetic instead of 64-bit vector multiplies per lane-load)
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lr   = lane >> 4;  // row of the wave-load
   const int cg   = lane & 15;  // quad of columns within the block
   T* const data  = static_cast<T*>(a.data);
@@ -206,29 +231,32 @@ __device__ __forceinline__ void gram_rows_body(const GramArgs& a, int unit, int 
       mean[s][j] = (mu != nullptr && ok[s][j]) ? mu[col[s][j]] : T(0);
     }
   }
-  const bool stream = a.npairs == 1;  // read once: keep it out of the caches
 
   acc_t acc[kTilesPerPair];
 #pragma unroll
   for (int t = 0; t < kTilesPerPair; ++t)
     acc[t] = acc_t{0, 0, 0, 0};
 
-  constexpr int kStepRows = 4 * kRowLoads;
-  const int64_t G         = (int64_t)a.S * kWaves;  // waves that share the rows of a pair
-  const int64_t g         = (int64_t)slab * kWaves + wave;
-  const int64_t nfull     = a.N / kStepRows;
+  // A unit is UL wave-loads of four rows each: UR adjacent rows of the block(s).  Units are
+  // dealt round-robin over the G waves that share the rows of a pair, the four waves of a
+  // workgroup side by side, so the grid reads one compact, advancing window of the matrix
+  // in contiguous pieces of 4 * UR rows per workgroup.
+  const int64_t G     = (int64_t)a.S * kWaves;
+  const int64_t g     = (int64_t)slab * kWaves + wave;
+  const int64_t nfull = a.N / UR;
+  const int64_t K     = g < nfull ? (nfull - g + G - 1) / G : 0;  // whole units of this wave
 
-  // one step: kRowLoads wave-loads of four rows for block bi (and bj off the diagonal)
-  auto load_step = [&](Quad<T> (&x)[NS][kRowLoads], int64_t step, bool guard) {
+  auto load_unit = [&](Quad<T> (&x)[NS][UL], int64_t q, bool guard) {
 #pragma unroll
-    for (int u = 0; u < kRowLoads; ++u) {
-      int64_t r = step * kStepRows + u * 4 + lr;
-      if (guard && r >= a.N) r = a.N - 1;
-      const T* rp = data + r * D;
+    for (int u = 0; u < UL; ++u) {
+      // the wave's first row of this load (uniform) plus the lane's row within it
+      const int64_t r0 = q * UR + u * 4;
+      const int64_t dr = (guard && r0 + lr >= a.N) ? a.N - 1 - r0 : lr;
+      const T* rp      = data + r0 * D + dr * D;
 #pragma unroll
       for (int s = 0; s < NS; ++s) {
         if constexpr (VEC) {
-          x[s][u] = load_quad<T>(rp + col[s][0], stream);
+          x[s][u] = load_quad<T, STREAM>(rp + col[s][0]);
         } else {
 #pragma unroll
           for (int j = 0; j < 4; ++j)
@@ -237,24 +265,27 @@ __device__ __forceinline__ void gram_rows_body(const GramArgs& a, int unit, int 
       }
     }
   };
-  auto fold_step = [&](const Quad<T> (&x)[NS][kRowLoads], int64_t step, bool guard) {
+  // `live`: the unit exists (wave-uniform); `guard`: its rows may run past the matrix
+  auto fold_unit = [&](const Quad<T> (&x)[NS][UL], int64_t q, bool live, bool guard) {
 #pragma unroll
-    for (int u = 0; u < kRowLoads; ++u) {
-      const int64_t r = step * kStepRows + u * 4 + lr;
-      const bool live = !guard || r < a.N;
+    for (int u = 0; u < UL; ++u) {
+      const int64_t r = q * UR + u * 4 + lr;
+      const bool in   = live && (!guard || r < a.N);
       T xa[4], xb[4];
 #pragma unroll
       for (int j = 0; j < 4; ++j)
-        xa[j] = (ok[0][j] && live) ? x[0][u].v[j] - mean[0][j] : T(0);
+        xa[j] = (ok[0][j] && in) ? x[0][u].v[j] - mean[0][j] : T(0);
       if constexpr (DIAG) {
-        if (a.center && live) {
+        // (CENTER is a template parameter: a store behind a run-time flag, even one that is
+        // never taken, makes the compiler wait for every load of the ring at the loop's top)
+        if (CENTER && in) {
           if constexpr (VEC) {
             if (ok[0][0]) {
-              Quad<T> q;
+              Quad<T> w;
 #pragma unroll
               for (int j = 0; j < 4; ++j)
-                q.v[j] = xa[j];
-              store_quad<T>(data + r * D + col[0][0], q);
+                w.v[j] = xa[j];
+              store_quad<T>(data + r * D + col[0][0], w);
             }
           } else {
 #pragma unroll
@@ -270,7 +301,7 @@ __device__ __forceinline__ void gram_rows_body(const GramArgs& a, int unit, int 
       } else {
 #pragma unroll
         for (int j = 0; j < 4; ++j)
-          xb[j] = (ok[NS - 1][j] && live) ? x[NS - 1][u].v[j] - mean[NS - 1][j] : T(0);
+          xb[j] = (ok[NS - 1][j] && in) ? x[NS - 1][u].v[j] - mean[NS - 1][j] : T(0);
 #pragma unroll
         for (int ja = 0; ja < 4; ++ja)
 #pragma unroll
@@ -280,28 +311,36 @@ __device__ __forceinline__ void gram_rows_body(const GramArgs& a, int unit, int 
     }
   };
 
-  // Steps are dealt round-robin over the G waves, so the grid reads one compact,
-  // advancing window of the matrix; a wave's next step is in flight while it feeds the
-  // current one to the matrix cores.
-  int64_t step = g;
-  Quad<T> x[NS][kRowLoads];
-  if (step < nfull) load_step(x, step, false);
-  while (step < nfull) {
-    const int64_t next = step + G;
-    Quad<T> y[NS][kRowLoads];
-    if (next < nfull) load_step(y, next, false);
-    fold_step(x, step, false);
+  // A ring of P units: every slot is used and at once refilled with the unit P further on, so
+  // the other slots' loads stay in flight behind the matrix instructions and no register is
+  // copied.  All of it is unconditional (past the end a slot reloads the wave's last unit and
+  // counts as zero): behind a branch, or with a copy of the prefetched registers at the loop's
+  // end, the compiler waits for the prefetch before the next step and nothing overlaps.
+  if (K > 0) {
+    Quad<T> ring[P][NS][UL];
 #pragma unroll
-    for (int s = 0; s < NS; ++s)
+    for (int i = 0; i < P; ++i) {
+      load_unit(ring[i], g + (i < K ? i : K - 1) * G, false);
+      // in slot order, like the refills: issued in another order, the loop's first wait would
+      // have to cover all of them on the way in, and so (the paths merge) on every trip
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    for (int64_t k0 = 0; k0 < K; k0 += P) {
 #pragma unroll
-      for (int u = 0; u < kRowLoads; ++u)
-        x[s][u] = y[s][u];
-    step = next;
+      for (int i = 0; i < P; ++i) {
+        const int64_t k = k0 + i;
+        fold_unit(ring[i], g + k * G, k < K, false);
+        __builtin_amdgcn_sched_barrier(0);
+        load_unit(ring[i], g + (k + P < K ? k + P : K - 1) * G, false);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
   }
-  // the rows after the last whole step
-  if (nfull * kStepRows < a.N && g == nfull % G) {
-    load_step(x, nfull, true);
-    fold_step(x, nfull, true);
+  // the rows after the last whole unit
+  if (nfull * UR < a.N && g == nfull % G) {
+    Quad<T> x[NS][UL];
+    load_unit(x, nfull, true);
+    fold_unit(x, nfull, true, true);
   }
 
   combine_waves<T, kTilesPerPair>(acc, sm, wave, lane);
@@ -315,7 +354,10 @@ __device__ __forceinline__ void gram_rows_body(const GramArgs& a, int unit, int 
   }
 }
 
-template <class T, bool VEC>
+// ONE: the matrix has one column block (D <= 64), so only the diagonal body is compiled in,
+// the kernel's register count is that body's, and the matrix, read once, is streamed past
+// the caches (with several blocks the pairs of a slab share their rows through the L2).
+template <class T, bool VEC, bool ONE, bool CENTER = false>
 __global__ __launch_bounds__(kThreads) void gram_rows_kernel(GramArgs a)
 {
   __shared__ T sm[kTilesPerPair * kTile];
@@ -325,27 +367,29 @@ __global__ __launch_bounds__(kThreads) void gram_rows_kernel(GramArgs a)
   int bi, bj;
   pair_blocks(unit - slab * a.npairs, a.nb, bi, bj);
   // one wave-uniform branch around two bodies whose loads are unconditional
-  if (bi == bj)
-    gram_rows_body<T, VEC, true>(a, unit, slab, bi, bj, sm);
-  else
-    gram_rows_body<T, VEC, false>(a, unit, slab, bi, bj, sm);
+  static_assert(ONE || !CENTER, "the centred data is written back by the one-block kernel only");
+  if (ONE || bi == bj) {
+    gram_rows_body<T, VEC, true, CENTER, ONE>(a, unit, slab, bi, bj, sm);
+  } else {
+    if constexpr (!ONE) gram_rows_body<T, VEC, false, false, false>(a, unit, slab, bi, bj, sm);
+  }
 }
 
 // ---------------------------------------------------------------------------
 // Col-major X: column c is N consecutive values at data + c * N.
 // ---------------------------------------------------------------------------
-template <class T, bool DIAG>
+template <class T, bool DIAG, bool CENTER, bool STREAM>
 __device__ __forceinline__ void gram_cols_body(const GramArgs& a, int unit, int slab, int bi, int bj,
                                                T* sm)
 {
   using M     = Mma<T>;
   using acc_t = typename M::acc_t;
-  constexpr int R  = M::kColRows;  // rows per lane, column group and step: two 16-byte loads
   constexpr int NS = DIAG ? 1 : 2;
+  constexpr int P  = ring_depth(NS * 16 * (int)sizeof(T) / 4);
 
   const int lane  = threadIdx.x & 63;
-  const int wave  = threadIdx.x >> 6;
-  const int rq    = lane >> 4;  // quarter of the step's rows
+  const int wave  = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform, see above
+  const int rq    = lane >> 4;  // quarter of the unit's rows
   const int cl    = lane & 15;  // column within a group of 16
   T* const data   = static_cast<T*>(a.data);
   const T* mu     = static_cast<const T*>(a.mu);
@@ -365,73 +409,58 @@ __device__ __forceinline__ void gram_cols_body(const GramArgs& a, int unit, int 
       mean[s][gq]     = (mu != nullptr && ok[s][gq]) ? mu[c] : T(0);
     }
   }
-  const bool stream = a.npairs == 1;
 
   acc_t acc[kTilesPerPair];
 #pragma unroll
   for (int t = 0; t < kTilesPerPair; ++t)
     acc[t] = acc_t{0, 0, 0, 0};
 
-  constexpr int kStepRows = 4 * R;
-  const int64_t G         = (int64_t)a.S * kWaves;
-  const int64_t g         = (int64_t)slab * kWaves + wave;
-  const int64_t nfull     = N / kStepRows;
+  // A unit is sixteen rows: every lane holds four consecutive rows of its column in each
+  // group, the four lane quarters four consecutive runs.
+  const int64_t G     = (int64_t)a.S * kWaves;
+  const int64_t g     = (int64_t)slab * kWaves + wave;
+  const int64_t nfull = N / kColUnitRows;
+  const int64_t K     = g < nfull ? (nfull - g + G - 1) / G : 0;
 
-  // x[s][gq][j]: row step * kStepRows + rq * R + j of the lane's column in group gq
-  auto load_step = [&](T (&x)[NS][4][R], int64_t step, bool guard) {
-    const int64_t r0 = step * kStepRows + rq * R;
+  auto load_unit = [&](Quad<T> (&x)[NS][4], int64_t q, bool guard) {
+    const int64_t r0 = q * kColUnitRows + rq * 4;
 #pragma unroll
     for (int s = 0; s < NS; ++s) {
 #pragma unroll
       for (int gq = 0; gq < 4; ++gq) {
         if (!guard) {
-#pragma unroll
-          for (int q = 0; q < R / 4; ++q) {
-            const Quad<T> v = load_quad<T>(colp[s][gq] + r0 + 4 * q, stream);
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-              x[s][gq][4 * q + j] = v.v[j];
-          }
+          x[s][gq] = load_quad<T, STREAM>(colp[s][gq] + r0);
         } else {
 #pragma unroll
-          for (int j = 0; j < R; ++j) {
-            const int64_t r = r0 + j < N ? r0 + j : N - 1;
-            x[s][gq][j]     = colp[s][gq][r];
-          }
+          for (int j = 0; j < 4; ++j)
+            x[s][gq].v[j] = colp[s][gq][r0 + j < N ? r0 + j : N - 1];
         }
       }
     }
   };
-  auto fold_step = [&](T (&x)[NS][4][R], int64_t step, bool guard) {
-    const int64_t r0 = step * kStepRows + rq * R;
+  auto fold_unit = [&](const Quad<T> (&x)[NS][4], int64_t q, bool live, bool guard) {
+    const int64_t r0 = q * kColUnitRows + rq * 4;
+    Quad<T> c[NS][4];
 #pragma unroll
-    for (int s = 0; s < NS; ++s) {
+    for (int s = 0; s < NS; ++s)
 #pragma unroll
       for (int gq = 0; gq < 4; ++gq)
 #pragma unroll
-        for (int j = 0; j < R; ++j) {
-          const bool live = ok[s][gq] && (!guard || r0 + j < N);
-          x[s][gq][j]     = live ? x[s][gq][j] - mean[s][gq] : T(0);
+        for (int j = 0; j < 4; ++j) {
+          const bool in = live && ok[s][gq] && (!guard || r0 + j < N);
+          c[s][gq].v[j] = in ? x[s][gq].v[j] - mean[s][gq] : T(0);
         }
-    }
     if constexpr (DIAG) {
-      if (a.center) {
+      if (CENTER && live) {
 #pragma unroll
         for (int gq = 0; gq < 4; ++gq) {
           if (!ok[0][gq]) continue;
           if (!guard) {
-#pragma unroll
-            for (int q = 0; q < R / 4; ++q) {
-              Quad<T> v;
-#pragma unroll
-              for (int j = 0; j < 4; ++j)
-                v.v[j] = x[0][gq][4 * q + j];
-              store_quad<T>(colp[0][gq] + r0 + 4 * q, v);
-            }
+            store_quad<T>(colp[0][gq] + r0, c[0][gq]);
           } else {
 #pragma unroll
-            for (int j = 0; j < R; ++j)
-              if (r0 + j < N) colp[0][gq][r0 + j] = x[0][gq][j];
+            for (int j = 0; j < 4; ++j)
+              if (r0 + j < N) colp[0][gq][r0 + j] = c[0][gq].v[j];
           }
         }
       }
@@ -441,31 +470,36 @@ __device__ __forceinline__ void gram_cols_body(const GramArgs& a, int unit, int 
 #pragma unroll
       for (int gb = DIAG ? ga : 0; gb < 4; ++gb) {
 #pragma unroll
-        for (int j = 0; j < R; ++j)
-          acc[ga * 4 + gb] = M::mma(x[0][ga][j], x[NS - 1][gb][j], acc[ga * 4 + gb]);
+        for (int j = 0; j < 4; ++j)
+          acc[ga * 4 + gb] = M::mma(c[0][ga].v[j], c[NS - 1][gb].v[j], acc[ga * 4 + gb]);
       }
   };
 
-  int64_t step = g;
-  T x[NS][4][R];
-  if (step < nfull) load_step(x, step, false);
-  while (step < nfull) {
-    const int64_t next = step + G;
-    T y[NS][4][R];
-    if (next < nfull) load_step(y, next, false);
-    fold_step(x, step, false);
+  // the same ring as gram_rows_body's
+  if (K > 0) {
+    Quad<T> ring[P][NS][4];
 #pragma unroll
-    for (int s = 0; s < NS; ++s)
+    for (int i = 0; i < P; ++i) {
+      load_unit(ring[i], g + (i < K ? i : K - 1) * G, false);
+      // in slot order, like the refills: issued in another order, the loop's first wait would
+      // have to cover all of them on the way in, and so (the paths merge) on every trip
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    for (int64_t k0 = 0; k0 < K; k0 += P) {
 #pragma unroll
-      for (int gq = 0; gq < 4; ++gq)
-#pragma unroll
-        for (int j = 0; j < R; ++j)
-          x[s][gq][j] = y[s][gq][j];
-    step = next;
+      for (int i = 0; i < P; ++i) {
+        const int64_t k = k0 + i;
+        fold_unit(ring[i], g + k * G, k < K, false);
+        __builtin_amdgcn_sched_barrier(0);
+        load_unit(ring[i], g + (k + P < K ? k + P : K - 1) * G, false);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
   }
-  if (nfull * kStepRows < N && g == nfull % G) {
-    load_step(x, nfull, true);
-    fold_step(x, nfull, true);
+  if (nfull * kColUnitRows < N && g == nfull % G) {
+    Quad<T> x[NS][4];
+    load_unit(x, nfull, true);
+    fold_unit(x, nfull, true, true);
   }
 
   combine_waves<T, kTilesPerPair>(acc, sm, wave, lane);
@@ -479,7 +513,7 @@ __device__ __forceinline__ void gram_cols_body(const GramArgs& a, int unit, int 
   }
 }
 
-template <class T>
+template <class T, bool ONE, bool CENTER = false>
 __global__ __launch_bounds__(kThreads) void gram_cols_kernel(GramArgs a)
 {
   __shared__ T sm[kTilesPerPair * kTile];
@@ -488,10 +522,12 @@ __global__ __launch_bounds__(kThreads) void gram_cols_kernel(GramArgs a)
   const int slab = unit / a.npairs;
   int bi, bj;
   pair_blocks(unit - slab * a.npairs, a.nb, bi, bj);
-  if (bi == bj)
-    gram_cols_body<T, true>(a, unit, slab, bi, bj, sm);
-  else
-    gram_cols_body<T, false>(a, unit, slab, bi, bj, sm);
+  static_assert(ONE || !CENTER, "the centred data is written back by the one-block kernel only");
+  if (ONE || bi == bj) {
+    gram_cols_body<T, true, CENTER, ONE>(a, unit, slab, bi, bj, sm);
+  } else {
+    if constexpr (!ONE) gram_cols_body<T, false, false, false>(a, unit, slab, bi, bj, sm);
+  }
 }
 
 // ---------------------------------------------------------------------------
