@@ -16,7 +16,9 @@ timed one by one after a 768 MB scratch sweep has evicted the caches (median and
 minimum of the repetitions; the method of the reference's benchmark fixture,
 cpp/bench/prims/common/benchmark.hpp:138-155).
 
-Prints one JSON line.  `roofline.achieved` = algorithmic bytes (input read once +
+Prints one JSON line; `roofline.by_config` holds ms per step, algorithmic bytes and the
+fraction of 8 TB/s for every workload (the long per-workload records go to
+bench_details.json).  `roofline.achieved` = algorithmic bytes (input read once +
 output written once) / average launch duration.  `roofline.traffic` is NOT measured in
 this run: it is read from profiles/traffic.json, which raft_amd/bench/profile_summary.py
 writes from rocprofv3 counter runs of this same program (the file names the commit it
@@ -79,44 +81,37 @@ def main():
     stream = torch.cuda.current_stream()
     sptr = stream.cuda_stream
 
-    def gen(seed):
-        g = torch.Generator(device=devc)
-        g.manual_seed(seed)
-        return g
+    # Inputs come from a counter-based generator (raft_amd/bench/synth.py): element i of a
+    # buffer is a function of (seed, i) alone, so the host can recompute any of them; the
+    # seeds are echoed in the output line.
+    from raft_amd.bench import synth
 
-    # ------------------------------------------------------------------
-    # workloads
-    # ------------------------------------------------------------------
     def mk_normal(rows, cols, seed, mean=0.0, std=1.0):
-        x = torch.randn(rows * cols, generator=gen(seed), device=devc, dtype=torch.float32)
-        if std != 1.0:
-            x.mul_(std)
-        if mean != 0.0:
-            x.add_(mean)
-        return x
+        return synth.normal_device(seed, rows * cols, mean, std, devc)
 
     def mk_uniform(rows, cols, seed):
-        x = torch.rand(rows * cols, generator=gen(seed), device=devc, dtype=torch.float32)
-        return x.mul_(2.0).sub_(1.0)
+        return synth.uniform_device(seed, rows * cols, devc)
 
     def mk_int8(rows, cols, seed):
-        return torch.randint(-128, 128, (rows * cols,), generator=gen(seed), device=devc,
-                             dtype=torch.int8)
+        return synth.int8_device(seed, rows * cols, devc)
 
     def mk_bf16(rows, cols, seed):
         return mk_uniform(rows, cols, seed).to(torch.bfloat16)
 
     def mk_logits_with_ties(rows, cols, seed):
+        # rows whose hash is 0 mod 100 (1 % of them) get their maximum copied to one to three
+        # further columns, all drawn from the same counter-based stream
         x = mk_normal(rows, cols, seed).view(rows, cols)
-        g = gen(seed + 1000)
-        n_tie = max(1, rows // 100)
-        tie_rows = torch.randperm(rows, generator=g, device=devc)[:n_tie]
+        h = torch.from_numpy(synth.bits_host(seed + 1000, np.arange(rows * 4)).view(np.int64)
+                             .reshape(rows, 4)).to(devc)
+        lsr = lambda z, k: (z >> k) & ((1 << (64 - k)) - 1)  # noqa: E731
+        tie_rows = torch.nonzero(lsr(h[:, 0], 8) % 100 == 0).view(-1)
         mx = x[tie_rows].amax(dim=1)
         for j in range(3):  # 1..3 further copies of the row maximum
-            pos = torch.randint(0, cols, (n_tie,), generator=g, device=devc)
-            keep = torch.rand(n_tie, generator=g, device=devc) < (1.0 if j == 0 else 0.5)
-            sel = tie_rows[keep]
-            x[sel, pos[keep]] = mx[keep]
+            hj = h[tie_rows, j + 1]
+            pos = lsr(hj, 20) % cols
+            keep = torch.ones_like(pos, dtype=torch.bool) if j == 0 else (hj & 1) == 1
+            x[tie_rows[keep], pos[keep]] = mx[keep]
         return x.view(-1)
 
     f32 = np.float32
@@ -621,6 +616,62 @@ def main():
                     pct_of_peak=100.0 * nb / (ms * 1e-3) / 1e9 / PEAK_HBM_GBPS,
                     check={"torch_fp64": ok})
 
+    def extra_cov():
+        # covariance of config 3's matrix around its column means: the one contraction on the
+        # path (matrix cores).  Two bounds: HBM (the matrix once + D^2 outputs) and the fp32
+        # matrix peak (2 N D^2 flop, half of it by symmetry, at 157.3 TFLOP/s); the tighter one
+        # (the longer time) is the roof.  `centered` times the reference's semantics (the call
+        # leaves x - mu in the data: read + write).
+        rows, cols = 10000000, 64
+        xs = [mk_normal(rows, cols, 3 + 7919 * i, 3.0, 2.0) for i in range(3)]
+        mus = [x.view(rows, cols).mean(dim=0, dtype=torch.float64).to(torch.float32) for x in xs]
+        out = torch.empty(cols * cols, dtype=torch.float32, device="cuda")
+        nws = lib.rmi_cov_workspace_bytes(api.F32, api.ROW_MAJOR, rows, cols)
+        ws = torch.empty(max(nws, 16), dtype=torch.uint8, device="cuda")
+
+        def call(i, flags):
+            return lib.rmi_cov(api.F32, api.ROW_MAJOR, rows, cols, 1, flags, xs[i % 3].data_ptr(),
+                               mus[i % 3].data_ptr(), out.data_ptr(), ws.data_ptr(), nws, sptr)
+        res = {}
+        n = max(10, args.steps // 4)
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        for name, flags in (("read_only", 0), ("centered", api.COV_CENTER_DATA)):
+            if flags == 0:
+                for i in range(3):
+                    rc = call(i, flags)
+                    assert rc == 0, api.status_string(rc)
+                torch.cuda.synchronize()
+                x = xs[2].view(rows, cols)
+                ref = torch.zeros(cols, cols, dtype=torch.float64, device="cuda")
+                for c in x.split(1 << 20):
+                    d = (c - mus[2][None, :]).to(torch.float64)
+                    ref += d.T @ d
+                ref /= rows - 1
+                sc = torch.sqrt(torch.outer(torch.diagonal(ref), torch.diagonal(ref)))
+                ok = bool(((out.view(cols, cols).double() - ref).abs() <= 1e-5 * sc).all())
+            e0.record(stream)
+            for i in range(n):
+                call(i, flags)
+            e1.record(stream)
+            torch.cuda.synchronize()
+            ms = e0.elapsed_time(e1) / n
+            nb = rows * cols * 4 * (2 if flags else 1) + cols * cols * 4
+            res[name] = dict(ms_per_step=ms, alg_bytes=nb, GBps=nb / (ms * 1e-3) / 1e9)
+        hbm_ms = (rows * cols * 4 + cols * cols * 4) / (PEAK_HBM_GBPS * 1e9) * 1e3
+        mfma_ms = rows * cols * cols / 157.3e12 * 1e3
+        ms = res["read_only"]["ms_per_step"]
+        return dict(workload="stats::cov fp32 10000000x64 row-major around its column means",
+                    ms_per_step=ms, alg_bytes=res["read_only"]["alg_bytes"],
+                    GBps=res["read_only"]["GBps"],
+                    pct_of_peak=100.0 * res["read_only"]["GBps"] / PEAK_HBM_GBPS,
+                    bounds_ms={"hbm": hbm_ms, "mfma_fp32_symmetric": mfma_ms},
+                    bound="hbm" if hbm_ms >= mfma_ms else "mfma",
+                    frac_of_bound=max(hbm_ms, mfma_ms) / ms,
+                    TFLOPs_symmetric=rows * cols * cols / (ms * 1e-3) / 1e12,
+                    centered=res["centered"],
+                    check={"torch_fp64": ok})
+
     results = {}
     cpu = {}
     for name in names:
@@ -633,6 +684,23 @@ def main():
         torch.cuda.empty_cache()
 
     head = results[HEADLINE]
+    extras = ({"row_normalize": extra_row_normalize(), "meanvar": extra_meanvar(),
+               "wide_columns": extra_wide_columns(), "dense_rows": extra_dense_rows(),
+               "cov": extra_cov()}
+              if args.configs == "all" else {})
+    # One short line: the contract's keys, and inside `roofline` / `config` / `cpu_baseline`
+    # what a reader needs to recompute every workload's fraction (ms per step and
+    # algorithmic bytes).  The long per-workload records go to a file beside the run.
+    by_config = {}
+    for name, r in list(results.items()) + list(extras.items()):
+        by_config[name] = {"ms": round(r["ms_per_step"], 6), "alg_bytes": r["alg_bytes"],
+                           "frac": round(r["GBps"] / PEAK_HBM_GBPS, 4),
+                           "traffic": PROFILE_TRAFFIC.get(name),
+                           "check": bool(all(v is True or not isinstance(v, bool)
+                                             for v in (r.get("check") or {}).values()))}
+        if "frac_of_bound" in r:
+            by_config[name]["frac_of_bound"] = round(r["frac_of_bound"], 4)
+            by_config[name]["bound"] = r["bound"]
     line = {
         "metric": "achieved HBM GB/s, L2 row norm fp32 1000000x128 (algorithmic bytes / kernel time)",
         "value": head["GBps"],
@@ -647,22 +715,31 @@ def main():
         "dtype": "f32",
         "data": "synthetic",
         "config": {"workload": WORK[HEADLINE]["desc"], "plan": head["plan"],
-                   "buffers_rotated": head["buffers"], "timing": "hip events on the launch stream"},
-        "rows_per_s": head["rows_per_s"],
-        "pct_of_hbm_peak": head["pct_of_peak"],
+                   "buffers_rotated": head["buffers"], "timing": "hip events on the launch stream",
+                   "generator": "splitmix64 counter-based (raft_amd/bench/synth.py); buffer i of a "
+                                "workload uses seed + 7919 * i",
+                   "seeds": {n: WORK[n]["seed"] for n in results}},
         "roofline": {"bound": "hbm", "achieved": head["GBps"], "peak": PEAK_HBM_GBPS,
                      "unit": "GB/s", "frac": head["GBps"] / PEAK_HBM_GBPS,
                      "traffic": PROFILE_TRAFFIC.get(HEADLINE),
-                     "traffic_source": PROFILE_SOURCE},
-        "cpu_baseline": cpu.get(HEADLINE),
+                     "traffic_source": PROFILE_SOURCE,
+                     "by_config": by_config},
+        "cpu_baseline": dict(cpu.get(HEADLINE) or {},
+                             by_config={n: round(c["value"], 2) for n, c in cpu.items()}) or None,
+        "rows_per_s": head["rows_per_s"],
         "launch_floor_us": launch_floor_us(),
-        "extras": ({"row_normalize": extra_row_normalize(), "meanvar": extra_meanvar(),
-                    "wide_columns": extra_wide_columns(), "dense_rows": extra_dense_rows()}
-                   if args.configs == "all" else {}),
-        "configs": results,
-        "cpu_baselines": cpu,
         "device": torch.cuda.get_device_name(0),
     }
+    details = {"configs": results, "extras": extras, "cpu_baselines": cpu}
+    for d in (ROOT / "gpurun_out", ROOT):
+        try:
+            if d.is_dir():
+                with open(d / "bench_details.json", "w") as f:
+                    json.dump(details, f, indent=1)
+                line["details_file"] = str((d / "bench_details.json").relative_to(ROOT))
+                break
+        except OSError:
+            continue
     print(json.dumps(line))
 
 
