@@ -159,7 +159,11 @@ typedef struct rmi_reduce_desc {
  * own), the last one to arrive folds the row's partials in index order (results stay
  * bitwise repeatable and equal to the two-launch plan's) and every counter wraps back to
  * zero, so the area is zero again when the call has run.  Without the flag the workspace
- * needs no initialisation and such rows take a second, folding launch. */
+ * needs no initialisation and such rows take a second, folding launch.
+ * The hand-off between the workgroups of that one launch is written for gfx942 / gfx950
+ * (write-through stores acknowledged by the memory side, device-scope atomics) and is
+ * outside the HIP memory model; the library refuses to build for other targets.  Ticket
+ * words are state: see rmi_workspace_reset for what leaves them non-zero and how to recover. */
 #define RMI_FLAG_WORKSPACE_ZEROED 1
 #define RMI_WORKSPACE_TICKET_BYTES 65536
 
@@ -252,6 +256,20 @@ RMI_API int rmi_reduce_noalloc(const rmi_reduce_desc* desc,
                                const void* in,
                                void* out,
                                void* stream);
+
+/* Zeroes the ticket words of a workspace (its first RMI_WORKSPACE_TICKET_BYTES bytes, or all
+ * of it when it is shorter) with a small kernel on `stream`: what a caller runs once on a
+ * fresh workspace before it passes RMI_FLAG_WORKSPACE_ZEROED, and again to recover one whose
+ * ticket words may have been left non-zero (a launch that was aborted or failed, calls that
+ * overlapped on two streams, a stray write).  Counters left non-zero are not detected: the
+ * rows they belong to are never folded and their outputs keep their old contents, on every
+ * later call, while the calls still return RMI_OK.  A kernel, not a memset, so the call may be
+ * recorded into a HIP graph.  No counterpart in the reference (its Thick plan takes a second
+ * launch, linalg/detail/coalesced_reduction-inl.cuh:595-625). */
+RMI_API int rmi_workspace_reset(void* workspace, size_t workspace_bytes, void* stream);
+
+/* The same for the static buffer of rmi_reduce_noalloc on the current device. */
+RMI_API int rmi_noalloc_reset(void* stream);
 
 /* Whole-array map + reduce to one scalar: replaces detail::mapThenReduceImpl
  * (linalg/detail/map_then_reduce.cuh:72-95) behind mapThenSumReduce /

@@ -80,6 +80,8 @@ SYMBOLS = {
     "rmi_reduce": (C.c_int, [C.POINTER(ReduceDesc), C.c_void_p, C.c_void_p, C.c_void_p,
                              C.c_size_t, C.c_void_p]),
     "rmi_reduce_noalloc": (C.c_int, [C.POINTER(ReduceDesc), C.c_void_p, C.c_void_p, C.c_void_p]),
+    "rmi_workspace_reset": (C.c_int, [C.c_void_p, C.c_size_t, C.c_void_p]),
+    "rmi_noalloc_reset": (C.c_int, [C.c_void_p]),
     "rmi_map_reduce_workspace_bytes": (C.c_size_t, [C.POINTER(ReduceDesc), C.c_int64]),
     "rmi_row_normalize": (C.c_int, [C.POINTER(ReduceDesc), C.c_void_p, C.c_void_p, C.c_double,
                                     C.c_void_p]),

@@ -13,6 +13,14 @@ static __device__ __align__(256) unsigned char scratch[RMI_NOALLOC_SCRATCH_BYTES
 
 namespace rmi {
 
+// Zero fill of a few KB on a stream: ticket words are cleared by a kernel so that the call
+// can be recorded into a HIP graph (memset nodes have replayed wrongly on this platform).
+__global__ __launch_bounds__(256) void zero_words_kernel(u32* p, size_t words)
+{
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < words; i += (size_t)gridDim.x * 256)
+    p[i] = 0;
+}
+
 // CU count of the current device, queried once per process.  Without a
 // visible device the MI355X figure is assumed so that planning works on a
 // build host.
@@ -335,6 +343,27 @@ int rmi_reduce_noalloc(const rmi_reduce_desc* desc, const void* in, void* out, v
   rc       = rmi::scratch_of_current_device(&ws);
   if (rc != RMI_OK) return rc;
   return rmi::reduce_planned(d, *p, in, out, ws, RMI_NOALLOC_SCRATCH_BYTES, stream);
+}
+
+int rmi_workspace_reset(void* workspace, size_t workspace_bytes, void* stream)
+{
+  if (workspace == nullptr) return workspace_bytes == 0 ? RMI_OK : RMI_ERR_NULL;
+  if (!rmi::aligned(workspace, 16)) return RMI_ERR_WORKSPACE;
+  const size_t bytes = workspace_bytes < RMI_WORKSPACE_TICKET_BYTES ? workspace_bytes
+                                                                    : (size_t)RMI_WORKSPACE_TICKET_BYTES;
+  const size_t words = bytes / 4;
+  if (words == 0) return RMI_OK;
+  hipLaunchKernelGGL(rmi::zero_words_kernel, dim3((unsigned)((words + 255) / 256)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), static_cast<rmi::u32*>(workspace), words);
+  return hipGetLastError() == hipSuccess ? RMI_OK : RMI_ERR_LAUNCH;
+}
+
+int rmi_noalloc_reset(void* stream)
+{
+  void* ws     = nullptr;
+  const int rc = rmi::scratch_of_current_device(&ws);
+  if (rc != RMI_OK) return rc;
+  return rmi_workspace_reset(ws, RMI_NOALLOC_SCRATCH_BYTES, stream);
 }
 
 size_t rmi_map_reduce_workspace_bytes(const rmi_reduce_desc* desc, int64_t len)

@@ -26,6 +26,7 @@
 #include <raft/util/cudart_utils.hpp>
 #include <raft/util/itertools.hpp>
 
+#include <chrono>
 #include <cstdint>
 #include <random>
 
@@ -826,6 +827,150 @@ void handle_copies_and_stream_changes()
   RAFT_HIP_TRY(hipStreamDestroy(s2));
 }
 
+// After a warm-up call a handle neither allocates nor makes the host wait: the column mean and
+// stddev (two-pass column plan), a split-row reduction (ticket counters in the handle's
+// workspace) and meanvar are recorded through one handle into a HIP graph; the graph is
+// replayed over new contents of the same buffers, with eager work in between, and every replay
+// is held to the host reference.
+void handle_calls_under_graph_capture()
+{
+  hipStream_t s;
+  RAFT_HIP_TRY(hipStreamCreate(&s));
+  {
+    raft::resources handle(s);
+    const int rows = 20000, cols = 64;        // column plans
+    const int lrows = 4, lcols = 1 << 20;      // rows split over several workgroups
+    auto data  = raft::make_device_matrix<float, int, raft::row_major>(handle, rows, cols);
+    auto mu    = raft::make_device_vector<float, int>(handle, cols);
+    auto sd    = raft::make_device_vector<float, int>(handle, cols);
+    auto mv_m  = raft::make_device_vector<float, int>(handle, cols);
+    auto mv_v  = raft::make_device_vector<float, int>(handle, cols);
+    auto ldata = raft::make_device_matrix<float, int, raft::row_major>(handle, lrows, lcols);
+    auto lout  = raft::make_device_vector<float, int>(handle, lrows);
+    auto run   = [&] {
+      auto dv = raft::make_const_mdspan(data.view());
+      raft::stats::mean(handle, dv, mu.view());
+      raft::stats::stddev(handle, dv, raft::make_const_mdspan(mu.view()), sd.view(), true);
+      raft::stats::meanvar(handle, dv, mv_m.view(), mv_v.view(), true);
+      raft::linalg::reduce<raft::Apply::ALONG_ROWS>(handle, raft::make_const_mdspan(ldata.view()),
+                                                    lout.view(), 0.0f);
+    };
+    auto fill = [&](unsigned long long seed, std::vector<float>& h, std::vector<float>& lh) {
+      h  = normal<float>((size_t)rows * cols, 3.0, 2.0, seed);
+      lh = uniform<float>((size_t)lrows * lcols, -1.0, 1.0, seed + 1);
+      raft::update_device(data.data_handle(), h.data(), h.size(), s);
+      raft::update_device(ldata.data_handle(), lh.data(), lh.size(), s);
+      RAFT_HIP_TRY(hipStreamSynchronize(s));
+    };
+    auto check = [&](const std::vector<float>& h, const std::vector<float>& lh) {
+      auto add = [](double a, double b) { return a + b; };
+      auto idm = [](double x, int) { return x; };
+      auto idf = [](double x) { return x; };
+      std::vector<double> wm(cols), ws(cols), wv(cols);
+      for (int j = 0; j < cols; ++j) {
+        double a = 0, q = 0;
+        for (int i = 0; i < rows; ++i)
+          a += h[(size_t)i * cols + j];
+        a /= rows;
+        for (int i = 0; i < rows; ++i) {
+          const double d = h[(size_t)i * cols + j] - a;
+          q += d * d;
+        }
+        wm[j] = a, wv[j] = q / (rows - 1), ws[j] = std::sqrt(wv[j]);
+      }
+      CHECK(all_close(to_host(mu.data_handle(), (size_t)cols, s), wm, 1e-5));
+      CHECK(all_close(to_host(sd.data_handle(), (size_t)cols, s), ws, 1e-4));
+      CHECK(all_close(to_host(mv_m.data_handle(), (size_t)cols, s), wm, 1e-5));
+      CHECK(all_close(to_host(mv_v.data_handle(), (size_t)cols, s), wv, 1e-5));
+      CHECK(all_close(to_host(lout.data_handle(), (size_t)lrows, s),
+                      host_reduce(lh, lrows, lcols, true, true, 0.0, nullptr, idm, add, idf), 1e-5));
+    };
+    std::vector<float> h, lh;
+    fill(1, h, lh);
+    run();  // warm-up: the workspace reaches its size, the ticket words are cleared
+    check(h, lh);
+
+    // the recorded calls must find the workspace as the warm-up left it: same buffer, no growth
+    void* const ws_before = handle.workspace(1);
+    size_t free_before = 0, free_after = 0, total = 0;
+    RAFT_HIP_TRY(hipMemGetInfo(&free_before, &total));
+    hipGraph_t graph;
+    hipGraphExec_t exec;
+    RAFT_HIP_TRY(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal));
+    run();
+    RAFT_HIP_TRY(hipStreamEndCapture(s, &graph));
+    RAFT_HIP_TRY(hipMemGetInfo(&free_after, &total));
+    CHECK(handle.workspace(1) == ws_before);
+    CHECK(free_after == free_before);  // nothing was allocated while recording
+    RAFT_HIP_TRY(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0));
+    for (unsigned long long rep = 0; rep < 3; ++rep) {
+      fill(100 + 7 * rep, h, lh);
+      RAFT_HIP_TRY(hipGraphLaunch(exec, s));
+      check(h, lh);
+      run();  // eager work between the replays, through the same workspace
+      check(h, lh);
+    }
+    RAFT_HIP_TRY(hipGraphExecDestroy(exec));
+    RAFT_HIP_TRY(hipGraphDestroy(graph));
+  }
+  RAFT_HIP_TRY(hipStreamDestroy(s));
+}
+
+// A change of the handle's stream costs no host wait: with several milliseconds of reductions
+// queued on the first stream, the first call on the second returns at once, and its
+// result is right although both calls share the workspace.
+void handle_stream_change_does_not_block()
+{
+  hipStream_t s1, s2;
+  RAFT_HIP_TRY(hipStreamCreate(&s1));
+  RAFT_HIP_TRY(hipStreamCreate(&s2));
+  {
+    raft::resources handle(s1);
+    const int rows = 4, cols = 16 << 20;  // 256 MB, rows split over workgroups
+    auto big  = raft::make_device_matrix<float, int, raft::row_major>(handle, rows, cols);
+    auto bout = raft::make_device_vector<float, int>(handle, rows);
+    auto h    = uniform<float>((size_t)rows * (1 << 20), -1.0, 1.0, 21);
+    auto small = raft::make_device_matrix<float, int, raft::row_major>(handle, rows, 1 << 20);
+    auto sout  = raft::make_device_vector<float, int>(handle, rows);
+    RAFT_HIP_TRY(hipMemsetAsync(big.data_handle(), 0, sizeof(float) * (size_t)rows * cols, s1));
+    raft::update_device(small.data_handle(), h.data(), h.size(), s1);
+    auto call_big = [&] {
+      raft::linalg::reduce<raft::Apply::ALONG_ROWS>(handle, raft::make_const_mdspan(big.view()),
+                                                    bout.view(), 0.0f);
+    };
+    call_big();  // warm-up
+    RAFT_HIP_TRY(hipDeviceSynchronize());
+    auto now = [] { return std::chrono::steady_clock::now(); };
+    const auto t0 = now();
+    for (int i = 0; i < 200; ++i)
+      call_big();  // 200 x 256 MB: about 8 ms of device work on s1
+    const auto t1 = now();
+    raft::resource::set_cuda_stream(handle, s2);
+    raft::linalg::reduce<raft::Apply::ALONG_ROWS>(handle, raft::make_const_mdspan(small.view()),
+                                                  sout.view(), 0.0f);
+    const auto t2 = now();
+    const bool s1_busy = hipStreamQuery(s1) == hipErrorNotReady;
+    RAFT_HIP_TRY(hipStreamSynchronize(s1));
+    const auto t3 = now();
+    const double enqueue_ms = std::chrono::duration<double, std::milli>(t1 - t0).count();
+    const double switch_ms  = std::chrono::duration<double, std::milli>(t2 - t1).count();
+    const double drain_ms   = std::chrono::duration<double, std::milli>(t3 - t2).count();
+    std::printf("  200 calls enqueued in %.2f ms, call after the stream change %.3f ms, "
+                "first stream drained %.2f ms later\n", enqueue_ms, switch_ms, drain_ms);
+    CHECK(s1_busy);            // the first stream still had work when the second call returned
+    CHECK(switch_ms < 1.0);    // ... so the call did not wait for it on the host
+    auto add = [](double a, double b) { return a + b; };
+    auto idm = [](double x, int) { return x; };
+    auto idf = [](double x) { return x; };
+    CHECK(all_close(to_host(sout.data_handle(), (size_t)rows, s2),
+                    host_reduce(h, rows, 1 << 20, true, true, 0.0, nullptr, idm, add, idf), 1e-5));
+    CHECK(all_close(to_host(bout.data_handle(), (size_t)rows, s1),
+                    std::vector<double>(rows, 0.0), 1e-6));
+  }
+  RAFT_HIP_TRY(hipStreamDestroy(s1));
+  RAFT_HIP_TRY(hipStreamDestroy(s2));
+}
+
 // cpp/tests/linalg/normalize.cu:40-135: row_normalize against rowNorm followed by a
 // per-row division, rows {11,101,12345} x cols {2,3,7,12,33,125,254} x {L1,L2,Linf}
 template <typename T, typename Idx>
@@ -897,6 +1042,8 @@ TEST_CASE(ArgFixturesD) { arg_fixtures<double>(); }
 TEST_CASE(MapReduce) { map_reduce_cases(); }
 TEST_CASE(HandleWorkspaceReuse) { handle_workspace_reuse(); }
 TEST_CASE(HandleCopiesAndStreamChanges) { handle_copies_and_stream_changes(); }
+TEST_CASE(HandleCallsUnderGraphCapture) { handle_calls_under_graph_capture(); }
+TEST_CASE(HandleStreamChangeDoesNotBlock) { handle_stream_change_does_not_block(); }
 
 int main()
 {
