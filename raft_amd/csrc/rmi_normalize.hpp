@@ -104,22 +104,24 @@ __device__ __forceinline__ void store16(void* p, const u32x4& v)
 // x / d for many x and one d, as the reference's element-wise division computes it, at three
 // instructions per element instead of the ten or more of a division: with r = RN(1 / d), the
 // quotient estimate q = RN(x * r) is corrected once with the exact residual, q' = RN(q + RN(x -
-// q * d) * r), which is the correctly rounded x / d (Markstein) as long as r and the residual
-// stay in the normal range.  A divisor outside [2^-100, 2^100] (fp32; 2^-900, 2^900 fp64), an
-// infinite or a NaN one takes the division itself.
+// q * d) * r), which is the correctly rounded x / d (Markstein) as long as r is normal and the
+// residual x - q * d, some 2^-24 (2^-53) of x, is exactly representable.  A divisor outside
+// [2^-100, 2^100] (fp32; 2^-900, 2^900 fp64), an infinite or a NaN one, and every element
+// smaller than 2^-100 (2^-900) in magnitude, whose residual would fall below the subnormal
+// spacing, take the division itself.
 template <class T>
 struct Quot {
   T d, r;
   bool fast;
+  static constexpr T lo = sizeof(T) == 4 ? (T)7.888609052210118e-31 : (T)1.183e-271;   // 2^-100, ~2^-900
+  static constexpr T hi = sizeof(T) == 4 ? (T)1.2676506002282294e30 : (T)8.452e270;    // 2^100, ~2^900
   __device__ __forceinline__ explicit Quot(T divisor) : d(divisor), r((T)1 / divisor)
   {
-    constexpr T lo = sizeof(T) == 4 ? (T)7.888609052210118e-31 : (T)1.183e-271;   // 2^-100, ~2^-900
-    constexpr T hi = sizeof(T) == 4 ? (T)1.2676506002282294e30 : (T)8.452e270;    // 2^100, ~2^900
     fast = fabs(divisor) >= lo && fabs(divisor) <= hi;
   }
   __device__ __forceinline__ T operator()(T x) const
   {
-    if (!fast) return x / d;
+    if (!fast || fabs(x) < lo) return x / d;
     const T q  = x * r;
     const T q2 = fma(fma(-q, d, x), r, q);
     // an infinite x has no residual (inf - inf): its product with r already is the quotient

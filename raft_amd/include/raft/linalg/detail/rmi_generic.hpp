@@ -30,6 +30,9 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
+#include <map>
+#include <mutex>
+#include <string>
 #include <type_traits>
 
 #include <raft/core/error.hpp>
@@ -469,6 +472,29 @@ inline int ilog2(int x)
   return l;
 }
 
+// CUs of the current device, asked once per device (the library's planner does the same);
+// grids that aim at "k workgroups per CU" are sized from it.
+inline int cu_count()
+{
+  static std::mutex guard;
+  static std::map<int, int> by_device;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) {
+    (void)hipGetLastError();
+    return 256;
+  }
+  std::lock_guard<std::mutex> lock(guard);
+  auto it = by_device.find(dev);
+  if (it != by_device.end()) return it->second;
+  int n = 0;
+  if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
+    (void)hipGetLastError();
+    n = 256;
+  }
+  by_device.emplace(dev, n);
+  return n;
+}
+
 inline void check_launch(const char* what)
 {
   const hipError_t e = hipGetLastError();
@@ -530,7 +556,7 @@ void coalesced(Dst* dots, const In* data, Idx D, Idx N, Out init, hipStream_t st
   // chunks are whole multiples of one block sweep (256 lanes x 4 loads x V elements), so
   // every chunk starts on a vector boundary of its row
   constexpr std::int64_t quantum = (std::int64_t)kBlock * 4 * V;
-  std::int64_t B = (1024 + (std::int64_t)N - 1) / (std::int64_t)N;
+  std::int64_t B = ((std::int64_t)4 * cu_count() + (std::int64_t)N - 1) / (std::int64_t)N;
   const std::int64_t max_b = ((std::int64_t)D + quantum - 1) / quantum;
   if (B > max_b) B = max_b;
   if (B < 1) B = 1;
@@ -560,11 +586,11 @@ void launch_cols(Dst* dots, const In* data, Idx D, Idx N, Out init, hipStream_t 
   const int TX             = (int)((lanes + cuts - 1) / cuts);
   const int TY             = kBlock / TX;
   const std::int64_t gridx = (lanes + TX - 1) / TX;
-  // 16-byte lane loads: two workgroups per CU of a 256-CU device read one compact, advancing
-  // window of the matrix (measured 74 % of 8 TB/s on 10M x 64 floats where 1024 workgroups
-  // give 63 %); element loads want eight times as many in flight.  At least four steps each.
-  // (rounded down: a 513th workgroup lands on a CU that then finishes last)
-  std::int64_t B           = (V > 1 ? 512 : 4096) / gridx;
+  // 16-byte lane loads: two workgroups per CU read one compact, advancing window of the
+  // matrix (measured 74 % of 8 TB/s on 10M x 64 floats where 1024 workgroups give 63 %);
+  // element loads want eight times as many in flight.  At least four steps each.
+  // (rounded down: one workgroup more lands on a CU that then finishes last)
+  std::int64_t B           = ((std::int64_t)cu_count() * (V > 1 ? 2 : 16)) / gridx;
   const std::int64_t max_b = ((std::int64_t)N + 4 * TY - 1) / (4 * TY);
   if (B > max_b) B = max_b;
   if (B < 1) B = 1;
@@ -590,7 +616,9 @@ void launch_cols(Dst* dots, const In* data, Idx D, Idx N, Out init, hipStream_t 
 // slots are dealt densely over the lane-loads of `rb` adjacent rows (a bundle): slot k of
 // thread t is lane-load (256 k + t) % piece of row (256 k + t) / piece, so a slot always meets
 // the same columns.  R bundles are in flight, every load issued before the first use and none
-// under a condition (idle slots load the piece's first vector and are dropped).  At the end the
+// under a condition (idle slots load the piece's first vector, run the caller's main_op and
+// reduce_op on it like every other slot, and are dropped: functors must be free of side
+// effects, as the reference's are).  At the end the
 // rows of a bundle are combined through LDS in row order and the partials are stored
 // [workgroup][column], whole lines at a time; fold_rows_kernel is the second pass.
 template <typename Out, int V>
@@ -742,7 +770,7 @@ bool launch_cols_wide(Dst* dots, const In* data, Idx D, Idx N, Out init, hipStre
                       bool inplace, Main main_op, Red red, Fin fin)
 {
   constexpr int K          = cols_wide_slots<Out, V>();
-  constexpr int kCus       = 256;  // one workgroup per CU of the device this is tuned for
+  const int kCus           = cu_count();  // one workgroup per CU
   const std::int64_t lanes = ((std::int64_t)D + V - 1) / V;
   const std::int64_t slots = (std::int64_t)kBlock * K;
   const std::int64_t cuts  = (lanes + slots - 1) / slots;

@@ -231,11 +231,13 @@ def encode_out(out_dtype, values):
 
 
 def gpu_reduce(desc: api.ReduceDesc, data: np.ndarray, *, old_raw=None, aux_raw=None,
-               misalign_elems: int = 0):
+               misalign_elems: int = 0, workspace=None):
     """Upload `data`, run rmi_reduce through the C ABI on cuda:0, return the raw output
     array (numpy, output dtype).  `old_raw` seeds the output buffer (inplace);
     `aux_raw` is uploaded and passed as final_aux; `misalign_elems` shifts the input's
-    device address by that many elements to exercise the element-wise load path."""
+    device address by that many elements to exercise the element-wise load path;
+    `workspace` is a device tensor to use instead of a fresh one (a shared, zeroed
+    workspace for descriptors that carry RMI_FLAG_WORKSPACE_ZEROED)."""
     import torch
     from raft_amd import device as dev
 
@@ -256,7 +258,7 @@ def gpu_reduce(desc: api.ReduceDesc, data: np.ndarray, *, old_raw=None, aux_raw=
     if aux_raw is not None:
         aux_t = torch.from_numpy(np.ascontiguousarray(aux_raw).view(np.uint8).reshape(-1)).cuda()
         d.final_aux = aux_t.data_ptr()
-    dev.reduce(d, buf, out, in_ptr=buf.data_ptr() + pad)
+    dev.reduce(d, buf, out, workspace, in_ptr=buf.data_ptr() + pad)
     torch.cuda.synchronize()
     raw = out.cpu().numpy()[: n * odt.itemsize].view(odt).copy()
     return raw

@@ -204,6 +204,29 @@ def test_quotients_are_correctly_rounded(gpu, dt, npdt, cols):
     assert np.array_equal(got, want), np.argwhere(got != want)[:5]
 
 
+# Elements far below their row's norm: the residual of the reciprocal-and-correct quotient is
+# not representable there (it falls below the subnormal spacing), so such elements must take
+# the division itself.  Norm near 1, elements from 1e-30 down into the subnormals (fp32) and
+# from 1e-290 down (fp64), held to numpy's division bit for bit.
+@pytest.mark.parametrize("dt,npdt,lo_exp,hi_exp", [(api.F32, np.float32, -44.0, -30.0),
+                                                    (api.F64, np.float64, -322.0, -290.0)])
+def test_quotients_of_tiny_elements(gpu, dt, npdt, lo_exp, hi_exp):
+    rows, cols = 64, 257
+    rng = np.random.default_rng(5)
+    m = (10.0 ** rng.uniform(lo_exp, hi_exp, (rows, cols)) * rng.choice([-1.0, 1.0], (rows, cols)))
+    m[:, 0] = rng.uniform(0.05, 3000.0, rows)      # the row's L-inf norm
+    m[:, 1] = rng.uniform(0.01, 0.04, rows) * m[:, 0]
+    m = m.astype(npdt)
+    main, red, fin = NORMS["linf"]
+    d = api.make_desc(dt, dt, rows, cols, main_op=main, reduce_op=red, final_op=fin)
+    got = _gpu(d, m.reshape(-1), np.zeros(rows * cols, dtype=npdt), 0.0).reshape(rows, cols)
+    with np.errstate(under="ignore"):
+        want = m / np.abs(m).max(axis=1, keepdims=True)
+    assert want.dtype == npdt
+    assert np.array_equal(got, want), (np.argwhere(got != want)[:5], got[got != want][:5],
+                                       want[got != want][:5])
+
+
 def test_full_size_embedding_shape(gpu):
     """1,000,000 x 128 fp32 (the shape of benchmark config 2): unit L2 rows, and the
     oracle on a slice."""

@@ -514,13 +514,16 @@ def test_split_rows_single_launch(gpu, in_dt, out_dt, kw):
     import torch
     lib = api.load()
     sptr = torch.cuda.current_stream().cuda_stream
-    ws = torch.zeros(1 << 20, dtype=torch.uint8, device="cuda")   # zeroed once, then only reused
-    scratch = torch.empty(1 << 20, dtype=torch.uint8, device="cuda")
+    ws = torch.zeros(4 << 20, dtype=torch.uint8, device="cuda")   # zeroed once, then only reused
+    scratch = torch.empty(4 << 20, dtype=torch.uint8, device="cuda")
     rng = np.random.default_rng(in_dt * 7 + out_dt)
     odt = u.out_numpy_dtype(out_dt)
+    # (the last three: two levels of counters with about a hundred rows, and more than sixteen
+    # groups of sixteen chunks per row)
     shapes = [(8, 300_001, api.PLAN_AUTO), (1, 2_000_000, api.PLAN_AUTO), (3, 70_001, api.PLAN_ROW_SPLIT),
               (40, 80_000, api.PLAN_ROW_SPLIT), (2, 1_000_003, api.PLAN_AUTO), (512, 70_000, api.PLAN_ROW_SPLIT),
-              (5, 100_003, api.PLAN_ROW_SPLIT)]
+              (5, 100_003, api.PLAN_ROW_SPLIT), (100, 200_003, api.PLAN_ROW_SPLIT),
+              (96, 150_000, api.PLAN_AUTO), (1, 6_000_001, api.PLAN_AUTO)]
     for rows, cols, hint in shapes:
         data = _rand(rng, in_dt, rows * cols)
         x = torch.from_numpy(data.view(np.uint8).reshape(-1)).cuda()
@@ -563,6 +566,46 @@ def test_split_rows_single_launch(gpu, in_dt, out_dt, kw):
         assert lib.rmi_reduce(C.byref(dc), xc.data_ptr(), oc.data_ptr(), ws.data_ptr(), ws.numel(), sptr) == api.OK
         torch.cuda.synchronize()
         assert bool((oc == 5000).all()) and int(ws[: api.WORKSPACE_TICKET_BYTES].max().item()) == 0
+
+
+# Ticket words that were left non-zero (here: random bytes) are recovered by rmi_workspace_reset,
+# a kernel on the caller's stream; rmi_noalloc_reset does the same for the static buffer.
+def test_workspace_reset_recovers_ticket_words(gpu):
+    import ctypes as C
+    import torch
+    lib = api.load()
+    sptr = torch.cuda.current_stream().cuda_stream
+    rng = np.random.default_rng(77)
+    rows, cols = 6, 400_003
+    data = rng.uniform(-1, 1, rows * cols).astype(np.float32)
+    x = torch.from_numpy(data).cuda()
+    d0 = api.make_desc(api.F32, api.F32, rows, cols)
+    want = u.gpu_reduce(d0, data)
+    df = api.make_desc(api.F32, api.F32, rows, cols, flags=api.FLAG_WORKSPACE_ZEROED)
+    assert api.plan_query(df).passes == 1
+    ws = torch.empty(1 << 20, dtype=torch.uint8, device="cuda").random_(1, 255)
+    assert lib.rmi_workspace_reset(ws.data_ptr(), ws.numel(), sptr) == api.OK
+    assert int(ws[: api.WORKSPACE_TICKET_BYTES].max().item()) == 0
+    assert int(ws[api.WORKSPACE_TICKET_BYTES:].min().item()) >= 1   # nothing past the ticket words
+    for _ in range(2):
+        out = torch.zeros(rows, device="cuda")
+        assert lib.rmi_reduce(C.byref(df), x.data_ptr(), out.data_ptr(), ws.data_ptr(), ws.numel(), sptr) == api.OK
+        torch.cuda.synchronize()
+        assert np.array_equal(out.cpu().numpy(), want)
+    # a short workspace is cleared whole, nothing beyond it
+    small = torch.empty(4096, dtype=torch.uint8, device="cuda").random_(1, 255)
+    assert lib.rmi_workspace_reset(small.data_ptr(), 1024, sptr) == api.OK
+    torch.cuda.synchronize()
+    assert int(small[:1024].max().item()) == 0 and int(small[1024:].min().item()) >= 1
+    assert lib.rmi_workspace_reset(None, 0, sptr) == api.OK
+    assert lib.rmi_workspace_reset(None, 16, sptr) == api.ERR_NULL
+    assert lib.rmi_workspace_reset(small.data_ptr() + 4, 16, sptr) == api.ERR_WORKSPACE
+    # the static buffer of rmi_reduce_noalloc
+    assert lib.rmi_noalloc_reset(sptr) == api.OK
+    out = torch.zeros(rows, device="cuda")
+    assert lib.rmi_reduce_noalloc(C.byref(d0), x.data_ptr(), out.data_ptr(), sptr) == api.OK
+    torch.cuda.synchronize()
+    assert np.array_equal(out.cpu().numpy(), want)
 
 
 # More rows than ticket words: the plan falls back to the folding launch.

@@ -84,7 +84,72 @@ def test_random_case(gpu, seed):
         old = u.encode_out(out_dt, rng.integers(-3, 4, n).astype(np.float64))
     label = (f"seed {seed}: {kind} {api.DTYPE_NAME[in_dt]}->{api.DTYPE_NAME[out_dt]} {rows}x{cols} "
              f"layout {kw['layout']} apply {kw['apply']} +{shift} {kw}")
-    u.check_against_oracle(d, data, old_raw=old, misalign_elems=shift, label=label)
+    raw = u.check_against_oracle(d, data, old_raw=old, misalign_elems=shift, label=label)
+    if seed % 2 == 0:
+        # every other case once more with RMI_FLAG_WORKSPACE_ZEROED through ONE workspace that
+        # all such cases share (zeroed once, then only used by the library): the same bits
+        _same_bits_with_shared_workspace(in_dt, out_dt, rows, cols, kw, data, old, shift, raw, label)
+
+
+_shared = {}
+
+
+def _shared_workspace():
+    import torch
+    if "ws" not in _shared:
+        _shared["ws"] = torch.zeros(64 << 20, dtype=torch.uint8, device="cuda")
+    return _shared["ws"]
+
+
+def _same_bits_with_shared_workspace(in_dt, out_dt, rows, cols, kw, data, old, shift, raw, label):
+    ws = _shared_workspace()
+    df = api.make_desc(in_dt, out_dt, rows, cols, flags=api.FLAG_WORKSPACE_ZEROED, **kw)
+    assert api.plan_query(df).workspace_bytes <= ws.numel(), label
+    got = u.gpu_reduce(df, data, old_raw=old, misalign_elems=shift, workspace=ws)
+    if got.dtype.names:   # key-value records: field by field (a record may hold padding bytes)
+        same = all(np.array_equal(np.ascontiguousarray(got[f]).view(np.uint8),
+                                  np.ascontiguousarray(raw[f]).view(np.uint8)) for f in got.dtype.names)
+    else:
+        same = np.array_equal(got.view(np.uint8), raw.view(np.uint8))
+    assert same, f"{label}: the flagged plan differs from the plain one"
+    assert int(ws[: api.WORKSPACE_TICKET_BYTES].max().item()) == 0, f"{label}: ticket words left non-zero"
+
+
+# Rows long enough to be split over several workgroups are rare in the draw above: few rows of
+# 70 thousand to 3 million elements, every accumulator family, counters in one level (up to
+# 16 chunks per row) and in two, through the shared workspace with the flag and through a
+# scratch one without it: the same bits, and the oracle's values.
+@pytest.mark.parametrize("seed", range(int(os.environ.get("RMI_RANDOM_CASES", "400")) // 8))
+def test_random_split_rows(gpu, seed):
+    rng = np.random.default_rng(40_000 + seed)
+    kind = rng.choice(["sum", "sum", "minmax", "arg"])
+    rows = int(rng.choice([1, 1, 2, 3, 5, 8, 17, 40, 100]))
+    cols = int(np.exp(rng.uniform(np.log(70_000), np.log(max(80_000, 4_000_000 // rows)))))
+    cols += int(rng.integers(0, 9))
+    kw = {}
+    if kind == "sum":
+        in_dt, out_dt = SUM_TYPES[rng.integers(len(SUM_TYPES))]
+        kw["main_op"] = int(rng.choice([api.MAIN_IDENTITY, api.MAIN_SQ, api.MAIN_ABS]))
+        kw["inplace"] = bool(rng.random() < 0.25)
+    elif kind == "minmax":
+        in_dt, out_dt = MINMAX_TYPES[rng.integers(len(MINMAX_TYPES))]
+        mx = rng.random() < 0.5
+        kw.update(reduce_op=api.RED_MAX if mx else api.RED_MIN,
+                  init_f=-np.inf if mx else np.inf, init_i=-2**62 if mx else 2**62)
+    else:
+        in_dt, out_dt = ARG_TYPES[rng.integers(len(ARG_TYPES))]
+        mx = rng.random() < 0.5
+        kw.update(main_op=api.MAIN_KVP, reduce_op=api.RED_ARGMAX if mx else api.RED_ARGMIN,
+                  init_f=-np.inf if mx else np.inf)
+    hint = api.PLAN_ROW_SPLIT if rng.random() < 0.5 else api.PLAN_AUTO
+    data = _rand(rng, in_dt, rows * cols)
+    d = api.make_desc(in_dt, out_dt, rows, cols, plan_hint=hint, **kw)
+    old = u.encode_out(out_dt, rng.integers(-3, 4, rows).astype(np.float64)) if kw.get("inplace") else None
+    shift = int(rng.choice([0, 0, 1, 3]))
+    label = f"seed {seed}: split rows {kind} {api.DTYPE_NAME[in_dt]}->{api.DTYPE_NAME[out_dt]} {rows}x{cols} +{shift} {kw}"
+    raw = u.check_against_oracle(d, data, old_raw=old, misalign_elems=shift, label=label)
+    _same_bits_with_shared_workspace(in_dt, out_dt, rows, cols, dict(kw, plan_hint=hint), data, old,
+                                     shift, raw, label)
 
 
 # The same for row normalisation and the one-pass mean / variance.

@@ -23,11 +23,21 @@ def _both(desc, x, out_dtype_bytes, n_out):
     b = torch.full((n_out * out_dtype_bytes,), 0xA5, dtype=torch.uint8, device="cuda")
     rc = lib.rmi_reduce(C.byref(desc), x.data_ptr(), a.data_ptr(), ws.data_ptr(), nws, sptr)
     assert rc == api.OK, api.status_string(rc)
-    before = torch.cuda.memory_allocated()
+    # "allocates nothing" is held to the device's own count of free memory, which sees any
+    # allocation of any library (torch's allocator counter would only see torch's): the first
+    # call on this device looked the buffer's address up, so from here on nothing may move
     rc = lib.rmi_reduce_noalloc(C.byref(desc), x.data_ptr(), b.data_ptr(), sptr)
     assert rc == api.OK, api.status_string(rc)
-    assert torch.cuda.memory_allocated() == before
     torch.cuda.synchronize()
+    free_before, _ = torch.cuda.mem_get_info()
+    before = torch.cuda.memory_allocated()
+    for _ in range(3):
+        rc = lib.rmi_reduce_noalloc(C.byref(desc), x.data_ptr(), b.data_ptr(), sptr)
+        assert rc == api.OK, api.status_string(rc)
+    torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info()
+    assert free_after == free_before, (free_before, free_after)
+    assert torch.cuda.memory_allocated() == before
     return a.cpu().numpy(), b.cpu().numpy(), nws
 
 
