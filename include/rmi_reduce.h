@@ -331,8 +331,12 @@ RMI_API int rmi_meanvar(int dtype,
  * cuBLAS GEMM X^T X scaled by alpha) behind raft::stats::cov (stats/cov.cuh:38-50 pointer
  * form, :77-106 mdspan form).  `dtype` is F32 or F64 (data, mu and covar share it), `layout`
  * the rmi_layout of `data`; `covar` is [n_cols][n_cols] and symmetric, so its layout does not
- * matter.  The contraction runs on the matrix cores in `dtype` (fp32 or fp64 products and
- * sums), partial sums of row slabs are added in f64.  `mu` may be NULL: the data is taken
+ * matter.  The contraction runs on the matrix cores: F64 data with fp64 products and sums;
+ * F32 data split exactly into three bf16 terms per value, six of the nine cross terms
+ * multiplied (the three left out are below 2^-23 of the product, one fp32 rounding) and
+ * summed in fp32.  Partial sums of row slabs are added in f64.  (An infinite F32 input gives
+ * NaN where an fp32 product would give an infinity; subnormal terms of the split may be
+ * flushed.)  `mu` may be NULL: the data is taken
  * as centred already.  With RMI_COV_CENTER_DATA in `flags` the call leaves x - mu in `data`,
  * which is what the reference documents ("this will get mean-centered at the end!") and its
  * callers rely on; without it `data` is only read and the matrix is moved once instead of

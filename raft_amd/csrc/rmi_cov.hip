@@ -39,7 +39,8 @@ int make_cov_plan(int dtype, int layout, int64_t N, int64_t D, CovPlan& p)
   p.npairs = (int)(nb * (nb + 1) / 2);
   p.vec    = D % 4 == 0;
   const int es          = dtype == RMI_F32 ? 4 : 8;
-  const int step_rows   = layout == RMI_ROW_MAJOR ? cov::kRowUnitRows : cov::kColUnitRows;
+  const int step_rows   = dtype == RMI_F32 ? cov::kBf16UnitRows
+                                           : (layout == RMI_ROW_MAJOR ? cov::kRowUnitRows : cov::kColUnitRows);
   const int64_t steps   = N / step_rows > 0 ? N / step_rows : 1;
   const int n_cu        = cu_count();
   int64_t S             = p.npairs <= 1 ? (int64_t)kWgPerCuOnePair * n_cu
@@ -118,8 +119,9 @@ int launch(const CovPlan& pl, int layout, int64_t N, int64_t D, int sample, bool
   f.permuted = layout == RMI_ROW_MAJOR ? 1 : 0;
   // the reference's scalar: Type(1) / Type(N - 1 | N), handed to the GEMM in Type
   f.alpha = N == 0 ? 0.0 : (double)(T(1) / (sample ? T(N - 1) : T(N)));  // no rows: zeros, as a GEMM with k = 0
-  hipLaunchKernelGGL((cov::cov_fold_kernel<T>), dim3((unsigned)(pl.npairs * cov::kTilesPerPair)),
-                     dim3(cov::kTile * cov::kFoldSplit), 0, st, f);
+  hipLaunchKernelGGL((cov::cov_fold_kernel<T>),
+                     dim3((unsigned)(pl.npairs * cov::kTilesPerPair * (cov::kTile / cov::kFoldElems))),
+                     dim3(cov::kFoldElems * cov::kFoldSplit), 0, st, f);
   return hipGetLastError() == hipSuccess ? RMI_OK : RMI_ERR_LAUNCH;
 }
 

@@ -5,15 +5,17 @@
 // The columns are cut into blocks of 64; a workgroup owns one pair of blocks (bi <= bj: the
 // upper triangle, the fold mirrors it) and one of S interleaved sets of rows (a slab), and
 // accumulates that pair's 64 x 64 piece of X^T X as sixteen 16 x 16 tiles (ten on the
-// diagonal) with v_mfma_f32_16x16x4_f32 / v_mfma_f64_16x16x4_f64.  The operands go from
-// global memory straight into the registers the instruction reads them from:
+// diagonal): fp64 data with v_mfma_f64_16x16x4_f64, fp32 data, split into three bf16 terms
+// per value, with v_mfma_f32_16x16x32_bf16 (see gram_rows_body_bf16).  The operands go from
+// global memory straight into the registers the instruction reads them from; for the
+// 16 x 16 x 4 instruction:
 //
 //   row-major X   lane l loads four consecutive columns 4 * (l % 16) .. + 3 of row l / 16 of
 //                 a wave-load of four rows; register j then holds, for the lanes 16 k .. 16 k
 //                 + 15, the columns {4 m + j} of row k, which is the A (and B) operand of a
 //                 16 x 16 x 4 step.  The result tile (ja, jb) is therefore the columns
 //                 {4 m + ja} x {4 n + jb}: a permutation the fold undoes.
-//   col-major X   lane l loads R consecutive rows of column 16 a + l % 16, the four lane
+//   col-major X   lane l loads four consecutive rows of column 16 a + l % 16, the four lane
 //                 quarters reading four consecutive runs of rows; register j of column group
 //                 a and register j of group b are one 16 x 16 x 4 step of tile (a, b).
 //
@@ -28,6 +30,8 @@
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+
+#include <type_traits>
 
 #include "rmi_reduce.h"
 
@@ -49,7 +53,7 @@ constexpr int kRowUnitLoads = RMI_COV_ROW_UNIT_LOADS;  // row-major: wave-loads 
 constexpr int kRowRing      = RMI_COV_ROW_RING;        // ... and units in the ring
 constexpr int kRowUnitRows  = 4 * kRowUnitLoads;      // rows of a unit
 constexpr int kColUnitRows  = 16;   // col-major: rows of a unit (four per lane quarter)
-constexpr int kFoldSplit    = 4;    // fold: threads that share the slabs of one element
+constexpr int kFoldSplit    = 16;   // fold: threads that share the slabs of one element
 
 // units a wave keeps in flight, given the 32-bit registers one unit takes: about 64
 // registers' worth, at least two and at most eight
@@ -354,6 +358,376 @@ __device__ __forceinline__ void gram_rows_body(const GramArgs& a, int unit, int 
   }
 }
 
+
+// ---------------------------------------------------------------------------
+// fp32 data on the bf16 matrix cores.  v_mfma_f32_16x16x4_f32 runs at 1/16 of the bf16
+// rate (and, fed random data, at a clock that the power limit pulls down to 1.7-1.9 GHz), so
+// fp32 Gram matrices are bound by it from 64 columns on.  Instead every centred value is
+// split exactly into three bf16 terms, x = h + m + l with eight significant bits each (two
+// truncations and two exact subtractions), and the product x * y is taken as
+//   h h' + h m' + m h' + m m' + h l' + l h'
+// with v_mfma_f32_16x16x32_bf16: products of bf16 values are exact in the fp32 accumulator,
+// and the three terms left out (m l', l m', l l') are below 2^-23 |x y|, the size of one
+// fp32 rounding of the product.  Six bf16 instructions of 32 rows take 96 cycles where eight
+// fp32 ones take 256; the splitting is 5.5 vector instructions per value.
+//
+// Operand layout of the 16 x 16 x 32 instruction: lane l supplies, for row (A) or column (B)
+// l % 16 of the tile, the eight k values 8 * (l / 16) .. + 7.  A unit is therefore 32 rows and
+// a lane holds eight of them: rows 8 * (l / 16) + r of its four columns (row-major, load r)
+// or eight consecutive rows of its column in each of the four groups (col-major).
+// ---------------------------------------------------------------------------
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+constexpr int kBf16UnitRows = 32;
+
+struct Split3 {
+  u32x4 h, m, l;  // eight bf16 each, value 2 w in the low half of word w
+};
+
+__device__ __forceinline__ Split3 split_bf16x3(const float (&x)[8])
+{
+  Split3 s;
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    const float a = x[2 * w], b = x[2 * w + 1];
+    const float ah = __uint_as_float(__float_as_uint(a) & 0xFFFF0000u);
+    const float bh = __uint_as_float(__float_as_uint(b) & 0xFFFF0000u);
+    const float ar = a - ah, br = b - bh;  // exact: the low 16 bits of the significand
+    const float am = __uint_as_float(__float_as_uint(ar) & 0xFFFF0000u);
+    const float bm = __uint_as_float(__float_as_uint(br) & 0xFFFF0000u);
+    const float al = ar - am, bl = br - bm;  // exact, eight significant bits or fewer
+    // the upper halves of two words side by side (v_perm_b32)
+    s.h[w] = __builtin_amdgcn_perm(__float_as_uint(b), __float_as_uint(a), 0x07060302u);
+    s.m[w] = __builtin_amdgcn_perm(__float_as_uint(br), __float_as_uint(ar), 0x07060302u);
+    s.l[w] = __builtin_amdgcn_perm(__float_as_uint(bl), __float_as_uint(al), 0x07060302u);
+  }
+  return s;
+}
+
+using f32x4 = float __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ f32x4 mma_bf16(const u32x4& a, const u32x4& b, f32x4 c)
+{
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a),
+                                                 __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+
+// acc[ca * 4 + cb] += A-class ca x B-class cb over the unit's 32 rows, term by term so that
+// consecutive instructions never wait for each other's accumulator
+template <bool DIAG>
+__device__ __forceinline__ void mma_unit_bf16(f32x4 (&acc)[kTilesPerPair], const Split3 (&A)[4],
+                                              const Split3 (&B)[4])
+{
+#define RMI_COV_TERM(TA, TB)                                                      \
+  _Pragma("unroll") for (int ca = 0; ca < 4; ++ca)                                \
+    _Pragma("unroll") for (int cb = DIAG ? ca : 0; cb < 4; ++cb)                  \
+      acc[ca * 4 + cb] = mma_bf16(A[ca].TA, B[cb].TB, acc[ca * 4 + cb]);
+  RMI_COV_TERM(l, h)
+  RMI_COV_TERM(h, l)
+  RMI_COV_TERM(m, m)
+  RMI_COV_TERM(m, h)
+  RMI_COV_TERM(h, m)
+  RMI_COV_TERM(h, h)
+#undef RMI_COV_TERM
+}
+
+// The matrix instruction adds into its accumulator with truncation: over the hundreds of
+// instructions of a wave's share of the rows a sum of squares came out 1e-5 too small.  So
+// the instruction's accumulator is kept short-lived: every kBf16FlushTrips trips of the ring
+// (a handful of units) it is added (an ordinary, correctly rounded fp32 addition) to a second
+// set of totals and cleared, which leaves a bias of about 3 * units * 2^-25.
+#ifndef RMI_COV_BF16_RING
+#define RMI_COV_BF16_RING 3
+#endif
+constexpr int kBf16Ring       = RMI_COV_BF16_RING;  // units of 32 rows a wave keeps loaded or in flight
+constexpr int kBf16FlushTrips = 2;
+__device__ __forceinline__ void flush_tiles(f32x4 (&total)[kTilesPerPair], f32x4 (&acc)[kTilesPerPair])
+{
+#pragma unroll
+  for (int t = 0; t < kTilesPerPair; ++t) {
+    total[t] += acc[t];
+    acc[t] = f32x4{0, 0, 0, 0};
+  }
+}
+
+template <bool VEC, bool DIAG, bool CENTER, bool STREAM>
+__device__ __forceinline__ void gram_rows_body_bf16(const GramArgs& a, int unit, int slab, int bi,
+                                                    int bj, float* sm)
+{
+  using T          = float;
+  constexpr int NS = DIAG ? 1 : 2;
+  constexpr int UR = kBf16UnitRows;
+  constexpr int P  = kBf16Ring;
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform, see above
+  const int g    = lane >> 4;  // the lane holds rows 8 g .. 8 g + 7 of a unit
+  const int cg   = lane & 15;  // quad of columns within the block
+  T* const data  = static_cast<T*>(a.data);
+  const T* mu    = static_cast<const T*>(a.mu);
+  const int64_t D = a.D;
+
+  int64_t col[NS][4];
+  bool ok[NS][4];
+  T mean[NS][4];
+#pragma unroll
+  for (int s = 0; s < NS; ++s) {
+    const int64_t c0 = (int64_t)(s == 0 ? bi : bj) * kBlockCols + 4 * cg;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      ok[s][j]   = c0 + j < D;
+      col[s][j]  = ok[s][j] ? c0 + j : 0;
+      mean[s][j] = (mu != nullptr && ok[s][j]) ? mu[col[s][j]] : T(0);
+    }
+  }
+
+  f32x4 acc[kTilesPerPair], total[kTilesPerPair];
+#pragma unroll
+  for (int t = 0; t < kTilesPerPair; ++t)
+    acc[t] = total[t] = f32x4{0, 0, 0, 0};
+
+  const int64_t G     = (int64_t)a.S * kWaves;
+  const int64_t gw    = (int64_t)slab * kWaves + wave;
+  const int64_t nfull = a.N / UR;
+  const int64_t K     = gw < nfull ? (nfull - gw + G - 1) / G : 0;
+
+  auto load_unit = [&](Quad<T> (&x)[NS][8], int64_t q, bool guard) {
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+      const int64_t r0 = q * UR + r;   // uniform part of the row; the lane adds 8 g
+      const int64_t dr = (guard && r0 + 8 * g >= a.N) ? a.N - 1 - r0 : 8 * g;
+      const T* rp      = data + r0 * D + dr * D;
+#pragma unroll
+      for (int s = 0; s < NS; ++s) {
+        if constexpr (VEC) {
+          x[s][r] = load_quad<T, STREAM>(rp + col[s][0]);
+        } else {
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            x[s][r].v[j] = rp[col[s][j]];
+        }
+      }
+    }
+  };
+  auto fold_unit = [&](const Quad<T> (&x)[NS][8], int64_t q, bool live, bool guard) {
+    Split3 ops[NS][4];
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        float v[8];
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {
+          const bool in = live && (!guard || q * UR + 8 * g + r < a.N);
+          v[r]          = (ok[s][j] && in) ? x[s][r].v[j] - mean[s][j] : T(0);
+        }
+        ops[s][j] = split_bf16x3(v);
+      }
+    }
+    if constexpr (DIAG && CENTER) {
+#pragma unroll
+      for (int r = 0; r < 8; ++r) {
+        const int64_t row = q * UR + 8 * g + r;
+        if (live && (!guard || row < a.N)) {
+          if constexpr (VEC) {
+            if (ok[0][0]) {
+              Quad<T> w;
+#pragma unroll
+              for (int j = 0; j < 4; ++j)
+                w.v[j] = x[0][r].v[j] - mean[0][j];
+              store_quad<T>(data + row * D + col[0][0], w);
+            }
+          } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+              if (ok[0][j]) data[row * D + col[0][j]] = x[0][r].v[j] - mean[0][j];
+          }
+        }
+      }
+    }
+    mma_unit_bf16<DIAG>(acc, ops[0], ops[NS - 1]);
+  };
+
+  // the ring of gram_rows_body: the other units in flight while one is split and multiplied
+  if (K > 0) {
+    Quad<T> ring[P][NS][8];
+#pragma unroll
+    for (int i = 0; i < P; ++i) {
+      load_unit(ring[i], gw + (i < K ? i : K - 1) * G, false);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    int trips = 0;
+    for (int64_t k0 = 0; k0 < K; k0 += P) {
+#pragma unroll
+      for (int i = 0; i < P; ++i) {
+        const int64_t k = k0 + i;
+        fold_unit(ring[i], gw + k * G, k < K, false);
+        __builtin_amdgcn_sched_barrier(0);
+        load_unit(ring[i], gw + (k + P < K ? k + P : K - 1) * G, false);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if (++trips == kBf16FlushTrips) {
+        flush_tiles(total, acc);
+        trips = 0;
+      }
+    }
+  }
+  if (nfull * UR < a.N && gw == nfull % G) {
+    Quad<T> x[NS][8];
+    load_unit(x, nfull, true);
+    fold_unit(x, nfull, true, true);
+  }
+
+  flush_tiles(total, acc);
+  combine_waves<T, kTilesPerPair>(total, sm, wave, lane);
+  if (wave == 0) {
+    T* out = static_cast<T*>(a.partial) + (int64_t)unit * kTilesPerPair * kTile;
+#pragma unroll
+    for (int ja = 0; ja < 4; ++ja)
+#pragma unroll
+      for (int jb = 0; jb < 4; ++jb)
+        if (!DIAG || jb >= ja) store_tile<T>(out + (ja * 4 + jb) * kTile, total[ja * 4 + jb], lane);
+  }
+}
+
+template <bool DIAG, bool CENTER, bool STREAM>
+__device__ __forceinline__ void gram_cols_body_bf16(const GramArgs& a, int unit, int slab, int bi,
+                                                    int bj, float* sm)
+{
+  using T          = float;
+  constexpr int NS = DIAG ? 1 : 2;
+  constexpr int UR = kBf16UnitRows;
+  constexpr int P  = kBf16Ring;
+
+  const int lane  = threadIdx.x & 63;
+  const int wave  = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int g     = lane >> 4;  // the lane holds rows 8 g .. 8 g + 7 of a unit
+  const int cl    = lane & 15;  // column within a group of 16
+  T* const data   = static_cast<T*>(a.data);
+  const T* mu     = static_cast<const T*>(a.mu);
+  const int64_t N = a.N;
+
+  T* colp[NS][4];
+  bool ok[NS][4];
+  T mean[NS][4];
+#pragma unroll
+  for (int s = 0; s < NS; ++s) {
+#pragma unroll
+    for (int gq = 0; gq < 4; ++gq) {
+      const int64_t c = (int64_t)(s == 0 ? bi : bj) * kBlockCols + 16 * gq + cl;
+      ok[s][gq]       = c < a.D;
+      colp[s][gq]     = data + (ok[s][gq] ? c : 0) * N;
+      mean[s][gq]     = (mu != nullptr && ok[s][gq]) ? mu[c] : T(0);
+    }
+  }
+
+  f32x4 acc[kTilesPerPair], total[kTilesPerPair];
+#pragma unroll
+  for (int t = 0; t < kTilesPerPair; ++t)
+    acc[t] = total[t] = f32x4{0, 0, 0, 0};
+
+  const int64_t G     = (int64_t)a.S * kWaves;
+  const int64_t gw    = (int64_t)slab * kWaves + wave;
+  const int64_t nfull = N / UR;
+  const int64_t K     = gw < nfull ? (nfull - gw + G - 1) / G : 0;
+
+  // x[s][gq][h]: rows 8 g + 4 h .. + 3 of the unit in the lane's column of group gq
+  auto load_unit = [&](Quad<T> (&x)[NS][4][2], int64_t q, bool guard) {
+    const int64_t r0 = q * UR + 8 * g;
+#pragma unroll
+    for (int s = 0; s < NS; ++s)
+#pragma unroll
+      for (int gq = 0; gq < 4; ++gq)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          if (!guard) {
+            x[s][gq][h] = load_quad<T, STREAM>(colp[s][gq] + r0 + 4 * h);
+          } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              const int64_t r  = r0 + 4 * h + j;
+              x[s][gq][h].v[j] = colp[s][gq][r < N ? r : N - 1];
+            }
+          }
+        }
+  };
+  auto fold_unit = [&](const Quad<T> (&x)[NS][4][2], int64_t q, bool live, bool guard) {
+    const int64_t r0 = q * UR + 8 * g;
+    Split3 ops[NS][4];
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+#pragma unroll
+      for (int gq = 0; gq < 4; ++gq) {
+        float v[8];
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {
+          const bool in = live && ok[s][gq] && (!guard || r0 + r < N);
+          v[r]          = in ? x[s][gq][r >> 2].v[r & 3] - mean[s][gq] : T(0);
+        }
+        if constexpr (DIAG && CENTER) {
+          if (s == 0 && live && ok[0][gq]) {
+            if (!guard) {
+#pragma unroll
+              for (int h = 0; h < 2; ++h) {
+                Quad<T> w;
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                  w.v[j] = v[4 * h + j];
+                store_quad<T>(colp[0][gq] + r0 + 4 * h, w);
+              }
+            } else {
+#pragma unroll
+              for (int r = 0; r < 8; ++r)
+                if (r0 + r < N) colp[0][gq][r0 + r] = v[r];
+            }
+          }
+        }
+        ops[s][gq] = split_bf16x3(v);
+      }
+    }
+    mma_unit_bf16<DIAG>(acc, ops[0], ops[NS - 1]);
+  };
+
+  if (K > 0) {
+    Quad<T> ring[P][NS][4][2];
+#pragma unroll
+    for (int i = 0; i < P; ++i) {
+      load_unit(ring[i], gw + (i < K ? i : K - 1) * G, false);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    int trips = 0;
+    for (int64_t k0 = 0; k0 < K; k0 += P) {
+#pragma unroll
+      for (int i = 0; i < P; ++i) {
+        const int64_t k = k0 + i;
+        fold_unit(ring[i], gw + k * G, k < K, false);
+        __builtin_amdgcn_sched_barrier(0);
+        load_unit(ring[i], gw + (k + P < K ? k + P : K - 1) * G, false);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if (++trips == kBf16FlushTrips) {
+        flush_tiles(total, acc);
+        trips = 0;
+      }
+    }
+  }
+  if (nfull * UR < N && gw == nfull % G) {
+    Quad<T> x[NS][4][2];
+    load_unit(x, nfull, true);
+    fold_unit(x, nfull, true, true);
+  }
+
+  flush_tiles(total, acc);
+  combine_waves<T, kTilesPerPair>(total, sm, wave, lane);
+  if (wave == 0) {
+    T* out = static_cast<T*>(a.partial) + (int64_t)unit * kTilesPerPair * kTile;
+#pragma unroll
+    for (int ga = 0; ga < 4; ++ga)
+#pragma unroll
+      for (int gb = 0; gb < 4; ++gb)
+        if (!DIAG || gb >= ga) store_tile<T>(out + (ga * 4 + gb) * kTile, total[ga * 4 + gb], lane);
+  }
+}
+
 // ONE: the matrix has one column block (D <= 64), so only the diagonal body is compiled in,
 // the kernel's register count is that body's, and the matrix, read once, is streamed past
 // the caches (with several blocks the pairs of a slab share their rows through the L2).
@@ -368,7 +742,13 @@ __global__ __launch_bounds__(kThreads) void gram_rows_kernel(GramArgs a)
   pair_blocks(unit - slab * a.npairs, a.nb, bi, bj);
   // one wave-uniform branch around two bodies whose loads are unconditional
   static_assert(ONE || !CENTER, "the centred data is written back by the one-block kernel only");
-  if (ONE || bi == bj) {
+  if constexpr (std::is_same_v<T, float>) {  // bf16 matrix cores, three exact terms per value
+    if (ONE || bi == bj) {
+      gram_rows_body_bf16<VEC, true, CENTER, ONE>(a, unit, slab, bi, bj, sm);
+    } else {
+      if constexpr (!ONE) gram_rows_body_bf16<VEC, false, false, false>(a, unit, slab, bi, bj, sm);
+    }
+  } else if (ONE || bi == bj) {
     gram_rows_body<T, VEC, true, CENTER, ONE>(a, unit, slab, bi, bj, sm);
   } else {
     if constexpr (!ONE) gram_rows_body<T, VEC, false, false, false>(a, unit, slab, bi, bj, sm);
@@ -523,7 +903,13 @@ __global__ __launch_bounds__(kThreads) void gram_cols_kernel(GramArgs a)
   int bi, bj;
   pair_blocks(unit - slab * a.npairs, a.nb, bi, bj);
   static_assert(ONE || !CENTER, "the centred data is written back by the one-block kernel only");
-  if (ONE || bi == bj) {
+  if constexpr (std::is_same_v<T, float>) {
+    if (ONE || bi == bj) {
+      gram_cols_body_bf16<true, CENTER, ONE>(a, unit, slab, bi, bj, sm);
+    } else {
+      if constexpr (!ONE) gram_cols_body_bf16<false, false, false>(a, unit, slab, bi, bj, sm);
+    }
+  } else if (ONE || bi == bj) {
     gram_cols_body<T, true, CENTER, ONE>(a, unit, slab, bi, bj, sm);
   } else {
     if constexpr (!ONE) gram_cols_body<T, false, false, false>(a, unit, slab, bi, bj, sm);
@@ -531,46 +917,53 @@ __global__ __launch_bounds__(kThreads) void gram_cols_kernel(GramArgs a)
 }
 
 // ---------------------------------------------------------------------------
-// Second pass: one workgroup per (pair, tile).  Thread (e, q) sums the slabs q, q + 4, ...
-// of element e in f64, the four meet in LDS in q order, the total is scaled and written
-// to covar[r][c] and covar[c][r].
+// Second pass: one workgroup per (pair, tile, quarter of the tile's 256 elements).  Thread
+// (e, q) sums the slabs q, q + 16, ... of element e in f64, eight loads in flight, the
+// sixteen meet in LDS in q order, the total is scaled and written to covar[r][c] and
+// covar[c][r].
 // ---------------------------------------------------------------------------
+constexpr int kFoldElems = 64;  // elements of a tile per workgroup
+
 template <class T>
-__global__ __launch_bounds__(kTile* kFoldSplit) void cov_fold_kernel(FoldArgs a)
+__global__ __launch_bounds__(kFoldElems* kFoldSplit) void cov_fold_kernel(FoldArgs a)
 {
   using M = Mma<T>;
-  __shared__ double sm[kFoldSplit][kTile];
-  const int pair = blockIdx.x / kTilesPerPair;
-  const int tile = blockIdx.x - pair * kTilesPerPair;
+  __shared__ double sm[kFoldSplit][kFoldElems];
+  constexpr int kParts = kTile / kFoldElems;
+  const int part = blockIdx.x % kParts;
+  const int pt   = blockIdx.x / kParts;
+  const int pair = pt / kTilesPerPair;
+  const int tile = pt - pair * kTilesPerPair;
   const int ta   = tile >> 2;
   const int tb   = tile & 3;
   int bi, bj;
   pair_blocks(pair, a.nb, bi, bj);
   if (bi == bj && tb < ta) return;  // the lower triangle is the mirror of the upper
 
-  const int e = threadIdx.x & (kTile - 1);
-  const int q = threadIdx.x / kTile;
-  const T* p  = static_cast<const T*>(a.partial) + ((int64_t)pair * kTilesPerPair + tile) * kTile + e;
+  const int le = threadIdx.x & (kFoldElems - 1);
+  const int q  = threadIdx.x / kFoldElems;
+  const int e  = part * kFoldElems + le;
+  const T* p   = static_cast<const T*>(a.partial) + ((int64_t)pair * kTilesPerPair + tile) * kTile + e;
   const int64_t slab_stride = (int64_t)a.npairs * kTilesPerPair * kTile;
   double sum = 0.0;
   int s      = q;
-  for (; s + 3 * kFoldSplit < a.S; s += 4 * kFoldSplit) {
-    const T v0 = p[(int64_t)s * slab_stride];
-    const T v1 = p[(int64_t)(s + kFoldSplit) * slab_stride];
-    const T v2 = p[(int64_t)(s + 2 * kFoldSplit) * slab_stride];
-    const T v3 = p[(int64_t)(s + 3 * kFoldSplit) * slab_stride];
-    sum += (double)v0;
-    sum += (double)v1;
-    sum += (double)v2;
-    sum += (double)v3;
+  constexpr int U = 8;
+  for (; s + (U - 1) * kFoldSplit < a.S; s += U * kFoldSplit) {
+    T v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      v[u] = p[(int64_t)(s + u * kFoldSplit) * slab_stride];
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      sum += (double)v[u];
   }
   for (; s < a.S; s += kFoldSplit)
     sum += (double)p[(int64_t)s * slab_stride];
-  sm[q][e] = sum;
+  sm[q][le] = sum;
   __syncthreads();
   if (q != 0) return;
   for (int k = 1; k < kFoldSplit; ++k)
-    sum += sm[k][e];
+    sum += sm[k][le];
 
   const int lane = e & 63;
   const int m    = M::row(lane, e >> 6);
@@ -578,11 +971,14 @@ __global__ __launch_bounds__(kTile* kFoldSplit) void cov_fold_kernel(FoldArgs a)
   const int64_t r = (int64_t)bi * kBlockCols + (a.permuted ? 4 * m + ta : 16 * ta + m);
   const int64_t c = (int64_t)bj * kBlockCols + (a.permuted ? 4 * n + tb : 16 * tb + n);
   if (r >= a.D || c >= a.D) return;
+  // A diagonal tile holds both (r, c) and (c, r), summed in two orders that may differ in the
+  // last bit: its upper half is kept and mirrored like every other tile, so the result is
+  // symmetric bit for bit.
+  if (bi == bj && ta == tb && r > c) return;
   const T val = (T)(sum * a.alpha);
   T* out      = static_cast<T*>(a.out);
   out[r * a.D + c] = val;
-  // a diagonal tile holds both (r, c) and (c, r); everything else is mirrored
-  if (!(bi == bj && ta == tb)) out[c * a.D + r] = val;
+  if (r != c) out[c * a.D + r] = val;
 }
 
 // ---------------------------------------------------------------------------
