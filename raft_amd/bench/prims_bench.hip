@@ -449,6 +449,96 @@ void bench_copy_roof(Harness& h)
   (void)hipEventDestroy(e1);
 }
 
+// ---- roof of 16-byte accesses off a 16-byte boundary -------------------------------------
+// Rows whose byte length is no multiple of 16 (33 bf16, 129 floats, 70 int8) put every lane's
+// 16-byte load and store at an address that is only element-aligned.  The same streaming copy
+// and read as above, with both pointers moved 2, 4 or 8 bytes off a 16-byte boundary, is the
+// ceiling for such shapes: what the memory pipeline sustains when no access is aligned.
+typedef u32x4_t u32x4_any_t __attribute__((aligned(1)));
+
+template <bool NT>
+__global__ __launch_bounds__(256) void offset_copy(const char* __restrict__ in, char* __restrict__ out)
+{
+  const size_t i       = ((size_t)blockIdx.x * 256 + threadIdx.x) * 16;
+  const u32x4_any_t* p = reinterpret_cast<const u32x4_any_t*>(in + i);
+  u32x4_any_t* q       = reinterpret_cast<u32x4_any_t*>(out + i);
+  if (NT)
+    __builtin_nontemporal_store(__builtin_nontemporal_load(p), q);
+  else
+    *q = *p;
+}
+
+template <bool NT>
+__global__ __launch_bounds__(256) void offset_read(const char* __restrict__ in, unsigned* __restrict__ out)
+{
+  u32x4_t acc = {0u, 0u, 0u, 0u};
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const size_t i       = (((size_t)blockIdx.x * 4 + u) * 256 + threadIdx.x) * 16;
+    const u32x4_any_t* p = reinterpret_cast<const u32x4_any_t*>(in + i);
+    acc ^= NT ? __builtin_nontemporal_load(p) : *p;
+  }
+  if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x9e3779b9u) out[blockIdx.x & 1023] = acc[0];
+}
+
+void bench_offset_roof(Harness& h)
+{
+  if (!h.wanted("offset_roof")) return;
+  hipEvent_t e0, e1;
+  RAFT_HIP_TRY(hipEventCreate(&e0));
+  RAFT_HIP_TRY(hipEventCreate(&e1));
+  const size_t bytes = (size_t)256 << 20;
+  const int nbuf     = 4;
+  std::vector<char*> src(nbuf), dst(nbuf);
+  for (int i = 0; i < nbuf; ++i) {
+    RAFT_HIP_TRY(hipMalloc(&src[i], bytes + 256));
+    RAFT_HIP_TRY(hipMalloc(&dst[i], bytes + 256));
+    fill_words<<<2048, 256, 0, h.stream()>>>(reinterpret_cast<unsigned*>(src[i]), (bytes + 256) / 4, 5u + i);
+  }
+  unsigned* sink = nullptr;
+  RAFT_HIP_TRY(hipMalloc(&sink, 4096));
+  RAFT_HIP_TRY(hipStreamSynchronize(h.stream()));
+  const unsigned copy_grid = (unsigned)(bytes / 16 / 256);
+  const unsigned read_grid = copy_grid / 4;
+  for (int off : {0, 2, 4, 8}) {
+    for (int nt = 0; nt < 2; ++nt) {
+      for (int what = 0; what < 2; ++what) {  // 0: copy, 1: read
+        auto launch = [&](int i) {
+          const char* a = src[i % nbuf] + off;
+          char* b       = dst[i % nbuf] + off;
+          if (what == 0 && nt) offset_copy<true><<<copy_grid, 256, 0, h.stream()>>>(a, b);
+          if (what == 0 && !nt) offset_copy<false><<<copy_grid, 256, 0, h.stream()>>>(a, b);
+          if (what == 1 && nt) offset_read<true><<<read_grid, 256, 0, h.stream()>>>(a, sink);
+          if (what == 1 && !nt) offset_read<false><<<read_grid, 256, 0, h.stream()>>>(a, sink);
+        };
+        const int reps = 40;
+        for (int i = 0; i < 5; ++i)
+          launch(i);
+        RAFT_HIP_TRY(hipEventRecord(e0, h.stream()));
+        for (int i = 0; i < reps; ++i)
+          launch(i);
+        RAFT_HIP_TRY(hipEventRecord(e1, h.stream()));
+        RAFT_HIP_TRY(hipEventSynchronize(e1));
+        float ms = 0.f;
+        RAFT_HIP_TRY(hipEventElapsedTime(&ms, e0, e1));
+        const double us   = ms * 1e3 / reps;
+        const double gbps = (what == 0 ? 2.0 : 1.0) * bytes / (us * 1e-6) / 1e9;
+        char name[96];
+        std::snprintf(name, sizeof name, "%s +%d bytes non-temporal=%d", what == 0 ? "copy" : "read", off, nt);
+        std::printf("%-34s %-22s %10.2f us %9.1f GB/s  %4.1f %% of 8 TB/s  %s\n", "offset_roof",
+                    what == 0 ? "256MiB+256MiB" : "256MiB", us, gbps, gbps / 80.0, name);
+      }
+    }
+  }
+  for (int i = 0; i < nbuf; ++i) {
+    (void)hipFree(src[i]);
+    (void)hipFree(dst[i]);
+  }
+  (void)hipFree(sink);
+  (void)hipEventDestroy(e0);
+  (void)hipEventDestroy(e1);
+}
+
 // ---- read roof ------------------------------------------------------------------------
 // What the GPU sustains when a kernel only reads: every lane XORs its 16-byte loads into a
 // register and one word per workgroup is written at the end (so that nothing can be dropped).
@@ -677,6 +767,7 @@ int main(int argc, char** argv)
   bench_mat_vec_op<double, true>(h);
   bench_copy_roof(h);
   bench_read_roof(h);
+  bench_offset_roof(h);
   bench_call_path(h);
   return 0;
 }

@@ -3,7 +3,7 @@
 
 Run the three profiler passes on the GPU box from the repository root (TMPDIR=/tmp):
 
-  ALL=cfg1,cfg2,cfg3_mean,cfg3_stddev,cfg4,cfg5a,cfg5b,cfg5c
+  ALL=cfg1,cfg2,cfg3_mean,cfg3_stddev,cfg3_stddev_sample,cfg4,cfg4_keys,cfg5a,cfg5b,cfg5c
   rocprofv3 --kernel-trace --stats -d OUT/kt -o kt --output-format csv -- \\
       python3 bench.py --only-kernel $ALL --steps 100 --warmup 10
   rocprofv3 --pmc FETCH_SIZE -d OUT/fetch -o fetch --output-format csv -- \\
@@ -45,8 +45,14 @@ CONFIGS = {
                   "fold_kernel<rmi::PolF<float, 0, 0>", 2560000000, 256),
     "cfg3_stddev": ("column stddev fp32 10000000x64 (sum of squares + epilogue)",
                     "col_kernel<rmi::PolF<float, 1, 0>", "fold_kernel<rmi::PolF<float, 1, 0>", 2560000000, 256),
+    # (the sample stddev runs the same kernels as the population one, and the index-only
+    # arg-max the same kernel as the key-value one: their launches are averaged together)
+    "cfg3_stddev_sample": ("column stddev (sample) fp32 10000000x64", "col_kernel<rmi::PolF<float, 1, 0>",
+                           "fold_kernel<rmi::PolF<float, 1, 0>", 2560000000, 256),
     "cfg4": ("row argmax fp32 65536x32000 -> {i32,f32}", "row_block_kernel<rmi::PolKvp<float, int, true>", None,
              8388608000, 524288),
+    "cfg4_keys": ("matrix::argmax fp32 65536x32000 -> i32", "row_block_kernel<rmi::PolKvp<float, int, true>", None,
+                  8388608000, 262144),
     "cfg5a": ("int8 4096x16384 -> int64", "row_block_kernel<rmi::PolI<signed char, 0, 0>", None, 67108864, 32768),
     "cfg5b": ("int8 16777216x8 -> int64", "row_lanes_kernel<rmi::PolI<signed char, 0, 0>", None, 134217728,
               134217728),
@@ -109,7 +115,7 @@ def main():
     w("")
     w(f"Library at commit {commit}.  Commands (run from the repository root on the GPU box, TMPDIR=/tmp):")
     w("")
-    w("  ALL=cfg1,cfg2,cfg3_mean,cfg3_stddev,cfg4,cfg5a,cfg5b,cfg5c")
+    w("  ALL=cfg1,cfg2,cfg3_mean,cfg3_stddev,cfg3_stddev_sample,cfg4,cfg4_keys,cfg5a,cfg5b,cfg5c")
     w("  rocprofv3 --kernel-trace --stats -d OUT/kt -o kt --output-format csv -- \\")
     w("      python3 bench.py --only-kernel $ALL --steps 100 --warmup 10")
     w("  rocprofv3 --pmc FETCH_SIZE -d OUT/fetch -o fetch --output-format csv -- \\")
@@ -120,6 +126,9 @@ def main():
     w("")
     w("GB/s = algorithmic bytes (input once + output once) / (kernel + fold average duration);")
     w("%peak against 8000 GB/s.  fetch / write MB = counters scaled by the copy-kernel factors.")
+    w("Durations under the tracer run up to about 4 % above the same launches timed with HIP events")
+    w("in bench.py on another box (tracing overhead and box-to-box spread): a kernel average here can")
+    w("exceed bench.py's ms_per_step of the same workload by that much.")
     w("")
     w(f"Counter scaling from the 512 MiB device copy ({COPY_KERNEL}, {COPY_KIB} KiB read and written):")
     w(f"  FETCH_SIZE reads {copy_f:.2f} -> multiply by {ff:.4f} for KiB;  "
@@ -177,7 +186,7 @@ def extras(out: Path, commit: str):
     kt = {r["Name"]: r for r in rows}
     lines = []
     w = lines.append
-    w("rocprofv3 summary: row_normalize, meanvar, wide-row column sums and dense-slot row sums, one MI355X (gfx950)")
+    w("rocprofv3 summary: row_normalize, meanvar, wide-row column sums, dense-slot row sums and cov, one MI355X (gfx950)")
     w("=" * 88)
     w("")
     w(f"Library at commit {commit}.  Command (run from the repository root on the GPU box, TMPDIR=/tmp):")
@@ -195,7 +204,11 @@ def extras(out: Path, commit: str):
             ("column sum fp32 32768x4097 (whole rows)", "col_wide_kernel<rmi::PolF<float, 0, 0>",
              "fold_rows_kernel<rmi::PolF<float, 0, 0>", 32768 * 4097 * 4 + 4097 * 4),
             ("row sum fp32 2000000x66 (dense slots)", "row_dense_kernel<rmi::PolF<float, 0, 0>", None,
-             2000000 * 67 * 4)]
+             2000000 * 67 * 4),
+            ("stats::cov fp32 10000000x64 (data read only)", "gram_rows_kernel<float, true, true, false>",
+             "cov_fold_kernel<float>", 2560016384),
+            ("stats::cov fp32 10000000x64 (data centred in place)", "gram_rows_kernel<float, true, true, true>",
+             "cov_fold_kernel<float>", 2 * 2560000000 + 16384)]
     for label, k1, k2, alg in work:
         s1 = pick(kt, k1)
         if s1 is None:
@@ -214,7 +227,7 @@ def extras(out: Path, commit: str):
     w("single timed calls, so launch counts include those):")
     for n, r in kt.items():
         if "rmi::" in n and "normalize" not in n and "MeanVar" not in n and "col_wide" not in n \
-                and "fold_rows" not in n and "row_dense" not in n:
+                and "fold_rows" not in n and "row_dense" not in n and "cov::" not in n:
             w(f"  {n[:100]:100s} {r['Calls']:>6s} {float(r['AverageNs']):12.1f}")
     (ROOT / "profiles" / "row_normalize_meanvar_rocprofv3.txt").write_text("\n".join(lines) + "\n")
     print("\n".join(lines[:16]))
