@@ -8,11 +8,12 @@ int cu_count();  // rmi_api.hip
 namespace {
 
 // Workgroups per CU when one pair of column blocks covers the matrix (D <= 64, the
-// shape that is bound by HBM as much as by the matrix cores), and the number of queued
-// workgroups per CU otherwise (diagonal pairs issue 10 matrix instructions per wave-load,
-// the others 16: small units even the CUs out).
+// shape that is bound by HBM as much as by the matrix cores): the kernels hold more than
+// 256 registers, so a CU holds one workgroup at a time and a second one per CU would only
+// queue behind the first.  Otherwise the number of queued workgroups per CU (diagonal pairs
+// issue 10 matrix instructions per wave-load, the others 16: small units even the CUs out).
 #ifndef RMI_COV_WG_PER_CU
-#define RMI_COV_WG_PER_CU 2
+#define RMI_COV_WG_PER_CU 1
 #endif
 constexpr int kWgPerCuOnePair = RMI_COV_WG_PER_CU;
 constexpr int kWgPerCuPairs   = 8;
@@ -88,15 +89,25 @@ int launch(const CovPlan& pl, int layout, int64_t N, int64_t D, int sample, bool
   const dim3 grid((unsigned)pl.grid);
   const dim3 block(cov::kThreads);
   const bool one = pl.npairs == 1;
+  // fp32, exactly one whole block of columns: the kernels without column masks
+  constexpr bool kF32 = std::is_same_v<T, float>;
+  const bool full     = kF32 && D == cov::kBlockCols;
   if (write_back) {  // one column block: the same pass leaves x - mu behind
-    if (layout != RMI_ROW_MAJOR)
-      hipLaunchKernelGGL((cov::gram_cols_kernel<T, true, true>), grid, block, 0, st, g);
+    if (layout != RMI_ROW_MAJOR) {
+      if (full)
+        hipLaunchKernelGGL((cov::gram_cols_kernel<T, true, true, kF32>), grid, block, 0, st, g);
+      else
+        hipLaunchKernelGGL((cov::gram_cols_kernel<T, true, true>), grid, block, 0, st, g);
+    } else if (full)
+      hipLaunchKernelGGL((cov::gram_rows_kernel<T, true, true, true, kF32>), grid, block, 0, st, g);
     else if (pl.vec)
       hipLaunchKernelGGL((cov::gram_rows_kernel<T, true, true, true>), grid, block, 0, st, g);
     else
       hipLaunchKernelGGL((cov::gram_rows_kernel<T, false, true, true>), grid, block, 0, st, g);
   } else if (layout == RMI_ROW_MAJOR) {
-    if (pl.vec && one)
+    if (full)
+      hipLaunchKernelGGL((cov::gram_rows_kernel<T, true, true, false, kF32>), grid, block, 0, st, g);
+    else if (pl.vec && one)
       hipLaunchKernelGGL((cov::gram_rows_kernel<T, true, true>), grid, block, 0, st, g);
     else if (pl.vec)
       hipLaunchKernelGGL((cov::gram_rows_kernel<T, true, false>), grid, block, 0, st, g);
@@ -104,6 +115,8 @@ int launch(const CovPlan& pl, int layout, int64_t N, int64_t D, int sample, bool
       hipLaunchKernelGGL((cov::gram_rows_kernel<T, false, true>), grid, block, 0, st, g);
     else
       hipLaunchKernelGGL((cov::gram_rows_kernel<T, false, false>), grid, block, 0, st, g);
+  } else if (full) {
+    hipLaunchKernelGGL((cov::gram_cols_kernel<T, true, false, kF32>), grid, block, 0, st, g);
   } else if (one) {
     hipLaunchKernelGGL((cov::gram_cols_kernel<T, true>), grid, block, 0, st, g);
   } else {

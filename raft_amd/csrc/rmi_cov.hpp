@@ -131,7 +131,10 @@ __device__ __forceinline__ Quad<T> load_quad(const T* p)
     q.v[j] = x[j];
   return q;
 }
-template <class T>
+// STREAM: the centred rows are not read again by this kernel; measured 3 % faster streamed
+// where a store instruction writes whole lines (row-major), 6 % slower where it writes 16-byte
+// pieces of 64 lines (col-major).
+template <class T, bool STREAM = false>
 __device__ __forceinline__ void store_quad(T* p, const Quad<T>& q)
 {
   typedef T full_t __attribute__((ext_vector_type(4)));
@@ -140,7 +143,10 @@ __device__ __forceinline__ void store_quad(T* p, const Quad<T>& q)
 #pragma unroll
   for (int j = 0; j < 4; ++j)
     x[j] = q.v[j];
-  *reinterpret_cast<vec_t*>(p) = x;
+  if constexpr (STREAM)
+    __builtin_nontemporal_store(x, reinterpret_cast<vec_t*>(p));
+  else
+    *reinterpret_cast<vec_t*>(p) = x;
 }
 
 // Workgroup ids are dealt round-robin over the 8 XCDs, each with an L2 of its own.  The
@@ -440,6 +446,31 @@ __device__ __forceinline__ void mma_unit_bf16(f32x4 (&acc)[kTilesPerPair], const
 #endif
 constexpr int kBf16Ring       = RMI_COV_BF16_RING;  // units of 32 rows a wave keeps loaded or in flight
 constexpr int kBf16FlushTrips = 2;
+// The diagonal body (one column block against itself, the whole job when D <= 64) runs one
+// wave per SIMD, so nothing but the wave's own instruction order can overlap the ~230 vector
+// instructions that split a unit with the 60 matrix instructions that multiply one.  Its loop
+// is therefore pipelined by hand: while unit k is multiplied, unit k + 1 is split into a
+// second set of operands, and the scheduler is told to issue kPipeValuPerMma vector
+// instructions behind every matrix instruction (a 16 x 16 x 32 instruction occupies the
+// matrix core for 16 cycles and the issue port for 4).
+#ifndef RMI_COV_BF16_PIPE_RING
+#define RMI_COV_BF16_PIPE_RING 4
+#endif
+#ifndef RMI_COV_BF16_PIPE_VALU
+#define RMI_COV_BF16_PIPE_VALU 4
+#endif
+constexpr int kPipeRing       = RMI_COV_BF16_PIPE_RING;  // even: the operand sets alternate
+constexpr int kPipeValuPerMma = RMI_COV_BF16_PIPE_VALU;
+constexpr int kPipeMmas       = 60;  // six terms of the ten tiles on and above the diagonal
+static_assert(kPipeRing % 2 == 0, "operand sets alternate with the ring slots");
+__device__ __forceinline__ void interleave_split_with_mma()
+{
+#pragma unroll
+  for (int i = 0; i < kPipeMmas; ++i) {
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                // one matrix instruction
+    __builtin_amdgcn_sched_group_barrier(0x002, kPipeValuPerMma, 0);  // vector instructions
+  }
+}
 __device__ __forceinline__ void flush_tiles(f32x4 (&total)[kTilesPerPair], f32x4 (&acc)[kTilesPerPair])
 {
 #pragma unroll
@@ -449,7 +480,11 @@ __device__ __forceinline__ void flush_tiles(f32x4 (&total)[kTilesPerPair], f32x4
   }
 }
 
-template <bool VEC, bool DIAG, bool CENTER, bool STREAM>
+// FULL: the block has all of its 64 columns (and VEC holds), so nothing in the loop depends
+// on a lane's column mask; together with a main loop over units that are all live this
+// leaves the centring stores unconditional, and the loop body one basic block that the
+// interleaving above applies to.
+template <bool VEC, bool DIAG, bool CENTER, bool STREAM, bool FULL = false>
 __device__ __forceinline__ void gram_rows_body_bf16(const GramArgs& a, int unit, int slab, int bi,
                                                     int bj, float* sm)
 {
@@ -508,8 +543,8 @@ __device__ __forceinline__ void gram_rows_body_bf16(const GramArgs& a, int unit,
       }
     }
   };
-  auto fold_unit = [&](const Quad<T> (&x)[NS][8], int64_t q, bool live, bool guard) {
-    Split3 ops[NS][4];
+  auto split_unit = [&](Split3 (&ops)[NS][4], const Quad<T> (&x)[NS][8], int64_t q, bool live,
+                        bool guard) {
 #pragma unroll
     for (int s = 0; s < NS; ++s) {
 #pragma unroll
@@ -518,7 +553,7 @@ __device__ __forceinline__ void gram_rows_body_bf16(const GramArgs& a, int unit,
 #pragma unroll
         for (int r = 0; r < 8; ++r) {
           const bool in = live && (!guard || q * UR + 8 * g + r < a.N);
-          v[r]          = (ok[s][j] && in) ? x[s][r].v[j] - mean[s][j] : T(0);
+          v[r]          = ((FULL || ok[s][j]) && in) ? x[s][r].v[j] - mean[s][j] : T(0);
         }
         ops[s][j] = split_bf16x3(v);
       }
@@ -529,12 +564,12 @@ __device__ __forceinline__ void gram_rows_body_bf16(const GramArgs& a, int unit,
         const int64_t row = q * UR + 8 * g + r;
         if (live && (!guard || row < a.N)) {
           if constexpr (VEC) {
-            if (ok[0][0]) {
+            if (FULL || ok[0][0]) {
               Quad<T> w;
 #pragma unroll
               for (int j = 0; j < 4; ++j)
                 w.v[j] = x[0][r].v[j] - mean[0][j];
-              store_quad<T>(data + row * D + col[0][0], w);
+              store_quad<T, STREAM>(data + row * D + col[0][0], w);
             }
           } else {
 #pragma unroll
@@ -544,9 +579,52 @@ __device__ __forceinline__ void gram_rows_body_bf16(const GramArgs& a, int unit,
         }
       }
     }
+  };
+  auto fold_unit = [&](const Quad<T> (&x)[NS][8], int64_t q, bool live, bool guard) {
+    Split3 ops[NS][4];
+    split_unit(ops, x, q, live, guard);
     mma_unit_bf16<DIAG>(acc, ops[0], ops[NS - 1]);
   };
 
+  if constexpr (DIAG) {
+    // pipelined: slot s of the ring holds the units s, s + PD, ...; unit k is multiplied from
+    // operand set k % 2 while unit k + 1 is split into the other and its slot is refilled
+    constexpr int PD = kPipeRing;
+    if (K > 0) {
+      Quad<T> ring[PD][NS][8];
+#pragma unroll
+      for (int i = 0; i < PD; ++i) {
+        load_unit(ring[i], gw + (i < K ? i : K - 1) * G, false);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      Split3 ops[2][NS][4];
+      split_unit(ops[0], ring[0], gw, true, false);
+      __builtin_amdgcn_sched_barrier(0);
+      load_unit(ring[0], gw + (PD < K ? PD : K - 1) * G, false);
+      __builtin_amdgcn_sched_barrier(0);
+      // a trip of PD units; `all_live`: none of its units is past the wave's last one
+      auto trip = [&](int64_t k0, auto all_live) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < PD; ++i) {
+          const int64_t k = k0 + i;
+          const int slot  = (i + 1) % PD;
+          const bool live = decltype(all_live)::value || k + 1 < K;
+          split_unit(ops[(i + 1) & 1], ring[slot], gw + (k + 1) * G, live, false);
+          mma_unit_bf16<true>(acc, ops[i & 1][0], ops[i & 1][0]);
+          interleave_split_with_mma();
+          __builtin_amdgcn_sched_barrier(0);
+          load_unit(ring[slot], gw + (k + 1 + PD < K ? k + 1 + PD : K - 1) * G, false);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        flush_tiles(total, acc);
+      };
+      int64_t k0 = 0;
+      for (; k0 + PD < K; k0 += PD)
+        trip(k0, std::true_type{});
+      for (; k0 < K; k0 += PD)
+        trip(k0, std::false_type{});
+    }
+  } else
   // the ring of gram_rows_body: the other units in flight while one is split and multiplied
   if (K > 0) {
     Quad<T> ring[P][NS][8];
@@ -589,7 +667,7 @@ __device__ __forceinline__ void gram_rows_body_bf16(const GramArgs& a, int unit,
   }
 }
 
-template <bool DIAG, bool CENTER, bool STREAM>
+template <bool DIAG, bool CENTER, bool STREAM, bool FULL = false>
 __device__ __forceinline__ void gram_cols_body_bf16(const GramArgs& a, int unit, int slab, int bi,
                                                     int bj, float* sm)
 {
@@ -630,9 +708,10 @@ __device__ __forceinline__ void gram_cols_body_bf16(const GramArgs& a, int unit,
   const int64_t nfull = N / UR;
   const int64_t K     = gw < nfull ? (nfull - gw + G - 1) / G : 0;
 
-  // x[s][gq][h]: rows 8 g + 4 h .. + 3 of the unit in the lane's column of group gq
+  // x[s][gq][h]: rows kLaneRows g + kHalfRows h .. + 3 of the unit in the lane's column of group gq
+  constexpr int kLaneRows = 8, kHalfRows = 4;
   auto load_unit = [&](Quad<T> (&x)[NS][4][2], int64_t q, bool guard) {
-    const int64_t r0 = q * UR + 8 * g;
+    const int64_t r0 = q * UR + kLaneRows * g;
 #pragma unroll
     for (int s = 0; s < NS; ++s)
 #pragma unroll
@@ -640,19 +719,19 @@ __device__ __forceinline__ void gram_cols_body_bf16(const GramArgs& a, int unit,
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
           if (!guard) {
-            x[s][gq][h] = load_quad<T, STREAM>(colp[s][gq] + r0 + 4 * h);
+            x[s][gq][h] = load_quad<T, STREAM>(colp[s][gq] + r0 + kHalfRows * h);
           } else {
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-              const int64_t r  = r0 + 4 * h + j;
+              const int64_t r  = r0 + kHalfRows * h + j;
               x[s][gq][h].v[j] = colp[s][gq][r < N ? r : N - 1];
             }
           }
         }
   };
-  auto fold_unit = [&](const Quad<T> (&x)[NS][4][2], int64_t q, bool live, bool guard) {
-    const int64_t r0 = q * UR + 8 * g;
-    Split3 ops[NS][4];
+  auto split_unit = [&](Split3 (&ops)[NS][4], const Quad<T> (&x)[NS][4][2], int64_t q, bool live,
+                        bool guard) {
+    const int64_t r0 = q * UR + kLaneRows * g;
 #pragma unroll
     for (int s = 0; s < NS; ++s) {
 #pragma unroll
@@ -660,11 +739,11 @@ __device__ __forceinline__ void gram_cols_body_bf16(const GramArgs& a, int unit,
         float v[8];
 #pragma unroll
         for (int r = 0; r < 8; ++r) {
-          const bool in = live && ok[s][gq] && (!guard || r0 + r < N);
+          const bool in = live && (FULL || ok[s][gq]) && (!guard || r0 + kHalfRows * (r >> 2) + (r & 3) < N);
           v[r]          = in ? x[s][gq][r >> 2].v[r & 3] - mean[s][gq] : T(0);
         }
         if constexpr (DIAG && CENTER) {
-          if (s == 0 && live && ok[0][gq]) {
+          if (s == 0 && live && (FULL || ok[0][gq])) {
             if (!guard) {
 #pragma unroll
               for (int h = 0; h < 2; ++h) {
@@ -672,22 +751,64 @@ __device__ __forceinline__ void gram_cols_body_bf16(const GramArgs& a, int unit,
 #pragma unroll
                 for (int j = 0; j < 4; ++j)
                   w.v[j] = v[4 * h + j];
-                store_quad<T>(colp[0][gq] + r0 + 4 * h, w);
+                store_quad<T>(colp[0][gq] + r0 + kHalfRows * h, w);
               }
             } else {
 #pragma unroll
               for (int r = 0; r < 8; ++r)
-                if (r0 + r < N) colp[0][gq][r0 + r] = v[r];
+                if (r0 + kHalfRows * (r >> 2) + (r & 3) < N)
+                  colp[0][gq][r0 + kHalfRows * (r >> 2) + (r & 3)] = v[r];
             }
           }
         }
         ops[s][gq] = split_bf16x3(v);
       }
     }
+  };
+  auto fold_unit = [&](const Quad<T> (&x)[NS][4][2], int64_t q, bool live, bool guard) {
+    Split3 ops[NS][4];
+    split_unit(ops, x, q, live, guard);
     mma_unit_bf16<DIAG>(acc, ops[0], ops[NS - 1]);
   };
 
-  if (K > 0) {
+  if constexpr (DIAG) {
+    // pipelined as in gram_rows_body_bf16
+    constexpr int PD = kPipeRing;
+    if (K > 0) {
+      Quad<T> ring[PD][NS][4][2];
+#pragma unroll
+      for (int i = 0; i < PD; ++i) {
+        load_unit(ring[i], gw + (i < K ? i : K - 1) * G, false);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      Split3 ops[2][NS][4];
+      split_unit(ops[0], ring[0], gw, true, false);
+      __builtin_amdgcn_sched_barrier(0);
+      load_unit(ring[0], gw + (PD < K ? PD : K - 1) * G, false);
+      __builtin_amdgcn_sched_barrier(0);
+      // a trip of PD units; `all_live`: none of its units is past the wave's last one
+      auto trip = [&](int64_t k0, auto all_live) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < PD; ++i) {
+          const int64_t k = k0 + i;
+          const int slot  = (i + 1) % PD;
+          const bool live = decltype(all_live)::value || k + 1 < K;
+          split_unit(ops[(i + 1) & 1], ring[slot], gw + (k + 1) * G, live, false);
+          mma_unit_bf16<true>(acc, ops[i & 1][0], ops[i & 1][0]);
+          interleave_split_with_mma();
+          __builtin_amdgcn_sched_barrier(0);
+          load_unit(ring[slot], gw + (k + 1 + PD < K ? k + 1 + PD : K - 1) * G, false);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        flush_tiles(total, acc);
+      };
+      int64_t k0 = 0;
+      for (; k0 + PD < K; k0 += PD)
+        trip(k0, std::true_type{});
+      for (; k0 < K; k0 += PD)
+        trip(k0, std::false_type{});
+    }
+  } else if (K > 0) {
     Quad<T> ring[P][NS][4][2];
 #pragma unroll
     for (int i = 0; i < P; ++i) {
@@ -731,7 +852,7 @@ __device__ __forceinline__ void gram_cols_body_bf16(const GramArgs& a, int unit,
 // ONE: the matrix has one column block (D <= 64), so only the diagonal body is compiled in,
 // the kernel's register count is that body's, and the matrix, read once, is streamed past
 // the caches (with several blocks the pairs of a slab share their rows through the L2).
-template <class T, bool VEC, bool ONE, bool CENTER = false>
+template <class T, bool VEC, bool ONE, bool CENTER = false, bool FULL = false>
 __global__ __launch_bounds__(kThreads) void gram_rows_kernel(GramArgs a)
 {
   __shared__ T sm[kTilesPerPair * kTile];
@@ -742,9 +863,10 @@ __global__ __launch_bounds__(kThreads) void gram_rows_kernel(GramArgs a)
   pair_blocks(unit - slab * a.npairs, a.nb, bi, bj);
   // one wave-uniform branch around two bodies whose loads are unconditional
   static_assert(ONE || !CENTER, "the centred data is written back by the one-block kernel only");
+  static_assert(!FULL || (ONE && VEC && std::is_same_v<T, float>), "FULL: one whole block of floats");
   if constexpr (std::is_same_v<T, float>) {  // bf16 matrix cores, three exact terms per value
     if (ONE || bi == bj) {
-      gram_rows_body_bf16<VEC, true, CENTER, ONE>(a, unit, slab, bi, bj, sm);
+      gram_rows_body_bf16<VEC, true, CENTER, ONE, FULL>(a, unit, slab, bi, bj, sm);
     } else {
       if constexpr (!ONE) gram_rows_body_bf16<VEC, false, false, false>(a, unit, slab, bi, bj, sm);
     }
@@ -893,7 +1015,7 @@ __device__ __forceinline__ void gram_cols_body(const GramArgs& a, int unit, int 
   }
 }
 
-template <class T, bool ONE, bool CENTER = false>
+template <class T, bool ONE, bool CENTER = false, bool FULL = false>
 __global__ __launch_bounds__(kThreads) void gram_cols_kernel(GramArgs a)
 {
   __shared__ T sm[kTilesPerPair * kTile];
@@ -905,7 +1027,10 @@ __global__ __launch_bounds__(kThreads) void gram_cols_kernel(GramArgs a)
   static_assert(ONE || !CENTER, "the centred data is written back by the one-block kernel only");
   if constexpr (std::is_same_v<T, float>) {
     if (ONE || bi == bj) {
-      gram_cols_body_bf16<true, CENTER, ONE>(a, unit, slab, bi, bj, sm);
+      // plain loads: the eight 16-byte pieces of a column's line are read by eight
+      // instructions, and a streamed line may be gone before the next piece is asked for
+      // (10M x 64: 500 -> 450 us)
+      gram_cols_body_bf16<true, CENTER, false, FULL>(a, unit, slab, bi, bj, sm);
     } else {
       if constexpr (!ONE) gram_cols_body_bf16<false, false, false>(a, unit, slab, bi, bj, sm);
     }

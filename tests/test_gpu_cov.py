@@ -104,6 +104,22 @@ def test_ragged_shapes(dt, layout, center):
             _check(dt, layout, rows, cols, sample, m, center)
 
 
+@pytest.mark.parametrize("layout", [api.ROW_MAJOR, api.COL_MAJOR])
+@pytest.mark.parametrize("center", [False, True])
+def test_one_block_few_units_per_wave(layout, center):
+    """One whole block of 64 fp32 columns and so few rows that a wave gets 0 to 9 units of 32
+    rows, with and without a ragged last unit: every entry and exit of the pipelined loop
+    (prologue only, partial first trip, whole trips, the trip that ends on a dead unit)."""
+    rng = np.random.default_rng(11 + layout)
+    for rows in (32, 33, 64, 127, 128, 129, 160, 255, 256, 257, 384, 511, 512, 513, 640, 768,
+                 1000, 1024, 1056, 1151, 1152, 1153, 1280, 2047, 2048, 2081):
+        m = (rng.normal(-1.0, 3.0, (rows, 64)) * rng.uniform(0.5, 2.0, 64)).astype(np.float32)
+        _check(api.F32, layout, rows, 64, True, m, center)
+    for cols in (60, 32, 8):  # the same loops with masked columns
+        m = rng.normal(0.5, 1.0, (1153, cols)).astype(np.float32)
+        _check(api.F32, layout, 1153, cols, False, m, center)
+
+
 @pytest.mark.parametrize("dt", [api.F32, api.F64])
 @pytest.mark.parametrize("layout", [api.ROW_MAJOR, api.COL_MAJOR])
 def test_without_mean_vector(dt, layout):
