@@ -636,20 +636,14 @@ def main():
         n = max(10, args.steps // 4)
         e0 = torch.cuda.Event(enable_timing=True)
         e1 = torch.cuda.Event(enable_timing=True)
+        # Timing first, the fp64 check after it: a second of fp64 matrix products right before
+        # the timed loop leaves the GPU at its power limit, and the loop then measures the
+        # limiter (the same kernel 380 us per call before, 590 us after), not the kernel.
         for name, flags in (("read_only", 0), ("centered", api.COV_CENTER_DATA)):
-            if flags == 0:
-                for i in range(3):
-                    rc = call(i, flags)
-                    assert rc == 0, api.status_string(rc)
-                torch.cuda.synchronize()
-                x = xs[2].view(rows, cols)
-                ref = torch.zeros(cols, cols, dtype=torch.float64, device="cuda")
-                for c in x.split(1 << 20):
-                    d = (c - mus[2][None, :]).to(torch.float64)
-                    ref += d.T @ d
-                ref /= rows - 1
-                sc = torch.sqrt(torch.outer(torch.diagonal(ref), torch.diagonal(ref)))
-                ok = bool(((out.view(cols, cols).double() - ref).abs() <= 1e-5 * sc).all())
+            for i in range(10):
+                rc = call(i, flags)
+                assert rc == 0, api.status_string(rc)
+            torch.cuda.synchronize()
             e0.record(stream)
             for i in range(n):
                 call(i, flags)
@@ -658,6 +652,21 @@ def main():
             ms = e0.elapsed_time(e1) / n
             nb = rows * cols * 4 * (2 if flags else 1) + cols * cols * 4
             res[name] = dict(ms_per_step=ms, alg_bytes=nb, GBps=nb / (ms * 1e-3) / 1e9)
+        # the centred loop left x - mu in the buffers: check a call on the third matrix regenerated
+        del xs[:]
+        fresh = mk_normal(rows, cols, 3 + 7919 * 2, 3.0, 2.0)
+        rc = lib.rmi_cov(api.F32, api.ROW_MAJOR, rows, cols, 1, 0, fresh.data_ptr(), mus[2].data_ptr(),
+                         out.data_ptr(), ws.data_ptr(), nws, sptr)
+        assert rc == 0, api.status_string(rc)
+        torch.cuda.synchronize()
+        x = fresh.view(rows, cols)
+        ref = torch.zeros(cols, cols, dtype=torch.float64, device="cuda")
+        for c in x.split(1 << 20):
+            d = (c - mus[2][None, :]).to(torch.float64)
+            ref += d.T @ d
+        ref /= rows - 1
+        sc = torch.sqrt(torch.outer(torch.diagonal(ref), torch.diagonal(ref)))
+        ok = bool(((out.view(cols, cols).double() - ref).abs() <= 1e-5 * sc).all())
         hbm_ms = (rows * cols * 4 + cols * cols * 4) / (PEAK_HBM_GBPS * 1e9) * 1e3
         mfma_ms = rows * cols * cols / 157.3e12 * 1e3
         ms = res["read_only"]["ms_per_step"]

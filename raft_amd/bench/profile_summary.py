@@ -205,9 +205,9 @@ def extras(out: Path, commit: str):
              "fold_rows_kernel<rmi::PolF<float, 0, 0>", 32768 * 4097 * 4 + 4097 * 4),
             ("row sum fp32 2000000x66 (dense slots)", "row_dense_kernel<rmi::PolF<float, 0, 0>", None,
              2000000 * 67 * 4),
-            ("stats::cov fp32 10000000x64 (data read only)", "gram_rows_kernel<float, true, true, false>",
+            ("stats::cov fp32 10000000x64 (data read only)", "gram_rows_kernel<float, true, true, false, true>",
              "cov_fold_kernel<float>", 2560016384),
-            ("stats::cov fp32 10000000x64 (data centred in place)", "gram_rows_kernel<float, true, true, true>",
+            ("stats::cov fp32 10000000x64 (data centred in place)", "gram_rows_kernel<float, true, true, true, true>",
              "cov_fold_kernel<float>", 2 * 2560000000 + 16384)]
     for label, k1, k2, alg in work:
         s1 = pick(kt, k1)

@@ -207,7 +207,7 @@ def test_empty_and_errors():
 
 
 def test_full_size_10m_by_64():
-    """BASELINE config 3's matrix (10,000,000 x 64 fp32, N(3, 2)): the covariance against an
+    """The column-statistics benchmark matrix (10,000,000 x 64 fp32, N(3, 2)): the covariance against an
     independent fp64 contraction on the device, the first 100,000 rows against the oracle as a
     problem of their own, and the centred data against x - mu."""
     import torch
