@@ -412,7 +412,6 @@ int rmi_row_normalize(const rmi_reduce_desc* desc,
   if (in == nullptr || out == nullptr) return RMI_ERR_NULL;
   const int es = dtype_size(d.in_dtype);
   if (!aligned(in, es) || !aligned(out, es)) return RMI_ERR_ALIGNMENT;
-  const NormPlan pl = make_norm_plan(d.n_rows, d.n_cols, es);
   NormArgs a{};
   a.in        = in;
   a.out       = out;
@@ -422,6 +421,16 @@ int rmi_row_normalize(const rmi_reduce_desc* desc,
   a.final_op  = d.final_op;
   a.init      = d.init.f;
   a.eps       = eps;
+  const NormPlan flat = make_flat_norm_plan(d.n_rows, d.n_cols, es, in, out);
+  if (flat.kind == 3) {
+    const int rc = fn(flat, a, static_cast<hipStream_t>(stream));
+    if (rc != RMI_OK || flat.flat_rows == d.n_rows) return rc;
+    // the last few rows, which do not end on a 16-byte boundary, go the ordinary way
+    a.in     = static_cast<const char*>(in) + flat.flat_rows * a.row_bytes;
+    a.out    = static_cast<char*>(out) + flat.flat_rows * a.row_bytes;
+    a.n_rows = d.n_rows - flat.flat_rows;
+  }
+  const NormPlan pl = make_norm_plan(a.n_rows, d.n_cols, es);
   return fn(pl, a, static_cast<hipStream_t>(stream));
 }
 

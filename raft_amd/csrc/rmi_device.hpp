@@ -281,6 +281,8 @@ struct PolF {
   using acc_t              = double;
   static constexpr int VEC = In<InT>::VEC;
   static constexpr int CLS = kClsFloat;
+  static constexpr int kMain = MAIN;
+  static constexpr int kRed  = RED;
   // How the overlapping last vector of a row (its first VEC - tail elements were already
   // counted) is folded: kTailZero: those elements are zeroed and the vector is pushed whole
   // (sums: every main op maps 0 to 0); kTailDup: the vector is pushed whole as it is (min,
@@ -367,6 +369,8 @@ struct PolKbn {
   using acc_t              = kbn_t;
   static constexpr int VEC = In<InT>::VEC;
   static constexpr int CLS = kClsFloat;
+  static constexpr int kMain = MAIN;
+  static constexpr int kRed  = RMI_RED_ADD;
   static constexpr int kTail = kTailZero;
 
   static __device__ __forceinline__ acc_t neutral() { return kbn_t{0.0, 0.0}; }

@@ -210,7 +210,69 @@ struct NormPlan {
   int64_t grid = 0;
   int64_t nvec = 0;
   int tail     = 0;
+  // kind 3, the flat kernel: `flat_rows` rows (ending on a 16-byte boundary) in chunks of
+  // `chunk_rows`, 2^logL lanes per row for the fold; the rows after them take another plan
+  int chunk_rows    = 0;
+  int logL          = 0;
+  int64_t flat_rows = 0;
 };
+
+// Rows that the flat kernel (normalize_flat_kernel) takes, or kind != 3 when it does not apply.
+// It needs rows of 16 bytes or more and input and output on a 16-byte boundary, and it is
+// chosen where the row-wise kernels' accesses do not fall on whole 128-byte lines, i.e. row
+// bytes that are no multiple of 128: measured over 512 MB + 512 MB, fp32 rows of 5 to 1001
+// elements 53-72 % -> 74-78.5 % of 8 TB/s (D = 129: 60 -> 76, 500: 63 -> 78), bf16 and fp16
+// rows of 9 to 2000 43-70 % -> 72-78 %, fp64 rows of 25 to 250 56-67 % -> 65-68 %.  Not chosen,
+// by the same measurements: rows of 16, 32 or 64 bytes (whole rows per power-of-two lane group:
+// 75-80 % against 70-77 %), fp64 rows below 192 bytes (-2 to -20 %), and rows so long that the
+// whole rows of a chunk fill less than 85 % of a workgroup's vector slots.
+#ifndef RMI_NORM_FLAT_MAX_ROW_BYTES
+#define RMI_NORM_FLAT_MAX_ROW_BYTES 4096
+#endif
+inline NormPlan make_flat_norm_plan(int64_t n_rows, int64_t len, int elem_bytes, const void* in,
+                                    const void* out)
+{
+  NormPlan p;
+  const int64_t rb = len * elem_bytes;
+  if (rb < 16 || rb % 128 == 0 || rb > RMI_NORM_FLAT_MAX_ROW_BYTES) return p;
+  if ((rb & (rb - 1)) == 0) return p;
+  if (elem_bytes == 8 && rb < 192) return p;
+  if (reinterpret_cast<uintptr_t>(in) % 16 != 0 || reinterpret_cast<uintptr_t>(out) % 16 != 0) return p;
+  int g = 16, r = (int)(rb % 16);
+  while (r != 0) {  // gcd(16, rb)
+    const int q = g % r;
+    g = r, r = q;
+  }
+  const int m0 = 16 / g;  // rows after which a row starts on a 16-byte boundary again
+  int chunk_rows = (int)((int64_t)kFlatMaxVec * 16 / rb / m0 * m0);
+  if (chunk_rows <= 0 || n_rows < m0) return p;
+  // a chunk that fills less than 85 % of the workgroup's 1024 vector slots leaves too many idle
+  if ((int64_t)chunk_rows * rb * 100 < (int64_t)kFlatChunkVec * 16 * 85) return p;
+  {
+    // chunks of whole 128-byte lines where that still fills the workgroup well enough: chunk
+    // edges inside a line make two workgroups read and write parts of it
+    int g128 = 128, r128 = (int)(rb % 128);
+    while (r128 != 0) {
+      const int q = g128 % r128;
+      g128 = r128, r128 = q;
+    }
+    const int m128   = 128 / g128;
+    const int aligned_rows = (int)((int64_t)kFlatMaxVec * 16 / rb / m128 * m128);
+    if (aligned_rows > 0 &&
+        (int64_t)aligned_rows * rb * 100 >= (int64_t)kFlatChunkVec * 16 * 90)
+      chunk_rows = aligned_rows;
+  }
+  const int vec_per_row = (int)((rb + 15) / 16);
+  int L = 1, logL = 0;
+  while (2 * L <= kWave && 2 * L * chunk_rows <= kBlock && 2 * L <= 2 * vec_per_row) L *= 2, ++logL;
+  p.kind       = 3;
+  p.vec16      = true;
+  p.chunk_rows = chunk_rows;
+  p.logL       = logL;
+  p.flat_rows  = n_rows - n_rows % m0;
+  p.grid       = ceildiv(p.flat_rows, (int64_t)chunk_rows);
+  return p;
+}
 
 inline NormPlan make_norm_plan(int64_t n_rows, int64_t len, int elem_bytes)
 {
@@ -288,7 +350,13 @@ int run_normalize(const NormPlan& pl, const NormArgs& args, hipStream_t st)
   a.invG     = 65536u / (unsigned)(pl.G > 0 ? pl.G : 1) + 1;
   if (pl.grid > 0x7fffffffLL) return RMI_ERR_BAD_SHAPE;
   const dim3 grid((unsigned)pl.grid);
-  if (pl.kind == 0) {
+  if (pl.kind == 3) {
+    a.n_rows        = pl.flat_rows;
+    a.chunk_rows    = pl.chunk_rows;
+    a.logL          = pl.logL;
+    a.inv_row_bytes = 1.0f / (float)a.row_bytes;
+    hipLaunchKernelGGL((normalize_flat_kernel<P>), grid, dim3(kBlock), 0, st, a);
+  } else if (pl.kind == 0) {
     if (!pl.vec16) {
       hipLaunchKernelGGL((normalize_wave_kernel<P, false>), grid, dim3(kBlock), 0, st, a);
     } else if ((a.row_bytes % 128 == 0 || (pl.L == 1 && ((kWave / pl.G) * a.row_bytes) % 128 == 0)) &&

@@ -27,6 +27,10 @@ struct NormArgs {
   int final_op;
   double init;
   double eps;
+  // flat kernel: a workgroup takes `chunk_rows` whole rows that start on a 16-byte boundary
+  int chunk_rows;
+  int logL;        // 2^logL lanes sum the partial norms of one row
+  float inv_row_bytes;
 };
 
 // Element stores, the inverse of In<T>::get.
@@ -427,6 +431,185 @@ __global__ __launch_bounds__(1024) void normalize_sweep_kernel(NormArgs a)
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u)
       if (v + (i64)u * T < nload) write_scaled<P, true, true, true>(a, orow, x[u], v + (i64)u * T, norm);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Flat kernel, for rows whose lane-loads would straddle 16-byte boundaries (row bytes no
+// multiple of 16) when input and output start on one: the matrix is read and written as a
+// flat run of ALIGNED 16-byte vectors, whatever the row length.  A workgroup takes a chunk of
+// whole rows that starts on a 16-byte boundary (a multiple of 16 / gcd(16, row bytes) rows,
+// at most 16 KB), each thread kFlatVecs vectors of it, all loaded before anything else
+// happens.  A vector holds elements of at most two rows (rows are 16 bytes or longer): every
+// thread reduces the two parts of each of its vectors and leaves them in LDS; 2^logL lanes
+// per row then fold the row's parts in vector order (fixed order: repeatable bits) and leave
+// the norm in LDS; every thread scales the elements of its vectors by their rows' norms and
+// stores the vectors whole.  Rows whose norm is <= eps must not be written: a vector that
+// touches such a row stores its other elements one by one.  In place is safe: a chunk is
+// in registers before any of it is written, and chunks do not overlap.
+// 16-bit elements take their products and the sums inside a vector in fp32 (products of
+// 8- and 11-bit significands are exact there; the sum of a vector's eight is rounded, 2^-22
+// of it at most, far below the 2^-9 / 2^-12 the outputs are rounded to), everything else in
+// the accumulator type as in the other kernels.
+// ---------------------------------------------------------------------------
+constexpr int kFlatVecs     = 4;                   // vectors per thread
+constexpr int kFlatChunkVec = kBlock * kFlatVecs;  // 1024 vector slots, 16 KB
+// Thread t takes the vectors t + 256 k - s of its chunk, s = the chunk's offset into its
+// 128-byte line in vectors (taken from the output address): every wave-wide load and store
+// instruction then covers eight whole lines, not seven and two halves that another
+// instruction completes.  The first s slots of a workgroup fall before its chunk and idle, so a
+// chunk holds up to kFlatChunkVec - 7 vectors.
+constexpr int kFlatMaxVec = kFlatChunkVec - 7;
+
+template <int MAIN>
+__device__ __forceinline__ float main_f32(float x)
+{
+  if constexpr (MAIN == RMI_MAIN_SQ) return x * x;
+  if constexpr (MAIN == RMI_MAIN_ABS) return fabsf(x);
+  return x;
+}
+template <int RED>
+__device__ __forceinline__ float red_f32(float a, float b)
+{
+  if constexpr (RED == RMI_RED_MAX) return fmaxf(a, b);
+  if constexpr (RED == RMI_RED_MIN) return fminf(a, b);
+  return a + b;
+}
+template <int RED>
+__device__ __forceinline__ float neutral_f32()
+{
+  if constexpr (RED == RMI_RED_MAX) return -__builtin_inff();
+  if constexpr (RED == RMI_RED_MIN) return __builtin_inff();
+  return 0.0f;
+}
+
+template <class P>
+__global__ __launch_bounds__(kBlock) void normalize_flat_kernel(NormArgs a)
+{
+  using in_t  = typename P::in_t;
+  using acc_t = typename P::acc_t;
+  using nat   = typename P::nat;
+  constexpr bool k16 = sizeof(in_t) == 2;
+  using part_t       = std::conditional_t<k16, float, acc_t>;
+  constexpr int VEC  = P::VEC;
+  constexpr int ES   = (int)sizeof(in_t);
+  __shared__ part_t part0[kFlatChunkVec];  // a vector's elements of the row it starts in
+  __shared__ part_t part1[kFlatChunkVec];  // ... and of the next row
+  __shared__ nat norms[kFlatChunkVec];     // a chunk has no more rows than vectors
+
+  const int t         = threadIdx.x;
+  const int rb        = (int)a.row_bytes;
+  const i64 row0      = (i64)blockIdx.x * a.chunk_rows;
+  const i64 left      = a.n_rows - row0;
+  const int rows      = left < a.chunk_rows ? (int)left : a.chunk_rows;
+  const int nvec      = (rows * rb) >> 4;  // whole vectors: the caller passes rows that end on a boundary
+  const char* base    = static_cast<const char*>(a.in) + row0 * rb;
+  char* obase         = static_cast<char*>(a.out) + row0 * rb;
+  const int shift     = (int)((reinterpret_cast<uintptr_t>(obase) >> 4) & 7);
+
+  u32x4 x[kFlatVecs];
+#pragma unroll
+  for (int k = 0; k < kFlatVecs; ++k) {  // unconditional, clamped
+    const int v = t + k * kBlock - shift;
+    x[k]        = load16(base + 16 * (i64)(v < 0 ? 0 : (v < nvec ? v : nvec - 1)));
+  }
+  int r0v[kFlatVecs], split[kFlatVecs];
+#pragma unroll
+  for (int k = 0; k < kFlatVecs; ++k) {
+    const int v = t + k * kBlock - shift;
+    const int b = 16 * (v < 0 ? 0 : v);
+    // row that byte b belongs to: b < 16384, so the float quotient is off by one at most
+    int r0 = (int)((float)b * a.inv_row_bytes);
+    if ((r0 + 1) * rb <= b) ++r0;
+    if (r0 * rb > b) --r0;
+    const int own = (r0 + 1) * rb - b;  // bytes from b on that belong to row r0
+    r0v[k]        = r0;
+    split[k]      = own < 16 ? own / ES : VEC;
+    if constexpr (k16) {
+      float s0 = neutral_f32<P::kRed>(), s1 = neutral_f32<P::kRed>();
+      static_for<VEC>([&](auto j) {
+        const float m = main_f32<P::kMain>(In<in_t>::template get<decltype(j)::value>(x[k]));
+        const bool lo = decltype(j)::value < split[k];
+        s0            = red_f32<P::kRed>(s0, lo ? m : neutral_f32<P::kRed>());
+        s1            = red_f32<P::kRed>(s1, lo ? neutral_f32<P::kRed>() : m);
+      });
+      if (v >= 0 && v < nvec) part0[v] = s0, part1[v] = s1;
+    } else {
+      acc_t s0 = P::neutral(), s1 = P::neutral();
+      static_for<VEC>([&](auto j) {
+        const nat e = In<in_t>::template get<decltype(j)::value>(x[k]);
+        if (decltype(j)::value < split[k]) P::push(s0, e, 0);
+        else P::push(s1, e, 0);
+      });
+      if (v >= 0 && v < nvec) part0[v] = s0, part1[v] = s1;
+    }
+  }
+  __syncthreads();
+  {
+    const int L    = 1 << a.logL;
+    const int c    = t & (L - 1);
+    const int step = kBlock >> a.logL;
+    const int npass = (rows + step - 1) / step;  // uniform: every lane of a group takes part in its exchanges
+    for (int pass = 0; pass < npass; ++pass) {
+      const int r  = pass * step + (t >> a.logL);
+      const int rr = r < rows ? r : rows - 1;
+      const int bs = rr * rb;
+      const int vf = bs >> 4, vl = (bs + rb - 1) >> 4;
+      acc_t acc    = P::neutral();
+      for (int v = vf + c; v <= vl; v += L) {
+        acc_t p;
+        if constexpr (k16) p = P::from_f64((double)((v == vf && (bs & 15)) ? part1[v] : part0[v]));
+        else p = (v == vf && (bs & 15)) ? part1[v] : part0[v];
+        P::merge(acc, p);
+      }
+      group_allreduce<P>(acc, L);
+      if (c == 0 && r < rows) norms[r] = row_norm<P>(a, acc);
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int k = 0; k < kFlatVecs; ++k) {
+    const int v = t + k * kBlock - shift;
+    if (v < 0 || v >= nvec) continue;
+    const int r0  = r0v[k];
+    const nat n0  = norms[r0];
+    const nat n1  = norms[r0 + 1 < rows ? r0 + 1 : r0];
+    const bool k0 = n0 <= (nat)a.eps;                       // rows that are left untouched
+    const bool k1 = split[k] < VEC && n1 <= (nat)a.eps;     // (a NaN norm is not: the row becomes NaN)
+    u32x4 y       = x[k];
+    if constexpr (k16) {
+      const float i0 = 1.0f / n0, i1 = 1.0f / n1;
+      static_for<VEC>([&](auto j) {
+        constexpr int J = decltype(j)::value;
+        Put<in_t>::template at<J>(y, In<in_t>::template get<J>(x[k]) * (J < split[k] ? i0 : i1));
+      });
+    } else {
+      const Quot<nat> q0(n0), q1(n1);
+      static_for<VEC>([&](auto j) {
+        constexpr int J = decltype(j)::value;
+        Quot<nat> q     = q0;
+        if (J >= split[k]) q = q1;
+        Put<in_t>::template at<J>(y, q(In<in_t>::template get<J>(x[k])));
+      });
+    }
+    if (!(k0 || k1)) {
+      store16<true>(obase + 16 * (i64)v, y);
+    } else {
+      in_t* o = reinterpret_cast<in_t*>(obase + 16 * (i64)v);
+      static_for<VEC>([&](auto j) {
+        constexpr int J = decltype(j)::value;
+        if (!(J < split[k] ? k0 : k1)) {
+          if constexpr (ES == 2) {
+            reinterpret_cast<uint16_t*>(o)[J] = (uint16_t)(y[J / 2] >> (16 * (J & 1)));
+          } else if constexpr (ES == 4) {
+            reinterpret_cast<u32*>(o)[J] = y[J];
+          } else {
+            reinterpret_cast<u32*>(o)[2 * J]     = y[2 * J];
+            reinterpret_cast<u32*>(o)[2 * J + 1] = y[2 * J + 1];
+          }
+        }
+      });
+    }
   }
 }
 

@@ -168,7 +168,8 @@ def round_to_16(out_dtype, values):
     best, bestd = o0.copy(), np.abs(from_bf16(b0).astype(np.float64) - v)
     for step in (-1, 1):
         c = o0 + step
-        d = np.abs(from_bf16(_bits16(c)).astype(np.float64) - v)
+        with np.errstate(invalid="ignore"):
+            d = np.abs(from_bf16(_bits16(c)).astype(np.float64) - v)
         take = np.isfinite(d) & (d < bestd)
         best, bestd = np.where(take, c, best), np.where(take, d, bestd)
     return np.where(np.isfinite(v), _bits16(best), b0).astype(np.uint16)

@@ -227,6 +227,81 @@ def test_quotients_of_tiny_elements(gpu, dt, npdt, lo_exp, hi_exp):
                                        want[got != want][:5])
 
 
+# Rows whose byte length is no multiple of 128 are normalised as a flat run of aligned
+# 16-byte vectors (a vector holds parts of two rows; chunks of whole rows per workgroup).
+# Row counts around the chunk sizes, every vector-to-row split, rows that must stay untouched
+# (norm <= eps: their neighbours in the same vector are still written), NaN rows, outputs that
+# start at every 16-byte offset into a 128-byte line, in place, and the few last rows that do
+# not end on a 16-byte boundary (they take the row-wise kernels).
+def _flat_case(dt, npdt, rows, cols, norm, in_off, out_off, inplace, seed):
+    import torch
+    from raft_amd import device as dev
+    rng = np.random.default_rng(seed)
+    m = rng.standard_normal((rows, cols)) * np.exp(rng.uniform(-2, 2, (rows, 1)))
+    if rows > 3:
+        m[rng.integers(0, rows, max(1, rows // 7))] = 0.0              # norm 0: untouched
+        m[rng.integers(0, rows, max(1, rows // 11))] *= 1e-14           # norm below eps: untouched
+    if rows > 5:
+        m[rows // 2, cols // 3] = np.nan
+    if dt == api.BF16:
+        data = u.to_bf16(m.astype(np.float32).reshape(-1))
+    else:
+        data = m.astype(npdt).reshape(-1)
+    es = data.dtype.itemsize
+    main, red, fin = NORMS[norm]
+    d = api.make_desc(dt, dt, rows, cols, main_op=main, reduce_op=red, final_op=fin)
+    nbytes = rows * cols * es
+    xbuf = torch.zeros(nbytes + 256, dtype=torch.uint8, device="cuda")
+    xbuf[in_off:in_off + nbytes] = torch.from_numpy(data.view(np.uint8)).cuda()
+    sentinel = np.full(rows * cols, 7.0, dtype=np.float32)
+    prev = u.to_bf16(sentinel) if dt == api.BF16 else sentinel.astype(npdt)
+    if inplace:
+        obuf, out_off, prev_f64 = xbuf, in_off, _as_f64(dt, data)
+    else:
+        obuf = torch.zeros(nbytes + 256, dtype=torch.uint8, device="cuda")
+        obuf[out_off:out_off + nbytes] = torch.from_numpy(prev.view(np.uint8)).cuda()
+        prev_f64 = _as_f64(dt, prev)
+    rc = api.load().rmi_row_normalize(C.byref(d), xbuf.data_ptr() + in_off, obuf.data_ptr() + out_off,
+                                      1e-6, dev.current_stream_ptr())
+    assert rc == 0, api.status_string(rc)
+    torch.cuda.synchronize()
+    got = obuf[out_off:out_off + nbytes].cpu().numpy().view(data.dtype).copy()
+    assert (obuf[:out_off] == 0).all() and (obuf[out_off + nbytes:] == 0).all(), "wrote outside the matrix"
+    exp = _oracle(d, data, prev_f64, 1e-6)
+    if dt in (api.BF16, api.F16):
+        ok = u.ulp16_ok(dt, got, exp)
+    else:
+        ok = u.approx_ok(got, exp, 1e-5 if dt == api.F32 else 1e-8)
+    assert ok.all(), (rows, cols, norm, in_off, out_off, np.argwhere(~ok)[:4])
+    if not inplace:  # untouched rows keep the output's old bits
+        keep = exp.reshape(rows, cols) == 7.0
+        assert (got.reshape(rows, cols)[keep] == prev.reshape(rows, cols)[keep]).all()
+
+
+@pytest.mark.parametrize("dt,npdt,colset", [
+    (api.F32, np.float32, (5, 9, 33, 100, 129, 250, 500, 1001)),
+    (api.BF16, None, (9, 33, 100, 130, 1004)),
+    (api.F16, np.float16, (12, 33, 500)),
+    (api.F64, np.float64, (25, 33, 65, 250))])
+def test_flat_rows(gpu, dt, npdt, colset):
+    seed = 0
+    for cols in colset:
+        es = 2 if dt in (api.BF16, api.F16) else (4 if dt == api.F32 else 8)
+        chunk = max(1, 16272 // (cols * es))
+        for rows in sorted({1, 2, 7, 8, 9, 31, chunk - 1, chunk, chunk + 1, 2 * chunk + 3, 4099}):
+            if rows < 1:
+                continue
+            seed += 1
+            _flat_case(dt, npdt, rows, cols, ("l2", "l1", "linf")[seed % 3], 0, 0, seed % 4 == 0, seed)
+
+
+@pytest.mark.parametrize("out_off", [16, 32, 48, 64, 80, 96, 112])
+def test_flat_rows_at_line_offsets(gpu, out_off):
+    for dt, npdt, cols in ((api.F32, np.float32, 129), (api.BF16, None, 33), (api.F64, np.float64, 33)):
+        _flat_case(dt, npdt, 3001, cols, "l2", (out_off * 3) % 128, out_off, False, out_off + cols)
+        _flat_case(dt, npdt, 3001, cols, "l2", out_off, out_off, True, out_off + cols + 1)
+
+
 def test_full_size_embedding_shape(gpu):
     """1,000,000 x 128 fp32 (the shape of benchmark config 2): unit L2 rows, and the
     oracle on a slice."""
