@@ -54,6 +54,8 @@ struct RowArgs {
                    // line; the workgroup that takes a row's last ticket folds its partials
                    // (nullptr: a second launch does)
   int LB;          // ... with LB lanes (a power of two <= 64), as fold_kernel would
+  int chunk_rows;  // row_flat_kernel: whole rows of a workgroup's chunk; logG: log2 of the lanes
+  float inv_row_bytes;  // ... that fold one row, and 1 / row_bytes
   Epilogue epi;
 };
 
@@ -977,6 +979,141 @@ __global__ __launch_bounds__(kBlock) void row_dense_kernel(RowArgs a)
       }
     }
     __syncthreads();
+  }
+}
+
+constexpr int kFlatVecs     = 4;                   // vectors per thread
+constexpr int kFlatChunkVec = kBlock * kFlatVecs;  // 1024 vector slots, 16 KB
+// Thread t takes the vectors t + 256 k - s of its chunk, s = the chunk's offset into its
+// 128-byte line in vectors (taken from the output address): every wave-wide load and store
+// instruction then covers eight whole lines, not seven and two halves that another
+// instruction completes.  The first s slots of a workgroup fall before its chunk and idle, so a
+// chunk holds up to kFlatChunkVec - 7 vectors.
+constexpr int kFlatMaxVec = kFlatChunkVec - 7;
+
+
+// ---------------------------------------------------------------------------
+// Flat row reduction, for rows whose length is no multiple of a 128-byte line when the
+// input starts on a 16-byte boundary.  The matrix is read as a flat run of ALIGNED 16-byte
+// vectors, whatever the row length: a workgroup takes a chunk of whole rows that starts on
+// a 16-byte boundary (a multiple of 16 / gcd(16, row bytes) rows, at most 16 KB), each
+// thread kFlatVecs vectors of it, all loaded before anything else happens.  A vector holds
+// elements of at most two rows (rows are 16 bytes or longer): every thread reduces the two
+// parts of each of its vectors and leaves them in LDS, and 2^logG lanes per row then fold the
+// row's parts in vector order (a fixed order: repeatable bits) and run the epilogue.  The
+// matrix's last vector may be a partial one: it is read as the 16 bytes that END at the
+// matrix's end and shifted down, so nothing is read past the input.
+// ---------------------------------------------------------------------------
+// mask of the bytes below s of a 32-bit word (s may be negative or beyond 4)
+__device__ __forceinline__ u32 low_bytes_mask(int s)
+{
+  return s >= 4 ? ~0u : (s <= 0 ? 0u : ((1u << (8 * s)) - 1u));
+}
+// the vector moved down by k bytes (k in 1..15), zeros moving in at the top
+__device__ __forceinline__ u32x4 shift_down_bytes(const u32x4& x, int k)
+{
+  const int wq = k >> 2, bq = k & 3;
+  u32 e[8];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    e[i] = x[i], e[i + 4] = 0u;
+  u32x4 y;
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    u32 lo = 0u, hi = 0u;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {  // a select chain: wq is a run-time value
+      if (wq == i) lo = e[w + i], hi = e[w + i + 1];
+    }
+    y[w] = bq == 0 ? lo : ((lo >> (8 * bq)) | (hi << (32 - 8 * bq)));
+  }
+  return y;
+}
+
+template <class P>
+__global__ __launch_bounds__(kBlock) void row_flat_kernel(RowArgs a)
+{
+  using in_t  = typename P::in_t;
+  using acc_t = typename P::acc_t;
+  constexpr int VEC = P::VEC;
+  constexpr int ES  = (int)sizeof(in_t);
+  static_assert(sizeof(acc_t) <= 16, "two accumulators per vector slot are kept in LDS");
+  __shared__ acc_t part0[kFlatChunkVec];  // a vector's elements of the row it starts in
+  __shared__ acc_t part1[kFlatChunkVec];  // ... and of the next row
+
+  const int t      = threadIdx.x;
+  const int rb     = (int)a.row_bytes;
+  const i64 row0   = (i64)blockIdx.x * a.chunk_rows;
+  const i64 left   = a.n_out - row0;
+  const int rows   = left < a.chunk_rows ? (int)left : a.chunk_rows;
+  const int bytes  = rows * rb;
+  const int rem    = bytes & 15;              // only the matrix's last chunk can end off a boundary
+  const int nvec   = (bytes + 15) >> 4;       // vectors of the chunk, the partial one included
+  const char* base = static_cast<const char*>(a.in) + row0 * rb;
+  const int shift  = (int)((reinterpret_cast<uintptr_t>(base) >> 4) & 7);  // see kFlatMaxVec
+
+  u32x4 x[kFlatVecs];
+#pragma unroll
+  for (int k = 0; k < kFlatVecs; ++k) {  // unconditional, clamped
+    const int v  = t + k * kBlock - shift;
+    const int vc = v < 0 ? 0 : (v < nvec ? v : nvec - 1);
+    // the partial last vector: the 16 bytes that end at the chunk's end
+    x[k] = load16((rem != 0 && vc == nvec - 1) ? base + bytes - 16 : base + 16 * (i64)vc);
+  }
+#pragma unroll
+  for (int k = 0; k < kFlatVecs; ++k) {
+    const int v = t + k * kBlock - shift;
+    const int b = 16 * (v < 0 ? 0 : v);
+    u32x4 xv    = x[k];
+    int valid   = 16;  // bytes of the vector that belong to the matrix
+    if (rem != 0 && v == nvec - 1) {
+      xv    = shift_down_bytes(xv, 16 - rem);
+      valid = rem;
+    }
+    // row that byte b belongs to: b < 16384, so the float quotient is off by one at most
+    int r0 = (int)((float)b * a.inv_row_bytes);
+    if ((r0 + 1) * rb <= b) ++r0;
+    if (r0 * rb > b) --r0;
+    const int own  = (r0 + 1) * rb - b;           // bytes from b on that belong to row r0
+    const int sb   = own < valid ? own : valid;   // bytes of part 0
+    const i64 idx0 = (b - r0 * rb) / ES;          // position in row r0 of the vector's first element
+    acc_t s0 = P::neutral(), s1 = P::neutral();
+    if constexpr (P::kTail == kTailZero) {
+      // sums: cleared elements count for nothing, each part is pushed as a whole vector
+      u32x4 lowv, highv;  // bytes [0, sb) and [sb, valid) of the vector
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        const u32 m0 = low_bytes_mask(sb - 4 * w);
+        lowv[w]      = xv[w] & m0;
+        highv[w]     = xv[w] & low_bytes_mask(valid - 4 * w) & ~m0;
+      }
+      P::push_vec(s0, lowv, idx0);
+      P::push_vec(s1, highv, 0);
+    } else {
+      static_for<VEC>([&](auto j) {
+        constexpr int J = decltype(j)::value;
+        const auto e    = In<in_t>::template get<J>(xv);
+        if (J * ES < sb) P::push(s0, e, idx0 + J);
+        else if (J * ES < valid) P::push(s1, e, (i64)J - sb / ES);
+      });
+    }
+    if (v >= 0 && v < nvec) part0[v] = s0, part1[v] = s1;
+  }
+  __syncthreads();
+  const int L     = 1 << a.logG;
+  const int c     = t & (L - 1);
+  const int step  = kBlock >> a.logG;
+  const int npass = (rows + step - 1) / step;  // uniform: every lane of a group takes part in its exchanges
+  for (int pass = 0; pass < npass; ++pass) {
+    const int r  = pass * step + (t >> a.logG);
+    const int rr = r < rows ? r : rows - 1;
+    const int bs = rr * rb;
+    const int vf = bs >> 4, vl = (bs + rb - 1) >> 4;
+    acc_t acc    = P::neutral();
+    for (int v = vf + c; v <= vl; v += L)
+      P::merge(acc, (v == vf && (bs & 15)) ? part1[v] : part0[v]);
+    group_allreduce<P>(acc, L);
+    if (c == 0 && r < rows) finish<P>(a.epi, row0 + r, acc);
   }
 }
 

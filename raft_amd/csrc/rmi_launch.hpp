@@ -65,7 +65,8 @@ int run(const PlanX& pl, const Problem& pr, hipStream_t st)
   static_assert(col_wide_bundles(1) == col_wide_bundles_of(1) && col_wide_bundles(2) == col_wide_bundles_of(2) &&
                   col_wide_bundles(3) == col_wide_bundles_of(3) && col_wide_bundles(4) == col_wide_bundles_of(4) &&
                   col_wide_bundles(5) == col_wide_bundles_of(5) && kColWideMaxSets == 5 &&
-                  kDenseSlots == kPlanDenseSlots && kDenseBundles == kPlanDenseBundles,
+                  kDenseSlots == kPlanDenseSlots && kDenseBundles == kPlanDenseBundles &&
+                  kFlatChunkVec == kPlanFlatChunkVec && kFlatMaxVec == kPlanFlatMaxVec,
                 "plan selector and wide-row column kernel must agree on rows per step");
   int rc = RMI_OK;
   switch (pl.kind) {
@@ -103,7 +104,15 @@ int run(const PlanX& pl, const Problem& pr, hipStream_t st)
           default: rc = RMI_ERR_UNSUPPORTED;
         }
       } else if (pl.kind == RMI_PLAN_ROW_WAVE && !pl.team_kernel) {
-        if (pl.dense_rows) {
+        if (pl.flat_rows) {
+          if constexpr (sizeof(typename P::in_t) == 1 && P::kTail == kTailZero) {  // the planner's rule
+            a.chunk_rows    = pl.chunk_rows;
+            a.inv_row_bytes = 1.0f / (float)pl.row_bytes;
+            hipLaunchKernelGGL((row_flat_kernel<P>), grid, dim3(kBlock), 0, st, a);
+          } else {
+            rc = RMI_ERR_UNSUPPORTED;
+          }
+        } else if (pl.dense_rows) {
           a.R = (kBlock * kDenseSlots) / pl.G;
           const size_t lds_bytes =
             (size_t)kDenseBundles * a.R * pl.G * sizeof(typename P::acc_t);  // at most 32 KB

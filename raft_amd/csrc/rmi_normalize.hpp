@@ -452,15 +452,6 @@ __global__ __launch_bounds__(1024) void normalize_sweep_kernel(NormArgs a)
 // of it at most, far below the 2^-9 / 2^-12 the outputs are rounded to), everything else in
 // the accumulator type as in the other kernels.
 // ---------------------------------------------------------------------------
-constexpr int kFlatVecs     = 4;                   // vectors per thread
-constexpr int kFlatChunkVec = kBlock * kFlatVecs;  // 1024 vector slots, 16 KB
-// Thread t takes the vectors t + 256 k - s of its chunk, s = the chunk's offset into its
-// 128-byte line in vectors (taken from the output address): every wave-wide load and store
-// instruction then covers eight whole lines, not seven and two halves that another
-// instruction completes.  The first s slots of a workgroup fall before its chunk and idle, so a
-// chunk holds up to kFlatChunkVec - 7 vectors.
-constexpr int kFlatMaxVec = kFlatChunkVec - 7;
-
 template <int MAIN>
 __device__ __forceinline__ float main_f32(float x)
 {

@@ -29,6 +29,8 @@ constexpr int kColBlocksPerCu = 2;
 constexpr int kColMaxLanes = 128;     // COL_TILE: most lanes of a workgroup along one row
 constexpr int kPlanDenseSlots   = 2;  // ROW_WAVE, dense rows: load slots per thread
 constexpr int kPlanDenseBundles = 4;  // ... and bundles of rows in flight
+constexpr int kPlanFlatChunkVec = 1024;  // ROW_WAVE, flat rows: vector slots of a workgroup
+constexpr int kPlanFlatMaxVec   = kPlanFlatChunkVec - 7;  // ... and the most vectors of its chunk
 constexpr int kColWideMaxSets = 5;    // COL_TILE, wide rows: most load slots per thread
 // row bundles in flight in the wide-row column kernel whose threads have K load slots
 constexpr int col_wide_bundles_of(int K) { return (10 + K - 1) / K; }
@@ -66,6 +68,9 @@ struct PlanX {
   bool any_g      = false;  // short_rows with G = the row's lane-load count (not a power of two)
   bool dense_rows = false;  // ROW_WAVE: G = the row's lane-load count, a workgroup's load slots
                             // dealt over whole adjacent rows, rows combined through LDS
+  bool flat_rows  = false;  // ROW_WAVE: the matrix is read as a flat run of aligned vectors, chunks
+                            // of `chunk_rows` whole rows per workgroup, 2^logG lanes fold a row
+  int chunk_rows  = 0;
   bool team_kernel = false; // served by the team-per-row kernel
   bool stage_ok    = false; // ROW_WAVE: rows could be staged through LDS
   bool staged      = false; // ROW_WAVE: rows are staged through LDS (line-aligned span reads)
@@ -517,6 +522,52 @@ inline int make_plan(const rmi_reduce_desc& d,
       p.short_rows = false;
       p.any_g      = false;
       p.G          = (int)nload;
+    }
+    // The flat kernel (row_flat_kernel): aligned 16-byte vectors whatever the row length.  It
+    // is bound by its index arithmetic and its pass through LDS at about 60 % of 8 TB/s for 2-
+    // to 8-byte elements (the lane-group plans read the same shapes at 70-88 %) and at 66-71 %
+    // for byte rows, so it serves byte sums only, and there the rows that are no whole 32-bit
+    // words, where the lane-group plans fall to 44-67 % (int8 D = 17 / 33 / 47 / 50 / 65 / 70 / 85:
+    // 49 / 44 / 55 / 56 / 58 / 60 / 59 % -> 71 / 71 / 67 / 67 / 68 / 70 / 65 %; rows of whole words keep
+    // their 75-80 %, and from 100 bytes on the lane groups win again).
+    {
+      bool flat_ok = p.vec16 && es == 1 && (key.family == kFamInt || key.family == kFamFloat) &&
+                     key.red_op == RMI_RED_ADD && (row_bytes % 4) != 0 && row_bytes <= 96 &&
+                     (in_misalign % 16) == 0 && acc_bytes <= 16 && hint == RMI_PLAN_AUTO;
+      if (flat_ok) {
+        int g = 16, r = (int)(row_bytes % 16);
+        while (r != 0) {  // gcd(16, row_bytes)
+          const int q = g % r;
+          g = r, r = q;
+        }
+        const int m0   = 16 / g;  // rows after which a row starts on a 16-byte boundary again
+        int chunk_rows = (int)((int64_t)kPlanFlatMaxVec * 16 / row_bytes / m0 * m0);
+        // a chunk that fills less than 85 % of the workgroup's vector slots leaves too many idle
+        if (chunk_rows <= 0 || (int64_t)chunk_rows * row_bytes * 100 < (int64_t)kPlanFlatChunkVec * 16 * 85)
+          flat_ok = false;
+        if (flat_ok) {
+          int g128 = 128, r128 = (int)(row_bytes % 128);
+          while (r128 != 0) {
+            const int q = g128 % r128;
+            g128 = r128, r128 = q;
+          }
+          const int m128         = 128 / g128;  // chunks of whole lines where they fill well enough
+          const int aligned_rows = (int)((int64_t)kPlanFlatMaxVec * 16 / row_bytes / m128 * m128);
+          if (aligned_rows > 0 && (int64_t)aligned_rows * row_bytes * 100 >= (int64_t)kPlanFlatChunkVec * 16 * 90)
+            chunk_rows = aligned_rows;
+          int L = 1, logL = 0;
+          while (2 * L <= 64 && 2 * L * chunk_rows <= kPlanBlock && L <= nload) L *= 2, ++logL;
+          p.flat_rows   = true;
+          p.short_rows  = false;
+          p.any_g       = false;
+          p.dense_rows  = false;
+          p.chunk_rows  = chunk_rows;
+          p.G           = L;
+          p.logG        = logL;
+          p.grid_blocks = ceildiv(p.n_out, (int64_t)chunk_rows);
+          return RMI_OK;
+        }
+      }
     }
     p.logG               = (p.any_g || p.dense_rows) ? 0 : ilog2(p.G);
     const int64_t rows_w = p.dense_rows ? 1 : (int64_t)(64 / p.G) * (p.short_rows ? kPlanUnroll : 1);

@@ -15,6 +15,7 @@ long staged_plans = 0;
 long grouped_plans = 0;
 long wide_plans = 0;
 long dense_plans = 0;
+long flat_plans = 0;
 #define REQUIRE(cond)                                                              \
   do {                                                                             \
     if (!(cond)) {                                                                 \
@@ -83,6 +84,21 @@ void check(const rmi_reduce_desc& d, int n_cu, uintptr_t in_misalign)
       REQUIRE(!p.strided);
       if (p.team_kernel) {
         REQUIRE(p.threads == 64 && p.B == 1 && p.chunk == p.nvec);
+      } else if (p.flat_rows) {
+        ++flat_plans;
+        // byte sums over rows that are no whole words: chunks of whole rows that start on a
+        // 16-byte boundary and fit the workgroup's vector slots, a power-of-two lane group per
+        // row for the fold, one workgroup per chunk
+        REQUIRE(p.vec16 && !p.short_rows && !p.any_g && !p.dense_rows && !p.staged);
+        REQUIRE(p.elem_bytes == 1 && p.row_bytes % 4 != 0 && p.row_bytes >= 17 && p.row_bytes <= 96);
+        REQUIRE(in_misalign % 16 == 0 && p.acc_bytes <= 16);
+        REQUIRE(p.chunk_rows >= 1 && ((int64_t)p.chunk_rows * p.row_bytes) % 16 == 0);
+        REQUIRE((int64_t)p.chunk_rows * p.row_bytes <= (int64_t)rmi::kPlanFlatMaxVec * 16);
+        REQUIRE((int64_t)p.chunk_rows * p.row_bytes * 100 >= (int64_t)rmi::kPlanFlatChunkVec * 16 * 85);
+        REQUIRE(p.G >= 1 && p.G <= 64 && (1 << p.logG) == p.G);
+        REQUIRE(p.G == 1 || (int64_t)p.G * p.chunk_rows <= kPlanBlock);
+        REQUIRE(p.grid_blocks * p.chunk_rows >= p.n_out && (p.grid_blocks - 1) * p.chunk_rows < p.n_out);
+        REQUIRE(p.passes == 1 && p.ws_bytes == 0 && p.lds_reserve == 0);
       } else if (p.dense_rows) {
         ++dense_plans;
         // one lane-load per load slot, whole adjacent rows per workgroup, rows met in LDS
@@ -222,6 +238,21 @@ int main()
       check(d, n_cu, mis);
     ++cases;
   }
+  // byte rows of 17 to 100 elements, the shapes the flat row plan is chosen from
+  for (int cols = 17; cols <= 100; ++cols)
+    for (int dt : {RMI_I8, RMI_U8})
+      for (int64_t rows : {(int64_t)1, (int64_t)15, (int64_t)16, (int64_t)1000, (int64_t)1 << 20, (int64_t)33554431})
+        for (uintptr_t mis : {(uintptr_t)0, (uintptr_t)16, (uintptr_t)3}) {
+          rmi_reduce_desc d{};
+          d.in_dtype  = dt;
+          d.out_dtype = rows % 2 ? RMI_I64 : RMI_F32;
+          d.main_op   = cols % 3 == 0 ? RMI_MAIN_SQ : RMI_MAIN_IDENTITY;
+          d.reduce_op = RMI_RED_ADD;
+          d.n_rows    = rows;
+          d.n_cols    = cols;
+          check(d, 256, mis);
+          ++cases;
+        }
   // the extremes the header promises to reject
   {
     rmi_reduce_desc d{};
@@ -235,10 +266,10 @@ int main()
       ++failures;
     }
   }
-  std::printf("plans checked: lanes %ld wave %ld block %ld split %ld col %ld (whole rows %ld) empty %ld, dense rows %ld\n",
+  std::printf("plans checked: lanes %ld wave %ld block %ld split %ld col %ld (whole rows %ld) empty %ld, dense rows %ld, flat rows %ld\n",
               planned[RMI_PLAN_ROW_LANES], planned[RMI_PLAN_ROW_WAVE], planned[RMI_PLAN_ROW_BLOCK],
               planned[RMI_PLAN_ROW_SPLIT], planned[RMI_PLAN_COL_TILE], wide_plans, planned[RMI_PLAN_EMPTY],
-              dense_plans);
+              dense_plans, flat_plans);
   for (int k = RMI_PLAN_ROW_LANES; k <= RMI_PLAN_EMPTY; ++k)
     if (planned[k] < 1000) {
       std::printf("  plan kind %d was hardly exercised\n", k);
@@ -254,6 +285,10 @@ int main()
   }
   if (dense_plans < 1000) {
     std::printf("  dense row plans were hardly exercised (%ld)\n", dense_plans);
+    ++failures;
+  }
+  if (flat_plans < 1000) {
+    std::printf("  flat row plans were hardly exercised (%ld)\n", flat_plans);
     ++failures;
   }
   if (staged_plans < 1000) {
