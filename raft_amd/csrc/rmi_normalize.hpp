@@ -123,6 +123,11 @@ struct Quot {
   {
     fast = fabs(divisor) >= lo && fabs(divisor) <= hi;
   }
+  // with the reciprocal RN(1 / divisor) computed elsewhere
+  __device__ __forceinline__ Quot(T divisor, T recip) : d(divisor), r(recip)
+  {
+    fast = fabs(divisor) >= lo && fabs(divisor) <= hi;
+  }
   __device__ __forceinline__ T operator()(T x) const
   {
     if (!fast || fabs(x) < lo) return x / d;
@@ -487,6 +492,10 @@ __global__ __launch_bounds__(kBlock) void normalize_flat_kernel(NormArgs a)
   __shared__ part_t part0[kFlatChunkVec];  // a vector's elements of the row it starts in
   __shared__ part_t part1[kFlatChunkVec];  // ... and of the next row
   __shared__ nat norms[kFlatChunkVec];     // a chunk has no more rows than vectors
+  // 1 / norm, computed once per row; not for fp64 rows, whose accumulators already take 32 KB
+  // of LDS: 8 KB more cost a resident workgroup and 4-6 % there
+  constexpr bool kRecips = sizeof(nat) < 8;
+  __shared__ nat recips[kRecips ? kFlatChunkVec : 1];
 
   const int t         = threadIdx.x;
   const int rb        = (int)a.row_bytes;
@@ -554,7 +563,11 @@ __global__ __launch_bounds__(kBlock) void normalize_flat_kernel(NormArgs a)
         P::merge(acc, p);
       }
       group_allreduce<P>(acc, L);
-      if (c == 0 && r < rows) norms[r] = row_norm<P>(a, acc);
+      if (c == 0 && r < rows) {
+        const nat n = row_norm<P>(a, acc);
+        norms[r]    = n;
+        if constexpr (kRecips) recips[r] = (nat)1 / n;
+      }
     }
   }
   __syncthreads();
@@ -563,19 +576,28 @@ __global__ __launch_bounds__(kBlock) void normalize_flat_kernel(NormArgs a)
     const int v = t + k * kBlock - shift;
     if (v < 0 || v >= nvec) continue;
     const int r0  = r0v[k];
+    const int r1  = r0 + 1 < rows ? r0 + 1 : r0;
     const nat n0  = norms[r0];
-    const nat n1  = norms[r0 + 1 < rows ? r0 + 1 : r0];
+    const nat n1  = norms[r1];
+    const nat i0  = kRecips ? recips[r0] : (nat)1 / n0;
+    const nat i1  = kRecips ? recips[r1] : (nat)1 / n1;
     const bool k0 = n0 <= (nat)a.eps;                       // rows that are left untouched
     const bool k1 = split[k] < VEC && n1 <= (nat)a.eps;     // (a NaN norm is not: the row becomes NaN)
     u32x4 y       = x[k];
     if constexpr (k16) {
-      const float i0 = 1.0f / n0, i1 = 1.0f / n1;
-      static_for<VEC>([&](auto j) {
-        constexpr int J = decltype(j)::value;
-        Put<in_t>::template at<J>(y, In<in_t>::template get<J>(x[k]) * (J < split[k] ? i0 : i1));
+      // two products rounded to 16 bits (nearest even) and packed by one conversion
+      typedef float f32x2 __attribute__((ext_vector_type(2)));
+      using half_t = std::conditional_t<std::is_same_v<in_t, bf16_t>, __bf16, _Float16>;
+      typedef half_t h16x2 __attribute__((ext_vector_type(2)));
+      static_for<VEC / 2>([&](auto w) {
+        constexpr int W = decltype(w)::value;
+        f32x2 p;
+        p[0] = In<in_t>::template get<2 * W>(x[k]) * (2 * W < split[k] ? i0 : i1);
+        p[1] = In<in_t>::template get<2 * W + 1>(x[k]) * (2 * W + 1 < split[k] ? i0 : i1);
+        y[W] = __builtin_bit_cast(u32, __builtin_convertvector(p, h16x2));
       });
     } else {
-      const Quot<nat> q0(n0), q1(n1);
+      const Quot<nat> q0(n0, i0), q1(n1, i1);
       static_for<VEC>([&](auto j) {
         constexpr int J = decltype(j)::value;
         Quot<nat> q     = q0;
