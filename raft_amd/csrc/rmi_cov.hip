@@ -59,11 +59,30 @@ int make_cov_plan(int dtype, int layout, int64_t N, int64_t D, CovPlan& p)
 
 bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 
+// Matrices of 4, 8, 16 or 32 columns whose row count is a multiple of f = 64 / D are contracted
+// as matrices of 64 columns and N / f rows: every load and every matrix instruction then does
+// useful work, where a 64-column block with masked columns reads 20M x 32 floats at 55 % of the
+// rate of 10M x 64 (20M x 32: 572 -> 383 us, 40M x 16: 934 -> 386 us, fp64 10M x 32: 874 -> 525 us).
+// It costs one more small launch, so matrices below 4M elements stay as they are (32768 x 32:
+// 14 us against 17.6).  Returns f, or 1.
+int fold_factor(int64_t N, int64_t D)
+{
+  if (D != 4 && D != 8 && D != 16 && D != 32) return 1;
+  const int f = (int)(cov::kBlockCols / D);
+  return (N % f == 0 && N * D >= ((int64_t)1 << 22)) ? f : 1;
+}
+constexpr size_t kWideBytes = (size_t)cov::kBlockCols * cov::kBlockCols * sizeof(double);
+
 template <class T>
-int launch(const CovPlan& pl, int layout, int64_t N, int64_t D, int sample, bool center, T* data,
+int launch(const CovPlan& pl, int layout, int64_t N_in, int64_t D_in, int sample, bool center, T* data,
            const T* mu, T* covar, void* ws, hipStream_t st)
 {
+  // `pl` is the plan of the matrix as it is contracted: N / f rows of 64 columns when folded
+  const int fold  = fold_factor(N_in, D_in);
+  const int64_t N = N_in / fold, D = D_in * fold;
   cov::GramArgs g{};
+  g.mu_div = layout == RMI_ROW_MAJOR ? 1 : fold;
+  g.mu_mod = fold > 1 ? (int)D_in : 0;
   g.data    = data;
   g.mu      = mu;
   g.partial = ws;
@@ -131,10 +150,20 @@ int launch(const CovPlan& pl, int layout, int64_t N, int64_t D, int sample, bool
   f.S        = pl.S;
   f.permuted = layout == RMI_ROW_MAJOR ? 1 : 0;
   // the reference's scalar: Type(1) / Type(N - 1 | N), handed to the GEMM in Type
-  f.alpha = N == 0 ? 0.0 : (double)(T(1) / (sample ? T(N - 1) : T(N)));  // no rows: zeros, as a GEMM with k = 0
+  f.alpha = N_in == 0 ? 0.0 : (double)(T(1) / (sample ? T(N_in - 1) : T(N_in)));  // no rows: zeros, as a GEMM with k = 0
+  // folded: the 64 x 64 sums go to the workspace behind the partials, then their diagonal blocks
+  // are added up into the D x D result
+  double* wide = fold > 1 ? reinterpret_cast<double*>(static_cast<char*>(ws) + pl.ws_bytes) : nullptr;
+  f.wide       = wide;
   hipLaunchKernelGGL((cov::cov_fold_kernel<T>),
                      dim3((unsigned)(pl.npairs * cov::kTilesPerPair * (cov::kTile / cov::kFoldElems))),
                      dim3(cov::kFoldElems * cov::kFoldSplit), 0, st, f);
+  if (fold > 1) {
+    const int cells = (int)(D_in * D_in);
+    hipLaunchKernelGGL((cov::cov_blocks_kernel<T>), dim3((unsigned)((cells + cov::kThreads - 1) / cov::kThreads)),
+                       dim3(cov::kThreads), 0, st, wide, covar, (int)D_in, fold,
+                       layout == RMI_ROW_MAJOR ? 1 : 0);
+  }
   return hipGetLastError() == hipSuccess ? RMI_OK : RMI_ERR_LAUNCH;
 }
 
@@ -146,8 +175,9 @@ extern "C" {
 size_t rmi_cov_workspace_bytes(int dtype, int layout, int64_t n_rows, int64_t n_cols)
 {
   rmi::CovPlan pl;
-  if (rmi::make_cov_plan(dtype, layout, n_rows, n_cols, pl) != RMI_OK) return 0;
-  return n_cols > 0 ? pl.ws_bytes : 0;
+  const int fold = rmi::fold_factor(n_rows, n_cols);
+  if (rmi::make_cov_plan(dtype, layout, n_rows / fold, n_cols * fold, pl) != RMI_OK) return 0;
+  return n_cols > 0 ? pl.ws_bytes + (fold > 1 ? rmi::kWideBytes : 0) : 0;
 }
 
 int rmi_cov(int dtype,
@@ -166,14 +196,16 @@ int rmi_cov(int dtype,
   using namespace rmi;
   if ((flags & ~RMI_COV_CENTER_DATA) != 0) return RMI_ERR_BAD_ENUM;
   CovPlan pl;
-  const int rc = make_cov_plan(dtype, layout, n_rows, n_cols, pl);
+  const int fold = fold_factor(n_rows, n_cols);
+  const int rc   = make_cov_plan(dtype, layout, n_rows / fold, n_cols * fold, pl);
   if (rc != RMI_OK) return rc;
   if (n_cols == 0) return RMI_OK;
   if (covar == nullptr) return RMI_ERR_NULL;
   if (n_rows > 0 && data == nullptr) return RMI_ERR_NULL;
   const size_t es = dtype == RMI_F32 ? 4 : 8;
   if (!aligned(data, es) || !aligned(mu, es) || !aligned(covar, es)) return RMI_ERR_ALIGNMENT;
-  if (workspace == nullptr || workspace_bytes < pl.ws_bytes || !aligned(workspace, 16))
+  if (workspace == nullptr || workspace_bytes < pl.ws_bytes + (fold > 1 ? kWideBytes : 0) ||
+      !aligned(workspace, 16))
     return RMI_ERR_WORKSPACE;
   hipStream_t st    = static_cast<hipStream_t>(stream);
   const bool center = (flags & RMI_COV_CENTER_DATA) != 0;

@@ -95,7 +95,16 @@ struct GramArgs {
   int npairs;        // nb * (nb + 1) / 2
   int S;             // slabs
   int total;         // S * npairs workgroups do work; the grid is rounded up to 8
+  // A matrix of 4, 8, 16 or 32 columns is contracted as one of 64: f = 64 / D consecutive rows
+  // (row-major) or the f pieces of a column (col-major) side by side.  Column c of the wide
+  // matrix then has the mean mu[(c / mu_div) % mu_mod]; mu_mod == 0: mu[c].
+  int mu_div;
+  int mu_mod;
 };
+__device__ __forceinline__ int64_t mean_index(const GramArgs& a, int64_t c)
+{
+  return a.mu_mod == 0 ? c : (c / a.mu_div) % a.mu_mod;
+}
 
 struct FoldArgs {
   const void* partial;
@@ -106,6 +115,8 @@ struct FoldArgs {
   int S;
   int permuted;      // tiles hold the columns {4 m + ja} x {4 n + jb} (row-major kernel)
   double alpha;      // 1 / (N - 1) or 1 / N, rounded to T as the reference's scalar is
+  double* wide;      // not null: the scaled sums go here as [D][D] doubles instead of `out`
+                     // (the 64-column contraction of a narrower matrix, see cov_blocks_kernel)
 };
 
 // Four elements at any element-aligned address (gfx950 serves unaligned vector loads).
@@ -238,7 +249,7 @@ __device__ __forceinline__ void gram_rows_body(const GramArgs& a, int unit, int 
     for (int j = 0; j < 4; ++j) {
       ok[s][j]   = c0 + j < D;
       col[s][j]  = ok[s][j] ? c0 + j : 0;
-      mean[s][j] = (mu != nullptr && ok[s][j]) ? mu[col[s][j]] : T(0);
+      mean[s][j] = (mu != nullptr && ok[s][j]) ? mu[mean_index(a, col[s][j])] : T(0);
     }
   }
 
@@ -511,7 +522,7 @@ __device__ __forceinline__ void gram_rows_body_bf16(const GramArgs& a, int unit,
     for (int j = 0; j < 4; ++j) {
       ok[s][j]   = c0 + j < D;
       col[s][j]  = ok[s][j] ? c0 + j : 0;
-      mean[s][j] = (mu != nullptr && ok[s][j]) ? mu[col[s][j]] : T(0);
+      mean[s][j] = (mu != nullptr && ok[s][j]) ? mu[mean_index(a, col[s][j])] : T(0);
     }
   }
 
@@ -694,7 +705,7 @@ __device__ __forceinline__ void gram_cols_body_bf16(const GramArgs& a, int unit,
       const int64_t c = (int64_t)(s == 0 ? bi : bj) * kBlockCols + 16 * gq + cl;
       ok[s][gq]       = c < a.D;
       colp[s][gq]     = data + (ok[s][gq] ? c : 0) * N;
-      mean[s][gq]     = (mu != nullptr && ok[s][gq]) ? mu[c] : T(0);
+      mean[s][gq]     = (mu != nullptr && ok[s][gq]) ? mu[mean_index(a, c)] : T(0);
     }
   }
 
@@ -908,7 +919,7 @@ __device__ __forceinline__ void gram_cols_body(const GramArgs& a, int unit, int 
       const int64_t c = (int64_t)(s == 0 ? bi : bj) * kBlockCols + 16 * gq + cl;
       ok[s][gq]       = c < a.D;
       colp[s][gq]     = data + (ok[s][gq] ? c : 0) * N;
-      mean[s][gq]     = (mu != nullptr && ok[s][gq]) ? mu[c] : T(0);
+      mean[s][gq]     = (mu != nullptr && ok[s][gq]) ? mu[mean_index(a, c)] : T(0);
     }
   }
 
@@ -1100,10 +1111,38 @@ __global__ __launch_bounds__(kFoldElems* kFoldSplit) void cov_fold_kernel(FoldAr
   // last bit: its upper half is kept and mirrored like every other tile, so the result is
   // symmetric bit for bit.
   if (bi == bj && ta == tb && r > c) return;
+  if (a.wide != nullptr) {
+    a.wide[r * a.D + c] = sum * a.alpha;
+    if (r != c) a.wide[c * a.D + r] = sum * a.alpha;
+    return;
+  }
   const T val = (T)(sum * a.alpha);
   T* out      = static_cast<T*>(a.out);
   out[r * a.D + c] = val;
   if (r != c) out[c * a.D + r] = val;
+}
+
+// A matrix of D = 64 / f columns contracted as one of 64 (f consecutive rows side by side,
+// row-major; the f pieces of every column side by side, col-major): its covariance is the sum
+// of the f diagonal D x D blocks of the wide result (row-major: rows and columns b D + r; col-
+// major: r f + b), summed in block order in f64 and rounded once.  One thread per element of
+// the upper half; the lower half is its mirror.
+template <class T>
+__global__ __launch_bounds__(kThreads) void cov_blocks_kernel(const double* wide, T* out, int D, int f,
+                                                              int row_major)
+{
+  const int i = blockIdx.x * kThreads + threadIdx.x;
+  if (i >= D * D) return;
+  const int r = i / D, c = i - r * D;
+  if (r > c) return;
+  double sum = 0.0;
+  for (int b = 0; b < f; ++b) {
+    const int wr = row_major ? b * D + r : r * f + b;
+    const int wc = row_major ? b * D + c : c * f + b;
+    sum += wide[wr * kBlockCols + wc];
+  }
+  out[r * D + c] = (T)sum;
+  if (r != c) out[c * D + r] = (T)sum;
 }
 
 // ---------------------------------------------------------------------------

@@ -90,7 +90,13 @@ def test_known_answer(dt):
 
 
 SHAPES = [(1, 1), (2, 3), (3, 2), (15, 5), (16, 4), (17, 63), (31, 64), (33, 65), (100, 100),
-          (257, 129), (1000, 130), (4099, 200), (513, 260), (64, 8), (5000, 66)]
+          (257, 129), (1000, 130), (4099, 200), (513, 260), (64, 8), (5000, 66),
+          (2, 32), (1000, 32), (1001, 32), (4096, 16), (40, 8), (96, 4)]
+
+# 4, 8, 16 or 32 columns and 4M elements or more: contracted as 64 columns when the row count is
+# a multiple of 64 / D, as they are otherwise
+NARROW = [(131072, 32), (131073, 32), (262144, 16), (262148, 16), (262146, 16), (524288, 8),
+          (524292, 8), (1048576, 4), (1048592, 4), (1048577, 4)]
 
 
 @pytest.mark.parametrize("dt", [api.F32, api.F64])
@@ -102,6 +108,16 @@ def test_ragged_shapes(dt, layout, center):
         m = (rng.normal(3.0, 2.0, (rows, cols)) * rng.uniform(0.25, 4.0, cols)).astype(NP[dt])
         for sample in ((False, True) if rows > 1 else (False,)):
             _check(dt, layout, rows, cols, sample, m, center)
+
+
+@pytest.mark.parametrize("dt", [api.F32, api.F64])
+@pytest.mark.parametrize("layout", [api.ROW_MAJOR, api.COL_MAJOR])
+@pytest.mark.parametrize("center", [False, True])
+def test_narrow_matrices(dt, layout, center):
+    rng = np.random.default_rng(21 + dt + 10 * layout)
+    for rows, cols in NARROW:
+        m = (rng.normal(1.0, 2.0, (rows, cols)) * rng.uniform(0.25, 4.0, cols)).astype(NP[dt])
+        _check(dt, layout, rows, cols, rows % 2 == 0, m, center)
 
 
 @pytest.mark.parametrize("layout", [api.ROW_MAJOR, api.COL_MAJOR])
