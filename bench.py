@@ -486,10 +486,10 @@ def main():
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) / 200 * 1e3
 
-    def extra_row_normalize():
+    def extra_row_normalize(rows=1000000, cols=128):
         # the step after config 2 in an embedding pipeline: x / ||x||_2 per row, same
-        # matrix shape; algorithmic bytes = matrix read once + written once
-        rows, cols = 1000000, 128
+        # matrix shape; algorithmic bytes = matrix read once + written once.  With 129
+        # columns the rows are no multiple of a cache line and the flat kernel takes them.
         xs = [mk_normal(rows, cols, 2 + 7919 * i) for i in range(3)]
         os_ = [torch.empty_like(x) for x in xs]
         d = api.make_desc(api.F32, api.F32, rows, cols, main_op=api.MAIN_SQ, final_op=api.FIN_SQRT)
@@ -510,7 +510,7 @@ def main():
         ms = e0.elapsed_time(e1) / n
         nb = 2 * rows * cols * 4
         norms = torch.linalg.vector_norm(os_[0].view(rows, cols).double(), dim=1)
-        return dict(workload="row_normalize L2 fp32 1000000x128 (read + write)", ms_per_step=ms,
+        return dict(workload=f"row_normalize L2 fp32 {rows}x{cols} (read + write)", ms_per_step=ms,
                     alg_bytes=nb, GBps=nb / (ms * 1e-3) / 1e9,
                     pct_of_peak=100.0 * nb / (ms * 1e-3) / 1e9 / PEAK_HBM_GBPS,
                     check={"unit_rows": bool(torch.allclose(norms, torch.ones_like(norms), atol=1e-6))})
@@ -693,7 +693,8 @@ def main():
         torch.cuda.empty_cache()
 
     head = results[HEADLINE]
-    extras = ({"row_normalize": extra_row_normalize(), "meanvar": extra_meanvar(),
+    extras = ({"row_normalize": extra_row_normalize(), "row_normalize_129": extra_row_normalize(1000000, 129),
+               "meanvar": extra_meanvar(),
                "wide_columns": extra_wide_columns(), "dense_rows": extra_dense_rows(),
                "cov": extra_cov()}
               if args.configs == "all" else {})

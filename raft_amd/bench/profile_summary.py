@@ -199,6 +199,8 @@ def extras(out: Path, commit: str):
     w(f"{'workload':50s} {'kernel':58s} {'calls':>5s} {'avg us':>8s} {'alg MB':>8s} {'GB/s':>6s} {'%peak':>6s}")
     work = [("row_normalize L2 fp32 1000000x128 (read + write)", "normalize_wave_kernel<rmi::PolF<float, 1, 0>", None,
              1024000000),
+            ("row_normalize L2 fp32 1000000x129 (flat kernel)", "normalize_flat_kernel<rmi::PolF<float, 1, 0>", None,
+             2 * 1000000 * 129 * 4),
             ("meanvar fp32 10000000x64 row-major (one read)", "col_kernel<rmi::PolMeanVar<float>",
              "fold_kernel<rmi::PolMeanVar<float>", 2560000512),
             ("column sum fp32 32768x4097 (whole rows)", "col_wide_kernel<rmi::PolF<float, 0, 0>",
