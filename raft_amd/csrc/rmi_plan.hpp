@@ -565,6 +565,7 @@ inline int make_plan(const rmi_reduce_desc& d,
           p.G           = L;
           p.logG        = logL;
           p.grid_blocks = ceildiv(p.n_out, (int64_t)chunk_rows);
+          if (p.grid_blocks > 0x7fffffffLL) return RMI_ERR_BAD_SHAPE;
           return RMI_OK;
         }
       }
