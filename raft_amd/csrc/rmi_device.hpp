@@ -275,6 +275,9 @@ __device__ __forceinline__ void static_for(F&& f)
 // reference's per-thread Kahan-Babuska-Neumaier compensation
 // (linalg/detail/coalesced_reduction-inl.cuh:37-46) at a third of the ALU cost.
 template <class InT, int MAIN, int RED>
+struct PolI;
+
+template <class InT, int MAIN, int RED>
 struct PolF {
   using in_t               = InT;
   using nat                = typename In<InT>::nat;
@@ -306,8 +309,22 @@ struct PolF {
   {
     a = red(a, main_f64<MAIN>((double)x));
   }
+  // Sums of bytes into a floating output: the terms are small integers, so a vector is folded
+  // in 32-bit integer arithmetic (the dot-product instructions of PolI) and column terms gather
+  // in 32-bit accumulators; both are exact, and so is every f64 sum of them below 2^53.
+  static constexpr bool kBytes     = sizeof(InT) == 1 && RED == RMI_RED_ADD;
+  static constexpr bool kColNarrow = kBytes;
+  static constexpr int kColFlush   = 128;
+  static __device__ __forceinline__ void push_cols_narrow(int32_t (&a)[VEC], const u32x4& v)
+  {
+    static_for<VEC>([&](auto j) { a[j] += main_i32<MAIN>((int32_t)In<InT>::template get<j>(v)); });
+  }
   static __device__ __forceinline__ void push_vec(acc_t& a, const u32x4& v, i64)
   {
+    if constexpr (kBytes) {
+      a += (double)PolI<InT, MAIN, RMI_RED_ADD>::vec_i32(v);
+      return;
+    }
     // Pairwise tree inside the vector (fixed order, so results do not depend
     // on the launch plan's scheduling), then one dependent step into `a`.
     double t[VEC];

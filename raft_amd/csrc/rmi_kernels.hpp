@@ -1134,10 +1134,13 @@ __global__ __launch_bounds__(kBlock) void row_flat_kernel(RowArgs a)
 // At the end the bundle's rows are combined through LDS in row order, and the partials are
 // stored [B][n_out], whole lines per workgroup; the epilogue is left to the second pass.
 // ---------------------------------------------------------------------------
+// (byte sums gather in 32-bit accumulators, see PolI::kColNarrow: four slots instead of two;
+// the launch keeps the terms per slot below 2^17, so that nothing overflows)
 template <class P>
 constexpr int col_wide_sets()
 {
-  constexpr int k = 256 / (P::VEC * (int)sizeof(typename P::acc_t));
+  constexpr int acc = col_narrow<P>::value ? 4 : (int)sizeof(typename P::acc_t);
+  constexpr int k   = 256 / (P::VEC * acc);
   return k < 1 ? 1 : (k > 5 ? 5 : k);
 }
 constexpr int col_wide_bundles(int K) { return (10 + K - 1) / K; }
@@ -1150,8 +1153,10 @@ __global__ __launch_bounds__(kBlock) void col_wide_kernel(ColArgs a)
   constexpr int S = P::VEC;
   constexpr int K = col_wide_sets<P>();
   constexpr int R = col_wide_bundles(K);
+  constexpr bool NARROW = col_narrow<P>::value;
+  using slot_t          = std::conditional_t<NARROW, int32_t, acc_t>;  // what a slot accumulates in
   extern __shared__ __align__(16) unsigned char col_wide_lds[];
-  acc_t* sm       = reinterpret_cast<acc_t*>(col_wide_lds);  // [rows of a bundle][nload * S]
+  slot_t* sm      = reinterpret_cast<slot_t*>(col_wide_lds);  // [rows of a bundle][nload * S]
   const int t     = threadIdx.x;
   const int piece = a.TX;  // lane-loads of this workgroup's piece of a row (the whole row
                            // when it fits the slots), the last piece may hold fewer
@@ -1175,12 +1180,18 @@ __global__ __launch_bounds__(kBlock) void col_wide_kernel(ColArgs a)
     live[k]          = (int)q < rb && lane[k] < nload;
     off[k]           = live[k] ? (i64)q * a.row_bytes + offset_of(l0 + lane[k]) : offset_of(l0);
   }
-  acc_t acc[K][S];
+  slot_t acc[K][S];
 #pragma unroll
   for (int k = 0; k < K; ++k)
 #pragma unroll
-    for (int j = 0; j < S; ++j)
-      acc[k][j] = P::neutral();
+    for (int j = 0; j < S; ++j) {
+      if constexpr (NARROW) acc[k][j] = 0;
+      else acc[k][j] = P::neutral();
+    }
+  auto push = [&](slot_t (&s)[S], const u32x4& v, i64 row) __attribute__((always_inline)) {
+    if constexpr (NARROW) P::push_cols_narrow(s, v);
+    else P::push_cols(s, v, row);
+  };
 
   const char* inb  = static_cast<const char*>(a.in);
   const i64 step   = (i64)R * rb;  // rows per step
@@ -1200,14 +1211,14 @@ __global__ __launch_bounds__(kBlock) void col_wide_kernel(ColArgs a)
     for (int q = 0; q < R; ++q)
 #pragma unroll
       for (int k = 0; k < K; ++k)
-        P::push_cols(acc[k], x[q][k], r + (i64)q * rb + sub[k]);
+        push(acc[k], x[q][k], r + (i64)q * rb + sub[k]);
   }
   // the rows after the last whole step go to the workgroup whose turn it is, bundle by bundle
   for (; r < a.len; r += rb) {
 #pragma unroll
     for (int k = 0; k < K; ++k)
       if (live[k] && r + sub[k] < a.len)
-        P::push_cols(acc[k], load16(inb + r * a.row_bytes + off[k]), r + sub[k]);
+        push(acc[k], load16(inb + r * a.row_bytes + off[k]), r + sub[k]);
   }
 
   const int width = nload * S;
@@ -1227,9 +1238,9 @@ __global__ __launch_bounds__(kBlock) void col_wide_kernel(ColArgs a)
     // the last, partial lane-load holds the row's last S columns; its first S - tail are
     // already covered by the lane-load before it
     if (l == a.nvec && j < S - a.tail) continue;
-    acc_t v = sm[idx];
+    acc_t v = (acc_t)sm[idx];
     for (int q = 1; q < rb; ++q)
-      P::merge(v, sm[q * width + idx]);
+      P::merge(v, (acc_t)sm[q * width + idx]);
     out[l < a.nvec ? l * S + j : a.n_out - S + j] = v;
   }
 }

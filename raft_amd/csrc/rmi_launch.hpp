@@ -173,12 +173,12 @@ int run(const PlanX& pl, const Problem& pr, hipStream_t st)
       }
       const dim3 grid((unsigned)pl.gridx, (unsigned)pl.B);
       if (pl.wide > 0) {
-        if constexpr (P::CLS != kClsFloat) {
-          return RMI_ERR_UNSUPPORTED;  // planned for plain and compensated floating sums only
+        if constexpr (P::CLS != kClsFloat && !col_narrow<P>::value) {
+          return RMI_ERR_UNSUPPORTED;  // planned for floating sums and byte sums only
         } else {
           if (col_wide_sets<P>() != pl.wide) return RMI_ERR_UNSUPPORTED;
-          const size_t lds_bytes =
-            (size_t)pl.TY * pl.TX * P::VEC * sizeof(typename P::acc_t);  // at most 64 KB
+          const size_t lds_bytes = (size_t)pl.TY * pl.TX * P::VEC *
+                                   (col_narrow<P>::value ? 4 : sizeof(typename P::acc_t));  // at most 64 KB
           hipLaunchKernelGGL((col_wide_kernel<P>), grid, dim3(kBlock), lds_bytes, st, a);
           FoldArgs f{};
           f.partial = partials_of(pr.ws);

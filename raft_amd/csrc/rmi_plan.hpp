@@ -344,9 +344,16 @@ inline int make_plan(const rmi_reduce_desc& d,
     // 4097: 67 / 78, 8191: 71 / 77, 11000: 66 / 81, 14000: 67 / 78, 22000: 66 / 79, 50000: 70 / 77,
     // 200000: 66 / 72 (640 and 1024: 84 / 81 and 82 / 81); fp64 D = 300: 76 / 82, 1025: 67 / 82,
     // 4097: 61 / 80, 8191: 70 / 79; bf16 D = 1030: 72 / 80, 10000: 62 / 72, 16400: 59 / 75.
+    // Byte sums gather in 32-bit accumulators here (four slots per thread), which bounds the
+    // rows a slot may see: a term is at most 2^14, so 100000 of them stay below 2^31.
+#ifndef RMI_COL_WIDE_BYTES
+#define RMI_COL_WIDE_BYTES 1
+#endif
+    const bool byte_sums = RMI_COL_WIDE_BYTES != 0 && (key.family == kFamInt || key.family == kFamFloat) &&
+                           es == 1 && key.red_op == RMI_RED_ADD;
     if (p.group == 0 && p.vec16 && lanes > kColMaxLanes &&
-        (key.family == kFamFloat || key.family == kFamKbn)) {
-      int K = 256 / (p.step * acc_bytes);
+        (key.family == kFamFloat || key.family == kFamKbn || byte_sums)) {
+      int K = 256 / (p.step * (byte_sums ? 4 : acc_bytes));
       K     = K < 1 ? 1 : (K > kColWideMaxSets ? kColWideMaxSets : K);
       const int64_t slots = (int64_t)kPlanBlock * K;
       const int64_t cuts  = ceildiv(lanes, slots);
@@ -357,7 +364,13 @@ inline int make_plan(const rmi_reduce_desc& d,
         const int64_t B      = (int64_t)n_cu / cuts;
         const size_t ws      = kTicketBytes + (size_t)p.n_out * B * acc_bytes;
         const bool too_large = (d.flags & kFlagSmallWorkspace) != 0 && ws > RMI_NOALLOC_SCRATCH_BYTES;
-        if (rows >= B * step * 16 && !too_large) {
+        // (byte sums have 1024 slots and no room to deal them finely: rows that use less than
+        // three quarters of them, or that are whole multiples of 64 lane-loads, keep the layout
+        // above: int8 D = 8200 / 16400 / 20000 lose 9-18 % here, 4096 / 8192 3-4 %, while D =
+        // 2100 / 3000 / 4100 / 5000 / 50000 go from 60-70 % to 70-74 %)
+        const bool bytes_ok = !byte_sums || (rows <= 100000 * B * bundle && bundle * piece * 4 >= slots * 3 &&
+                                             (lanes % 64 != 0 || p.tail > 0));
+        if (rows >= B * step * 16 && !too_large && bytes_ok) {
           p.wide        = K;
           p.TX          = (int)piece;
           p.TY          = (int)bundle;

@@ -151,15 +151,24 @@ void check(const rmi_reduce_desc& d, int n_cu, uintptr_t in_misalign)
         // threads hold TY adjacent rows of TX lane-loads, more than half of them in use, in at
         // most 64 KB of LDS at the end; no more workgroups than CUs
         const int64_t slots = (int64_t)kPlanBlock * p.wide;
-        REQUIRE(p.wide >= 1 && p.wide <= rmi::kColWideMaxSets && p.wide * p.step * p.acc_bytes <= 256);
-        REQUIRE(key.family == rmi::kFamFloat || key.family == rmi::kFamKbn);
+        // byte sums gather in 32-bit slot accumulators: terms of at most 2^14, at most 100000
+        // of them per slot, and rows that fill three quarters of the slots
+        const bool byte_sums = p.elem_bytes == 1 && d.reduce_op == RMI_RED_ADD &&
+                               (key.family == rmi::kFamInt || key.family == rmi::kFamFloat);
+        const int slot_bytes = byte_sums ? 4 : p.acc_bytes;
+        REQUIRE(p.wide >= 1 && p.wide <= rmi::kColWideMaxSets && p.wide * p.step * slot_bytes <= 256);
+        REQUIRE(key.family == rmi::kFamFloat || key.family == rmi::kFamKbn || byte_sums);
+        if (byte_sums) {
+          REQUIRE(p.wide == 4 && (int64_t)p.TY * p.TX * 4 >= slots * 3);
+          REQUIRE(p.len <= (int64_t)100000 * p.B * p.TY && (nload % 64 != 0 || p.tail > 0));
+        }
         REQUIRE(p.group == 0 && p.vec16 && nload > rmi::kColMaxLanes && p.TX <= slots);
         REQUIRE(p.gridx >= 1 && p.gridx <= n_cu && p.gridx * p.TX >= nload && (p.gridx - 1) * p.TX < nload);
         REQUIRE(p.gridx == (nload + slots - 1) / slots);
         if (p.gridx > 1) REQUIRE(nload % 64 != 0 || p.tail > 0);
         REQUIRE(p.TY >= 1 && (int64_t)p.TY * p.TX <= slots && (int64_t)(p.TY + 1) * p.TX > slots);
         REQUIRE((int64_t)p.TY * p.TX * 2 > slots);
-        REQUIRE((int64_t)p.TY * p.TX * p.step * p.acc_bytes <= 65536);
+        REQUIRE((int64_t)p.TY * p.TX * p.step * slot_bytes <= 65536);
         REQUIRE(p.B == n_cu / p.gridx && p.B >= 1 && p.grid_blocks == p.B * p.gridx && p.grid_blocks <= n_cu);
         REQUIRE(p.passes == 2);
         REQUIRE(p.len >= (int64_t)p.B * p.TY * rmi::col_wide_bundles_of(p.wide) * 16);

@@ -751,6 +751,12 @@ def _whole_row_rows(lanes, slots_per_thread, bundles):
     (api.F64, api.F64, dict(reduce_op=api.RED_MIN, init_f=np.inf), 5, 2, (301, 1281)),
     (api.BF16, api.F32, {}, 4, 3, (1025, 1030, 2056, 5500, 8191, 8192)),
     (api.F16, api.F32, dict(main_op=api.MAIN_ABS), 4, 3, (1100, 2741)),
+    # byte sums: 32-bit slot accumulators, rows that fill three quarters of the 1024 slots
+    (api.I8, api.I64, {}, 4, 3, (2100, 2730, 3000, 4100, 5000, 12300, 16000)),
+    (api.I8, api.I32, dict(main_op=api.MAIN_SQ), 4, 3, (4100, 13000)),
+    (api.U8, api.I64, dict(main_op=api.MAIN_NZ), 4, 3, (2500, 5001)),
+    (api.I8, api.F32, dict(main_op=api.MAIN_ABS), 4, 3, (3001, 4100)),
+    (api.U8, api.F16, dict(final_op=api.FIN_MUL_CONST, final_scalar=1e-4), 4, 3, (4099,)),
 ])
 @pytest.mark.parametrize("extra,shift,col_major,inplace", [(0, 0, False, False), (37, 1, False, True),
                                                            (5, 0, True, False)])
