@@ -783,19 +783,65 @@ __device__ __forceinline__ void gram_cols_body_bf16(const GramArgs& a, int unit,
   };
 
   if constexpr (DIAG) {
-    // pipelined as in gram_rows_body_bf16
-    constexpr int PD = kPipeRing;
+    // Pipelined as in gram_rows_body_bf16.  The operand layout (lane = column, the lane groups
+    // four runs of eight rows) makes a load instruction touch 64 lines, 16 bytes of each; the
+    // units are therefore loaded in a coalesced layout instead (eight consecutive lanes read the
+    // 128 bytes that a column has in the unit, eight columns per instruction) and turned into
+    // the operand layout through the wave's own piece of LDS when they are split (10M x 64:
+    // 458 -> 440 us; what is left to the row-major kernel's 380 us goes with the number of
+    // columns, i.e. of streams 40 MB apart that every wave reads side by side).
+    constexpr int PD      = kPipeRing;
+    constexpr int kColLds = 128 + 16;  // bytes of a column in LDS: its 32 rows and a pad
+    __shared__ __align__(16) char turn_lds[kWaves][kBlockCols * kColLds];
+    char* const turn = turn_lds[wave];
+    const int c8     = lane >> 3;  // coalesced layout: column 8 i + c8 of load i ...
+    const int p8     = lane & 7;   // ... rows 4 p8 .. + 3 of the unit
+    const T* cop[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int64_t c = (int64_t)bi * kBlockCols + 8 * i + c8;
+      cop[i]          = data + ((FULL || c < a.D) ? c : 0) * N + 4 * p8;
+    }
+    auto load_unit_co = [&](Quad<T> (&x)[8], int64_t q) __attribute__((always_inline)) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        x[i] = load_quad<T, STREAM>(cop[i] + q * UR);
+    };
+    auto turn_unit = [&](Quad<T> (&x)[NS][4][2], const Quad<T> (&c)[8]) __attribute__((always_inline)) {
+      typedef T full_t __attribute__((ext_vector_type(4)));
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        full_t v;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          v[j] = c[i].v[j];
+        *reinterpret_cast<full_t*>(turn + (8 * i + c8) * kColLds + 16 * p8) = v;
+      }
+#pragma unroll
+      for (int gq = 0; gq < 4; ++gq)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const full_t v = *reinterpret_cast<const full_t*>(turn + (16 * gq + cl) * kColLds + 16 * (2 * g + h));
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            x[0][gq][h].v[j] = v[j];
+        }
+    };
     if (K > 0) {
-      Quad<T> ring[PD][NS][4][2];
+      Quad<T> ring[PD][8];
 #pragma unroll
       for (int i = 0; i < PD; ++i) {
-        load_unit(ring[i], gw + (i < K ? i : K - 1) * G, false);
+        load_unit_co(ring[i], gw + (i < K ? i : K - 1) * G);
         __builtin_amdgcn_sched_barrier(0);
       }
       Split3 ops[2][NS][4];
-      split_unit(ops[0], ring[0], gw, true, false);
+      {
+        Quad<T> x[NS][4][2];
+        turn_unit(x, ring[0]);
+        split_unit(ops[0], x, gw, true, false);
+      }
       __builtin_amdgcn_sched_barrier(0);
-      load_unit(ring[0], gw + (PD < K ? PD : K - 1) * G, false);
+      load_unit_co(ring[0], gw + (PD < K ? PD : K - 1) * G);
       __builtin_amdgcn_sched_barrier(0);
       // a trip of PD units; `all_live`: none of its units is past the wave's last one
       auto trip = [&](int64_t k0, auto all_live) __attribute__((always_inline)) {
@@ -804,11 +850,13 @@ __device__ __forceinline__ void gram_cols_body_bf16(const GramArgs& a, int unit,
           const int64_t k = k0 + i;
           const int slot  = (i + 1) % PD;
           const bool live = decltype(all_live)::value || k + 1 < K;
-          split_unit(ops[(i + 1) & 1], ring[slot], gw + (k + 1) * G, live, false);
+          Quad<T> x[NS][4][2];
+          turn_unit(x, ring[slot]);
+          split_unit(ops[(i + 1) & 1], x, gw + (k + 1) * G, live, false);
           mma_unit_bf16<true>(acc, ops[i & 1][0], ops[i & 1][0]);
           interleave_split_with_mma();
           __builtin_amdgcn_sched_barrier(0);
-          load_unit(ring[slot], gw + (k + 1 + PD < K ? k + 1 + PD : K - 1) * G, false);
+          load_unit_co(ring[slot], gw + (k + 1 + PD < K ? k + 1 + PD : K - 1) * G);
           __builtin_amdgcn_sched_barrier(0);
         }
         flush_tiles(total, acc);
