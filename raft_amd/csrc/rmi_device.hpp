@@ -576,6 +576,41 @@ struct PolKvp {
     const KeyT k0 = (KeyT)idx0;
     static_for<VEC>([&](auto j) { take(a, (KeyT)(k0 + j), In<InT>::template get<j>(v)); });
   }
+  // A batch of vectors that a lane holds in registers is scanned from its highest index down.
+  // Every candidate's key is then below the holder's, so the rule shrinks to "not worse"
+  // (`>=` for arg-max): a compare and two selects per element where `take` needs seven
+  // instructions, and the key that travels is the element's slot in the batch, a constant of
+  // the instruction.  An element met twice (the overlapping last vector of a row) is harmless
+  // as long as the last visits go down in index.  The batch's winner then enters the
+  // accumulator under the full rule; a batch of NaNs only has no winner (slot -1).
+  struct scan_t {
+    int slot;
+    val_t value;
+  };
+  static __device__ __forceinline__ scan_t scan_begin() { return scan_t{-1, neutral().value}; }
+  template <int SLOT0>
+  static __device__ __forceinline__ void scan_vec(scan_t& s, const u32x4& v)
+  {
+    static_for<VEC>([&](auto jj) {
+      constexpr int j = VEC - 1 - decltype(jj)::value;
+      const val_t x   = In<InT>::template get<j>(v);
+      const bool win  = IS_MAX ? (x >= s.value) : (x <= s.value);
+      s.value         = win ? x : s.value;
+      s.slot          = win ? SLOT0 + j : s.slot;
+    });
+  }
+  // `key`: the index of the element in slot s.slot.  FRESH: the accumulator is known to be the
+  // neutral one, which the winner replaces.
+  template <bool FRESH = false>
+  static __device__ __forceinline__ void scan_end(acc_t& a, const scan_t& s, KeyT key)
+  {
+    const KeyT k = s.slot < 0 ? kKeyMax : key;
+    if constexpr (FRESH) {
+      a = acc_t{k, s.value};
+    } else {
+      take(a, k, s.value);
+    }
+  }
   static __device__ __forceinline__ void push_cols(acc_t (&a)[VEC], const u32x4& v, i64 idx)
   {
     static_for<VEC>([&](auto j) { take(a[j], (KeyT)idx, In<InT>::template get<j>(v)); });

@@ -161,6 +161,29 @@ struct Held {
   }
 };
 
+// Policies that scan a batch of vectors downwards (P::scan_t, see PolKvp).
+template <class P, class = void>
+struct scans_batches : std::false_type {};
+template <class P>
+struct scans_batches<P, std::void_t<typename P::scan_t>> : std::true_type {};
+
+// The vectors x[u] with live(u) of one lane's batch into the accumulator; base(u) is the index
+// of the first element of x[u] along the row, and rises with u.
+template <class P, bool FRESH, int N, class Live, class Base>
+__device__ __forceinline__ void scan_batch(typename P::acc_t& acc, const u32x4 (&x)[N], Live live, Base base)
+{
+  typename P::scan_t s = P::scan_begin();
+  static_for<N>([&](auto uu) {
+    constexpr int u = N - 1 - decltype(uu)::value;
+    if (live(u)) P::template scan_vec<u * P::VEC>(s, x[u]);
+  });
+  static_assert((P::VEC & (P::VEC - 1)) == 0, "slots split into vector and element by shifts");
+  constexpr int kLogVec = P::VEC == 1 ? 0 : P::VEC == 2 ? 1 : P::VEC == 4 ? 2 : P::VEC == 8 ? 3 : 4;
+  static_assert((1 << kLogVec) == P::VEC, "vectors of 1 to 16 elements");
+  const int u = s.slot < 0 ? 0 : s.slot >> kLogVec;
+  P::template scan_end<FRESH>(acc, s, (decltype(acc.key))(base(u) + (s.slot & (P::VEC - 1))));
+}
+
 // Accumulator held by lane `src` of the wave (ds_bpermute, word by word).
 template <class P>
 __device__ __forceinline__ typename P::acc_t shfl_acc(const typename P::acc_t& a, int src)
@@ -279,9 +302,15 @@ __device__ __forceinline__ void last_batch(typename P::acc_t& acc, const char* r
     const IdxT vl = v + u * stride < end ? v + u * stride : end - 1;
     x[u]          = H::load_any(rp, vl, nvec, len);
   }
+  if constexpr (VEC16 && scans_batches<P>::value) {
+    scan_batch<P, false>(
+      acc, x, [&](int u) { return v + u * stride < end; },
+      [&](int u) { return v + u * stride < (IdxT)nvec ? (i64)(v + u * stride) * P::VEC : len - P::VEC; });
+  } else {
 #pragma unroll
-  for (int u = 0; u < N; ++u)
-    if (v + u * stride < end) H::push_any(acc, x[u], v + u * stride, nvec, len, tail);
+    for (int u = 0; u < N; ++u)
+      if (v + u * stride < end) H::push_any(acc, x[u], v + u * stride, nvec, len, tail);
+  }
 }
 
 // n = 1 .. 4 lane-loads per lane, wave-uniform
@@ -337,7 +366,15 @@ __global__ __launch_bounds__(kBlock) void row_short_kernel(RowArgs a)
 #pragma unroll
   for (int t = 0; t < kUnroll; ++t) {
     acc[t] = P::neutral();
-    if (incol && row[t] < a.n_out) H::push_any(acc[t], x[t], c, a.nvec, a.len, a.tail);
+    if constexpr (VEC16 && scans_batches<P>::value) {
+      const u32x4 one[1] = {x[t]};
+      const bool live    = incol && row[t] < a.n_out;
+      scan_batch<P, true>(
+        acc[t], one, [&](int) { return live; },
+        [&](int) { return c < a.nvec ? (i64)c * P::VEC : a.len - P::VEC; });
+    } else {
+      if (incol && row[t] < a.n_out) H::push_any(acc[t], x[t], c, a.nvec, a.len, a.tail);
+    }
   }
   const i64 wave_row0 = wid * kUnroll * R;
   if constexpr (ANYG) {
@@ -464,9 +501,14 @@ __global__ __launch_bounds__(kBlock) void row_wave_kernel(RowArgs a)
         const i64 v = c + u * G < nvec ? c + u * G : nvec - 1;  // clamped, not masked: see above
         x[u]        = *reinterpret_cast<const u32x4*>(rp + v * 16);
       }
+      if constexpr (scans_batches<P>::value) {
+        scan_batch<P, true>(
+          acc, x, [&](int u) { return c + u * G < nvec; }, [&](int u) { return (i64)(c + u * G) * S; });
+      } else {
 #pragma unroll
-      for (int u = 0; u < kUnroll; ++u)
-        if (c + u * G < nvec) P::push_vec(acc, x[u], (i64)(c + u * G) * S);
+        for (int u = 0; u < kUnroll; ++u)
+          if (c + u * G < nvec) P::push_vec(acc, x[u], (i64)(c + u * G) * S);
+      }
     }
   } else if (row < a.n_out) {
     const char* rp = static_cast<const char*>(a.in) + row * a.row_bytes;
@@ -481,9 +523,14 @@ __global__ __launch_bounds__(kBlock) void row_wave_kernel(RowArgs a)
 #pragma unroll
       for (int u = 0; u < kUnroll; ++u)
         x[u] = H::load(rp, v + u * G);
+      if constexpr (VEC16 && scans_batches<P>::value) {
+        scan_batch<P, false>(
+          acc, x, [](int) { return true; }, [&](int u) { return (v + u * G) * S; });
+      } else {
 #pragma unroll
-      for (int u = 0; u < kUnroll; ++u)
-        H::push(acc, x[u], (v + u * G) * S);
+        for (int u = 0; u < kUnroll; ++u)
+          H::push(acc, x[u], (v + u * G) * S);
+      }
     }
     const i64 nload = nvec + (a.tail > 0 ? 1 : 0);  // the tail is one more lane-load
     // the last batch: what is left of the row, up to kUnroll lane-loads per lane; the
@@ -595,9 +642,14 @@ __global__ __launch_bounds__(1024) void row_block_kernel(RowArgs a)
 #pragma unroll
         for (int u = 0; u < W; ++u)
           x[u] = H::load(rp, vb + t + (i64)u * T);
+        if constexpr (VEC16 && scans_batches<P>::value) {
+          scan_batch<P, false>(
+            acc, x, [](int) { return true; }, [&](int u) { return (vb + t + (i64)u * T) * S; });
+        } else {
 #pragma unroll
-        for (int u = 0; u < W; ++u)
-          H::push(acc, x[u], (vb + t + (i64)u * T) * S);
+          for (int u = 0; u < W; ++u)
+            H::push(acc, x[u], (vb + t + (i64)u * T) * S);
+        }
       }
     }
     // Whole batches of U lane-loads; the next batch is issued before the current one is
@@ -617,9 +669,14 @@ __global__ __launch_bounds__(1024) void row_block_kernel(RowArgs a)
           for (int u = 0; u < U; ++u)
             y[u] = H::load(rp, vn + t + (i64)u * T);
         }
+        if constexpr (VEC16 && scans_batches<P>::value) {
+          scan_batch<P, false>(
+            acc, x, [](int) { return true; }, [&](int u) { return (vb + t + (i64)u * T) * S; });
+        } else {
 #pragma unroll
-        for (int u = 0; u < U; ++u)
-          H::push(acc, x[u], (vb + t + (i64)u * T) * S);
+          for (int u = 0; u < U; ++u)
+            H::push(acc, x[u], (vb + t + (i64)u * T) * S);
+        }
         vb = vn;
         if (!more) break;
 #pragma unroll
@@ -962,7 +1019,14 @@ __global__ __launch_bounds__(kBlock) void row_dense_kernel(RowArgs a)
 #pragma unroll
       for (int k = 0; k < K; ++k) {
         acc_t v = P::neutral();
-        H::push_any(v, x[q][k], lane[k], a.nvec, a.len, a.tail);
+        if constexpr (scans_batches<P>::value) {
+          const u32x4 one[1] = {x[q][k]};
+          scan_batch<P, true>(
+            v, one, [](int) { return true; },
+            [&](int) { return lane[k] < a.nvec ? (i64)lane[k] * P::VEC : a.len - P::VEC; });
+        } else {
+          H::push_any(v, x[q][k], lane[k], a.nvec, a.len, a.tail);
+        }
         if (live[k]) sm[q * width + k * kBlock + t] = v;
       }
     __syncthreads();

@@ -395,6 +395,54 @@ def test_argmax_ties_and_specials(gpu, plan, cols):
     assert np.array_equal(keys, raw["key"])
 
 
+# Short rows (lane groups, the any-G and dense layouts, the overlapping last vector) scan a
+# lane's batch from its highest index down with a shortened rule: ties inside and across
+# vectors and in the row's tail, rows of NaN only, rows of the neutral value only (the lowest
+# index below the init's key wins, core/operators.hpp:187-203 applied element after element),
+# and an init whose key is not 0.
+@pytest.mark.parametrize("in_dt,out_dt", [(api.F32, api.KVP_I32_F32), (api.F64, api.KVP_I64_F64),
+                                          (api.BF16, api.KVP_I32_F32)])
+@pytest.mark.parametrize("red", [api.RED_ARGMAX, api.RED_ARGMIN])
+def test_arg_short_rows_specials(gpu, in_dt, out_dt, red):
+    is_max = red == api.RED_ARGMAX
+    worst = -np.inf if is_max else np.inf
+    best = 100.0 if is_max else -100.0
+    for cols in (5, 9, 17, 33, 37, 48, 62, 66, 100, 129, 130, 200, 300, 515, 1000):
+        rng = np.random.default_rng(cols * 2 + int(is_max))
+        rows = 700
+        m = np.round(rng.standard_normal((rows, cols)) * 4).astype(np.float64)   # many ties
+        for r in range(rows):
+            kind = r % 10
+            if kind == 0:      # the best value twice in the row's last elements
+                m[r, cols - 1] = m[r, max(0, cols - 3)] = best
+            elif kind == 1:    # ... in adjacent vectors
+                c = int(rng.integers(0, cols))
+                m[r, c] = m[r, min(cols - 1, c + 4)] = best
+            elif kind == 2:    # NaN only: the init stays
+                m[r, :] = np.nan
+            elif kind == 3:    # the neutral value only: index 0 beats the init's key
+                m[r, :] = worst
+            elif kind == 4:    # NaN, then the neutral value from some index on
+                c = int(rng.integers(0, cols))
+                m[r, :c] = np.nan
+                m[r, c:] = worst
+            elif kind == 5:    # NaN scattered over ordinary values
+                m[r, rng.random(cols) < 0.3] = np.nan
+            elif kind == 6:    # the best value in the first and in the last element
+                m[r, 0] = m[r, cols - 1] = best
+        flat = m.reshape(-1)
+        data = {api.F32: lambda: flat.astype(np.float32), api.F64: lambda: flat,
+                api.BF16: lambda: u.to_bf16(flat.astype(np.float32))}[in_dt]()
+        for init_i, init_f in ((0, worst), (7, worst), (3, 0.0)):
+            d = api.make_desc(in_dt, out_dt, rows, cols, main_op=api.MAIN_KVP, reduce_op=red,
+                              init_i=init_i, init_f=init_f)
+            raw = u.check_against_oracle(d, data, label=f"arg specials {rows}x{cols} init {init_i}")
+            if init_f == worst:
+                keys = raw["key"]
+                assert all(int(keys[r]) == init_i for r in range(2, rows, 10))          # NaN only
+                assert all(int(keys[r]) == 0 for r in range(3, rows, 10))               # neutral only
+
+
 # Arg reduction along the strided dimension (the reference restricts KVP outputs to the
 # contiguous dimension, linalg/strided_reduction.cuh:70-77; here it is supported).
 def test_kvp_strided(gpu):
