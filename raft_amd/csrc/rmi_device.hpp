@@ -615,6 +615,17 @@ struct PolKvp {
   {
     static_for<VEC>([&](auto j) { take(a[j], (KeyT)idx, In<InT>::template get<j>(v)); });
   }
+  // The same for a thread that walks DOWN the rows of its columns: every accumulator is the
+  // neutral one or holds a key above `idx`.
+  static __device__ __forceinline__ void push_cols_down(acc_t (&a)[VEC], const u32x4& v, i64 idx)
+  {
+    static_for<VEC>([&](auto j) {
+      const val_t x  = In<InT>::template get<j>(v);
+      const bool win = IS_MAX ? (x >= a[j].value) : (x <= a[j].value);
+      a[j].value     = win ? x : a[j].value;
+      a[j].key       = win ? (KeyT)idx : a[j].key;
+    });
+  }
   static __device__ __forceinline__ void merge(acc_t& a, const acc_t& b) { take(a, b.key, b.value); }
   template <int SEL>
   static __device__ __forceinline__ acc_t exchange(const acc_t& a)

@@ -786,6 +786,8 @@ __global__ __launch_bounds__(kBlock) void col_kernel(ColArgs a)
   constexpr bool NARROW = VEC16 && col_narrow<P>::value;
   // mean-and-variance accumulators: shift set once, count added once (see PolMeanVar)
   constexpr bool SHIFTED = VEC16 && P::CLS == kClsMeanVar;
+  // arg-reductions walk the rows downwards, where their rule takes three instructions, not seven
+  constexpr bool DOWN = VEC16 && scans_batches<P>::value;
   constexpr int W = kBlock / kWave;
   __shared__ acc_t sm[W * kWave * S];
 
@@ -829,6 +831,9 @@ __global__ __launch_bounds__(kBlock) void col_kernel(ColArgs a)
         }
       };
       i64 steps = 0;  // SHIFTED: vectors folded by the loop
+      // DOWN: the workgroup's tiles are dealt from the matrix's last whole tile backwards and a
+      // tile's rows are folded last to first, so a thread meets falling row indices throughout
+      auto tile_at = [&](i64 tl) { return DOWN ? n_full - 1 - tl : tl; };
       auto load_tile = [&](u32x4 (&v)[kColUnroll], i64 tl) {
 #pragma unroll
         for (int u = 0; u < kColUnroll; ++u)
@@ -846,6 +851,10 @@ __global__ __launch_bounds__(kBlock) void col_kernel(ColArgs a)
           for (int u = 0; u < kColUnroll; ++u)
             P::cols_steps(acc, v[u]);
           steps += kColUnroll;
+        } else if constexpr (DOWN) {
+#pragma unroll
+          for (int u = kColUnroll - 1; u >= 0; --u)
+            P::push_cols_down(acc, v[u], tl * RT + ty + (i64)u * TY);
         } else {
 #pragma unroll
           for (int u = 0; u < kColUnroll; ++u)
@@ -853,7 +862,7 @@ __global__ __launch_bounds__(kBlock) void col_kernel(ColArgs a)
         }
       };
       if (tile < n_full) {
-        load_tile(x, tile);
+        load_tile(x, tile_at(tile));
         if constexpr (SHIFTED) P::cols_set_shift(acc, x[0]);
       }
       // The next tile's loads are issued before the current tile is folded.  (Two register
@@ -863,8 +872,8 @@ __global__ __launch_bounds__(kBlock) void col_kernel(ColArgs a)
       while (tile < n_full) {
         const i64 next = tile + a.B;
         u32x4 y[kColUnroll];
-        if (next < n_full) load_tile(y, next);
-        fold_tile(x, tile);
+        if (next < n_full) load_tile(y, tile_at(next));
+        fold_tile(x, tile_at(tile));
 #pragma unroll
         for (int u = 0; u < kColUnroll; ++u)
           x[u] = y[u];
@@ -1256,26 +1265,39 @@ __global__ __launch_bounds__(kBlock) void col_wide_kernel(ColArgs a)
     if constexpr (NARROW) P::push_cols_narrow(s, v);
     else P::push_cols(s, v, row);
   };
+  // arg-reductions: the workgroup's whole steps are dealt from the matrix's last one backwards
+  // and a step's bundles are folded last to first, so a slot meets falling row indices
+  constexpr bool DOWN = !NARROW && scans_batches<P>::value;
 
-  const char* inb  = static_cast<const char*>(a.in);
-  const i64 step   = (i64)R * rb;  // rows per step
-  const i64 stride = (i64)a.B * step;
-  i64 r            = (i64)blockIdx.y * step;
+  const char* inb   = static_cast<const char*>(a.in);
+  const i64 step    = (i64)R * rb;  // rows per step
+  const i64 stride  = (i64)a.B * step;
+  const i64 n_steps = DOWN ? a.len / step : 0;
+  i64 r             = (i64)blockIdx.y * step;
   for (; r + step <= a.len; r += stride) {
+    const i64 r0 = DOWN ? (n_steps - 1) * step - r : r;  // the step's first row
     u32x4 x[R][K];
 #pragma unroll
     for (int q = 0; q < R; ++q)
 #pragma unroll
       for (int k = 0; k < K; ++k)
-        x[q][k] = load16(inb + (r + (i64)q * rb) * a.row_bytes + off[k]);
+        x[q][k] = load16(inb + (r0 + (i64)q * rb) * a.row_bytes + off[k]);
     // all of the step's loads first: left to itself the scheduler trades loads in flight for
     // registers and issues four or five of the ten before the first use
     __builtin_amdgcn_sched_barrier(0);
+    if constexpr (DOWN) {
 #pragma unroll
-    for (int q = 0; q < R; ++q)
+      for (int q = R - 1; q >= 0; --q)
 #pragma unroll
-      for (int k = 0; k < K; ++k)
-        push(acc[k], x[q][k], r + (i64)q * rb + sub[k]);
+        for (int k = 0; k < K; ++k)
+          P::push_cols_down(acc[k], x[q][k], r0 + (i64)q * rb + sub[k]);
+    } else {
+#pragma unroll
+      for (int q = 0; q < R; ++q)
+#pragma unroll
+        for (int k = 0; k < K; ++k)
+          push(acc[k], x[q][k], r0 + (i64)q * rb + sub[k]);
+    }
   }
   // the rows after the last whole step go to the workgroup whose turn it is, bundle by bundle
   for (; r < a.len; r += rb) {

@@ -456,6 +456,49 @@ def test_kvp_strided(gpu):
     assert int(raw["key"][3]) == 17
 
 
+# Columns walk their rows downwards with the shortened rule: ties between far rows, in the
+# rows after the last whole tile and in one tile, columns of NaN only and of the neutral value
+# only, an init whose key is not 0; narrow matrices, whole-row layouts and wide rows.
+@pytest.mark.parametrize("in_dt,out_dt", [(api.F32, api.KVP_I32_F32), (api.F64, api.KVP_I64_F64)])
+@pytest.mark.parametrize("red", [api.RED_ARGMAX, api.RED_ARGMIN])
+@pytest.mark.parametrize("rows,cols", [(20011, 5), (9001, 33), (6007, 130), (2503, 600),
+                                       (1201, 2049), (4099, 4100)])
+def test_arg_columns_specials(gpu, in_dt, out_dt, red, rows, cols):
+    is_max = red == api.RED_ARGMAX
+    worst = -np.inf if is_max else np.inf
+    best = 100.0 if is_max else -100.0
+    rng = np.random.default_rng(rows + cols + int(is_max))
+    m = np.round(rng.standard_normal((rows, cols)) * 4).astype(np.float64)   # many ties
+    for c in range(cols):
+        kind = c % 8
+        if kind == 0:      # the best value in two far rows
+            r = np.sort(rng.choice(rows, size=2, replace=False))
+            m[r, c] = best
+        elif kind == 1:    # ... in the last rows of the matrix
+            m[rows - 1, c] = m[rows - 2, c] = best
+        elif kind == 2:    # NaN only
+            m[:, c] = np.nan
+        elif kind == 3:    # the neutral value only
+            m[:, c] = worst
+        elif kind == 4:    # NaN, then the neutral value from some row on
+            r = int(rng.integers(0, rows))
+            m[:r, c] = np.nan
+            m[r:, c] = worst
+        elif kind == 5:    # NaN scattered
+            m[rng.random(rows) < 0.3, c] = np.nan
+        elif kind == 6:    # the best value in adjacent rows
+            r = int(rng.integers(0, rows - 1))
+            m[r, c] = m[r + 1, c] = best
+    data = m.reshape(-1).astype(np.float32) if in_dt == api.F32 else m.reshape(-1)
+    for init_i, init_f in ((0, worst), (7, worst)):
+        d = api.make_desc(in_dt, out_dt, rows, cols, apply=api.ALONG_COLUMNS, main_op=api.MAIN_KVP,
+                          reduce_op=red, init_i=init_i, init_f=init_f)
+        raw = u.check_against_oracle(d, data, label=f"arg columns {rows}x{cols} init {init_i}")
+        keys = raw["key"]
+        assert all(int(keys[c]) == init_i for c in range(2, cols, 8))   # NaN only
+        assert all(int(keys[c]) == 0 for c in range(3, cols, 8))        # the neutral value only
+
+
 # Inputs whose device address is not 16-byte aligned take the element-wise load path.
 @pytest.mark.parametrize("in_dt,out_dt", [(api.F32, api.F32), (api.I8, api.I64),
                                           (api.BF16, api.F32), (api.F64, api.F64)])
