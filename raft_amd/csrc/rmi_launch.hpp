@@ -173,8 +173,8 @@ int run(const PlanX& pl, const Problem& pr, hipStream_t st)
       }
       const dim3 grid((unsigned)pl.gridx, (unsigned)pl.B);
       if (pl.wide > 0) {
-        if constexpr (P::CLS != kClsFloat && !col_narrow<P>::value) {
-          return RMI_ERR_UNSUPPORTED;  // planned for floating sums and byte sums only
+        if constexpr (P::CLS != kClsFloat && P::CLS != kClsKvp && !col_narrow<P>::value) {
+          return RMI_ERR_UNSUPPORTED;  // planned for floating sums, arg-reductions and byte sums only
         } else {
           if (col_wide_sets<P>() != pl.wide) return RMI_ERR_UNSUPPORTED;
           const size_t lds_bytes = (size_t)pl.TY * pl.TX * P::VEC *

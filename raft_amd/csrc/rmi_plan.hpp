@@ -335,10 +335,12 @@ inline int make_plan(const rmi_reduce_desc& d,
     // workgroup would share a CU and finish last: 3 pieces x 86 workgroups ran 15 % slower than
     // the layout above, 3 x 85 run 20 % faster).  Taken when every workgroup gets sixteen steps
     // or more (4096 x 4097 floats lose 16 % with eight).  Accumulators whose step is
-    // arithmetic-bound at four waves per CU (arg-reductions 33-38 % slower, byte sums 25 %)
+    // arithmetic-bound at four waves per CU (byte sums in 64-bit accumulators: 25 % slower)
     // keep the layout above, and so do rows of several pieces that are whole multiples of 64
     // whole lane-loads, its best case (fp32 D = 32768 / 65536: 80 / 83 % there, 76 / 75 % this
-    // way).
+    // way).  Arg-reductions were such accumulators (33-38 % slower here) until they walked
+    // their rows downwards; now fp32 arg-max D = 1000 / 2049 / 4097 / 10000 runs 72 / 70 / 71 /
+    // 73 % there and 75 / 75 / 73 / 72 % this way.
     // Measured at 512 MB, % of 8 TB/s, the layout above / this one: fp32 D = 513: 76 / 81,
     // 768: 74 / 82, 1025: 70 / 80, 1536: 73 / 82, 2049: 66 / 80, 3000: 65 / 78, 4096: 72 / 81,
     // 4097: 67 / 78, 8191: 71 / 77, 11000: 66 / 81, 14000: 67 / 78, 22000: 66 / 79, 50000: 70 / 77,
@@ -352,7 +354,7 @@ inline int make_plan(const rmi_reduce_desc& d,
     const bool byte_sums = RMI_COL_WIDE_BYTES != 0 && (key.family == kFamInt || key.family == kFamFloat) &&
                            es == 1 && key.red_op == RMI_RED_ADD;
     if (p.group == 0 && p.vec16 && lanes > kColMaxLanes &&
-        (key.family == kFamFloat || key.family == kFamKbn || byte_sums)) {
+        (key.family == kFamFloat || key.family == kFamKbn || key.family == kFamKvp || byte_sums)) {
       int K = 256 / (p.step * (byte_sums ? 4 : acc_bytes));
       K     = K < 1 ? 1 : (K > kColWideMaxSets ? kColWideMaxSets : K);
       const int64_t slots = (int64_t)kPlanBlock * K;

@@ -157,7 +157,8 @@ void check(const rmi_reduce_desc& d, int n_cu, uintptr_t in_misalign)
                                (key.family == rmi::kFamInt || key.family == rmi::kFamFloat);
         const int slot_bytes = byte_sums ? 4 : p.acc_bytes;
         REQUIRE(p.wide >= 1 && p.wide <= rmi::kColWideMaxSets && p.wide * p.step * slot_bytes <= 256);
-        REQUIRE(key.family == rmi::kFamFloat || key.family == rmi::kFamKbn || byte_sums);
+        REQUIRE(key.family == rmi::kFamFloat || key.family == rmi::kFamKbn || key.family == rmi::kFamKvp ||
+                byte_sums);
         if (byte_sums) {
           REQUIRE(p.wide == 4 && (int64_t)p.TY * p.TX * 4 >= slots * 3);
           REQUIRE(p.len <= (int64_t)100000 * p.B * p.TY && (nload % 64 != 0 || p.tail > 0));

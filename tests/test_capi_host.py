@@ -220,8 +220,9 @@ def test_column_plans_of_wide_rows():
     """Floating sums, max and min down rows of more than 128 lane-loads: whole adjacent rows
     per workgroup (one workgroup per CU of the 256 a build host is planned for, one set of
     partials each, a second pass), rows beyond 1280 lane-loads in the fewest equal pieces;
-    byte sums likewise where their rows fill three quarters of the 1024 slots; arg-reductions,
-    short matrices and whole multiples of 64 lane-loads in several pieces keep the other layout;
+    byte sums likewise where their rows fill three quarters of the 1024 slots, arg-reductions
+    too; short matrices and whole multiples of 64 lane-loads in several pieces keep the other
+    layout;
     the library's own descriptor flag is refused."""
     lib = api.load()
     q = lambda rows, cols, in_dt=api.F32, out_dt=api.F32, **kw: api.plan_query(
@@ -236,7 +237,8 @@ def test_column_plans_of_wide_rows():
     assert q(8191, 4097).grid_blocks != 256              # fewer than sixteen steps per workgroup
     assert q(4096, 32768).grid_blocks > 256              # 8192 whole lane-loads: pieces of 64 lanes
     kvp = dict(main_op=api.MAIN_KVP, reduce_op=api.RED_ARGMAX)
-    assert q(32768, 4097, api.F32, api.KVP_I32_F32, **kvp).grid_blocks > 256
+    p = q(32768, 4097, api.F32, api.KVP_I32_F32, **kvp)
+    assert (p.passes, p.grid_blocks, p.blocks_per_out) == (2, 256, 256)
     p = q(131072, 4100, api.I8, api.I64)                 # 257 lane-loads, three rows per bundle
     assert (p.kind, p.passes, p.grid_blocks, p.blocks_per_out) == (api.PLAN_COL_TILE, 2, 256, 256)
     assert q(131072, 4100, api.I8, api.F32).grid_blocks == 256
