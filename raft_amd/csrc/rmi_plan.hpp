@@ -34,6 +34,10 @@ constexpr int kPlanFlatMaxVec   = kPlanFlatChunkVec - 7;  // ... and the most ve
 constexpr int kColWideMaxSets = 5;    // COL_TILE, wide rows: most load slots per thread
 // row bundles in flight in the wide-row column kernel whose threads have K load slots
 constexpr int col_wide_bundles_of(int K) { return (10 + K - 1) / K; }
+#ifndef RMI_COL_GROUP_OFF_WORDS
+#define RMI_COL_GROUP_OFF_WORDS 1
+#endif
+constexpr int64_t kGroupMaxRowBytes = 130;  // COL_TILE: longest row that is read in groups
 constexpr int64_t kGroupMinLen = 256;  // COL_TILE: fewest row groups worth reading rows in groups
 constexpr int kLdsPerCu       = 160 * 1024;  // LDS bytes of one gfx950 CU
 constexpr int64_t kBytesInFlightPerCu = 80 * 1024;  // target of the wave-per-row plan
@@ -296,9 +300,23 @@ inline int make_plan(const rmi_reduce_desc& d,
     // element.  Reductions that need the row index (arg-reductions) stay on the plain path,
     // as do inputs that do not start on a 16-byte boundary and matrices with fewer than
     // kGroupMinLen groups.
+    // Rows of up to 130 bytes that are an odd number of bytes or of 16-bit elements are grouped
+    // as well: their vectors would start 1 or 2 bytes off a 4-byte boundary, which costs a
+    // plain read a quarter of its rate (rows 4 or 8 bytes off read like aligned ones).  512 MB,
+    // % of 8 TB/s, plain / grouped: bf16 D = 9 / 17 / 33 / 65: 42 / 50 / 63 / 71 -> 78 / 78 / 78 / 73,
+    // int8 D = 17 / 18 / 33 / 50 / 65 / 126: 39 / 41 / 47 / 53 / 56 / 70 -> 71 / 75 / 72 / 74 / 65 / 73;
+    // longer rows lose (bf16 D = 101 / 127: 75 / 77 -> 72 / 71, int8 D = 127: 66 -> 63).
     int64_t lanes = nload, rows = p.len;
-    if (key.family != kFamKvp && row_bytes < 16 && (in_misalign % 16) == 0) {
-      const int64_t low = row_bytes & -row_bytes;  // largest power of two in row_bytes
+    const int64_t low = row_bytes & -row_bytes;  // largest power of two in row_bytes
+    const bool short_rows = row_bytes < 16;
+    // (a group multiplies the partials; the entry point without allocation keeps the plain
+    // layout where they would outgrow its buffer)
+    const bool off_words = RMI_COL_GROUP_OFF_WORDS != 0 && row_bytes > 16 && low <= 2 &&
+                           row_bytes <= kGroupMaxRowBytes && row_bytes / low <= kColMaxLanes &&
+                           !((d.flags & kFlagSmallWorkspace) != 0 &&
+                             kTicketBytes + (size_t)p.n_out * (16 / low) * ((size_t)n_cu * (kColBlocksPerCu + 1)) *
+                                 acc_bytes > RMI_NOALLOC_SCRATCH_BYTES);
+    if (key.family != kFamKvp && (short_rows || off_words) && (in_misalign % 16) == 0) {
       if (p.len / (16 / low) >= kGroupMinLen) {
         p.group      = (int)(16 / low);
         p.group_len  = p.len / p.group;

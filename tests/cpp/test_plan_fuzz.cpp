@@ -188,11 +188,14 @@ void check(const rmi_reduce_desc& d, int n_cu, uintptr_t in_misalign)
       }
       if (p.group > 0) {
         ++grouped_plans;
-        // rows shorter than a 16-byte vector, in groups that are whole vectors at aligned
+        // rows shorter than a 16-byte vector, or longer ones 1 or 2 bytes off whole words whose
+        // group fits a workgroup's lanes, in groups that are whole vectors at aligned
         // addresses, enough of them, no index-dependent reduction
-        REQUIRE(key.family != rmi::kFamKvp && in_misalign % 16 == 0 && p.row_bytes < 16);
+        REQUIRE(key.family != rmi::kFamKvp && in_misalign % 16 == 0);
+        REQUIRE(p.row_bytes < 16 || (p.row_bytes % 4 != 0 && p.row_bytes <= rmi::kGroupMaxRowBytes &&
+                                     p.group_nvec <= rmi::kColMaxLanes));
         REQUIRE(p.group >= 2 && p.group <= 16 && (p.group * p.row_bytes) % 16 == 0);
-        REQUIRE(p.group_nvec * 16 == p.group * p.row_bytes && p.group_nvec <= 15);
+        REQUIRE(p.group_nvec * 16 == p.group * p.row_bytes && (p.row_bytes >= 16 || p.group_nvec <= 15));
         REQUIRE(p.group_len == p.len / p.group && p.group_len >= rmi::kGroupMinLen);
         REQUIRE(p.passes == 2);
       }

@@ -744,6 +744,38 @@ def test_grouped_columns(gpu, in_dt, out_dt, kw, rows, cols, shift):
                            label=f"grouped {rows}x{cols} dt{in_dt} +{shift}")
 
 
+# Rows of 16 bytes or more that are 1 or 2 bytes off whole words (odd byte counts, odd counts of
+# 16-bit elements) are read in groups of 16 or 8 as well up to 130 bytes:
+# every row count around a whole group, sums, extrema and squares, in place.
+@pytest.mark.parametrize("in_dt,out_dt,kw", [
+    (api.BF16, api.F32, {}),
+    (api.F16, api.F32, dict(main_op=api.MAIN_SQ, final_op=api.FIN_SQRT)),
+    (api.BF16, api.BF16, dict(reduce_op=api.RED_MAX, init_f=-np.inf)),
+    (api.I8, api.I64, {}),
+    (api.U8, api.I32, dict(main_op=api.MAIN_SQ)),
+    (api.I8, api.F32, dict(main_op=api.MAIN_ABS)),
+    (api.I8, api.I32, dict(reduce_op=api.RED_MIN, init_i=127)),
+])
+@pytest.mark.parametrize("cols", [9, 17, 33, 65, 127])
+def test_grouped_columns_off_words(gpu, in_dt, out_dt, kw, cols):
+    es = api.load().rmi_dtype_size(in_dt)
+    rb = cols * es
+    group = 16 // np.gcd(16, rb)
+    for rows in [4096 + k for k in (0, 1, group - 1, group, group + 1)] + [50007]:
+        rng = np.random.default_rng(rows * 3 + cols)
+        data = _rand(rng, in_dt, rows * cols)
+        d = api.make_desc(in_dt, out_dt, rows, cols, apply=api.ALONG_COLUMNS, **kw)
+        pl = api.plan_query(d)
+        assert pl.kind == api.PLAN_COL_TILE
+        if 16 < rb <= 130 and rb % 4 != 0:
+            assert pl.passes == 2 and pl.blocks_per_out % group == 0, (rows, cols, pl.blocks_per_out)
+        first = u.check_against_oracle(d, data, label=f"grouped off words {rows}x{cols} dt{in_dt}")
+        d.inplace = 1
+        u.check_against_oracle(d, data, old_raw=first, label=f"grouped off words {rows}x{cols} dt{in_dt} inplace")
+        d.inplace = 0
+        u.check_against_oracle(d, data, misalign_elems=1, label=f"grouped off words {rows}x{cols} dt{in_dt} +1")
+
+
 # Byte rows that are no whole 32-bit words (17 to 96 bytes) are summed by the flat kernel:
 # the matrix as one run of aligned 16-byte vectors, a vector's two row parts folded through
 # LDS.  Row counts around the chunk sizes, matrices whose last vector is a partial one (it is
