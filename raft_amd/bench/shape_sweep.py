@@ -40,9 +40,18 @@ def shapes(api):
         out.append((f"rows f32 D={d}", f32, f32, 4_000_000 if d < 33 else 1_000_000, d, {}))
     for r, d in ((100_000, 2048), (100_000, 4096), (8192, 8192), (32768, 32768)):
         out.append((f"rows f32 {r}x{d}", f32, f32, r, d, {}))
+    # rows just beyond a whole batch of the team kernel
+    for d in (1025, 1100, 1500, 2049, 2500, 4097):
+        out.append((f"rows f32 D={d}", f32, f32, rows_of(d, 4), d, {}))
+    for d in (513, 600, 1025):
+        out.append((f"rows f64 D={d}", f64, f64, rows_of(d, 8), d, {}))
+    for d in (2049, 4097):
+        out.append((f"rows bf16 D={d}", bf16, f32, rows_of(d, 2), d, {}))
+    for d in (4097, 5000):
+        out.append((f"rows i8 D={d}", i8, api.I64, rows_of(d, 1), d, {}))
     for d in (9, 17, 25, 33, 35, 63, 65, 67, 129):
         out.append((f"rows f64 D={d}", f64, f64, 2_000_000, d, {}))
-    for d in (36, 66, 76, 100, 130, 132, 250, 260):
+    for d in (33, 36, 65, 66, 76, 100, 129, 130, 132, 250, 260, 513):
         out.append((f"rows bf16 D={d}", bf16, f32, 2_000_000, d, {}))
     for d in (17, 33, 47, 70, 90, 150, 270, 500):
         out.append((f"rows i8 D={d}", i8, api.I64, rows_of(d, 1, 256), d, {}))
@@ -51,8 +60,10 @@ def shapes(api):
     # column sums, 512 MB each
     for d in (1, 2, 3, 5, 7, 12, 16, 20, 33, 48, 63, 64, 65, 100, 128, 129, 200, 256, 260, 300):
         out.append((f"cols f32 D={d}", f32, f32, rows_of(d, 4), d, col))
-    for d in (3, 8, 33, 100, 128, 300):
+    for d in (3, 8, 9, 17, 33, 65, 100, 127, 128, 300):
         out.append((f"cols bf16 D={d}", bf16, f32, rows_of(d, 2), d, col))
+    for d in (17, 33, 50, 65, 127):
+        out.append((f"cols i8 D={d}", i8, api.I64, rows_of(d, 1), d, col))
     for d in (3, 33, 100):
         out.append((f"cols f64 D={d}", f64, f64, rows_of(d, 8), d, col))
     for d in (516, 600, 768, 1000, 1100, 1400, 1536, 2049, 2300, 3000, 3500, 4096, 4097, 5000, 5120,

@@ -327,6 +327,22 @@ __device__ __forceinline__ void last_batch_n(int n, typename P::acc_t& acc, cons
   }
 }
 
+// n = 1 .. 9 lane-loads per lane, wave-uniform (the team kernel's rows of one trip)
+template <class P, bool VEC16, class IdxT>
+__device__ __forceinline__ void last_batch_n9(int n, typename P::acc_t& acc, const char* rp,
+                                              IdxT v, IdxT stride, IdxT end, i64 nvec, i64 len,
+                                              int tail)
+{
+  switch (n) {
+    case 5: last_batch<P, VEC16, 5, IdxT>(acc, rp, v, stride, end, nvec, len, tail); break;
+    case 6: last_batch<P, VEC16, 6, IdxT>(acc, rp, v, stride, end, nvec, len, tail); break;
+    case 7: last_batch<P, VEC16, 7, IdxT>(acc, rp, v, stride, end, nvec, len, tail); break;
+    case 8: last_batch<P, VEC16, 8, IdxT>(acc, rp, v, stride, end, nvec, len, tail); break;
+    case 9: last_batch<P, VEC16, 9, IdxT>(acc, rp, v, stride, end, nvec, len, tail); break;
+    default: last_batch_n<P, VEC16, IdxT>(n, acc, rp, v, stride, end, nvec, len, tail); break;
+  }
+}
+
 // ---------------------------------------------------------------------------
 // Short rows: nvec <= G, one lane-load per lane per row, kUnroll tiles of
 // 64/G rows in flight per wave.  ANYG = false: G is a power of two.  true: G is
@@ -632,10 +648,18 @@ __global__ __launch_bounds__(1024) void row_block_kernel(RowArgs a)
     // condition would send the lanes with one more whole batch through a loop and the
     // others through the last batch, one after the other).
     i64 vb = v0;
+    // the chunk's lane-loads, the row's tail elements counting as one more for the last chunk
+    const i64 vend = v1 + ((a.tail > 0 && b == a.B - 1) ? 1 : 0);
+    // A chunk of at most 2 * U + 1 lane-loads per thread makes ONE trip to memory, whatever its
+    // length: every load is issued before the first is used, positions past the chunk re-read
+    // its last vector.  (Whole batches first and the rest behind them made two or three
+    // dependent trips of rows just beyond a whole batch: fp32 D = 1025 ... 1100 ran at 45-50 %,
+    // D = 2049 at 67 %.  The ninth load takes the one vector more of rows like D = 4097.)
+    const bool one_trip = vend - v0 <= (i64)(2 * U + 1) * T;
     // A chunk of fewer than three batches per thread is read 2 * U lane-loads at a
     // time: all of it is in flight at once and the accumulate step starts as the first
     // vectors arrive.
-    if (a.chunk < (i64)3 * U * T) {
+    if (!one_trip && a.chunk < (i64)3 * U * T) {
       constexpr int W = 2 * U;
       for (; vb + (i64)W * T <= v1; vb += (i64)W * T) {
         typename H::type x[W];
@@ -655,7 +679,7 @@ __global__ __launch_bounds__(1024) void row_block_kernel(RowArgs a)
     // Whole batches of U lane-loads; the next batch is issued before the current one is
     // accumulated, so its latency overlaps the arithmetic (the loop holds no stores:
     // gfx9 counts loads and stores in one in-order counter).
-    if (vb + (i64)U * T <= v1) {
+    if (!one_trip && vb + (i64)U * T <= v1) {
       typename H::type x[U];
 #pragma unroll
       for (int u = 0; u < U; ++u)
@@ -684,13 +708,11 @@ __global__ __launch_bounds__(1024) void row_block_kernel(RowArgs a)
           x[u] = y[u];
       }
     }
-    // what is left: fewer than U * T lane-loads, at most U per lane
-    if (vb < v1)
-      last_batch_n<P, VEC16, i64>((int)((v1 - vb + T - 1) >> (6 + a.logT)), acc, rp, vb + t, (i64)T,
-                                  v1, a.nvec, a.len, 0);
-    // the overlapping last vector of the row goes to the team that owns the last chunk
-    if (a.tail > 0 && b == a.B - 1 && t == 0)
-      H::push_any(acc, H::load_any(rp, a.nvec, a.nvec, a.len), a.nvec, a.nvec, a.len, a.tail);
+    // what is left (or the whole chunk in one trip): at most 2 * U + 1 lane-loads per lane, the
+    // overlapping last vector of the row among them
+    if (vb < vend)
+      last_batch_n9<P, VEC16, i64>((int)((vend - vb + T - 1) >> (6 + a.logT)), acc, rp, vb + t, (i64)T,
+                                   vend, a.nvec, a.len, a.tail);
   }
 
   wave_allreduce<P>(acc);

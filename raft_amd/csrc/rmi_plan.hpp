@@ -34,6 +34,9 @@ constexpr int kPlanFlatMaxVec   = kPlanFlatChunkVec - 7;  // ... and the most ve
 constexpr int kColWideMaxSets = 5;    // COL_TILE, wide rows: most load slots per thread
 // row bundles in flight in the wide-row column kernel whose threads have K load slots
 constexpr int col_wide_bundles_of(int K) { return (10 + K - 1) / K; }
+#ifndef RMI_TEAM_ONE_TRIP
+#define RMI_TEAM_ONE_TRIP 1
+#endif
 #ifndef RMI_COL_GROUP_OFF_WORDS
 #define RMI_COL_GROUP_OFF_WORDS 1
 #endif
@@ -463,12 +466,22 @@ inline int make_plan(const rmi_reduce_desc& d,
       // four to eight (arg-reductions, whose accumulate step is longer).  One wave
       // streaming a long row alone leaves thousands of row streams open at once, which
       // measured 3-7 points slower than 128- or 256-thread teams.
+      // Sums over rows of up to 2304 lane-loads take the narrowest team that reads the row in
+      // ONE trip of at most nine loads per thread (fp32 D = 1025 / 1100 / 2049: 45 / 50 / 67 % with
+      // whole batches of four first and the rest in further trips).
       {
         const bool kvp     = key.family == kFamKvp;
         const int64_t want = p.nvec / (kvp ? 16 : 8);
         int wide           = kvp ? 64 : 128;
         while (wide < 256 && wide * 2 <= want)
           wide *= 2;
+        if (!kvp && RMI_TEAM_ONE_TRIP != 0) {
+          int narrow = 64;
+          while (narrow < 256 && nload > (int64_t)(2 * kPlanTeamUnroll + 1) * narrow)
+            narrow *= 2;
+          // (where such teams fill the machine's wave slots; fewer rows keep the wider teams)
+          if (p.n_out * (narrow / 64) >= slots) wide = narrow;
+        }
         if (wide > threads) threads = wide;
       }
       if (threads == 1024 && p.n_out * 16 < slots &&

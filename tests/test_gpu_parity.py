@@ -776,6 +776,41 @@ def test_grouped_columns_off_words(gpu, in_dt, out_dt, kw, cols):
         u.check_against_oracle(d, data, misalign_elems=1, label=f"grouped off words {rows}x{cols} dt{in_dt} +1")
 
 
+# Rows of 257 to 2304 lane-loads are read by a team in ONE trip of up to nine loads per thread
+# (positions past the row re-read its last vector), the overlapping last vector among them: row
+# lengths around every boundary of the rule, with and without tail elements, few rows (wider
+# teams) and enough rows to fill the machine (the narrowest team), sums, extrema, arg-reductions.
+@pytest.mark.parametrize("in_dt,out_dt,kw", [
+    (api.F32, api.F32, {}),
+    (api.F32, api.F32, dict(reduce_op=api.RED_MAX, init_f=-np.inf)),
+    (api.F32, api.KVP_I32_F32, dict(main_op=api.MAIN_KVP, reduce_op=api.RED_ARGMIN, init_f=np.inf)),
+    (api.F64, api.F64, dict(main_op=api.MAIN_SQ, final_op=api.FIN_SQRT)),
+    (api.BF16, api.F32, {}),
+    (api.I8, api.I64, dict(main_op=api.MAIN_ABS)),
+])
+def test_team_rows_one_trip(gpu, in_dt, out_dt, kw):
+    es = api.load().rmi_dtype_size(in_dt)
+    vec = 16 // es
+    seed = 0
+    for nload in (257, 258, 300, 511, 512, 513, 576, 577, 1000, 1024, 1025, 1152, 1153, 2048, 2049, 2304, 2305):
+        for short in (0, 1, vec - 1):                 # whole vectors, one element short, one element over
+            cols = nload * vec - short
+            for rows in (5, 2100):
+                seed += 1
+                rng = np.random.default_rng(seed)
+                data = _rand(rng, in_dt, rows * cols)
+                if kw.get("main_op") == api.MAIN_KVP:   # ties for the arg-reduction
+                    data = np.round(data * 8).astype(data.dtype)
+                d = api.make_desc(in_dt, out_dt, rows, cols, **kw)
+                first = u.check_against_oracle(d, data, label=f"one trip {rows}x{cols} dt{in_dt}")
+                if seed % 4 == 0:
+                    d.inplace = 1
+                    u.check_against_oracle(d, data, old_raw=first, label=f"one trip {rows}x{cols} dt{in_dt} inplace")
+                    d.inplace = 0
+                if seed % 5 == 0:
+                    u.check_against_oracle(d, data, misalign_elems=1, label=f"one trip {rows}x{cols} dt{in_dt} +1")
+
+
 # Byte rows that are no whole 32-bit words (17 to 96 bytes) are summed by the flat kernel:
 # the matrix as one run of aligned 16-byte vectors, a vector's two row parts folded through
 # LDS.  Row counts around the chunk sizes, matrices whose last vector is a partial one (it is
