@@ -35,6 +35,15 @@ def shapes(api):
         return max(1, (mb << 20) // (d * es))
 
     # row sums
+    for d in (3, 5, 9):
+        out.append((f"rows f32 D={d}", f32, f32, rows_of(d, 4, 256), d, {}))
+    for d in (3, 9, 17):
+        out.append((f"rows bf16 D={d}", bf16, f32, rows_of(d, 2, 256), d, {}))
+    for d in (5, 11):
+        out.append((f"rows i8 D={d}", i8, api.I64, rows_of(d, 1, 128), d, {}))
+    for d in (3, 5):
+        out.append((f"rows f64 D={d}", f64, f64, rows_of(d, 8, 256), d, {}))
+    out.append(("rows argmax f32 D=3", f32, api.KVP_I32_F32, rows_of(3, 4, 256), 3, kvp))
     for d in (7, 12, 16, 20, 21, 24, 32, 33, 36, 40, 41, 45, 48, 50, 54, 58, 60, 62, 64, 66, 68, 72,
               79, 83, 90, 96, 100, 125, 128, 129, 160, 200, 256, 300, 384, 768, 1000):
         out.append((f"rows f32 D={d}", f32, f32, 4_000_000 if d < 33 else 1_000_000, d, {}))

@@ -62,6 +62,7 @@ int run(const PlanX& pl, const Problem& pr, hipStream_t st)
                   kTeamUnroll == kPlanTeamUnroll && kStageBytes == kStageBytesPerWave &&
                   kFan == kTicketFan && kLineWords * 4 == kTicketLineBytes,
                 "plan selector and kernels must agree on block size and unroll");
+  static_assert(kSmallBytes == kPlanSmallBytes, "the planner's chunk of small rows is the kernel's");
   static_assert(col_wide_bundles(1) == col_wide_bundles_of(1) && col_wide_bundles(2) == col_wide_bundles_of(2) &&
                   col_wide_bundles(3) == col_wide_bundles_of(3) && col_wide_bundles(4) == col_wide_bundles_of(4) &&
                   col_wide_bundles(5) == col_wide_bundles_of(5) && kColWideMaxSets == 5 &&
@@ -104,7 +105,10 @@ int run(const PlanX& pl, const Problem& pr, hipStream_t st)
           default: rc = RMI_ERR_UNSUPPORTED;
         }
       } else if (pl.kind == RMI_PLAN_ROW_WAVE && !pl.team_kernel) {
-        if (pl.flat_rows) {
+        if (pl.small_rows) {
+          a.chunk_rows = pl.chunk_rows;
+          hipLaunchKernelGGL((row_small_kernel<P>), grid, dim3(kBlock), 0, st, a);
+        } else if (pl.flat_rows) {
           if constexpr (sizeof(typename P::in_t) == 1 && P::kTail == kTailZero) {  // the planner's rule
             a.chunk_rows    = pl.chunk_rows;
             a.inv_row_bytes = 1.0f / (float)pl.row_bytes;

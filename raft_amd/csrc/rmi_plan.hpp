@@ -34,6 +34,10 @@ constexpr int kPlanFlatMaxVec   = kPlanFlatChunkVec - 7;  // ... and the most ve
 constexpr int kColWideMaxSets = 5;    // COL_TILE, wide rows: most load slots per thread
 // row bundles in flight in the wide-row column kernel whose threads have K load slots
 constexpr int col_wide_bundles_of(int K) { return (10 + K - 1) / K; }
+#ifndef RMI_SMALL_ROWS
+#define RMI_SMALL_ROWS 1
+#endif
+constexpr int kPlanSmallBytes = 16384;  // ROW_WAVE, small rows: bytes of a workgroup's chunk at most
 #ifndef RMI_TEAM_ONE_TRIP
 #define RMI_TEAM_ONE_TRIP 1
 #endif
@@ -79,6 +83,8 @@ struct PlanX {
                             // of `chunk_rows` whole rows per workgroup, 2^logG lanes fold a row
   int chunk_rows  = 0;
   bool team_kernel = false; // served by the team-per-row kernel
+  bool small_rows  = false; // ROW_WAVE: rows shorter than a vector that do not divide one, kPlanSmallChunk
+                            // whole rows per workgroup through LDS
   bool stage_ok    = false; // ROW_WAVE: rows could be staged through LDS
   bool staged      = false; // ROW_WAVE: rows are staged through LDS (line-aligned span reads)
   int elem_bytes  = 0;
@@ -499,6 +505,31 @@ inline int make_plan(const rmi_reduce_desc& d,
 
   if (kind == RMI_PLAN_ROW_WAVE) {
     p.kind = RMI_PLAN_ROW_WAVE;
+    // Rows through LDS (row_small_kernel): a workgroup reads a chunk of whole rows as aligned
+    // vectors into LDS and its threads reduce whole rows from there, element by element.
+    // Rows shorter than a vector that do not divide one (the others are ROW_LANES) would be read
+    // a lane per element: fp32 D = 3 34 -> 82 % of 8 TB/s, arg-max 39 -> 84, bf16 D = 3 / 5 / 7:
+    // 23 / 17 / 22 -> 74 / 82 / 82, int8 D = 3 ... 15: 16-26 -> 73-84.  Longer rows that are no whole
+    // vectors, as long as a chunk holds 32 of them: 16-bit elements (their lane-loads sit 2 bytes
+    // off whole words: bf16 D = 9 / 17 / 33 / 65 / 97 / 161: 46 / 43 / 58 / 63 / 68 / 69 -> 79 / 75 / 75 /
+    // 78 / 80 / 76, D = 193 / 225: 62 / 65 -> 61 / 68; 42-45 % from 514 bytes on) and 8-byte ones
+    // (compensated sums pay most for the steps between lanes: fp64 D = 3 / 5 / 9 / 17 / 33 / 49 / 63:
+    // 75 / 56 / 67 / 71 / 75 / 65 / 73 -> 80 / 76 / 76 / 77 / 81 / 77 / 82, D = 65: 76 -> 64); 4-byte rows
+    // up to 40 bytes (fp32 D = 6 / 9: 71 / 67 -> 78 / 75, D = 5 / 7 / 10 within 2 points; D = 11 / 13 /
+    // 25 lose 3 / 8 / 7).  Byte rows of 17 to 96 bytes keep the flat kernel (int8 D = 33 / 63: 68 /
+    // 67 % there, 61 / 58 % here).
+    const int64_t small_max = es == 1 ? 15 : es == 4 ? 40 : (es == 2 || es == 8) ? 512 : 15;
+    if (RMI_SMALL_ROWS != 0 && row_bytes <= small_max && (row_bytes % 16) != 0 &&
+        (16 % row_bytes) != 0 && (in_misalign % 16) == 0 && hint == RMI_PLAN_AUTO &&
+        kPlanSmallBytes / row_bytes >= 32) {
+      p.small_rows  = true;
+      p.G           = 1;
+      p.logG        = 0;
+      p.chunk_rows  = (int)(kPlanSmallBytes / row_bytes / 16 * 16);
+      p.grid_blocks = ceildiv(p.n_out, (int64_t)p.chunk_rows);
+      if (p.grid_blocks > 0x7fffffffLL) return RMI_ERR_BAD_SHAPE;
+      return RMI_OK;
+    }
     // An input that starts off a 16-byte boundary makes every 128-byte piece of the default
     // layout (8 or 16 lanes per row, several loads per lane) straddle two lines, and each
     // line is then asked for by two load instructions.  With one load per lane and the

@@ -16,6 +16,7 @@ long grouped_plans = 0;
 long wide_plans = 0;
 long dense_plans = 0;
 long flat_plans = 0;
+long small_plans = 0;
 #define REQUIRE(cond)                                                              \
   do {                                                                             \
     if (!(cond)) {                                                                 \
@@ -84,6 +85,15 @@ void check(const rmi_reduce_desc& d, int n_cu, uintptr_t in_misalign)
       REQUIRE(!p.strided);
       if (p.team_kernel) {
         REQUIRE(p.threads == 64 && p.B == 1 && p.chunk == p.nvec);
+      } else if (p.small_rows) {
+        ++small_plans;
+        // rows through LDS: a chunk of whole rows per workgroup, at most 16 KB
+        REQUIRE(p.row_bytes <= (es == 1 ? 15 : es == 4 ? 40 : 512) && p.row_bytes % 16 != 0 && 16 % p.row_bytes != 0);
+        REQUIRE(in_misalign % 16 == 0 && d.plan_hint == RMI_PLAN_AUTO);
+        REQUIRE(!p.short_rows && !p.any_g && !p.dense_rows && !p.flat_rows && p.passes == 1 && p.ws_bytes == 0);
+        REQUIRE(p.chunk_rows >= 32 && p.chunk_rows % 16 == 0 &&
+                (int64_t)p.chunk_rows * p.row_bytes <= rmi::kPlanSmallBytes);
+        REQUIRE(p.grid_blocks == (p.n_out + p.chunk_rows - 1) / p.chunk_rows);
       } else if (p.flat_rows) {
         ++flat_plans;
         // byte sums over rows that are no whole words: chunks of whole rows that start on a
@@ -296,7 +306,11 @@ int main()
     std::printf("  whole-row column plans were hardly exercised (%ld)\n", wide_plans);
     ++failures;
   }
-  if (dense_plans < 1000) {
+  if (small_plans < 1000) {
+    std::printf("  plans of rows through LDS were hardly exercised (%ld)\n", small_plans);
+    ++failures;
+  }
+  if (dense_plans < 500) {
     std::printf("  dense row plans were hardly exercised (%ld)\n", dense_plans);
     ++failures;
   }

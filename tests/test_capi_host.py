@@ -169,8 +169,8 @@ def test_null_and_workspace_errors_without_a_launch():
 def test_lane_groups_follow_the_row_length():
     """Rows whose lane-load count is far from a power of two get one lane per lane-load
     (5 lane-loads, and 6 or 9..17 with tail elements); the others keep power-of-two groups."""
-    lanes = lambda cols, dt=api.F32, out=api.F32: api.plan_query(
-        api.make_desc(dt, out, 1000000, cols)).lanes_per_row
+    lanes = lambda cols, dt=api.F32, out=api.F32, hint=api.PLAN_AUTO: api.plan_query(
+        api.make_desc(dt, out, 1000000, cols, plan_hint=hint)).lanes_per_row
     assert lanes(20) == 5 and lanes(17) == 5            # 5 lane-loads, without and with a tail
     assert lanes(33) == 9 and lanes(45) == 12 and lanes(62) == 16
     # 17, 18 and 33 lane-loads with a tail: the row's own count (slots dealt over whole rows)
@@ -180,12 +180,17 @@ def test_lane_groups_follow_the_row_length():
     assert lanes(24) == 8 and lanes(28) == 8            # 6 and 7 whole lane-loads stay on 8 lanes
     assert lanes(36) == 4                               # 9 whole vectors: 4 lanes x 3 loads
     assert lanes(128) == 8 and lanes(256) == 16
-    assert lanes(100, api.BF16) == 13                   # 12 whole + 4 elements
+    # 16-bit and 8-byte rows of up to 512 bytes that are no whole vectors go through LDS, a
+    # thread per row; the lane groups serve them when the plan is asked for (or the input
+    # starts off a 16-byte boundary)
+    W = api.PLAN_ROW_WAVE
+    assert lanes(100, api.BF16) == 1 and lanes(17, api.F64, api.F64) == 1 and lanes(9) == 1
+    assert lanes(100, api.BF16, hint=W) == 13           # 12 whole + 4 elements
     # 16-byte accumulators (f64 sums) keep it up to 12 lane-loads
-    assert lanes(17, api.F64, api.F64) == 9 and lanes(63, api.F64, api.F64) == 8
-    # ... and take their own count again from 5 to 18 lane-loads with a tail, whole rows dealt
-    # over the workgroup's load slots
-    assert lanes(25, api.F64, api.F64) == 13 and lanes(35, api.F64, api.F64) == 18
+    assert lanes(17, api.F64, api.F64, W) == 9 and lanes(63, api.F64, api.F64, W) == 8
+    # (with a tail they take their own count again from 5 to 18 lane-loads, whole rows dealt over
+    # the workgroup's load slots, under the automatic plan only: inputs off a 16-byte boundary)
+    assert lanes(25, api.F64, api.F64, W) == 8
     # arg-reductions follow the same rule
     d = api.make_desc(api.F32, api.KVP_I32_F32, 1000, 33, main_op=api.MAIN_KVP,
                       reduce_op=api.RED_ARGMAX)

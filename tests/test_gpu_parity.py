@@ -811,6 +811,48 @@ def test_team_rows_one_trip(gpu, in_dt, out_dt, kw):
                     u.check_against_oracle(d, data, misalign_elems=1, label=f"one trip {rows}x{cols} dt{in_dt} +1")
 
 
+# Rows through LDS: a workgroup reads a chunk of whole rows as aligned vectors and its threads
+# reduce whole rows element by element.  Rows shorter than a vector, 16-bit and 8-byte rows
+# that are no whole vectors, short fp32 rows; row counts around a chunk, matrices that end
+# inside a vector, every reduction, in place, an input off a 16-byte boundary (other plans).
+@pytest.mark.parametrize("in_dt,out_dt,kw,colset", [
+    (api.F32, api.F32, {}, (3, 5, 6, 7, 9, 10)),
+    (api.F32, api.F32, dict(main_op=api.MAIN_SQ, final_op=api.FIN_SQRT), (3, 9)),
+    (api.F32, api.KVP_I32_F32, dict(main_op=api.MAIN_KVP, reduce_op=api.RED_ARGMAX, init_f=-np.inf), (3, 7)),
+    (api.F32, api.F32, dict(reduce_op=api.RED_MIN, init_f=np.inf), (3, 10)),
+    (api.F64, api.F64, {}, (3, 5, 9, 33, 63)),
+    (api.F64, api.KVP_I64_F64, dict(main_op=api.MAIN_KVP, reduce_op=api.RED_ARGMIN, init_f=np.inf), (3, 17)),
+    (api.BF16, api.F32, {}, (3, 5, 7, 9, 17, 33, 100, 129, 255)),
+    (api.F16, api.F16, dict(main_op=api.MAIN_ABS, reduce_op=api.RED_MAX, init_f=0.0), (3, 11, 65)),
+    (api.I8, api.I64, {}, (3, 5, 7, 11, 15)),
+    (api.U8, api.I32, dict(main_op=api.MAIN_SQ), (6, 13)),
+    (api.I8, api.F32, dict(main_op=api.MAIN_NZ), (9,)),
+    (api.I32, api.I64, {}, (3, 6)),
+])
+def test_small_rows_through_lds(gpu, in_dt, out_dt, kw, colset):
+    es = api.load().rmi_dtype_size(in_dt)
+    seed = 0
+    for cols in colset:
+        chunk = 16384 // (cols * es) // 16 * 16
+        for rows in sorted({1, 2, 15, 16, 17, chunk - 1, chunk, chunk + 1, 2 * chunk + 3, 50001}):
+            seed += 1
+            rng = np.random.default_rng(seed * 11 + in_dt)
+            data = _rand(rng, in_dt, rows * cols)
+            if kw.get("main_op") == api.MAIN_KVP:       # ties
+                data = np.round(data * 4).astype(data.dtype)
+            d = api.make_desc(in_dt, out_dt, rows, cols, **kw)
+            pl = api.plan_query(d)
+            assert pl.kind == api.PLAN_ROW_WAVE and pl.passes == 1
+            assert pl.grid_blocks == -(-rows // chunk), (rows, cols, pl.grid_blocks)
+            first = u.check_against_oracle(d, data, label=f"small rows {rows}x{cols} dt{in_dt}")
+            if seed % 3 == 0:
+                d.inplace = 1
+                u.check_against_oracle(d, data, old_raw=first, label=f"small rows {rows}x{cols} dt{in_dt} inplace")
+                d.inplace = 0
+            if seed % 4 == 0:
+                u.check_against_oracle(d, data, misalign_elems=1, label=f"small rows {rows}x{cols} dt{in_dt} +1")
+
+
 # Byte rows that are no whole 32-bit words (17 to 96 bytes) are summed by the flat kernel:
 # the matrix as one run of aligned 16-byte vectors, a vector's two row parts folded through
 # LDS.  Row counts around the chunk sizes, matrices whose last vector is a partial one (it is
@@ -877,8 +919,13 @@ def test_dense_rows(gpu, in_dt, out_dt, kw, cols_list, rows, shift, inplace):
         pl = api.plan_query(d)
         assert pl.kind == api.PLAN_ROW_WAVE and pl.passes == 1
         es = api.load().rmi_dtype_size(in_dt)
-        assert pl.lanes_per_row == -(-cols * es // 16), (cols, pl.lanes_per_row)
-        assert pl.grid_blocks <= 4 * 256
+        if es in (2, 8) and cols * es <= 512 and (cols * es) % 16 != 0:
+            # from a 16-byte boundary such rows go through LDS, a thread per row (the query's
+            # answer); the dense slots serve them from any other start (shift != 0 below)
+            assert pl.lanes_per_row == 1
+        else:
+            assert pl.lanes_per_row == -(-cols * es // 16), (cols, pl.lanes_per_row)
+            assert pl.grid_blocks <= 4 * 256
         old = None
         if inplace and kw.get("main_op") != api.MAIN_KVP:
             old = u.encode_out(out_dt, rng.integers(1, 5, rows))
@@ -1006,7 +1053,10 @@ def test_any_lane_count_rows(gpu, in_dt, out_dt, kw, cols_list, rows, shift):
         d = api.make_desc(in_dt, out_dt, rows, cols, **kw)
         pl = api.plan_query(d)
         assert pl.kind == api.PLAN_ROW_WAVE
-        assert pl.lanes_per_row in (5, 6) + tuple(range(9, 17)) + tuple(range(18, 22)) + tuple(range(28, 33)), \
+        # (from a 16-byte boundary the 16-bit and 8-byte shapes, and fp32 rows of up to 40 bytes,
+        # go through LDS, a thread per row: the query answers 1 for them, and the lane groups
+        # serve them from any other start, shift != 0)
+        assert pl.lanes_per_row in (1, 5, 6) + tuple(range(9, 17)) + tuple(range(18, 22)) + tuple(range(28, 33)), \
             (cols, pl.lanes_per_row)
         u.check_against_oracle(d, data, misalign_elems=shift,
                                label=f"any-G {rows}x{cols} dt{in_dt} +{shift}")
