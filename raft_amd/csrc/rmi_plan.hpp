@@ -34,6 +34,9 @@ constexpr int kPlanFlatMaxVec   = kPlanFlatChunkVec - 7;  // ... and the most ve
 constexpr int kColWideMaxSets = 5;    // COL_TILE, wide rows: most load slots per thread
 // row bundles in flight in the wide-row column kernel whose threads have K load slots
 constexpr int col_wide_bundles_of(int K) { return (10 + K - 1) / K; }
+#ifndef RMI_LANES_AUTO
+#define RMI_LANES_AUTO 0
+#endif
 #ifndef RMI_SMALL_ROWS
 #define RMI_SMALL_ROWS 1
 #endif
@@ -437,8 +440,18 @@ inline int make_plan(const rmi_reduce_desc& d,
 
   // ---- contiguous-dimension plans ----
   // several whole rows per 16-byte vector
+  // (Left to itself the planner takes this plan for two rows per vector, for outputs narrower
+  // than 32 bits, which it packs, and for inputs off a 16-byte boundary: with four rows and
+  // more per vector the rows through LDS of the ROW_WAVE branch measured faster, a lane's K
+  // outputs being K separate stores here: int8 -> int64 D = 1 / 2 / 4: 6 / 10 / 59 -> 64 / 64 / 68 % of
+  // 8 TB/s, int8 -> int32 D = 1 / 2 / 4: 14 / 30 / 60 -> 63 / 70 / 82, bf16 -> fp32 D = 1 / 2: 66 / 76 ->
+  // 70 / 82, fp32 D = 1: 77 -> 82; bf16 -> bf16 D = 2: 67 here, 55 there.  Two rows per vector
+  // measured within a point on fp32 and bf16 and either way by 5 points with the matrix's size
+  // on int8 -> int64 D = 8: 8M / 17M / 34M / 67M rows 75 / 79 / 81 / 81 % here, 70 / 79 / 86 / 76 there.)
+  const bool lanes_auto = RMI_LANES_AUTO != 0 || 16 / row_bytes <= 2 || dtype_size(d.out_dtype) < 4 ||
+                          (in_misalign % 16) != 0;
   if (row_bytes < 16 && 16 % row_bytes == 0 &&
-      (hint == RMI_PLAN_AUTO || hint == RMI_PLAN_ROW_LANES)) {
+      ((hint == RMI_PLAN_AUTO && lanes_auto) || hint == RMI_PLAN_ROW_LANES)) {
     p.kind        = RMI_PLAN_ROW_LANES;
     p.vec16       = true;
     p.step        = 16 / es;
@@ -520,9 +533,10 @@ inline int make_plan(const rmi_reduce_desc& d,
     // 67 % there, 61 / 58 % here).
     const int64_t small_max = es == 1 ? 15 : es == 4 ? 40 : (es == 2 || es == 8) ? 512 : 15;
     if (RMI_SMALL_ROWS != 0 && row_bytes <= small_max && (row_bytes % 16) != 0 &&
-        (16 % row_bytes) != 0 && (in_misalign % 16) == 0 && hint == RMI_PLAN_AUTO &&
+        (in_misalign % 16) == 0 && hint == RMI_PLAN_AUTO &&
         kPlanSmallBytes / row_bytes >= 32) {
       p.small_rows  = true;
+      p.vec16       = true;  // the chunk is read as whole vectors
       p.G           = 1;
       p.logG        = 0;
       p.chunk_rows  = (int)(kPlanSmallBytes / row_bytes / 16 * 16);

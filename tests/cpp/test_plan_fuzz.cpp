@@ -72,7 +72,7 @@ void check(const rmi_reduce_desc& d, int n_cu, uintptr_t in_misalign)
   const int es = dtype_size(d.in_dtype);
   if (p.kind != RMI_PLAN_ROW_LANES) {
     REQUIRE(p.row_bytes == contiguous * es);
-    REQUIRE(p.vec16 == (p.row_bytes >= 16 || p.group > 0));
+    REQUIRE(p.vec16 == (p.row_bytes >= 16 || p.group > 0 || p.small_rows));
     REQUIRE(p.nvec * p.step + p.tail == contiguous);
     REQUIRE(p.tail >= 0 && p.tail < p.step);
   }
@@ -80,6 +80,10 @@ void check(const rmi_reduce_desc& d, int n_cu, uintptr_t in_misalign)
   switch (p.kind) {
     case RMI_PLAN_ROW_LANES:
       REQUIRE(!p.strided && p.K >= 2 && p.K <= 16 && p.K * contiguous * es == 16);
+      // asked for by name, two rows per vector, outputs narrower than 32 bits, or an input off a
+      // 16-byte boundary
+      REQUIRE(d.plan_hint == RMI_PLAN_ROW_LANES || p.K == 2 || dtype_size(d.out_dtype) < 4 ||
+              in_misalign % 16 != 0);
       break;
     case RMI_PLAN_ROW_WAVE:
       REQUIRE(!p.strided);
@@ -88,7 +92,9 @@ void check(const rmi_reduce_desc& d, int n_cu, uintptr_t in_misalign)
       } else if (p.small_rows) {
         ++small_plans;
         // rows through LDS: a chunk of whole rows per workgroup, at most 16 KB
-        REQUIRE(p.row_bytes <= (es == 1 ? 15 : es == 4 ? 40 : 512) && p.row_bytes % 16 != 0 && 16 % p.row_bytes != 0);
+        REQUIRE(p.row_bytes <= (es == 1 ? 15 : es == 4 ? 40 : 512) && p.row_bytes % 16 != 0);
+        // rows of which four or more fill a vector come here when their outputs have 32 bits or more
+        if (16 % p.row_bytes == 0) REQUIRE(dtype_size(d.out_dtype) >= 4 && 16 / p.row_bytes >= 4);
         REQUIRE(in_misalign % 16 == 0 && d.plan_hint == RMI_PLAN_AUTO);
         REQUIRE(!p.short_rows && !p.any_g && !p.dense_rows && !p.flat_rows && p.passes == 1 && p.ws_bytes == 0);
         REQUIRE(p.chunk_rows >= 32 && p.chunk_rows % 16 == 0 &&

@@ -145,6 +145,10 @@ TEST_CASE(plan_selector)
   CHECK(p.kind == RMI_PLAN_ROW_WAVE && p.lanes_per_row == 8 && p.vec_bytes == 16);
   p = plan(RMI_I8, RMI_I64, 16777216, 8);
   CHECK(p.kind == RMI_PLAN_ROW_LANES);
+  p = plan(RMI_I8, RMI_I64, 16777216, 4);
+  CHECK(p.kind == RMI_PLAN_ROW_WAVE && p.lanes_per_row == 1);  // four rows per vector: through LDS, a thread per row
+  p = plan(RMI_BF16, RMI_BF16, 16777216, 2);
+  CHECK(p.kind == RMI_PLAN_ROW_LANES);  // outputs narrower than 32 bits are packed by a lane
   p = plan(RMI_I8, RMI_I64, 4096, 16384);
   CHECK(p.kind == RMI_PLAN_ROW_BLOCK && p.passes == 1);
   p = plan(RMI_BF16, RMI_F32, 8, 4194304);
@@ -156,7 +160,7 @@ TEST_CASE(plan_selector)
   p = plan(RMI_F32, RMI_F32, 100, 7);
   CHECK(p.vec_bytes == 16);  // 28-byte rows: one 16-byte lane load and three tail elements
   p = plan(RMI_F32, RMI_F32, 100, 3);
-  CHECK(p.vec_bytes == 4);  // 12-byte rows are read element by element
+  CHECK(p.vec_bytes == 16 && p.lanes_per_row == 1);  // 12-byte rows go through LDS as whole vectors
   p = plan(RMI_F32, RMI_F32, 5, 0);
   CHECK(p.kind == RMI_PLAN_EMPTY);
   rmi_reduce_desc bad{};

@@ -68,6 +68,7 @@ BENCH_SHAPES = [
      dict(main_op=api.MAIN_KVP, reduce_op=api.RED_ARGMAX), api.PLAN_ROW_BLOCK, 1),
     (api.I8, api.I64, 4096, 16384, {}, api.PLAN_ROW_BLOCK, 1),
     (api.I8, api.I64, 16777216, 8, {}, api.PLAN_ROW_LANES, 1),
+    (api.I8, api.I64, 16777216, 4, {}, api.PLAN_ROW_WAVE, 1),           # four rows per vector: through LDS
     (api.BF16, api.F32, 8, 4194304, {}, api.PLAN_ROW_SPLIT, 2),
 ]
 
@@ -96,10 +97,13 @@ def test_plan_hints_and_fallbacks():
     assert p.kind == api.PLAN_ROW_SPLIT and p.blocks_per_out >= 2
     assert p.workspace_bytes == api.WORKSPACE_TICKET_BYTES + 4 * p.blocks_per_out * 8
     # rows of 7 floats (28 B) are one 16-byte vector plus three tail elements;
-    # rows of 3 floats (12 B) are read element by element
+    # rows of 3 floats (12 B) go through LDS as whole vectors, and are read element by element
+    # when the lane-group plan is asked for
     p = api.plan_query(api.make_desc(api.F32, api.F32, 1000, 7))
     assert p.vec_bytes == 16 and p.kind == api.PLAN_ROW_WAVE
     p = api.plan_query(api.make_desc(api.F32, api.F32, 1000, 3))
+    assert p.vec_bytes == 16 and p.kind == api.PLAN_ROW_WAVE and p.lanes_per_row == 1
+    p = api.plan_query(api.make_desc(api.F32, api.F32, 1000, 3, plan_hint=api.PLAN_ROW_WAVE))
     assert p.vec_bytes == 4 and p.kind == api.PLAN_ROW_WAVE
     # f64 sums carry a 16-byte (sum, compensation) accumulator through the partials
     d = api.make_desc(api.F64, api.F64, 4, 1 << 20, plan_hint=api.PLAN_ROW_SPLIT)

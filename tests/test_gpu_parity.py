@@ -219,7 +219,8 @@ def test_min_max(gpu, in_dt, out_dt, red, main):
 # the oracle (exactly: max / min select one of the inputs) and against numpy's nanmax / nanmin.
 NAN_SHAPES = [
     # rows, cols, apply, plan hint, expected plan kind
-    (5000, 2, api.ALONG_ROWS, api.PLAN_AUTO, api.PLAN_ROW_LANES),
+    (5000, 2, api.ALONG_ROWS, api.PLAN_ROW_LANES, api.PLAN_ROW_LANES),
+    (5000, 3, api.ALONG_ROWS, api.PLAN_AUTO, api.PLAN_ROW_WAVE),      # rows through LDS
     (3000, 21, api.ALONG_ROWS, api.PLAN_AUTO, api.PLAN_ROW_WAVE),     # one load per lane, any G, tail
     (3000, 30, api.ALONG_ROWS, api.PLAN_AUTO, api.PLAN_ROW_WAVE),     # one load per lane, G = 8, tail
     (1000, 259, api.ALONG_ROWS, api.PLAN_AUTO, api.PLAN_ROW_WAVE),    # lanes of a wave, tail
@@ -1110,9 +1111,15 @@ def test_rows_inside_a_vector(gpu, in_dt, out_dt, cols, final, rows):
         kw = dict(inplace=True)
     rng = np.random.default_rng(rows + cols)
     data = _rand(rng, in_dt, rows * cols)
-    d = api.make_desc(in_dt, out_dt, rows, cols, **kw)
-    assert api.plan_query(d).kind == api.PLAN_ROW_LANES
     old = None
     if final == "inplace":
         old = u.encode_out(out_dt, rng.integers(-5, 5, rows).astype(np.float64))
+    # the plan asked for by name, and what the planner takes by itself (rows through LDS where
+    # the output has 32 bits or more)
+    d = api.make_desc(in_dt, out_dt, rows, cols, plan_hint=api.PLAN_ROW_LANES, **kw)
+    assert api.plan_query(d).kind == api.PLAN_ROW_LANES
     u.check_against_oracle(d, data, old_raw=old, label=f"lanes {rows}x{cols} {final}")
+    d = api.make_desc(in_dt, out_dt, rows, cols, **kw)
+    through_lds = api.load().rmi_dtype_size(out_dt) >= 4 and 16 // (cols * api.load().rmi_dtype_size(in_dt)) >= 4
+    assert api.plan_query(d).kind == (api.PLAN_ROW_WAVE if through_lds else api.PLAN_ROW_LANES)
+    u.check_against_oracle(d, data, old_raw=old, label=f"lanes or LDS {rows}x{cols} {final}")
