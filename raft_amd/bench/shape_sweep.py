@@ -90,8 +90,9 @@ def shapes(api):
     for d in (5, 8, 16, 20, 32, 33, 50, 64, 100, 128, 129, 200, 220, 250, 256, 300, 401, 500, 512, 777, 1000,
               1024, 4096, 10000):
         out.append((f"normalize f32 D={d}", f32, f32, rows_of(d, 4), d, "normalize"))
-    for d in (9, 33, 100, 128, 130, 256, 1000, 4096):
+    for d in (3, 5, 9, 33, 100, 128, 130, 256, 1000, 4096):
         out.append((f"normalize bf16 D={d}", bf16, bf16, rows_of(d, 2), d, "normalize"))
+    out.append(("normalize f32 D=3", f32, f32, rows_of(3, 4), 3, "normalize"))
     for d in (25, 33, 65, 128, 250):
         out.append((f"normalize f64 D={d}", f64, f64, rows_of(d, 8), d, "normalize"))
     return out

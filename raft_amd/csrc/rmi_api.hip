@@ -421,6 +421,8 @@ int rmi_row_normalize(const rmi_reduce_desc* desc,
   a.final_op  = d.final_op;
   a.init      = d.init.f;
   a.eps       = eps;
+  const NormPlan small = make_small_norm_plan(d.n_rows, d.n_cols, es, in, out);
+  if (small.kind == 4) return fn(small, a, static_cast<hipStream_t>(stream));
   const NormPlan flat = make_flat_norm_plan(d.n_rows, d.n_cols, es, in, out);
   if (flat.kind == 3) {
     const int rc = fn(flat, a, static_cast<hipStream_t>(stream));

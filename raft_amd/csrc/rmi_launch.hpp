@@ -287,6 +287,26 @@ inline NormPlan make_flat_norm_plan(int64_t n_rows, int64_t len, int elem_bytes,
   return p;
 }
 
+// Rows shorter than a vector through LDS (normalize_small_kernel), or kind != 4 when it does not
+// apply: input and output on a 16-byte boundary.
+inline NormPlan make_small_norm_plan(int64_t n_rows, int64_t len, int elem_bytes, const void* in,
+                                     const void* out)
+{
+  NormPlan p;
+  const int64_t rb = len * elem_bytes;
+  if (rb >= 16 || rb < 1) return p;
+  if (reinterpret_cast<uintptr_t>(in) % 16 != 0 || reinterpret_cast<uintptr_t>(out) % 16 != 0) return p;
+  if (len < 2) return p;  // a row of one element: the lane-per-row kernels are as fast
+  int chunk_rows = (int)(kSmallBytes / rb / 16 * 16);
+  if (elem_bytes == 2 && len % 2 != 0 && chunk_rows > kSmallNormRows) chunk_rows = kSmallNormRows;
+  if (chunk_rows < 32 || chunk_rows > 32 * kBlock) return p;
+  p.kind       = 4;
+  p.vec16      = true;
+  p.chunk_rows = chunk_rows;
+  p.grid       = ceildiv(n_rows, (int64_t)chunk_rows);
+  return p;
+}
+
 inline NormPlan make_norm_plan(int64_t n_rows, int64_t len, int elem_bytes)
 {
   NormPlan p;
@@ -363,7 +383,16 @@ int run_normalize(const NormPlan& pl, const NormArgs& args, hipStream_t st)
   a.invG     = 65536u / (unsigned)(pl.G > 0 ? pl.G : 1) + 1;
   if (pl.grid > 0x7fffffffLL) return RMI_ERR_BAD_SHAPE;
   const dim3 grid((unsigned)pl.grid);
-  if (pl.kind == 3) {
+  if (pl.kind == 4) {
+    a.chunk_rows = pl.chunk_rows;
+    if constexpr (sizeof(typename P::in_t) == 2) {
+      if (a.len % 2 != 0) {  // rows that share 32-bit words: scaled on the way out
+        hipLaunchKernelGGL((normalize_small_kernel<P, true>), grid, dim3(kBlock), 0, st, a);
+        return hipGetLastError() == hipSuccess ? RMI_OK : RMI_ERR_LAUNCH;
+      }
+    }
+    hipLaunchKernelGGL((normalize_small_kernel<P, false>), grid, dim3(kBlock), 0, st, a);
+  } else if (pl.kind == 3) {
     a.n_rows        = pl.flat_rows;
     a.chunk_rows    = pl.chunk_rows;
     a.logL          = pl.logL;

@@ -626,4 +626,132 @@ __global__ __launch_bounds__(kBlock) void normalize_flat_kernel(NormArgs a)
   }
 }
 
+// ---------------------------------------------------------------------------
+// Rows shorter than a 16-byte vector (three floats, five halves): a lane per ELEMENT read and
+// wrote them at 20-45 % of the memory rate.  Here a workgroup reads a chunk of whole rows (a
+// multiple of 16 rows, at most 16 KB, from a 16-byte boundary of input and output) as aligned
+// vectors into LDS, every thread norms whole rows out of LDS, element by element, and the
+// chunk leaves as whole vectors, scaled with the arithmetic of the other kernels.
+//   PER_VECTOR = false: the thread that normed a row scales it in place in LDS.
+//   PER_VECTOR = true: the threads leave the reciprocals of their rows' norms in LDS and the
+//     chunk is scaled vector by vector on its way out, an element's row being its index over
+//     the row length (at most kSmallNormRows rows per chunk).  For 16-bit rows of an odd
+//     length, whose rows share 32-bit words of LDS: written by different lanes, they cost the
+//     first variant half of its rate.
+// A row whose norm is <= eps must not be written: a chunk that holds one is stored row by
+// row, element by element, by the threads that own its rows.
+// ---------------------------------------------------------------------------
+constexpr int kSmallNormRows = 2048;
+template <class P, bool PER_VECTOR>
+__global__ __launch_bounds__(kBlock) void normalize_small_kernel(NormArgs a)
+{
+  using in_t  = typename P::in_t;
+  using nat   = typename P::nat;
+  using acc_t = typename P::acc_t;
+  constexpr int ES  = (int)sizeof(in_t);
+  constexpr int VEC = P::VEC;
+  __shared__ __align__(16) unsigned char sm[kSmallBytes];
+  __shared__ nat recips[PER_VECTOR ? kSmallNormRows : 1];
+  __shared__ int any_skipped;
+  const int t     = threadIdx.x;
+  const int rb    = (int)a.row_bytes;
+  const i64 row0  = (i64)blockIdx.x * a.chunk_rows;
+  const i64 left  = a.n_rows - row0;
+  const int rows  = left < a.chunk_rows ? (int)left : a.chunk_rows;
+  const int bytes = rows * rb;   // kSmallBytes at most
+  const int nfull = bytes >> 4;  // whole vectors of the chunk
+  const char* base = static_cast<const char*>(a.in) + row0 * rb;
+  char* obase      = static_cast<char*>(a.out) + row0 * rb;
+  if (t == 0) any_skipped = 0;
+  if (nfull > 0) {
+    u32x4 x[kSmallVecs];
+#pragma unroll
+    for (int k = 0; k < kSmallVecs; ++k) {  // unconditional, clamped
+      const int v = t + k * kBlock;
+      x[k]        = load16(base + 16 * (v < nfull ? v : nfull - 1));
+    }
+#pragma unroll
+    for (int k = 0; k < kSmallVecs; ++k) {
+      const int v = t + k * kBlock;
+      if (v < nfull) *reinterpret_cast<u32x4*>(sm + 16 * v) = x[k];
+    }
+  }
+  // what follows the last whole vector (the matrix's last chunk only), element by element
+  for (int i = (nfull << 4) / ES + t; i < bytes / ES; i += kBlock)
+    reinterpret_cast<in_t*>(sm)[i] = reinterpret_cast<const in_t*>(base)[i];
+  __syncthreads();
+  in_t* e     = reinterpret_cast<in_t*>(sm);
+  const int D = (int)a.len;
+  // x / norm as the other kernels compute it: 16-bit elements times the reciprocal in fp32,
+  // fp32 and fp64 correctly rounded
+  auto scaled = [&](nat x, nat norm, nat recip) __attribute__((always_inline)) {
+    if constexpr (ES == 2) {
+      return x * recip;
+    } else {
+      return Quot<nat>(norm, recip)(x);
+    }
+  };
+  u32 skipped = 0;  // bit k: this thread's k-th row is left untouched (32 rows per thread at most)
+  int k       = 0;
+  for (int r = t; r < rows; r += kBlock, ++k) {
+    acc_t acc = P::neutral();
+    for (int j = 0; j < D; ++j)
+      P::push(acc, stored_to_nat<in_t>(e[r * D + j]), (i64)j);
+    const nat norm  = row_norm<P>(a, acc);
+    const nat recip = (nat)1 / norm;
+    if (norm <= (nat)a.eps) {  // a NaN norm is not skipped: the row becomes NaN
+      skipped |= 1u << k;
+      any_skipped = 1;
+    }
+    if constexpr (PER_VECTOR) {
+      recips[r] = recip;
+    } else if (!(norm <= (nat)a.eps)) {
+      for (int j = 0; j < D; ++j)
+        Put<in_t>::st(e + r * D + j, scaled(stored_to_nat<in_t>(e[r * D + j]), norm, recip));
+    }
+  }
+  __syncthreads();
+  if (any_skipped == 0) {
+    const float inv_len = 1.0f / (float)D;
+#pragma unroll
+    for (int q = 0; q < kSmallVecs; ++q) {
+      const int v = t + q * kBlock;
+      if (v < nfull) {
+        u32x4 y = *reinterpret_cast<const u32x4*>(sm + 16 * v);
+        if constexpr (PER_VECTOR) {
+          static_assert(!PER_VECTOR || ES == 2, "scaled by the reciprocal alone");
+          const u32x4 x = y;
+          static_for<VEC>([&](auto j) {
+            constexpr int J = decltype(j)::value;
+            // the element's row: its index is below 8192 and D below 16, so the quotient is exact
+            const int r = (int)(((float)(v * VEC + J) + 0.5f) * inv_len);
+            Put<in_t>::template at<J>(y, In<in_t>::template get<J>(x) * recips[r]);
+          });
+        }
+        store16<false>(obase + 16 * v, y);
+      }
+    }
+    for (int i = (nfull << 4) / ES + t; i < bytes / ES; i += kBlock) {
+      if constexpr (PER_VECTOR) {
+        Put<in_t>::st(reinterpret_cast<in_t*>(obase) + i,
+                      stored_to_nat<in_t>(e[i]) * recips[(int)(((float)i + 0.5f) * inv_len)]);
+      } else {
+        reinterpret_cast<in_t*>(obase)[i] = e[i];
+      }
+    }
+  } else {
+    k = 0;
+    for (int r = t; r < rows; r += kBlock, ++k) {
+      if ((skipped >> k) & 1u) continue;
+      for (int j = 0; j < D; ++j) {
+        if constexpr (PER_VECTOR) {
+          Put<in_t>::st(reinterpret_cast<in_t*>(obase) + r * D + j, stored_to_nat<in_t>(e[r * D + j]) * recips[r]);
+        } else {
+          reinterpret_cast<in_t*>(obase)[r * D + j] = e[r * D + j];
+        }
+      }
+    }
+  }
+}
+
 }  // namespace rmi

@@ -323,3 +323,46 @@ def test_full_size_embedding_shape(gpu):
     ds = api.make_desc(api.F32, api.F32, ns, cols, main_op=api.MAIN_SQ, final_op=api.FIN_SQRT)
     exp = _oracle(ds, sub, np.zeros(ns * cols), 1e-8)
     assert u.approx_ok(o[: ns * cols].cpu().numpy(), exp, 1e-5).all()
+
+
+# Rows shorter than a 16-byte vector go through LDS (a chunk of whole rows as aligned vectors, a
+# thread per row; 16-bit rows of an odd length are scaled vector by vector on the way out): row
+# counts around a chunk, rows of norm 0 and below eps (untouched: their chunk is stored row by
+# row), NaN, the three norms, in place, and starts off a 16-byte boundary (the other kernels).
+@pytest.mark.gpu
+@pytest.mark.parametrize("dt,npdt,colset", [
+    (api.F32, np.float32, (2, 3)),
+    (api.BF16, None, (2, 3, 4, 5, 6, 7)),
+    (api.F16, np.float16, (3, 6)),
+])
+def test_rows_shorter_than_a_vector(gpu, dt, npdt, colset):
+    es = 4 if dt == api.F32 else 2
+    seed = 0
+    for cols in colset:
+        chunk = 16384 // (cols * es) // 16 * 16
+        if es == 2 and cols % 2 == 1:
+            chunk = min(chunk, 2048)
+        for rows in sorted({1, 2, 17, chunk - 1, chunk, chunk + 1, 3 * chunk + 5}):
+            for norm in NORMS:
+                seed += 1
+                _flat_case(dt, npdt, rows, cols, norm, 0, 0, seed % 3 == 0, seed)
+            _flat_case(dt, npdt, rows, cols, "l2", 16, 48, False, seed + 1000)
+            _flat_case(dt, npdt, rows, cols, "l2", es, 0, False, seed + 2000)      # off a 16-byte boundary
+    # a chunk without any untouched row takes the whole-vector stores
+    import torch
+    from raft_amd import device as dev
+    rng = np.random.default_rng(5)
+    for cols in colset:
+        rows = 50001
+        m = rng.standard_normal((rows, cols)) + 3.0
+        data = u.to_bf16(m.astype(np.float32).reshape(-1)) if dt == api.BF16 else m.astype(npdt).reshape(-1)
+        d = api.make_desc(dt, dt, rows, cols, main_op=api.MAIN_SQ, final_op=api.FIN_SQRT)
+        x = torch.from_numpy(data.view(np.uint8)).cuda()
+        o = torch.zeros_like(x)
+        assert api.load().rmi_row_normalize(C.byref(d), x.data_ptr(), o.data_ptr(), 1e-6,
+                                            dev.current_stream_ptr()) == 0
+        torch.cuda.synchronize()
+        got = o.cpu().numpy().view(data.dtype)
+        exp = _oracle(d, data, np.zeros(rows * cols), 1e-6)
+        ok = u.ulp16_ok(dt, got, exp) if dt in (api.BF16, api.F16) else u.approx_ok(got, exp, 1e-5)
+        assert ok.all(), (cols, np.argwhere(~ok)[:4])
