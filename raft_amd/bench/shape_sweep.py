@@ -93,6 +93,8 @@ def shapes(api):
     for d in (3, 5, 9, 33, 100, 128, 130, 256, 1000, 4096):
         out.append((f"normalize bf16 D={d}", bf16, bf16, rows_of(d, 2), d, "normalize"))
     out.append(("normalize f32 D=3", f32, f32, rows_of(3, 4), 3, "normalize"))
+    out.append(("normalize f32 D=1100", f32, f32, rows_of(1100, 4), 1100, "normalize"))
+    out.append(("normalize bf16 D=2049", bf16, bf16, rows_of(2049, 2), 2049, "normalize"))
     for d in (25, 33, 65, 128, 250):
         out.append((f"normalize f64 D={d}", f64, f64, rows_of(d, 8), d, "normalize"))
     return out

@@ -239,6 +239,9 @@ struct NormPlan {
 // by the same measurements: rows of 16, 32 or 64 bytes (whole rows per power-of-two lane group:
 // 75-80 % against 70-77 %), fp64 rows below 192 bytes (-2 to -20 %), and rows so long that the
 // whole rows of a chunk fill less than 85 % of a workgroup's vector slots.
+#ifndef RMI_NORM_WAVE_LONG
+#define RMI_NORM_WAVE_LONG 1
+#endif
 #ifndef RMI_NORM_FLAT_MAX_ROW_BYTES
 #define RMI_NORM_FLAT_MAX_ROW_BYTES 4096
 #endif
@@ -349,6 +352,18 @@ inline NormPlan make_norm_plan(int64_t n_rows, int64_t len, int elem_bytes)
       p.logG = 0;
       p.grid = ceildiv(n_rows, (int64_t)(kWave / p.G) * kUnroll * (kBlock / kWave));
     }
+  } else if (RMI_NORM_WAVE_LONG != 0 && p.vec16 && nload < (int64_t)2 * kUnroll * kWave) {
+    // 257 to 511 lane-loads: one wave per row with five to eight loads per lane, where a
+    // 256-thread team holds one or two lane-loads per thread and a quarter to a half of its load
+    // slots (256 MB in + out, % of 8 TB/s: bf16 D = 2049 / 2555 / 3137 / 3999: 41 / 50 / 60 / 69 -> 80 /
+    // 80 / 80 / 79, fp32 D = 1025 / 1100 / 1500 / 2001: 66 / 71 / 75 / 74 -> 81 / 82 / 81 / 79, fp64 D = 513 /
+    // 601 / 901: 62 / 71 / 74 -> 79 / 81 / 79; exactly 512 lane-loads: 79 / 79 / 78 -> 76 / 77 / 77, left
+    // to the team)
+    p.G     = kWave;
+    p.logG  = 6;
+    p.L     = (int)ceildiv(nload, (int64_t)kWave);
+    p.tiles = 1;
+    p.grid  = ceildiv(n_rows, (int64_t)(kBlock / kWave));
   } else {
     p.grid = n_rows;
     if (nload <= 256 * 4) {

@@ -336,8 +336,15 @@ __global__ __launch_bounds__(kBlock) void normalize_wave_kernel(NormArgs a)
     else normalize_wave_body<P, VEC16, 2, 2, STREAM>(a);
   } else if (a.L == 3) {
     normalize_wave_body<P, VEC16, 3, 1, STREAM>(a);
-  } else {
+  } else if (a.L == 4) {
     normalize_wave_body<P, VEC16, 4, 1, STREAM>(a);
+  } else if constexpr (VEC16) {
+    // rows of 257 to 512 lane-loads on one wave: a 256-thread team would hold one or two
+    // lane-loads per thread and a quarter of its load slots
+    if (a.L == 5) normalize_wave_body<P, true, 5, 1, STREAM>(a);
+    else if (a.L == 6) normalize_wave_body<P, true, 6, 1, STREAM>(a);
+    else if (a.L == 7) normalize_wave_body<P, true, 7, 1, STREAM>(a);
+    else normalize_wave_body<P, true, 8, 1, STREAM>(a);
   }
 }
 

@@ -366,3 +366,21 @@ def test_rows_shorter_than_a_vector(gpu, dt, npdt, colset):
         exp = _oracle(d, data, np.zeros(rows * cols), 1e-6)
         ok = u.ulp16_ok(dt, got, exp) if dt in (api.BF16, api.F16) else u.approx_ok(got, exp, 1e-5)
         assert ok.all(), (cols, np.argwhere(~ok)[:4])
+
+
+# Rows of 257 to 511 lane-loads stay on one wave with five to eight loads per lane: every load
+# count, with and without tail elements, few rows and many, untouched and NaN rows, in place.
+@pytest.mark.gpu
+@pytest.mark.parametrize("dt,npdt,colset", [
+    (api.F32, np.float32, (1025, 1028, 1281, 1300, 1537, 1791, 1793, 2040, 2043)),
+    (api.BF16, None, (2049, 2056, 3000, 3585, 4081)),
+    (api.F64, np.float64, (513, 640, 641, 1000, 1021)),
+])
+def test_rows_of_five_to_eight_loads_per_lane(gpu, dt, npdt, colset):
+    seed = 0
+    for cols in colset:
+        for rows in (1, 5, 300):
+            for norm in ("l2", "linf"):
+                seed += 1
+                _flat_case(dt, npdt, rows, cols, norm, 0, 0, seed % 3 == 0, seed)
+        _flat_case(dt, npdt, 9, cols, "l1", 16, 64, False, seed + 500)
