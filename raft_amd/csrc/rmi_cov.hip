@@ -59,17 +59,25 @@ int make_cov_plan(int dtype, int layout, int64_t N, int64_t D, CovPlan& p)
 
 bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 
-// Matrices of 4, 8, 16 or 32 columns whose row count is a multiple of f = 64 / D are contracted
-// as matrices of 64 columns and N / f rows: every load and every matrix instruction then does
-// useful work, where a 64-column block with masked columns reads 20M x 32 floats at 55 % of the
-// rate of 10M x 64 (20M x 32: 572 -> 383 us, 40M x 16: 934 -> 386 us, fp64 10M x 32: 874 -> 525 us).
-// It costs one more small launch, so matrices below 4M elements stay as they are (32768 x 32:
-// 14 us against 17.6).  Returns f, or 1.
-int fold_factor(int64_t N, int64_t D)
+// Matrices of at most 32 columns are contracted as matrices of f D <= 64 columns and N / f rows:
+// every load and every matrix instruction then does useful work, where a 64-column block with
+// masked columns reads 20M x 32 floats at 55 % of the rate of 10M x 64 and 45M x 3 at 5 % (20M x
+// 32: 572 -> 383 us, 40M x 16: 934 -> 386 us, fp64 10M x 32: 874 -> 525 us; 45M x 3: 1359 us as it
+// was).  Row-major, f rows sit side by side; col-major, the first f pieces of N / f rows of every
+// column; the N % f rows left over are added by cov_blocks_kernel.  It costs one more small
+// launch, so matrices below 4M elements stay as they are (32768 x 32: 14 us against 17.6).
+// Returns f, or 1.
+int fold_factor(int layout, int64_t N, int64_t D)
 {
-  if (D != 4 && D != 8 && D != 16 && D != 32) return 1;
-  const int f = (int)(cov::kBlockCols / D);
-  return (N % f == 0 && N * D >= ((int64_t)1 << 22)) ? f : 1;
+  if (D < 1 || D > cov::kBlockCols / 2 || N * D < ((int64_t)1 << 22)) return 1;
+  const int f0 = (int)(cov::kBlockCols / D);
+  if (layout != RMI_ROW_MAJOR) return f0;
+  // row-major: rows of whole quads of columns are read as vectors, which is worth up to a
+  // quarter fewer rows side by side (45M x 3 as 21 rows of 63 columns: 156 us, as 20 of 60: see
+  // the measurements)
+  for (int f = f0; f >= 1 && f * 4 >= f0 * 3; --f)
+    if ((f * D) % 4 == 0) return f;
+  return f0;
 }
 constexpr size_t kWideBytes = (size_t)cov::kBlockCols * cov::kBlockCols * sizeof(double);
 
@@ -78,11 +86,13 @@ int launch(const CovPlan& pl, int layout, int64_t N_in, int64_t D_in, int sample
            const T* mu, T* covar, void* ws, hipStream_t st)
 {
   // `pl` is the plan of the matrix as it is contracted: N / f rows of 64 columns when folded
-  const int fold  = fold_factor(N_in, D_in);
+  const int fold  = fold_factor(layout, N_in, D_in);
   const int64_t N = N_in / fold, D = D_in * fold;
   cov::GramArgs g{};
   g.mu_div = layout == RMI_ROW_MAJOR ? 1 : fold;
   g.mu_mod = fold > 1 ? (int)D_in : 0;
+  g.col_ld = N_in;
+  g.col_f  = fold;
   g.data    = data;
   g.mu      = mu;
   g.partial = ws;
@@ -160,9 +170,19 @@ int launch(const CovPlan& pl, int layout, int64_t N_in, int64_t D_in, int sample
                      dim3(cov::kFoldElems * cov::kFoldSplit), 0, st, f);
   if (fold > 1) {
     const int cells = (int)(D_in * D_in);
+    // the rows that the contraction leaves over, still as they were given: the last N % fold
+    // rows of the matrix (row-major) or of every column (col-major)
+    const int left       = (int)(N_in - N * fold);
+    const bool rm        = layout == RMI_ROW_MAJOR;
+    T* tail              = rm ? data + N * fold * D_in : data + N * fold;
+    const int64_t rs     = rm ? D_in : 1;
+    const int64_t cs     = rm ? 1 : N_in;
     hipLaunchKernelGGL((cov::cov_blocks_kernel<T>), dim3((unsigned)((cells + cov::kThreads - 1) / cov::kThreads)),
-                       dim3(cov::kThreads), 0, st, wide, covar, (int)D_in, fold,
-                       layout == RMI_ROW_MAJOR ? 1 : 0);
+                       dim3(cov::kThreads), 0, st, wide, covar, (int)D_in, fold, rm ? 1 : 0, tail, mu, left, rs,
+                       cs, f.alpha);
+    if (left > 0 && center && mu != nullptr)  // ... and centred like the others afterwards
+      hipLaunchKernelGGL((cov::center_tail_kernel<T>), dim3(1), dim3(cov::kThreads), 0, st, tail, mu, left,
+                         (int)D_in, rs, cs);
   }
   return hipGetLastError() == hipSuccess ? RMI_OK : RMI_ERR_LAUNCH;
 }
@@ -175,7 +195,7 @@ extern "C" {
 size_t rmi_cov_workspace_bytes(int dtype, int layout, int64_t n_rows, int64_t n_cols)
 {
   rmi::CovPlan pl;
-  const int fold = rmi::fold_factor(n_rows, n_cols);
+  const int fold = rmi::fold_factor(layout, n_rows, n_cols);
   if (rmi::make_cov_plan(dtype, layout, n_rows / fold, n_cols * fold, pl) != RMI_OK) return 0;
   return n_cols > 0 ? pl.ws_bytes + (fold > 1 ? rmi::kWideBytes : 0) : 0;
 }
@@ -196,7 +216,7 @@ int rmi_cov(int dtype,
   using namespace rmi;
   if ((flags & ~RMI_COV_CENTER_DATA) != 0) return RMI_ERR_BAD_ENUM;
   CovPlan pl;
-  const int fold = fold_factor(n_rows, n_cols);
+  const int fold = fold_factor(layout, n_rows, n_cols);
   const int rc   = make_cov_plan(dtype, layout, n_rows / fold, n_cols * fold, pl);
   if (rc != RMI_OK) return rc;
   if (n_cols == 0) return RMI_OK;

@@ -95,15 +95,23 @@ struct GramArgs {
   int npairs;        // nb * (nb + 1) / 2
   int S;             // slabs
   int total;         // S * npairs workgroups do work; the grid is rounded up to 8
-  // A matrix of 4, 8, 16 or 32 columns is contracted as one of 64: f = 64 / D consecutive rows
-  // (row-major) or the f pieces of a column (col-major) side by side.  Column c of the wide
-  // matrix then has the mean mu[(c / mu_div) % mu_mod]; mu_mod == 0: mu[c].
+  // A matrix of at most 32 columns is contracted as one of f D <= 64: f consecutive rows (row-
+  // major) or the first f pieces of N rows of every column (col-major) side by side.  Column c
+  // of the wide matrix then has the mean mu[(c / mu_div) % mu_mod]; mu_mod == 0: mu[c].
   int mu_div;
   int mu_mod;
+  // col-major: column c of the (wide) matrix starts at (c / col_f) * col_ld + (c % col_f) * N
+  // (col_f pieces of the columns of a matrix whose columns are col_ld apart; 1: c * col_ld)
+  int64_t col_ld;
+  int col_f;
 };
 __device__ __forceinline__ int64_t mean_index(const GramArgs& a, int64_t c)
 {
   return a.mu_mod == 0 ? c : (c / a.mu_div) % a.mu_mod;
+}
+__device__ __forceinline__ int64_t col_offset(const GramArgs& a, int64_t c)
+{
+  return a.col_f <= 1 ? c * a.col_ld : (c / a.col_f) * a.col_ld + (c % a.col_f) * a.N;
 }
 
 struct FoldArgs {
@@ -704,7 +712,7 @@ __device__ __forceinline__ void gram_cols_body_bf16(const GramArgs& a, int unit,
     for (int gq = 0; gq < 4; ++gq) {
       const int64_t c = (int64_t)(s == 0 ? bi : bj) * kBlockCols + 16 * gq + cl;
       ok[s][gq]       = c < a.D;
-      colp[s][gq]     = data + (ok[s][gq] ? c : 0) * N;
+      colp[s][gq]     = data + col_offset(a, ok[s][gq] ? c : 0);
       mean[s][gq]     = (mu != nullptr && ok[s][gq]) ? mu[mean_index(a, c)] : T(0);
     }
   }
@@ -800,7 +808,7 @@ __device__ __forceinline__ void gram_cols_body_bf16(const GramArgs& a, int unit,
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const int64_t c = (int64_t)bi * kBlockCols + 8 * i + c8;
-      cop[i]          = data + ((FULL || c < a.D) ? c : 0) * N + 4 * p8;
+      cop[i]          = data + col_offset(a, (FULL || c < a.D) ? c : 0) + 4 * p8;
     }
     auto load_unit_co = [&](Quad<T> (&x)[8], int64_t q) __attribute__((always_inline)) {
 #pragma unroll
@@ -966,7 +974,7 @@ __device__ __forceinline__ void gram_cols_body(const GramArgs& a, int unit, int 
     for (int gq = 0; gq < 4; ++gq) {
       const int64_t c = (int64_t)(s == 0 ? bi : bj) * kBlockCols + 16 * gq + cl;
       ok[s][gq]       = c < a.D;
-      colp[s][gq]     = data + (ok[s][gq] ? c : 0) * N;
+      colp[s][gq]     = data + col_offset(a, ok[s][gq] ? c : 0);
       mean[s][gq]     = (mu != nullptr && ok[s][gq]) ? mu[mean_index(a, c)] : T(0);
     }
   }
@@ -1170,14 +1178,18 @@ __global__ __launch_bounds__(kFoldElems* kFoldSplit) void cov_fold_kernel(FoldAr
   if (r != c) out[c * a.D + r] = val;
 }
 
-// A matrix of D = 64 / f columns contracted as one of 64 (f consecutive rows side by side,
+// A matrix of D <= 32 columns contracted as one of f D <= 64 (f consecutive rows side by side,
 // row-major; the f pieces of every column side by side, col-major): its covariance is the sum
 // of the f diagonal D x D blocks of the wide result (row-major: rows and columns b D + r; col-
-// major: r f + b), summed in block order in f64 and rounded once.  One thread per element of
-// the upper half; the lower half is its mirror.
+// major: r f + b), summed in block order in f64 and rounded once.  The `left` rows that the
+// contraction leaves over (row k, column r at tail[k tail_rs + r tail_cs]) are added here, from
+// the data as it was given.
+// One thread per element of the upper half; the lower half is its mirror.
 template <class T>
 __global__ __launch_bounds__(kThreads) void cov_blocks_kernel(const double* wide, T* out, int D, int f,
-                                                              int row_major)
+                                                              int row_major, const T* tail, const T* mu,
+                                                              int left, int64_t tail_rs, int64_t tail_cs,
+                                                              double alpha)
 {
   const int i = blockIdx.x * kThreads + threadIdx.x;
   if (i >= D * D) return;
@@ -1187,10 +1199,28 @@ __global__ __launch_bounds__(kThreads) void cov_blocks_kernel(const double* wide
   for (int b = 0; b < f; ++b) {
     const int wr = row_major ? b * D + r : r * f + b;
     const int wc = row_major ? b * D + c : c * f + b;
-    sum += wide[wr * kBlockCols + wc];
+    sum += wide[wr * (f * D) + wc];  // the wide result has f D rows and columns
+  }
+  if (left > 0) {
+    const double mr = mu != nullptr ? (double)mu[r] : 0.0, mc = mu != nullptr ? (double)mu[c] : 0.0;
+    double rest     = 0.0;
+    for (int k = 0; k < left; ++k)
+      rest += ((double)tail[k * tail_rs + r * tail_cs] - mr) * ((double)tail[k * tail_rs + c * tail_cs] - mc);
+    sum += rest * alpha;
   }
   out[r * D + c] = (T)sum;
   if (r != c) out[c * D + r] = (T)sum;
+}
+
+// the rows left over, centred like the others (after cov_blocks_kernel has read them)
+template <class T>
+__global__ __launch_bounds__(kThreads) void center_tail_kernel(T* tail, const T* mu, int left, int D,
+                                                               int64_t tail_rs, int64_t tail_cs)
+{
+  for (int i = blockIdx.x * kThreads + threadIdx.x; i < left * D; i += gridDim.x * kThreads) {
+    const int k = i / D, r = i - k * D;
+    tail[k * tail_rs + r * tail_cs] -= mu[r];
+  }
 }
 
 // ---------------------------------------------------------------------------

@@ -93,10 +93,13 @@ SHAPES = [(1, 1), (2, 3), (3, 2), (15, 5), (16, 4), (17, 63), (31, 64), (33, 65)
           (257, 129), (1000, 130), (4099, 200), (513, 260), (64, 8), (5000, 66),
           (2, 32), (1000, 32), (1001, 32), (4096, 16), (40, 8), (96, 4)]
 
-# 4, 8, 16 or 32 columns and 4M elements or more: contracted as 64 columns when the row count is
-# a multiple of 64 / D, as they are otherwise
+# Up to 32 columns and 4M elements or more: contracted as f D <= 64 columns, f = 64 // D rows side
+# by side (row-major, the rows left over added separately) or the largest divisor of the row
+# count up to that (col-major: pieces of whole columns)
 NARROW = [(131072, 32), (131073, 32), (262144, 16), (262148, 16), (262146, 16), (524288, 8),
-          (524292, 8), (1048576, 4), (1048592, 4), (1048577, 4)]
+          (524292, 8), (1048576, 4), (1048592, 4), (1048577, 4),
+          (1398101, 3), (1398120, 3), (4194304, 1), (4194305, 1), (2097153, 2), (838861, 5), (838860, 5),
+          (600000, 7), (420001, 10), (349526, 12), (209716, 20), (209715, 20), (135301, 31), (190651, 22)]
 
 
 @pytest.mark.parametrize("dt", [api.F32, api.F64])
