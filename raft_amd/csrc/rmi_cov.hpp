@@ -272,7 +272,12 @@ __device__ __forceinline__ void gram_rows_body(const GramArgs& a, int unit, int 
   // in contiguous pieces of 4 * UR rows per workgroup.
   const int64_t G     = (int64_t)a.S * kWaves;
   const int64_t g     = (int64_t)slab * kWaves + wave;
-  const int64_t nfull = a.N / UR;
+  // Rows that are no whole quads of columns are read as quads all the same, the last quad of a
+  // row running up to three elements into the next row (masked like the columns beyond D): the
+  // units of the main loop therefore end before the matrix's last row, which the guarded unit
+  // reads element by element.  (Rows of one or two columns would reach beyond the next row.)
+  const bool quads    = VEC || D >= 3;
+  const int64_t nfull = (VEC || !quads) ? a.N / UR : (a.N - 1) / UR;
   const int64_t K     = g < nfull ? (nfull - g + G - 1) / G : 0;  // whole units of this wave
 
   auto load_unit = [&](Quad<T> (&x)[NS][UL], int64_t q, bool guard) {
@@ -284,7 +289,7 @@ __device__ __forceinline__ void gram_rows_body(const GramArgs& a, int unit, int 
       const T* rp      = data + r0 * D + dr * D;
 #pragma unroll
       for (int s = 0; s < NS; ++s) {
-        if constexpr (VEC) {
+        if (VEC || (quads && !guard)) {
           x[s][u] = load_quad<T, STREAM>(rp + col[s][0]);
         } else {
 #pragma unroll
@@ -541,7 +546,9 @@ __device__ __forceinline__ void gram_rows_body_bf16(const GramArgs& a, int unit,
 
   const int64_t G     = (int64_t)a.S * kWaves;
   const int64_t gw    = (int64_t)slab * kWaves + wave;
-  const int64_t nfull = a.N / UR;
+  // (rows that are no whole quads of columns: see gram_rows_body)
+  const bool quads    = VEC || D >= 3;
+  const int64_t nfull = (VEC || !quads) ? a.N / UR : (a.N - 1) / UR;
   const int64_t K     = gw < nfull ? (nfull - gw + G - 1) / G : 0;
 
   auto load_unit = [&](Quad<T> (&x)[NS][8], int64_t q, bool guard) {
@@ -552,7 +559,7 @@ __device__ __forceinline__ void gram_rows_body_bf16(const GramArgs& a, int unit,
       const T* rp      = data + r0 * D + dr * D;
 #pragma unroll
       for (int s = 0; s < NS; ++s) {
-        if constexpr (VEC) {
+        if (VEC || (quads && !guard)) {
           x[s][r] = load_quad<T, STREAM>(rp + col[s][0]);
         } else {
 #pragma unroll
