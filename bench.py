@@ -616,6 +616,36 @@ def main():
                     pct_of_peak=100.0 * nb / (ms * 1e-3) / 1e9 / PEAK_HBM_GBPS,
                     check={"torch_fp64": ok})
 
+    def extra_rows(rows, cols, what):
+        # L2 norms of short or awkward rows: `what` names the kernel the planner takes
+        xs = [mk_normal(rows, cols, 17 + 7919 * i) for i in range(3)]
+        out = torch.empty(rows, dtype=torch.float32, device="cuda")
+        d = api.make_desc(api.F32, api.F32, rows, cols, main_op=api.MAIN_SQ, final_op=api.FIN_SQRT)
+        ref = C.byref(d)
+
+        def call(i):
+            return lib.rmi_reduce(ref, xs[i % 3].data_ptr(), out.data_ptr(), None, 0, sptr)
+        for i in range(5):
+            rc = call(i)
+            assert rc == 0, api.status_string(rc)
+        torch.cuda.synchronize()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        n = max(10, args.steps // 4)
+        e0.record(stream)
+        for i in range(n):
+            call(i)
+        e1.record(stream)
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / n
+        nb = rows * cols * 4 + rows * 4
+        want = xs[(n - 1) % 3].view(rows, cols).double().pow(2).sum(dim=1).sqrt()
+        ok = bool(torch.allclose(out.double(), want, rtol=1e-5, atol=1e-5))
+        return dict(workload=f"L2 row norm fp32 {rows}x{cols} ({what})",
+                    ms_per_step=ms, alg_bytes=nb, GBps=nb / (ms * 1e-3) / 1e9,
+                    pct_of_peak=100.0 * nb / (ms * 1e-3) / 1e9 / PEAK_HBM_GBPS,
+                    check={"torch_fp64": ok})
+
     def extra_cov():
         # covariance of config 3's matrix around its column means: the one contraction on the
         # path (matrix cores).  Two bounds: HBM (the matrix once + D^2 outputs) and the fp32
@@ -696,6 +726,8 @@ def main():
     extras = ({"row_normalize": extra_row_normalize(), "row_normalize_129": extra_row_normalize(1000000, 129),
                "meanvar": extra_meanvar(),
                "wide_columns": extra_wide_columns(), "dense_rows": extra_dense_rows(),
+               "rows_of_3": extra_rows(40000000, 3, "rows shorter than a vector, through LDS"),
+               "rows_of_1100": extra_rows(120000, 1100, "one trip of five loads per thread"),
                "cov": extra_cov()}
               if args.configs == "all" else {})
     # One short line: the contract's keys, and inside `roofline` / `config` / `cpu_baseline`

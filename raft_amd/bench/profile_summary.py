@@ -207,6 +207,10 @@ def extras(out: Path, commit: str):
              "fold_rows_kernel<rmi::PolF<float, 0, 0>", 32768 * 4097 * 4 + 4097 * 4),
             ("row sum fp32 2000000x66 (dense slots)", "row_dense_kernel<rmi::PolF<float, 0, 0>", None,
              2000000 * 67 * 4),
+            ("L2 row norm fp32 40000000x3 (rows through LDS)", "row_small_kernel<rmi::PolF<float, 1, 0>", None,
+             40000000 * 4 * 4),
+            ("L2 row norm fp32 120000x1100 (one trip, 5 loads)", "row_block_kernel<rmi::PolF<float, 1, 0>", None,
+             120000 * 1101 * 4),
             ("stats::cov fp32 10000000x64 (data read only)", "gram_rows_kernel<float, true, true, false, true>",
              "cov_fold_kernel<float>", 2560016384),
             ("stats::cov fp32 10000000x64 (data centred in place)", "gram_rows_kernel<float, true, true, true, true>",
@@ -229,7 +233,8 @@ def extras(out: Path, commit: str):
     w("single timed calls, so launch counts include those):")
     for n, r in kt.items():
         if "rmi::" in n and "normalize" not in n and "MeanVar" not in n and "col_wide" not in n \
-                and "fold_rows" not in n and "row_dense" not in n and "cov::" not in n:
+                and "fold_rows" not in n and "row_dense" not in n and "cov::" not in n \
+                and "row_small" not in n:
             w(f"  {n[:100]:100s} {r['Calls']:>6s} {float(r['AverageNs']):12.1f}")
     (ROOT / "profiles" / "row_normalize_meanvar_rocprofv3.txt").write_text("\n".join(lines) + "\n")
     print("\n".join(lines[:16]))
