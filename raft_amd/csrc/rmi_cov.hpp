@@ -1101,10 +1101,11 @@ __global__ __launch_bounds__(kThreads) void gram_cols_kernel(GramArgs a)
   static_assert(ONE || !CENTER, "the centred data is written back by the one-block kernel only");
   if constexpr (std::is_same_v<T, float>) {
     if (ONE || bi == bj) {
-      // plain loads: the eight 16-byte pieces of a column's line are read by eight
-      // instructions, and a streamed line may be gone before the next piece is asked for
-      // (10M x 64: 500 -> 450 us)
-      gram_cols_body_bf16<true, CENTER, false, FULL>(a, unit, slab, bi, bj, sm);
+      // (streamed loads where the units are loaded line by line, i.e. the one-block kernel that
+      // does not write the data back: 10M x 64 437 -> 429 us; in the operand layout, where the
+      // eight 16-byte pieces of a column's line are read by eight instructions, a streamed line
+      // may be gone before the next piece is asked for: 450 -> 500 us)
+      gram_cols_body_bf16<true, CENTER, ONE && !CENTER, FULL>(a, unit, slab, bi, bj, sm);
     } else {
       if constexpr (!ONE) gram_cols_body_bf16<false, false, false>(a, unit, slab, bi, bj, sm);
     }
