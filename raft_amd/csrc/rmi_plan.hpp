@@ -47,6 +47,15 @@ constexpr int kPlanSmallBytes = 16384;  // ROW_WAVE, small rows: bytes of a work
 #ifndef RMI_COL_GROUP_OFF_WORDS
 #define RMI_COL_GROUP_OFF_WORDS 1
 #endif
+#ifndef RMI_SPLIT_FINE
+#define RMI_SPLIT_FINE 1
+#endif
+
+// ROW_SPLIT: long rows are cut into pieces of at least this many vectors (64 KB; twice that for
+// the mean-and-variance accumulators, whose merges at a workgroup's end cost more), at most
+// kSplitMaxPieces of them, also where fewer pieces would fill the machine's wave slots
+constexpr int64_t kSplitPieceVecs = 4096;
+constexpr int64_t kSplitMaxPieces = 32;
 constexpr int64_t kGroupMaxRowBytes = 130;  // COL_TILE: longest row that is read in groups
 constexpr int64_t kGroupMinLen = 256;  // COL_TILE: fewest row groups worth reading rows in groups
 constexpr int kLdsPerCu       = 160 * 1024;  // LDS bytes of one gfx950 CU
@@ -252,6 +261,24 @@ inline int classify(const rmi_reduce_desc& d, PolicyKey& key, int& acc_bytes)
 }
 
 // Shape -> plan.  desc.plan_hint forces a plan kind where it applies to the shape.
+// Few long rows on wide teams: `cap` teams are resident at once, and the teams of a last,
+// partly filled round each run at what their own loads in flight allow (a 1024-thread team
+// alone reads ~ 60 GB/s), so 525 rows take as long as 1024.  Rows of at least four pieces are
+// split instead (2 GB of fp32, 525 / 600 / 900 / 1300 / 1800 rows: 68 / 81 / 80 / 75 / 76 -> 82 / 86 /
+// 84 / 84 / 84 % of 8 TB/s; the mean-and-variance accumulators 512 MB, 525 / 900 / 1300 rows: 58 /
+// 63 / 68 -> 74 / 73 / 73 %; 512, 1024 and 2047 rows, whose rounds are full, stay whole: 86-88 %,
+// and so do last rounds that are nine tenths full).  Shorter rows get teams of half the width,
+// which all fit at once (128 MB, 525 / 768 / 1000 rows: 60 / 66 / 64 -> 64 / 72 / 76 %,
+// mean and variance 1000 / 1536 / 2047 rows: 34 / 44 / 39 -> 51 / 58 / 60 %; on rows long enough
+// to split, the half-filled machine measured 3-5 points slower than the wide teams).
+enum : int { kTailKeep = 0, kTailSplit = 1, kTailNarrow = 2 };
+inline int tail_round_rule(int64_t n_rows, int64_t cap, int64_t nvec, int64_t piece)
+{
+  if (cap < 1 || n_rows <= cap || n_rows % cap == 0) return kTailKeep;
+  if (nvec / piece < 4) return kTailNarrow;
+  return (n_rows % cap) * 10 < cap * 9 ? kTailSplit : kTailKeep;
+}
+
 inline int make_plan(const rmi_reduce_desc& d,
                      const PolicyKey& key,
                      int acc_bytes,
@@ -472,6 +499,7 @@ inline int make_plan(const rmi_reduce_desc& d,
   if (kind == RMI_PLAN_ROW_LANES || kind == RMI_PLAN_COL_TILE || kind == RMI_PLAN_EMPTY)
     kind = RMI_PLAN_AUTO;
   int threads = 64;
+  const int64_t split_piece = key.family == kFamMeanVar ? 2 * kSplitPieceVecs : kSplitPieceVecs;
   if (kind == RMI_PLAN_AUTO) {
     if (nload <= 4 * 64) {
       kind = RMI_PLAN_ROW_WAVE;
@@ -508,6 +536,11 @@ inline int make_plan(const rmi_reduce_desc& d,
         kind = RMI_PLAN_ROW_SPLIT;
       } else {
         kind = RMI_PLAN_ROW_BLOCK;
+        if (RMI_SPLIT_FINE != 0 && threads >= 512) {
+          const int rule = tail_round_rule(p.n_out, slots / (threads / 64), p.nvec, split_piece);
+          if (rule == kTailSplit) kind = RMI_PLAN_ROW_SPLIT;
+          if (rule == kTailNarrow) threads /= 2;
+        }
       }
     }
   } else if (kind == RMI_PLAN_ROW_BLOCK) {
@@ -727,6 +760,16 @@ inline int make_plan(const rmi_reduce_desc& d,
     int64_t B             = ceildiv(slots, p.n_out * (kPlanBlock / 64));
     const int64_t maxB    = p.nvec / quantum > 1 ? p.nvec / quantum : 1;
     if (B > maxB) B = maxB;
+    if (RMI_SPLIT_FINE != 0) {
+      // More pieces than the wave slots ask for: the workgroups of the last round, which run
+      // with the machine partly empty, are shorter (1 GB of fp32, 200 / 400 / 500 rows: 80 / 80 /
+      // 79 -> 83 / 84 / 82 % of 8 TB/s).
+      int64_t fine = p.nvec / split_piece;
+      if (fine > kSplitMaxPieces) fine = kSplitMaxPieces;
+      const bool fits = (d.flags & kFlagSmallWorkspace) == 0 ||
+                        kTicketBytes + (size_t)(p.n_out * fine) * acc_bytes <= RMI_NOALLOC_SCRATCH_BYTES;
+      if (fine > B && fits) B = fine;
+    }
     if (B < 2) B = 2;
     if (B > 4096) B = 4096;
     p.chunk       = ceildiv(ceildiv(p.nvec, B), quantum) * quantum;

@@ -72,7 +72,8 @@ def test_reduce_thick(gpu, in_dt, out_dt, rows, cols):
 
 # Many long rows: the automatic plan gives each row a team of 64, 128 or 256 threads
 # depending on the row's length and the accumulator; lengths straddle the team sizes and
-# leave ragged last batches and tail elements.
+# leave ragged last batches and tail elements.  (1100 rows would leave a last round of 76
+# wide teams: rows of four 64 KB pieces and more are split instead.)
 @pytest.mark.parametrize("in_dt,out_dt,kw", [
     (api.F32, api.F32, dict(main_op=api.MAIN_SQ)),
     (api.F64, api.F64, {}),
@@ -89,8 +90,43 @@ def test_many_long_rows(gpu, in_dt, out_dt, kw, rows, cols):
     data = _rand(rng, in_dt, rows * cols)
     d = api.make_desc(in_dt, out_dt, rows, cols, **kw)
     p = api.plan_query(d)
-    assert p.kind in (api.PLAN_ROW_WAVE, api.PLAN_ROW_BLOCK) and p.passes == 1
+    if rows == 1100 and p.kind == api.PLAN_ROW_SPLIT:
+        assert p.blocks_per_out >= 3 and cols * api.DTYPE_SIZE[in_dt] >= 4 * 65536
+    else:
+        assert p.kind in (api.PLAN_ROW_WAVE, api.PLAN_ROW_BLOCK) and p.passes == 1
     u.check_against_oracle(d, data, label=f"long rows {rows}x{cols} dt{in_dt}")
+
+
+# Row counts that would leave a partly filled last round of wide teams: rows of four 64 KB
+# pieces and more are split (with and without the single-launch fold), shorter ones get
+# teams of half the width; row counts that fill their rounds stay whole.
+@pytest.mark.parametrize("in_dt,out_dt,kw", [
+    (api.F32, api.F32, dict(main_op=api.MAIN_SQ, final_op=api.FIN_SQRT)),
+    (api.BF16, api.F32, {}),
+    (api.F64, api.F64, {}),
+    (api.I8, api.I64, dict(main_op=api.MAIN_ABS)),
+    (api.F32, api.KVP_I32_F32, dict(main_op=api.MAIN_KVP, reduce_op=api.RED_ARGMIN, init_f=np.inf)),
+])
+@pytest.mark.parametrize("rows,row_bytes,kind,threads", [
+    (525, 262144 + 52, api.PLAN_ROW_SPLIT, 256), (1100, 300000, api.PLAN_ROW_SPLIT, 256),
+    (1800, 262144, api.PLAN_ROW_SPLIT, 256),
+    (525, 140008, api.PLAN_ROW_BLOCK, 512), (1000, 140000, api.PLAN_ROW_BLOCK, 512),
+    (1300, 100000, api.PLAN_ROW_BLOCK, 256), (2047, 70000, api.PLAN_ROW_BLOCK, 256),
+    (512, 140000, api.PLAN_ROW_BLOCK, 1024), (1024, 300000, api.PLAN_ROW_BLOCK, 512),
+    (1000, 300000, api.PLAN_ROW_BLOCK, 1024),
+])
+def test_tail_round_rows(gpu, in_dt, out_dt, kw, rows, row_bytes, kind, threads):
+    es = api.DTYPE_SIZE[in_dt]
+    cols = row_bytes // es
+    rng = np.random.default_rng(rows + row_bytes + in_dt)
+    data = _rand(rng, in_dt, rows * cols)
+    for flags in (0, api.FLAG_WORKSPACE_ZEROED):
+        d = api.make_desc(in_dt, out_dt, rows, cols, flags=flags, **kw)
+        p = api.plan_query(d)
+        assert (p.kind, p.block_threads) == (kind, threads), (p.kind, p.block_threads, p.blocks_per_out)
+        if kind == api.PLAN_ROW_SPLIT:
+            assert 3 <= p.blocks_per_out <= 32
+        u.check_against_oracle(d, data, label=f"tail round {rows}x{cols} dt{in_dt} flags{flags}")
 
 
 # Rows that do not fill 128-byte lines, or that start off a line: the wave-per-row plan
