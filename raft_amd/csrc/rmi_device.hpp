@@ -641,7 +641,8 @@ struct PolKvp {
 // shift inside the data's range the subtraction loses a few bits at most, and an
 // element costs three f64 operations and no division.  Two states merge by the
 // pairwise update of Chan et al. that the reference's mean_var monoid uses
-// (stats/detail/meanvar.cuh:16-99); the merged state is stored with k = mean, sd = 0.
+// (stats/detail/meanvar.cuh:16-99), the merged state stored with k = mean, sd = 0; sets
+// of up to kMvReshiftMax values together merge by moving one's sums to the other's shift.
 struct mv_t {
   double w;
   double k;
@@ -657,6 +658,11 @@ __device__ __forceinline__ double mv_m2(const mv_t& a)
 {
   return a.w > 0.0 ? fmax(a.sdd - a.sd * a.sd / a.w, 0.0) : 0.0;
 }
+
+#ifndef RMI_MV_RESHIFT
+#define RMI_MV_RESHIFT 1
+#endif
+constexpr double kMvReshiftMax = 65536.0;  // largest merged set that keeps a member's shift
 
 template <class InT>
 struct PolMeanVar {
@@ -714,14 +720,32 @@ struct PolMeanVar {
   static __device__ __forceinline__ void merge(acc_t& a, const acc_t& b)
   {
     const double cw = a.w + b.w;
-    const double ma = mv_mean(a), mb = mv_mean(b);
-    const double sa = mv_m2(a), sb = mv_m2(b);
-    const double fb = cw > 0.0 ? b.w / cw : 0.0;
-    const double d  = mb - ma;
-    a.k             = ma + d * fb;
-    a.sdd           = (sa + sb) + d * d * (a.w * fb);
-    a.sd            = 0.0;
-    a.w             = cw;
+    double k, sd, sdd;
+    if (RMI_MV_RESHIFT != 0 && cw <= kMvReshiftMax) {
+      // Small sets: b's sums are moved to a's shift, sum(x - ka) = sd_b + w_b d and
+      // sum((x - ka)^2) = sdd_b + 2 d sd_b + w_b d^2 with d = kb - ka, which takes no
+      // division (the pairwise update takes three: six of them per row cost more than
+      // reading a row of 671 floats).  The shift stays a value of the set, so
+      // (mean - k)^2 <= w var and the subtraction in mv_m2 loses at most log2(w) bits
+      // of the 53.
+      k                = a.w == 0.0 ? b.k : a.k;
+      const double d   = b.k - k;
+      const double bwd = b.w * d;
+      sdd              = a.sdd + fma(d, 2.0 * b.sd + bwd, b.sdd);
+      sd               = a.sd + (b.sd + bwd);
+    } else {
+      const double ma = mv_mean(a), mb = mv_mean(b);
+      const double sa = mv_m2(a), sb = mv_m2(b);
+      const double fb = cw > 0.0 ? b.w / cw : 0.0;
+      const double d  = mb - ma;
+      k               = ma + d * fb;
+      sdd             = (sa + sb) + d * d * (a.w * fb);
+      sd              = 0.0;
+    }
+    a.k   = k;
+    a.sd  = sd;
+    a.sdd = sdd;
+    a.w   = cw;
   }
   template <int SEL>
   static __device__ __forceinline__ acc_t exchange(const acc_t& a)
