@@ -88,6 +88,20 @@ def test_shifted_data(gpu, layout):
     _check(api.F32, layout, rows, cols, True, stored)
 
 
+@pytest.mark.parametrize("layout", [api.ROW_MAJOR, api.COL_MAJOR])
+@pytest.mark.parametrize("rows,cols", [(671, 3000), (6710, 700), (60000, 40), (200000, 12)])
+def test_outlier_first_sample(gpu, layout, rows, cols):
+    """The worst case for sums that are shifted by a member of the set: every column's first
+    sample lies a million standard deviations off.  Sets of up to 65536 values merge by moving
+    their sums to one shift, which may cost log2(w) of the 53 bits; larger ones merge
+    pairwise."""
+    m = np.random.default_rng(rows + cols).normal(0.0, 1.0, (rows, cols))
+    m[0, :] = 1e6
+    for dt, tol in ((api.F64, 1e-8), (api.F32, 1e-5)):
+        stored = np.ascontiguousarray((m if layout == api.ROW_MAJOR else m.T).astype(NP[dt]))
+        _check(dt, layout, rows, cols, True, stored, tol=tol)
+
+
 def test_constant_columns(gpu):
     rows, cols = 10000, 40
     stored = np.full((rows, cols), 3.25, dtype=np.float32)
