@@ -54,6 +54,8 @@ struct RowArgs {
                    // line; the workgroup that takes a row's last ticket folds its partials
                    // (nullptr: a second launch does)
   int LB;          // ... with LB lanes (a power of two <= 64), as fold_kernel would
+  int head_skip;   // row_block_kernel, 1- and 2-byte elements: rows are read from their
+                   // first whole 32-bit word on, the elements before it by the first thread
   int chunk_rows;  // row_flat_kernel: whole rows of a workgroup's chunk; logG: log2 of the lanes
   float inv_row_bytes;  // ... that fold one row, and 1 / row_bytes
   Epilogue epi;
@@ -606,6 +608,17 @@ template <class P, bool COHERENT = false>
 __device__ __forceinline__ typename P::acc_t fold_lane(const typename P::acc_t* p, int B, int LB,
                                                        int lb);
 
+// A stored element as the type the policies accumulate.
+template <class T>
+__device__ __forceinline__ typename In<T>::nat stored_to_nat(const T& v)
+{
+  if constexpr (std::is_same_v<T, bf16_t>) {
+    return as_f32((u32)v.bits << 16);
+  } else {
+    return (typename In<T>::nat)v;
+  }
+}
+
 // ---------------------------------------------------------------------------
 // Teams of T = 64 << logT threads (1..16 waves); each team sweeps one chunk of
 // one row in batches of kTeamUnroll loads per lane.  A workgroup holds
@@ -640,16 +653,39 @@ __global__ __launch_bounds__(1024) void row_block_kernel(RowArgs a)
 
   acc_t acc = P::neutral();
   if (live) {
-    const i64 v0   = (i64)b * a.chunk;
-    const i64 v1   = (v0 + a.chunk < a.nvec) ? (v0 + a.chunk) : a.nvec;
     const char* rp = static_cast<const char*>(a.in) + row * a.row_bytes;
+    i64 nvec = a.nvec, len = a.len;
+    int tail = a.tail;
+    // Rows that start off a 32-bit word are read from their next whole word on; the one to
+    // three elements before it go to the first thread of the row's first chunk, which loads
+    // them here, ahead of its vectors, and accumulates them after those (used first, they
+    // would add a trip to memory to every row).
+    constexpr bool kHead = VEC16 && sizeof(typename P::in_t) < 4 && P::CLS != kClsKvp;
+    constexpr int kHeadMax = kHead ? 4 / (int)sizeof(typename P::in_t) - 1 : 1;
+    [[maybe_unused]] typename P::in_t hv[kHeadMax];
+    [[maybe_unused]] int he = 0;
+    if constexpr (kHead) {
+      using in_t       = typename P::in_t;
+      constexpr int es = (int)sizeof(in_t);
+      const int skip = a.head_skip != 0 ? (int)((4 - (reinterpret_cast<uintptr_t>(rp) & 3)) & 3) / es : 0;
+      he             = (t == 0 && b == 0) ? skip : 0;
+#pragma unroll
+      for (int j = 0; j < kHeadMax; ++j)
+        if (j < he) hv[j] = reinterpret_cast<const in_t*>(rp)[j];
+      rp += skip * es;
+      len -= skip;
+      nvec = len / P::VEC;
+      tail = (int)(len - nvec * P::VEC);
+    }
+    const i64 v0   = (i64)b * a.chunk;
+    const i64 v1   = (v0 + a.chunk < nvec) ? (v0 + a.chunk) : nvec;
     // `vb` is the first lane-load of the team's next batch: every loop condition below
     // is the same for all lanes of the team, so a wave follows one path (a per-lane
     // condition would send the lanes with one more whole batch through a loop and the
     // others through the last batch, one after the other).
     i64 vb = v0;
     // the chunk's lane-loads, the row's tail elements counting as one more for the last chunk
-    const i64 vend = v1 + ((a.tail > 0 && b == a.B - 1) ? 1 : 0);
+    const i64 vend = v1 + ((tail > 0 && b == a.B - 1) ? 1 : 0);
     // A chunk of at most 2 * U + 1 lane-loads per thread makes ONE trip to memory, whatever its
     // length: every load is issued before the first is used, positions past the chunk re-read
     // its last vector.  (Whole batches first and the rest behind them made two or three
@@ -712,7 +748,12 @@ __global__ __launch_bounds__(1024) void row_block_kernel(RowArgs a)
     // overlapping last vector of the row among them
     if (vb < vend)
       last_batch_n9<P, VEC16, i64>((int)((vend - vb + T - 1) >> (6 + a.logT)), acc, rp, vb + t, (i64)T,
-                                   vend, a.nvec, a.len, a.tail);
+                                   vend, nvec, len, tail);
+    if constexpr (kHead) {
+#pragma unroll
+      for (int j = 0; j < kHeadMax; ++j)
+        if (j < he) P::push(acc, stored_to_nat<typename P::in_t>(hv[j]), (i64)j);
+    }
   }
 
   wave_allreduce<P>(acc);
@@ -1088,15 +1129,6 @@ __global__ __launch_bounds__(kBlock) void row_dense_kernel(RowArgs a)
 // ---------------------------------------------------------------------------
 constexpr int kSmallVecs  = 4;                    // vectors per thread
 constexpr int kSmallBytes = kBlock * kSmallVecs * 16;  // bytes of a workgroup's chunk at most
-template <class T>
-__device__ __forceinline__ typename In<T>::nat stored_to_nat(const T& v)
-{
-  if constexpr (std::is_same_v<T, bf16_t>) {
-    return as_f32((u32)v.bits << 16);
-  } else {
-    return (typename In<T>::nat)v;
-  }
-}
 template <class P>
 __global__ __launch_bounds__(kBlock) void row_small_kernel(RowArgs a)
 {

@@ -93,6 +93,7 @@ int run(const PlanX& pl, const Problem& pr, hipStream_t st)
       a.logG    = pl.logG;
       a.B       = pl.B;
       a.logT    = ilog2(pl.threads / 64);
+      a.head_skip = pl.head_skip ? 1 : 0;
       a.epi     = pr.epi;
       const dim3 grid((unsigned)pl.grid_blocks);
       const unsigned lds = (unsigned)pl.lds_reserve;

@@ -50,6 +50,9 @@ constexpr int kPlanSmallBytes = 16384;  // ROW_WAVE, small rows: bytes of a work
 #ifndef RMI_SPLIT_FINE
 #define RMI_SPLIT_FINE 1
 #endif
+#ifndef RMI_HEAD_SKIP
+#define RMI_HEAD_SKIP 1
+#endif
 
 // ROW_SPLIT: long rows are cut into pieces of at least this many vectors (64 KB; twice that for
 // the mean-and-variance accumulators, whose merges at a workgroup's end cost more), at most
@@ -89,6 +92,9 @@ struct PlanX {
   bool vec16      = false;  // 16-byte lane loads
   bool short_rows = false;  // ROW_WAVE served by the one-load-per-lane kernel
   bool any_g      = false;  // short_rows with G = the row's lane-load count (not a power of two)
+  bool head_skip  = false;  // team kernel, rows of 1- or 2-byte elements: a row that starts
+                            // off a 32-bit word gives its first one to three elements to the
+                            // team's first thread and is read from the next whole word on
   bool dense_rows = false;  // ROW_WAVE: G = the row's lane-load count, a workgroup's load slots
                             // dealt over whole adjacent rows, rows combined through LDS
   bool flat_rows  = false;  // ROW_WAVE: the matrix is read as a flat run of aligned vectors, chunks
@@ -500,6 +506,8 @@ inline int make_plan(const rmi_reduce_desc& d,
     kind = RMI_PLAN_AUTO;
   int threads = 64;
   const int64_t split_piece = key.family == kFamMeanVar ? 2 * kSplitPieceVecs : kSplitPieceVecs;
+  const bool head_skip      = RMI_HEAD_SKIP != 0 && p.vec16 && es < 4 && key.family != kFamKvp &&
+                         ((row_bytes % 4) != 0 || (in_misalign % 4) != 0);
   if (kind == RMI_PLAN_AUTO) {
     if (nload <= 4 * 64) {
       kind = RMI_PLAN_ROW_WAVE;
@@ -740,6 +748,10 @@ inline int make_plan(const rmi_reduce_desc& d,
     p.threads     = threads;
     p.B           = 1;
     p.chunk       = p.nvec;
+    // 16-byte loads from addresses that are no multiples of four run at two thirds of the
+    // rate of the others (bf16 rows of odd length, every second of which starts 2 bytes off:
+    // D = 10531 ... 68709 56-63 % of 8 TB/s, even lengths 72-74 %)
+    p.head_skip = head_skip;
     const int teams = threads >= kPlanBlock ? 1 : kPlanBlock / threads;
     p.grid_blocks   = ceildiv(p.n_out, teams);
     if (threads <= kPlanBlock && p.vec16 && p.grid_blocks > (int64_t)8 * n_cu) {
@@ -756,6 +768,7 @@ inline int make_plan(const rmi_reduce_desc& d,
     p.kind        = RMI_PLAN_ROW_SPLIT;
     p.team_kernel = true;
     p.threads     = kPlanBlock;
+    p.head_skip   = head_skip;
     const int64_t quantum = (int64_t)kPlanBlock * 8;
     int64_t B             = ceildiv(slots, p.n_out * (kPlanBlock / 64));
     const int64_t maxB    = p.nvec / quantum > 1 ? p.nvec / quantum : 1;

@@ -97,6 +97,19 @@ def test_many_long_rows(gpu, in_dt, out_dt, kw, rows, cols):
     u.check_against_oracle(d, data, label=f"long rows {rows}x{cols} dt{in_dt}")
 
 
+def _same_with_zeroed_workspace(d, data, first, misalign_elems=0):
+    """The same reduction with RMI_FLAG_WORKSPACE_ZEROED and a zeroed workspace (split rows
+    then fold in the same launch where the ticket lines suffice): bit-identical, twice."""
+    import torch
+    d2 = api.ReduceDesc.from_buffer_copy(d)
+    d2.flags = api.FLAG_WORKSPACE_ZEROED
+    ws = torch.zeros(max(api.plan_query(d2).workspace_bytes, api.WORKSPACE_TICKET_BYTES),
+                     dtype=torch.uint8, device="cuda")
+    for _ in range(2):
+        again = u.gpu_reduce(d2, data, misalign_elems=misalign_elems, workspace=ws)
+        assert np.array_equal(np.asarray(first).view(np.uint8), np.asarray(again).view(np.uint8))
+
+
 # Row counts that would leave a partly filled last round of wide teams: rows of four 64 KB
 # pieces and more are split (with and without the single-launch fold), shorter ones get
 # teams of half the width; row counts that fill their rounds stay whole.
@@ -120,13 +133,38 @@ def test_tail_round_rows(gpu, in_dt, out_dt, kw, rows, row_bytes, kind, threads)
     cols = row_bytes // es
     rng = np.random.default_rng(rows + row_bytes + in_dt)
     data = _rand(rng, in_dt, rows * cols)
-    for flags in (0, api.FLAG_WORKSPACE_ZEROED):
-        d = api.make_desc(in_dt, out_dt, rows, cols, flags=flags, **kw)
-        p = api.plan_query(d)
-        assert (p.kind, p.block_threads) == (kind, threads), (p.kind, p.block_threads, p.blocks_per_out)
-        if kind == api.PLAN_ROW_SPLIT:
-            assert 3 <= p.blocks_per_out <= 32
-        u.check_against_oracle(d, data, label=f"tail round {rows}x{cols} dt{in_dt} flags{flags}")
+    d = api.make_desc(in_dt, out_dt, rows, cols, **kw)
+    p = api.plan_query(d)
+    assert (p.kind, p.block_threads) == (kind, threads), (p.kind, p.block_threads, p.blocks_per_out)
+    if kind == api.PLAN_ROW_SPLIT:
+        assert 3 <= p.blocks_per_out <= 32
+    first = u.check_against_oracle(d, data, label=f"tail round {rows}x{cols} dt{in_dt}")
+    _same_with_zeroed_workspace(d, data, first)
+
+
+# Long rows of 1- and 2-byte elements that start off a 32-bit word (odd lengths, inputs
+# shifted by one to three elements): the team kernel reads them from their next whole word
+# on and gives the elements before it to the row's first thread, whole rows and split ones,
+# sums (tails cleared), maxima (tails duplicated) and element-wise tails alike.
+@pytest.mark.parametrize("in_dt,out_dt,kw", [
+    (api.BF16, api.F32, {}),
+    (api.F16, api.F16, dict(main_op=api.MAIN_ABS, reduce_op=api.RED_MAX)),
+    (api.BF16, api.BF16, dict(main_op=api.MAIN_SQ, final_op=api.FIN_SQRT)),
+    (api.I8, api.I64, dict(main_op=api.MAIN_SQ)),
+    (api.I8, api.I32, dict(reduce_op=api.RED_MIN, init_i=127)),
+    (api.U8, api.I64, {}),
+    (api.BF16, api.KVP_I32_F32, dict(main_op=api.MAIN_KVP, reduce_op=api.RED_ARGMAX, init_f=-np.inf)),
+])
+@pytest.mark.parametrize("rows,cols,shift", [(37, 10531, 0), (37, 10531, 1), (300, 4689, 0), (64, 2071, 3),
+                                             (5, 262145, 0), (3, 300001, 1), (2, 1000003, 2),
+                                             (700, 70001, 0), (9, 1025, 1)])
+def test_long_rows_off_words(gpu, in_dt, out_dt, kw, rows, cols, shift):
+    rng = np.random.default_rng(rows + cols + shift + in_dt)
+    data = _rand(rng, in_dt, rows * cols)
+    d = api.make_desc(in_dt, out_dt, rows, cols, **kw)
+    first = u.check_against_oracle(d, data, misalign_elems=shift,
+                                   label=f"off words {rows}x{cols} dt{in_dt} +{shift}")
+    _same_with_zeroed_workspace(d, data, first, misalign_elems=shift)
 
 
 # Rows that do not fill 128-byte lines, or that start off a line: the wave-per-row plan
