@@ -616,15 +616,19 @@ def main():
                     pct_of_peak=100.0 * nb / (ms * 1e-3) / 1e9 / PEAK_HBM_GBPS,
                     check={"torch_fp64": ok})
 
-    def extra_rows(rows, cols, what):
-        # L2 norms of short or awkward rows: `what` names the kernel the planner takes
+    def extra_rows(rows, cols, what, l2=True):
+        # L2 norms (or plain sums) of short or awkward rows: `what` names the kernel the planner takes
         xs = [mk_normal(rows, cols, 17 + 7919 * i) for i in range(3)]
         out = torch.empty(rows, dtype=torch.float32, device="cuda")
-        d = api.make_desc(api.F32, api.F32, rows, cols, main_op=api.MAIN_SQ, final_op=api.FIN_SQRT)
+        d = (api.make_desc(api.F32, api.F32, rows, cols, main_op=api.MAIN_SQ, final_op=api.FIN_SQRT)
+             if l2 else api.make_desc(api.F32, api.F32, rows, cols))
         ref = C.byref(d)
+        nws = lib.rmi_reduce_workspace_bytes(ref)
+        ws = torch.empty(nws, dtype=torch.uint8, device="cuda") if nws else None
 
         def call(i):
-            return lib.rmi_reduce(ref, xs[i % 3].data_ptr(), out.data_ptr(), None, 0, sptr)
+            return lib.rmi_reduce(ref, xs[i % 3].data_ptr(), out.data_ptr(),
+                                  ws.data_ptr() if nws else None, nws, sptr)
         for i in range(5):
             rc = call(i)
             assert rc == 0, api.status_string(rc)
@@ -639,9 +643,10 @@ def main():
         torch.cuda.synchronize()
         ms = e0.elapsed_time(e1) / n
         nb = rows * cols * 4 + rows * 4
-        want = xs[(n - 1) % 3].view(rows, cols).double().pow(2).sum(dim=1).sqrt()
-        ok = bool(torch.allclose(out.double(), want, rtol=1e-5, atol=1e-5))
-        return dict(workload=f"L2 row norm fp32 {rows}x{cols} ({what})",
+        x64 = xs[(n - 1) % 3].view(rows, cols).double()
+        want = x64.pow(2).sum(dim=1).sqrt() if l2 else x64.sum(dim=1)
+        ok = bool(torch.allclose(out.double(), want, rtol=1e-5, atol=1e-5 if l2 else 1e-2))
+        return dict(workload=f"{'L2 row norm' if l2 else 'row sum'} fp32 {rows}x{cols} ({what})",
                     ms_per_step=ms, alg_bytes=nb, GBps=nb / (ms * 1e-3) / 1e9,
                     pct_of_peak=100.0 * nb / (ms * 1e-3) / 1e9 / PEAK_HBM_GBPS,
                     check={"torch_fp64": ok})
@@ -728,6 +733,7 @@ def main():
                "wide_columns": extra_wide_columns(), "dense_rows": extra_dense_rows(),
                "rows_of_3": extra_rows(40000000, 3, "rows shorter than a vector, through LDS"),
                "rows_of_1100": extra_rows(120000, 1100, "one trip of five loads per thread"),
+               "few_long_rows": extra_rows(525, 511305, "rows split: no partly filled last round of teams", l2=False),
                "cov": extra_cov()}
               if args.configs == "all" else {})
     # One short line: the contract's keys, and inside `roofline` / `config` / `cpu_baseline`

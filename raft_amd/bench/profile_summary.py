@@ -211,6 +211,8 @@ def extras(out: Path, commit: str):
              40000000 * 4 * 4),
             ("L2 row norm fp32 120000x1100 (one trip, 5 loads)", "row_block_kernel<rmi::PolF<float, 1, 0>", None,
              120000 * 1101 * 4),
+            ("row sum fp32 525x511305 (split rows)", "row_block_kernel<rmi::PolF<float, 0, 0>",
+             "fold_kernel<rmi::PolF<float, 0, 0>", 525 * 511306 * 4),
             ("stats::cov fp32 10000000x64 (data read only)", "gram_rows_kernel<float, true, true, false, true>",
              "cov_fold_kernel<float>", 2560016384),
             ("stats::cov fp32 10000000x64 (data centred in place)", "gram_rows_kernel<float, true, true, true, true>",

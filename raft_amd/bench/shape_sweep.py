@@ -58,6 +58,14 @@ def shapes(api):
         out.append((f"rows bf16 D={d}", bf16, f32, rows_of(d, 2), d, {}))
     for d in (4097, 5000):
         out.append((f"rows i8 D={d}", i8, api.I64, rows_of(d, 1), d, {}))
+    # few long rows: a last round of wide teams that would be partly filled (split rows, or
+    # teams of half the width where the rows are short)
+    for r, mb in ((525, 1024), (900, 1024), (1300, 1024), (1800, 1024), (525, 128), (1000, 128)):
+        d = (mb << 20) // (4 * r)
+        out.append((f"rows f32 {r}x{d}", f32, f32, r, d, {}))
+    # long 16-bit rows of odd length (every second row starts 2 bytes off a 32-bit word)
+    for d in (13593, 50337, 262145):
+        out.append((f"rows bf16 D={d}", bf16, f32, rows_of(d, 2), d, {}))
     for d in (9, 17, 25, 33, 35, 63, 65, 67, 129):
         out.append((f"rows f64 D={d}", f64, f64, 2_000_000, d, {}))
     for d in (33, 36, 65, 66, 76, 100, 129, 130, 132, 250, 260, 513):
