@@ -17,6 +17,8 @@ long wide_plans = 0;
 long dense_plans = 0;
 long flat_plans = 0;
 long small_plans = 0;
+long wide_team_plans = 0;
+long tail_split_plans = 0;
 #define REQUIRE(cond)                                                              \
   do {                                                                             \
     if (!(cond)) {                                                                 \
@@ -153,11 +155,24 @@ void check(const rmi_reduce_desc& d, int n_cu, uintptr_t in_misalign)
     case RMI_PLAN_ROW_BLOCK:
       REQUIRE(!p.strided && p.team_kernel && p.B == 1 && p.chunk == p.nvec);
       REQUIRE(p.threads >= 64 && p.threads <= 1024 && (p.threads & (p.threads - 1)) == 0);
+      if (d.plan_hint == RMI_PLAN_AUTO && p.threads >= 512) {
+        // wide teams either fit at once, fill their rounds, or leave a last round that is nine
+        // tenths full on rows long enough to split (shorter rows get narrower teams)
+        ++wide_team_plans;
+        const int64_t cap  = (int64_t)n_cu * rmi::kWavesPerCu / (p.threads / 64);
+        const int64_t last = p.n_out % cap;
+        REQUIRE(p.n_out <= cap || last == 0 || (last * 10 >= cap * 9 && p.nvec / rmi::kSplitPieceVecs >= 4));
+      }
       break;
     case RMI_PLAN_ROW_SPLIT:
       REQUIRE(!p.strided && p.team_kernel && p.B >= 2 && p.threads == kPlanBlock);
       REQUIRE(p.chunk > 0 && (int64_t)p.B * p.chunk >= p.nvec && (int64_t)(p.B - 1) * p.chunk < p.nvec);
       REQUIRE(p.grid_blocks == p.n_out * p.B);
+      // rows split for their last round: pieces of 64 KB and more, at most 32 of them
+      if (d.plan_hint == RMI_PLAN_AUTO && p.n_out * 16 >= (int64_t)n_cu * rmi::kWavesPerCu) {
+        ++tail_split_plans;
+        REQUIRE(p.B <= rmi::kSplitMaxPieces && p.chunk >= rmi::kSplitPieceVecs);
+      }
       break;
     case RMI_PLAN_COL_TILE:
       REQUIRE(p.strided);
@@ -218,6 +233,11 @@ void check(const rmi_reduce_desc& d, int n_cu, uintptr_t in_misalign)
       break;
     default: REQUIRE(false);
   }
+  // rows read from their first whole 32-bit word on: team kernel, 1- and 2-byte elements, no
+  // element indices
+  if (p.head_skip)
+    REQUIRE(p.team_kernel && p.vec16 && es < 4 && key.family != rmi::kFamKvp &&
+            (p.row_bytes % 4 != 0 || in_misalign % 4 != 0));
   rmi_plan out{};
   export_plan(p, out);
   REQUIRE(out.n_outputs == p.n_out && out.reduce_len == p.len && out.workspace_bytes == p.ws_bytes);
@@ -282,6 +302,20 @@ int main()
           check(d, 256, mis);
           ++cases;
         }
+  // few long rows: every row count from 500 to 2100 at three row lengths
+  for (int64_t rows = 500; rows <= 2100; ++rows)
+    for (int64_t cols : {(int64_t)20000, (int64_t)70001, (int64_t)524288})
+      for (int dt : {RMI_F32, RMI_BF16}) {
+        rmi_reduce_desc d{};
+        d.in_dtype  = dt;
+        d.out_dtype = RMI_F32;
+        d.reduce_op = RMI_RED_ADD;
+        d.n_rows    = rows;
+        d.n_cols    = cols;
+        d.flags     = rows % 2 ? RMI_FLAG_WORKSPACE_ZEROED : 0;
+        check(d, 256, rows % 3 == 0 ? 2 : 0);
+        ++cases;
+      }
   // the extremes the header promises to reject
   {
     rmi_reduce_desc d{};
@@ -310,6 +344,11 @@ int main()
   }
   if (wide_plans < 1000) {
     std::printf("  whole-row column plans were hardly exercised (%ld)\n", wide_plans);
+    ++failures;
+  }
+  if (wide_team_plans < 500 || tail_split_plans < 500) {
+    std::printf("  plans of few long rows were hardly exercised (%ld wide teams, %ld splits)\n", wide_team_plans,
+                tail_split_plans);
     ++failures;
   }
   if (small_plans < 1000) {
