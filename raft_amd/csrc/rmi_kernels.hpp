@@ -608,6 +608,9 @@ template <class P, bool COHERENT = false>
 __device__ __forceinline__ typename P::acc_t fold_lane(const typename P::acc_t* p, int B, int LB,
                                                        int lb);
 
+#ifndef RMI_HEAD_SKIP
+#define RMI_HEAD_SKIP 1
+#endif
 // A stored element as the type the policies accumulate.
 template <class T>
 __device__ __forceinline__ typename In<T>::nat stored_to_nat(const T& v)
@@ -660,7 +663,7 @@ __global__ __launch_bounds__(1024) void row_block_kernel(RowArgs a)
     // three elements before it go to the first thread of the row's first chunk, which loads
     // them here, ahead of its vectors, and accumulates them after those (used first, they
     // would add a trip to memory to every row).
-    constexpr bool kHead = VEC16 && sizeof(typename P::in_t) < 4 && P::CLS != kClsKvp;
+    constexpr bool kHead = RMI_HEAD_SKIP != 0 && VEC16 && sizeof(typename P::in_t) < 4 && P::CLS != kClsKvp;
     constexpr int kHeadMax = kHead ? 4 / (int)sizeof(typename P::in_t) - 1 : 1;
     [[maybe_unused]] typename P::in_t hv[kHeadMax];
     [[maybe_unused]] int he = 0;

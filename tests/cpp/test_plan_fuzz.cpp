@@ -237,7 +237,7 @@ void check(const rmi_reduce_desc& d, int n_cu, uintptr_t in_misalign)
   // element indices
   if (p.head_skip)
     REQUIRE(p.team_kernel && p.vec16 && es < 4 && key.family != rmi::kFamKvp &&
-            (p.row_bytes % 4 != 0 || in_misalign % 4 != 0));
+            (p.row_bytes % 4 != 0 || in_misalign % 4 != 0) && (es == 2 || p.nvec >= 512));
   rmi_plan out{};
   export_plan(p, out);
   REQUIRE(out.n_outputs == p.n_out && out.reduce_len == p.len && out.workspace_bytes == p.ws_bytes);
