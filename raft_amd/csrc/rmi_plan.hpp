@@ -53,6 +53,12 @@ constexpr int kPlanSmallBytes = 16384;  // ROW_WAVE, small rows: bytes of a work
 #ifndef RMI_HEAD_SKIP
 #define RMI_HEAD_SKIP 1
 #endif
+#ifndef RMI_TEAM_WG_ONE_TRIP
+#define RMI_TEAM_WG_ONE_TRIP 6
+#endif
+#ifndef RMI_TEAM_OT_LOADS
+#define RMI_TEAM_OT_LOADS 7
+#endif
 
 // ROW_SPLIT: long rows are cut into pieces of at least this many vectors (64 KB; twice that for
 // the mean-and-variance accumulators, whose merges at a workgroup's end cost more), at most
@@ -759,12 +765,18 @@ inline int make_plan(const rmi_reduce_desc& d,
     if (threads <= kPlanBlock && p.vec16 && p.grid_blocks > (int64_t)8 * n_cu) {
       // More workgroups than fit at once: the resident 256-thread workgroups per CU are
       // capped by a dynamic LDS reservation the kernel never touches.  4 keep 64-128 KB
-      // in flight per CU, which measured best across row lengths and accumulators; 3
+      // in flight per CU, which measured best for rows of several batches per thread; 3
       // gain another 3 points for sums over rows of 128 KB and more (eight or more
-      // batches per thread) and lose 20 on arg-reductions.
+      // batches per thread) and lose 20 on arg-reductions.  Rows read in one trip of at most
+      // seven loads per thread have less in flight per workgroup and no second batch to
+      // overlap their arithmetic with: 6 (as many as their registers allow) gain 7-10 points
+      // (fp32 D = 1100 76 -> 85 % of 8 TB/s, fp64 D = 600 73 -> 81, bf16 D = 4786 / 10530 72 / 75
+      // -> 81 / 85, int8 D = 20000 78 -> 84, arg-max D = 1100 75 -> 85), with eight or nine loads
+      // per thread they lose 2.
       const bool deep = threads == kPlanBlock && key.family != kFamKvp &&
                         p.nvec >= (int64_t)8 * kPlanTeamUnroll * kPlanBlock;
-      p.lds_reserve   = kLdsPerCu / (deep ? 3 : 4) - 768;
+      const bool one_trip = nload <= (int64_t)RMI_TEAM_OT_LOADS * threads;
+      p.lds_reserve       = kLdsPerCu / (deep ? 3 : one_trip ? RMI_TEAM_WG_ONE_TRIP : 4) - 768;
     }
   } else {
     p.kind        = RMI_PLAN_ROW_SPLIT;
