@@ -53,6 +53,9 @@ constexpr int kPlanSmallBytes = 16384;  // ROW_WAVE, small rows: bytes of a work
 #ifndef RMI_HEAD_SKIP
 #define RMI_HEAD_SKIP 1
 #endif
+#ifndef RMI_SPLIT_WG
+#define RMI_SPLIT_WG 4
+#endif
 #ifndef RMI_TEAM_WG_ONE_TRIP
 #define RMI_TEAM_WG_ONE_TRIP 6
 #endif
@@ -807,6 +810,9 @@ inline int make_plan(const rmi_reduce_desc& d,
       p.B     = 1;
       p.chunk = p.nvec;
     } else {
+      // more pieces than fit at once: four resident workgroups per CU, as for whole rows of
+      // several batches per thread (1 GB of fp32, 500 / 525 / 1800 rows: 82 / 84 / 83 -> 85 / 86 / 86 %)
+      if (RMI_SPLIT_WG < 8 && p.grid_blocks > (int64_t)8 * n_cu) p.lds_reserve = kLdsPerCu / RMI_SPLIT_WG - 768;
       p.ws_bytes   = kTicketBytes + (size_t)p.n_out * p.B * acc_bytes;
       p.fused_fold = (d.flags & RMI_FLAG_WORKSPACE_ZEROED) != 0 &&
                      p.n_out * ticket_lines_per_row(p.B) <= kTicketLines;
