@@ -389,6 +389,12 @@ using norm_fn = int (*)(const NormPlan&, const NormArgs&, hipStream_t);
 template <class P>
 int run_normalize(const NormPlan& pl, const NormArgs& args, hipStream_t st)
 {
+  // fp32 rows: six resident workgroups per CU instead of the eight that fit (an LDS reservation
+  // the kernels never touch): 512 MB in + out, D = 64 / 128 / 256 / 2048 / 4096 78.8 / 78.8 / 78.8 /
+  // 78.4 / 76.7 -> 81.1 / 81.2 / 80.4 / 80.9 / 78.5 % of 8 TB/s, D = 401 / 777 / 1100 +1 to +3; five lose
+  // 1-10 points at D <= 512 and 2048, four and three more; bf16 rows gain and lose by shape
+  // (D = 256 / 16384 -2, D = 2049 / 4096 +1 to +2) and keep eight.
+  const unsigned resident_lds = sizeof(typename P::in_t) == 4 ? (unsigned)(kLdsPerCu / 6 - 768) : 0u;
   NormArgs a = args;
   a.nvec     = pl.nvec;
   a.tail     = pl.tail;
@@ -421,19 +427,19 @@ int run_normalize(const NormPlan& pl, const NormArgs& args, hipStream_t st)
                reinterpret_cast<uintptr_t>(a.out) % 128 == 0) {
       // every store instruction writes whole cache lines (rows of whole lines, or the rows
       // of one wave step together) at an aligned address: streamed stores
-      hipLaunchKernelGGL((normalize_wave_kernel<P, true, true>), grid, dim3(kBlock), 0, st, a);
+      hipLaunchKernelGGL((normalize_wave_kernel<P, true, true>), grid, dim3(kBlock), resident_lds, st, a);
     } else {
-      hipLaunchKernelGGL((normalize_wave_kernel<P, true>), grid, dim3(kBlock), 0, st, a);
+      hipLaunchKernelGGL((normalize_wave_kernel<P, true>), grid, dim3(kBlock), resident_lds, st, a);
     }
   } else if (pl.kind == 1) {
     // rows of 4 KB and more always hold whole vectors
     const dim3 block((unsigned)pl.threads);
     if (pl.hold == 4)
-      hipLaunchKernelGGL((normalize_team_kernel<P, 4>), grid, block, 0, st, a);
+      hipLaunchKernelGGL((normalize_team_kernel<P, 4>), grid, block, resident_lds, st, a);
     else if (pl.hold == 8)
-      hipLaunchKernelGGL((normalize_team_kernel<P, 8>), grid, block, 0, st, a);
+      hipLaunchKernelGGL((normalize_team_kernel<P, 8>), grid, block, resident_lds, st, a);
     else
-      hipLaunchKernelGGL((normalize_team_kernel<P, 16>), grid, block, 0, st, a);
+      hipLaunchKernelGGL((normalize_team_kernel<P, 16>), grid, block, resident_lds, st, a);
   } else {
     hipLaunchKernelGGL((normalize_sweep_kernel<P>), grid, dim3(pl.threads), 0, st, a);
   }
